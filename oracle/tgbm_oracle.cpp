@@ -1,0 +1,1003 @@
+// TEST INFRASTRUCTURE ONLY.
+//
+// CPU restatement of ThunderGBM's single-GPU histogram trainer ("hist_single") and predictor.
+// It is the parity checker for the HIP library and the same-box CPU baseline of the benchmark.
+// Nothing in the shipped library links, loads or calls this file.
+//
+// The reference has no CPU training path (docs/faq.md:10-11) and is CUDA-only, so it cannot be
+// compiled here; every function below restates the algorithm of the cited reference lines.
+// Paths are relative to the reference checkout.
+//
+// What pins each function (tests/test_oracle_*.py):
+//   cut points      closed-form rule on hand inputs, invariants, the a1a fixture (one cut = 1.0 per feature)
+//   bin ids         brute force min(#cuts<=v, k-1) against numpy searchsorted
+//   gradients       float64 closed forms
+//   histogram       brute-force float64 accumulation; bin counts for squared loss
+//   split finding   brute-force enumeration of (feature, bin, direction) in numpy float64
+//   update/partition row counts equal hessian sums for squared loss; raw-value threshold consistency
+//   prune           hand-built 7-node trees
+//   predictor       equality with the training-time prediction on the training rows
+//   metrics         reference KATs src/test/test_metrics.cpp:70,84,96; tree size src/test/test_tree.cpp:68
+// Parity unpinned (no run of the reference is possible): the association order of the reference's
+// fp32 sums (atomics, thrust scan/reduce), device expf ulps, ordering of +0.0/-0.0 duplicates in
+// the cut-point sort.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+namespace {
+
+struct GH {
+    float g, h;
+};
+
+// Layout of Tree::TreeNode, include/thundergbm/tree.h:14-30 (48 bytes).
+struct Node {
+    int final_id, lch, rch, parent;
+    float gain, base_weight;
+    int split_fid;
+    float split_value;
+    unsigned char split_bid;
+    bool default_right, is_leaf, is_valid, is_pruned;
+    GH sum;
+};
+static_assert(sizeof(Node) == 48, "TreeNode must be 48 bytes");
+
+// Per-node best split, the information of SplitPoint in include/thundergbm/builder/shard.h:23-47
+// laid out for the tests (fixed 48 bytes).
+struct Split {
+    float gain;
+    GH missing;
+    GH lch_sum;
+    int default_right;
+    int nid;
+    int fid;
+    float fval;
+    int bid;         // local bin id (split_bid, truncated to unsigned char like the reference)
+    int best_index;  // global bin index of the winning candidate
+    int pad;
+};
+static_assert(sizeof(Split) == 48, "Split must be 48 bytes");
+
+inline float calc_weight(GH s, float lambda) { return -s.g / (s.h + lambda); }
+
+// compute_gain lambda, src/thundergbm/builder/hist_tree_builder_single.cu:282-289
+inline float compute_gain(GH f, GH l, GH r, float mcw, float lambda) {
+    if (l.h >= mcw && r.h >= mcw)
+        return (l.g * l.g) / (l.h + lambda) + (r.g * r.g) / (r.h + lambda) - (f.g * f.g) / (f.h + lambda);
+    return 0.f;
+}
+
+struct Oracle {
+    // data (DataSet, src/thundergbm/dataset.cpp:20-63)
+    int n = 0, F = 0;
+    long nnz = 0;
+    std::vector<float> val;
+    std::vector<int> col, row_ptr;
+    std::vector<float> y;      // mapped to class index for classification
+    std::vector<float> label;  // distinct labels
+    // params (GBMParam, include/thundergbm/common.h:86-111)
+    int depth = 6, n_trees = 40, max_num_bin = 255, num_class = 1, tree_per_rounds = 1;
+    float mcw = 1, lambda = 1, gamma = 1, rt_eps = 1e-6f, lr = 1, base_score = 0;
+    std::string objective = "reg:linear";
+    // cuts (HistCut)
+    std::vector<float> cut_val;
+    std::vector<int> cut_row_ptr, cut_fid;
+    int n_bins = 0;
+    std::vector<int> bin_id;  // global bin id per nnz
+    // training state
+    std::vector<float> y_pred;  // class-major
+    std::vector<GH> gh;         // class-major
+    std::vector<int> nid;
+    std::vector<Node> nodes;
+    std::vector<Split> sp;
+    int cur_class = 0;
+    int cur_level = -1;
+    bool keep_debug = false;
+    bool shadow64 = false;
+    // raw (unscanned) histograms of the current and previous level, node-major
+    std::vector<GH> hist_cur, hist_prev;
+    std::vector<double> hist64_cur, hist64_prev;  // g,h interleaved
+    // debug: per node of the whole tree
+    std::vector<float> dbg_score;   // [n_nodes][n_bins], signed gain of every candidate
+    std::vector<GH> dbg_hist;       // [n_nodes][n_bins], raw hist
+    std::vector<double> dbg_hist64; // [n_nodes][n_bins][2]
+    std::vector<int> dbg_built;     // [n_nodes] 1 if built from rows, 0 if by subtraction
+    std::vector<std::vector<Node>> model;  // iteration-major, class inside
+    std::vector<float> metric_log;
+    long rows_built_total = 0;      // rows visited by histogram builds (for byte accounting)
+    std::vector<long> rows_built_level;
+};
+
+// ---------------------------------------------------------------------------------------------
+// a1  HistCut::get_cut_points_single, src/thundergbm/hist_cut.cu:232-286 (sort/unique :205-228,
+// comparator :196-203, stride selection :259-265 with interval = n_unique / max_num_bins from
+// include/thundergbm/util/device_lambda.cuh:33-42).
+int cut_points(int F, long nnz, const float *val, const int *col, int max_bin, std::vector<float> &cut_val,
+               std::vector<int> &cut_row_ptr, std::vector<int> &cut_fid) {
+    std::vector<long> cnt(F + 1, 0);
+    for (long i = 0; i < nnz; ++i) cnt[col[i] + 1]++;
+    for (int f = 0; f < F; ++f) cnt[f + 1] += cnt[f];
+    std::vector<float> byf(nnz);
+    {
+        std::vector<long> pos(cnt.begin(), cnt.end() - 1);
+        for (long i = 0; i < nnz; ++i) byf[pos[col[i]]++] = val[i];
+    }
+    std::vector<std::vector<float>> per(F);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int f = 0; f < F; ++f) {
+        float *b = byf.data() + cnt[f], *e = byf.data() + cnt[f + 1];
+        if (b == e) continue;
+        std::sort(b, e);
+        e = std::unique(b, e);  // distinct by ==
+        long m = e - b;
+        long step = m / max_bin;
+        std::vector<float> &out = per[f];
+        if (step == 0) {
+            out.assign(b, e);
+        } else {
+            out.reserve(max_bin);
+            for (long j = 0; j < max_bin; ++j) out.push_back(b[j * step]);
+        }
+    }
+    cut_val.clear();
+    cut_fid.clear();
+    cut_row_ptr.assign(F + 1, 0);
+    for (int f = 0; f < F; ++f) {
+        cut_row_ptr[f] = (int)cut_val.size();
+        for (float v : per[f]) {
+            cut_val.push_back(v);
+            cut_fid.push_back(f);
+        }
+    }
+    cut_row_ptr[F] = (int)cut_val.size();
+    return (int)cut_val.size();
+}
+
+// a2  HistTreeBuilder_single::get_bin_ids, hist_tree_builder_single.cu:81-119: upper bound with
+// the right end clamped to the feature's last cut, plus the feature's global offset.
+inline int bin_of(const float *cut_val, const int *cut_row_ptr, int fid, float v) {
+    const float *begin = cut_val + cut_row_ptr[fid];
+    const float *end = cut_val + cut_row_ptr[fid + 1];
+    const float *left = begin, *right = end - 1;
+    while (left < right) {
+        const float *mid = left + (right - left) / 2;
+        if (*mid <= v)
+            left = mid + 1;
+        else
+            right = mid;
+    }
+    return (int)(left - begin) + cut_row_ptr[fid];
+}
+
+// a3  gradients. SquareLoss include/thundergbm/objective/regression_obj.h:130-134, LogisticLoss
+// :145-154, Softmax src/thundergbm/objective/multiclass_obj.cu:6-35.
+void gradient(const std::string &obj, int n, int num_class, const float *y, const float *yp, GH *gh) {
+    if (obj == "reg:linear") {
+#pragma omp parallel for
+        for (int i = 0; i < n; ++i) gh[i] = GH{yp[i] - y[i], 1.f};
+    } else if (obj == "binary:logistic" || obj == "reg:logistic") {
+#pragma omp parallel for
+        for (int i = 0; i < n; ++i) {
+            float p = 1 / (1 + expf(-yp[i]));
+            gh[i] = GH{p - y[i], fmaxf(p * (1 - p), 1e-16f)};
+        }
+    } else {  // multi:softmax / multi:softprob
+#pragma omp parallel for
+        for (int i = 0; i < n; ++i) {
+            float mx = yp[i];
+            for (int k = 1; k < num_class; ++k) mx = fmaxf(mx, yp[(long)k * n + i]);
+            float sum = 0;
+            for (int k = 0; k < num_class; ++k) sum += expf(yp[(long)k * n + i] - mx);
+            for (int k = 0; k < num_class; ++k) {
+                float p = expf(yp[(long)k * n + i] - mx) / sum;
+                float g = (k == y[i]) ? (p - 1) : (p - 0);
+                float h = fmaxf(2 * p * (1 - p), 1e-16f);
+                gh[(long)k * n + i] = GH{g, h};
+            }
+        }
+    }
+}
+
+// DataSet::group_label, src/thundergbm/dataset.cpp:83-101: distinct int-truncated labels in
+// ascending order; y is looked up by its exact float value, unknown keys map to 0.
+void group_label(std::vector<float> &y, std::vector<float> &label) {
+    std::vector<int> t(y.begin(), y.end());
+    std::sort(t.begin(), t.end());
+    t.erase(std::unique(t.begin(), t.end()), t.end());
+    std::map<float, int> m;
+    label.clear();
+    for (int v : t) {
+        m[(float)v] = (int)label.size();
+        label.push_back((float)v);
+    }
+    for (float &v : y) v = (float)m[v];
+}
+
+// a4  Tree::init2, src/thundergbm/tree.cu:8-39
+void tree_init(Oracle &o, int k) {
+    o.cur_class = k;
+    int n_max = (1 << (o.depth + 1)) - 1;
+    o.nodes.assign(n_max, Node{});
+    for (int i = 0; i < n_max; ++i) {
+        Node &nd = o.nodes[i];
+        std::memset(&nd, 0, sizeof(Node));
+        nd.final_id = i;
+        nd.split_fid = -1;
+        nd.is_valid = false;
+        nd.parent = i == 0 ? -1 : (i - 1) / 2;
+        if (i < n_max / 2) {
+            nd.is_leaf = false;
+            nd.lch = 2 * i + 1;
+            nd.rch = 2 * i + 2;
+        } else {
+            nd.is_leaf = true;
+            nd.lch = nd.rch = -1;
+        }
+    }
+    const GH *g = o.gh.data() + (long)k * o.n;
+    // fp32 reduction (the reference's thrust::reduce order is unspecified; pairwise per thread chunk)
+    double sg = 0, sh = 0;
+    float fg = 0, fh = 0;
+    const int CH = 4096;
+    long nch = (o.n + CH - 1) / CH;
+    std::vector<GH> part(nch);
+#pragma omp parallel for
+    for (long c = 0; c < nch; ++c) {
+        float a = 0, b = 0;
+        long e = std::min<long>(o.n, (c + 1) * CH);
+        for (long i = c * CH; i < e; ++i) {
+            a += g[i].g;
+            b += g[i].h;
+        }
+        part[c] = GH{a, b};
+    }
+    for (long c = 0; c < nch; ++c) {
+        fg += part[c].g;
+        fh += part[c].h;
+    }
+    (void)sg;
+    (void)sh;
+    Node &root = o.nodes[0];
+    root.sum = GH{fg, fh};
+    root.is_valid = true;
+    root.base_weight = calc_weight(root.sum, o.lambda);
+    std::fill(o.nid.begin(), o.nid.end(), 0);  // ins2node_id.resize(n) zero-fills, tree_builder.cu:156
+    o.cur_level = -1;
+    if (o.keep_debug) {
+        o.dbg_score.assign((size_t)n_max * o.n_bins, 0.f);
+        o.dbg_hist.assign((size_t)n_max * o.n_bins, GH{0, 0});
+        if (o.shadow64) o.dbg_hist64.assign((size_t)n_max * o.n_bins * 2, 0.0);
+        o.dbg_built.assign(n_max, -1);
+    }
+}
+
+// Histogram of one node from a list of rows (root: rows == nullptr means 0..cnt-1).
+// hist_tree_builder_single.cu:203-216 (root) and :485-505 (node): hist[global_bin] += (g,h) for every
+// stored entry of every row; zero g / zero h contributions are skipped (no effect on the sum).
+void build_hist(Oracle &o, const int *rows, long cnt, GH *out, double *out64) {
+    const int B = o.n_bins;
+    const GH *gh = o.gh.data() + (long)o.cur_class * o.n;
+    int nt = 1;
+#ifdef _OPENMP
+    nt = omp_get_max_threads();
+#endif
+    if (cnt < 4096) nt = 1;
+    std::vector<GH> priv((size_t)nt * B, GH{0, 0});
+    std::vector<double> priv64;
+    if (out64) priv64.assign((size_t)nt * B * 2, 0.0);
+#pragma omp parallel num_threads(nt)
+    {
+        int t = 0;
+#ifdef _OPENMP
+        t = omp_get_thread_num();
+#endif
+        GH *h = priv.data() + (size_t)t * B;
+        double *h64 = out64 ? priv64.data() + (size_t)t * B * 2 : nullptr;
+        long b = cnt * t / nt, e = cnt * (t + 1) / nt;
+        for (long r = b; r < e; ++r) {
+            int i = rows ? rows[r] : (int)r;
+            GH s = gh[i];
+            for (int j = o.row_ptr[i]; j < o.row_ptr[i + 1]; ++j) {
+                int bid = o.bin_id[j];
+                h[bid].g += s.g;
+                h[bid].h += s.h;
+                if (h64) {
+                    h64[2 * bid] += (double)s.g;
+                    h64[2 * bid + 1] += (double)s.h;
+                }
+            }
+        }
+    }
+    for (int b = 0; b < B; ++b) {
+        float g = 0, h = 0;
+        for (int t = 0; t < nt; ++t) {
+            g += priv[(size_t)t * B + b].g;
+            h += priv[(size_t)t * B + b].h;
+        }
+        out[b] = GH{g, h};
+    }
+    if (out64)
+        for (int b = 0; b < 2 * B; ++b) {
+            double s = 0;
+            for (int t = 0; t < nt; ++t) s += priv64[(size_t)t * B * 2 + b];
+            out64[b] = s;
+        }
+    o.rows_built_total += cnt;
+}
+
+// Scan + missing + gain + argmax + record for one node given its raw histogram.
+// hist_tree_builder_single.cu:257-390 (root) / :614-752 (pair member).
+void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
+    const int B = o.n_bins, F = o.F;
+    const Node &nd = o.nodes[node];
+    if (!nd.is_valid) {
+        std::memset(&s, 0, sizeof(Split));
+        s.fid = -1;
+        s.nid = -1;
+        return;
+    }
+    std::vector<GH> pre(B);
+    std::vector<GH> miss(F, GH{0, 0});
+    const GH S = nd.sum;
+    // inclusive_scan_by_key over cut_fid (:257, :614): fp32 running sums restarting per feature
+    for (int f = 0; f < F; ++f) {
+        float g = 0, h = 0;
+        for (int b = o.cut_row_ptr[f]; b < o.cut_row_ptr[f + 1]; ++b) {
+            g += raw[b].g;
+            h += raw[b].h;
+            pre[b] = GH{g, h};
+        }
+        // missing_gh (:265-274): only for splittable nodes and features with at least one cut
+        if (!nd.is_leaf && o.cut_row_ptr[f + 1] != o.cut_row_ptr[f]) {
+            GH last = pre[o.cut_row_ptr[f + 1] - 1];
+            miss[f] = GH{S.g - last.g, S.h - last.h};
+        }
+    }
+    int best = 0;
+    float best_score = 0;
+    bool first = true;
+    float *dbg = o.keep_debug ? o.dbg_score.data() + (size_t)node * B : nullptr;
+    for (int b = 0; b < B; ++b) {
+        int f = o.cut_fid[b];
+        GH l = GH{0, 0};
+        if (o.cut_row_ptr[f] != b) l = pre[b - 1];
+        GH r = GH{S.g - l.g, S.h - l.h};
+        float gr = fmaxf(0.f, compute_gain(S, l, r, o.mcw, o.lambda));
+        GH l2 = GH{l.g + miss[f].g, l.h + miss[f].h};
+        GH r2 = GH{S.g - l2.g, S.h - l2.h};
+        float gl = fmaxf(0.f, compute_gain(S, l2, r2, o.mcw, o.lambda));
+        float score = (gl > gr) ? gl : -gr;
+        if (dbg) dbg[b] = score;
+        // arg_abs_max (:330-335): larger |gain| wins, ties keep the smaller index
+        if (first || fabsf(score) > fabsf(best_score)) {
+            best = b;
+            best_score = score;
+            first = false;
+        }
+    }
+    std::memset(&s, 0, sizeof(Split));
+    if (B == 0) {  // no candidate at all: behaves as a zero-gain split point
+        s.nid = node;
+        s.fid = -1;
+        return;
+    }
+    int f = o.cut_fid[best];
+    s.fid = f;
+    s.nid = node;
+    s.gain = fabsf(best_score);
+    s.bid = (int)(unsigned char)(best - o.cut_row_ptr[f]);
+    s.missing = miss[f];
+    s.default_right = best_score < 0;
+    s.lch_sum = GH{0, 0};
+    float c0 = o.cut_val[o.cut_row_ptr[f]];
+    s.fval = (float)((double)(c0 - fabsf(c0)) - 1e-5);  // :383
+    if (best != o.cut_row_ptr[f]) {
+        s.lch_sum = pre[best - 1];
+        s.fval = o.cut_val[best - 1];
+    }
+    s.best_index = best;
+}
+
+void stash_debug(Oracle &o, int node, const GH *raw, const double *raw64, int built) {
+    if (!o.keep_debug) return;
+    std::copy(raw, raw + o.n_bins, o.dbg_hist.begin() + (size_t)node * o.n_bins);
+    if (o.shadow64 && raw64)
+        std::copy(raw64, raw64 + 2 * o.n_bins, o.dbg_hist64.begin() + (size_t)node * o.n_bins * 2);
+    o.dbg_built[node] = built;
+}
+
+// a5/a6  HistTreeBuilder_single::find_split, hist_tree_builder_single.cu:132-780
+void find_split(Oracle &o, int level) {
+    const int B = o.n_bins;
+    const int n_level = 1 << level;
+    const int off = n_level - 1;
+    o.sp.assign(n_level, Split{});
+    std::swap(o.hist_cur, o.hist_prev);
+    std::swap(o.hist64_cur, o.hist64_prev);
+    o.hist_cur.assign((size_t)n_level * B, GH{0, 0});
+    if (o.shadow64) o.hist64_cur.assign((size_t)n_level * B * 2, 0.0);
+    long built_rows_before = o.rows_built_total;
+    if (level == 0) {
+        build_hist(o, nullptr, o.n, o.hist_cur.data(), o.shadow64 ? o.hist64_cur.data() : nullptr);
+        stash_debug(o, 0, o.hist_cur.data(), o.shadow64 ? o.hist64_cur.data() : nullptr, 1);
+        evaluate_node(o, 0, o.hist_cur.data(), o.sp[0]);
+    } else {
+        // rows of every node of this level in ascending row order (stable radix sort by node id,
+        // :401-412)
+        std::vector<int> ptr(n_level + 1, 0);
+        for (int i = 0; i < o.n; ++i) {
+            int x = o.nid[i] - off;
+            if (x >= 0 && x < n_level) ptr[x + 1]++;
+        }
+        for (int x = 0; x < n_level; ++x) ptr[x + 1] += ptr[x];
+        std::vector<int> idx(ptr[n_level]);
+        {
+            std::vector<int> pos(ptr.begin(), ptr.end() - 1);
+            for (int i = 0; i < o.n; ++i) {
+                int x = o.nid[i] - off;
+                if (x >= 0 && x < n_level) idx[pos[x]++] = i;
+            }
+        }
+        for (int p = 0; p < n_level / 2; ++p) {
+            int a = 2 * p, b = 2 * p + 1;  // compute a, subtract b
+            int nl = ptr[a + 1] - ptr[a], nr = ptr[b + 1] - ptr[b];
+            if (std::max(nl, nr) == 0) {
+                // :454-465. Both siblings empty: invalid nodes are flagged. A valid pair without rows
+                // cannot occur (a split with an empty side has zero gain); it is flagged too instead
+                // of reproducing the reference's zero-initialised SplitPoint (which addresses node 0).
+                for (int j = 0; j < 2; ++j) {
+                    o.sp[2 * p + j].nid = -1;
+                    o.sp[2 * p + j].fid = -1;
+                }
+                continue;
+            }
+            if (nl > nr) std::swap(a, b);  // build the one with fewer rows, ties build the left one
+            GH *ha = o.hist_cur.data() + (size_t)a * B;
+            GH *hb = o.hist_cur.data() + (size_t)b * B;
+            double *ha64 = o.shadow64 ? o.hist64_cur.data() + (size_t)a * B * 2 : nullptr;
+            double *hb64 = o.shadow64 ? o.hist64_cur.data() + (size_t)b * B * 2 : nullptr;
+            build_hist(o, idx.data() + ptr[a], ptr[a + 1] - ptr[a], ha, ha64);
+            const GH *par = o.hist_prev.data() + (size_t)p * B;  // raw parent histogram (:526-540)
+            for (int i = 0; i < B; ++i) hb[i] = GH{par[i].g - ha[i].g, par[i].h - ha[i].h};
+            if (o.shadow64) {
+                const double *par64 = o.hist64_prev.data() + (size_t)p * B * 2;
+                for (int i = 0; i < 2 * B; ++i) hb64[i] = par64[i] - ha64[i];
+            }
+            stash_debug(o, off + a, ha, ha64, 1);
+            stash_debug(o, off + b, hb, hb64, 0);
+            evaluate_node(o, off + 2 * p, o.hist_cur.data() + (size_t)(2 * p) * B, o.sp[2 * p]);
+            evaluate_node(o, off + 2 * p + 1, o.hist_cur.data() + (size_t)(2 * p + 1) * B, o.sp[2 * p + 1]);
+        }
+    }
+    if ((int)o.rows_built_level.size() <= level) o.rows_built_level.resize(level + 1, 0);
+    o.rows_built_level[level] += o.rows_built_total - built_rows_before;
+    o.cur_level = level;
+}
+
+// a7  HistTreeBuilder_single::update_tree, hist_tree_builder_single.cu:847-902
+void update_tree(Oracle &o) {
+    for (size_t i = 0; i < o.sp.size(); ++i) {
+        const Split &s = o.sp[i];
+        if (s.gain > o.rt_eps) {
+            if (s.nid == -1) continue;
+            Node &nd = o.nodes[s.nid];
+            nd.gain = s.gain;
+            Node &l = o.nodes[nd.lch];
+            Node &r = o.nodes[nd.rch];
+            l.is_valid = true;
+            r.is_valid = true;
+            nd.split_fid = s.fid;
+            nd.split_value = s.fval;
+            nd.split_bid = (unsigned char)s.bid;
+            l.sum = s.lch_sum;
+            if (!s.default_right) {
+                l.sum = GH{l.sum.g + s.missing.g, l.sum.h + s.missing.h};
+                nd.default_right = false;
+            } else {
+                nd.default_right = true;
+            }
+            r.sum = GH{nd.sum.g - l.sum.g, nd.sum.h - l.sum.h};
+            l.base_weight = calc_weight(l.sum, o.lambda);
+            r.base_weight = calc_weight(r.sum, o.lambda);
+        } else {
+            if (s.nid == -1) continue;
+            Node &nd = o.nodes[s.nid];
+            nd.is_leaf = true;
+            o.nodes[nd.lch].is_valid = false;
+            o.nodes[nd.rch].is_valid = false;
+        }
+    }
+}
+
+// a8  HistTreeBuilder_single::update_ins2node_id, hist_tree_builder_single.cu:908-1020. The
+// reference's bounded binary search (:941-966) finds the row's stored bin that lies in the split
+// feature's bin range; rows must have ascending column indices.
+int update_ins2node(Oracle &o) {
+    int has_split = 0;
+#pragma omp parallel for reduction(| : has_split)
+    for (int i = 0; i < o.n; ++i) {
+        int x = o.nid[i];
+        const Node &nd = o.nodes[x];
+        int f = nd.split_fid;
+        if (!nd.is_leaf && nd.is_valid && f >= 0 && f < o.F) {
+            has_split |= 1;
+            int cb = o.cut_row_ptr[f], ce = o.cut_row_ptr[f + 1];
+            int split_bid = (int)nd.split_bid + cb;
+            long lo = o.row_ptr[i], hi = o.row_ptr[i + 1];
+            int bid = -1;
+            long prev = -1;
+            while (lo != hi) {
+                long mid = lo + (hi - lo) / 2;
+                if (mid == prev) break;
+                prev = mid;
+                int t = o.bin_id[mid];
+                if (t >= cb && t < ce) {
+                    bid = t;
+                    break;
+                } else if (t < cb)
+                    lo = mid;
+                else
+                    hi = mid;
+            }
+            bool to_left = true;
+            if ((bid == -1 && nd.default_right) || (bid >= split_bid && bid >= 0)) to_left = false;
+            o.nid[i] = to_left ? nd.lch : nd.rch;
+        }
+    }
+    return has_split;
+}
+
+// a9  Tree::prune_self, src/thundergbm/tree.cu:85-128
+int try_prune_leaf(std::vector<Node> &nodes, int x, int np, float gamma, std::vector<int> &cnt) {
+    int p = nodes[x].parent;
+    if (p == -1) return np;
+    Node &pn = nodes[p];
+    Node &l = nodes[pn.lch];
+    Node &r = nodes[pn.rch];
+    cnt[p]++;
+    if (cnt[p] >= 2 && pn.gain < gamma) {
+        l.is_pruned = true;
+        r.is_pruned = true;
+        pn.is_leaf = true;
+        return try_prune_leaf(nodes, p, np + 2, gamma, cnt);
+    }
+    return np;
+}
+
+int prune(std::vector<Node> &nodes, float gamma) {
+    std::vector<int> cnt(nodes.size(), 0);
+    int np = 0;
+    for (size_t i = 0; i < nodes.size(); ++i)
+        if (nodes[i].is_leaf && nodes[i].is_valid) np = try_prune_leaf(nodes, (int)i, np, gamma, cnt);
+    int id = 0;
+    for (size_t i = 0; i < nodes.size(); ++i)
+        if (nodes[i].is_valid && !nodes[i].is_pruned) nodes[i].final_id = id++;
+    return np;
+}
+
+// a10  TreeBuilder::predict_in_training, src/thundergbm/builder/tree_builder.cu:62-74
+void predict_in_training(Oracle &o, int k) {
+    float *yp = o.y_pred.data() + (long)k * o.n;
+#pragma omp parallel for
+    for (int i = 0; i < o.n; ++i) {
+        int x = o.nid[i];
+        while (x != -1 && o.nodes[x].is_pruned) x = o.nodes[x].parent;
+        yp[i] += o.lr * o.nodes[x].base_weight;
+    }
+}
+
+// a12  metrics: RMSE src/thundergbm/metric/pointwise_metric.cu:8-22, accuracy / error
+// src/thundergbm/metric/multiclass_metric.cu:9-46
+float metric(const std::string &obj, int n, int num_class, const float *y, const float *yp) {
+    if (obj == "reg:linear" || obj == "reg:logistic") {
+        float s = 0;
+        for (int i = 0; i < n; ++i) {
+            float e = yp[i] - y[i];
+            s += e * e;
+        }
+        return sqrtf(s / n);
+    }
+    if (obj == "binary:logistic") {
+        int t = 0;
+        for (int i = 0; i < n; ++i) {
+            int k = (1 / (1 + exp(-(double)yp[i])) > 0.5) ? 1 : 0;
+            t += (k == y[i]);
+        }
+        float acc = t / (float)n;
+        return 1 - acc;
+    }
+    int t = 0;
+    for (int i = 0; i < n; ++i) {
+        int mk = 0;
+        float mp = yp[i];
+        for (int k = 1; k < num_class; ++k)
+            if (yp[(long)k * n + i] > mp) {
+                mp = yp[(long)k * n + i];
+                mk = k;
+            }
+        t += (mk == y[i]);
+    }
+    return t / (float)n;
+}
+
+// a3b  init_base_score, regression_obj.h:35-53 / :95-114, called from booster.h:66-73
+void init_base_score(Oracle &o) {
+    if (o.objective == "reg:linear" || o.objective == "reg:logistic" || o.objective == "binary:logistic") {
+        gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+        float sg = 0, sh = 0;
+        const int CH = 4096;
+        for (long c = 0; c < o.n; c += CH) {
+            float a = 0, b = 0;
+            for (long i = c; i < std::min<long>(o.n, c + CH); ++i) {
+                a += o.gh[i].g;
+                b += o.gh[i].h;
+            }
+            sg += a;
+            sh += b;
+        }
+        float w = (float)(-sg / fmax((double)sh, 1e-6));
+        if (o.objective == "binary:logistic") {
+            w = 1 / (1 + expf(-w));
+            o.base_score = -logf(1.0f / w - 1.0f);
+        } else {
+            o.base_score = w;
+        }
+        std::fill(o.y_pred.begin(), o.y_pred.end(), o.base_score);
+    } else {
+        o.base_score = 0;  // objective_function.h:21-24: not implemented for softmax
+    }
+}
+
+// a11  TreeBuilder::build_approximate, tree_builder.cu:147-194
+void build_tree(Oracle &o, int k) {
+    tree_init(o, k);
+    for (int level = 0; level < o.depth; ++level) {
+        find_split(o, level);
+        update_tree(o);
+        if (!update_ins2node(o)) break;
+    }
+    prune(o.nodes, o.gamma);
+    predict_in_training(o, k);
+}
+
+// Booster::boost, include/thundergbm/booster.h:76-93
+void boost_round(Oracle &o) {
+    gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+    std::vector<Node> round_trees;
+    for (int k = 0; k < o.tree_per_rounds; ++k) {
+        build_tree(o, k);
+        round_trees.insert(round_trees.end(), o.nodes.begin(), o.nodes.end());
+    }
+    o.model.push_back(round_trees);
+    o.metric_log.push_back(metric(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data()));
+}
+
+// a13  Predictor::predict_raw, src/thundergbm/predictor.cu:32-189. double accumulation when the
+// dense shared-memory path would be taken (n_features * 128 * 4 <= 48 KB), float otherwise.
+void predict_raw(int n, int F, const float *val, const int *row_ptr, const int *col, const Node *model, int n_iter,
+                 int n_class_trees, int n_nodes, float lr, float base_score, float *out) {
+    if (n_class_trees > 1) base_score = 0;
+    bool dense_path = (size_t)F * 128 * sizeof(float) <= 48 * 1024;
+#pragma omp parallel for
+    for (int i = 0; i < n; ++i) {
+        const int *ci = col + row_ptr[i];
+        const float *cv = val + row_ptr[i];
+        int len = row_ptr[i + 1] - row_ptr[i];
+        for (int t = 0; t < n_class_trees; ++t) {
+            double sd = base_score;
+            float sf = base_score;
+            for (int it = 0; it < n_iter; ++it) {
+                const Node *nd = model + ((size_t)it * n_class_trees + t) * n_nodes;
+                int cur = 0;
+                while (!nd[cur].is_leaf) {
+                    int f = nd[cur].split_fid;
+                    const int *p = std::lower_bound(ci, ci + len, f);
+                    if (p != ci + len && *p == f) {
+                        float v = cv[p - ci];
+                        cur = v < nd[cur].split_value ? nd[cur].lch : nd[cur].rch;
+                    } else {
+                        cur = nd[cur].default_right ? nd[cur].rch : nd[cur].lch;
+                    }
+                }
+                sd += lr * nd[cur].base_weight;  // float product promoted to double (:126)
+                sf += lr * nd[cur].base_weight;
+            }
+            out[(size_t)t * n + i] += dense_path ? (float)sd : sf;
+        }
+    }
+}
+
+// a14  predict_transform: regression_obj.h:27-32 / :76-92, multiclass_obj.cu:44-88.
+// Returns the number of outputs.
+long predict_transform(const std::string &obj, int n, int num_class, const float *label, float *y) {
+    if (obj == "binary:logistic") {
+        for (int i = 0; i < n; ++i) y[i] = label[y[i] > 0 ? 1 : 0];
+        return n;
+    }
+    if (obj == "multi:softmax") {
+        int nc = num_class == 2 ? 1 : num_class;
+        for (int i = 0; i < n; ++i) {
+            int mk = 0;
+            float mp = y[i];
+            for (int k = 1; k < nc; ++k)
+                if (mp < y[(long)k * n + i]) {
+                    mp = y[(long)k * n + i];
+                    mk = k;
+                }
+            y[i] = label[mk];
+        }
+        return n;
+    }
+    if (obj == "multi:softprob") {
+        for (int i = 0; i < n; ++i) {
+            float mx = y[i];
+            for (int k = 1; k < num_class; ++k) mx = fmaxf(mx, y[(long)k * n + i]);
+            float sum = 0;
+            for (int k = 0; k < num_class; ++k) {
+                y[(long)k * n + i] = expf(y[(long)k * n + i] - mx);
+                sum += y[(long)k * n + i];
+            }
+            for (int k = 0; k < num_class; ++k) y[(long)k * n + i] /= sum;
+        }
+        return (long)n * num_class;
+    }
+    if (obj == "reg:logistic") {
+        for (int i = 0; i < n; ++i) y[i] = 1 / (1 + expf(-y[i]));
+        return n;
+    }
+    return n;  // reg:linear identity
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------
+extern "C" {
+
+// DataSet::load_from_sparse (dataset.cpp:20-63) + the class bookkeeping of TreeTrainer::train
+// (trainer.cu:24-37).
+void *orc_create(int n, const float *val, const int *row_ptr, const int *col, const float *y, int depth, int n_trees,
+                 float min_child_weight, float lambda, float gamma, int max_num_bin, float learning_rate,
+                 const char *objective, int num_class) {
+    Oracle *o = new Oracle;
+    o->n = n;
+    o->nnz = row_ptr[n];
+    o->val.assign(val, val + o->nnz);
+    o->col.assign(col, col + o->nnz);
+    o->row_ptr.assign(row_ptr, row_ptr + n + 1);
+    o->y.assign(y, y + n);
+    int mx = 0;
+    for (long i = 0; i < o->nnz; ++i) mx = std::max(mx, col[i]);
+    o->F = mx + 1;
+    o->depth = depth;
+    o->n_trees = n_trees;
+    o->mcw = min_child_weight;
+    o->lambda = lambda;
+    o->gamma = gamma;
+    o->max_num_bin = max_num_bin;
+    o->lr = learning_rate;
+    o->objective = objective;
+    o->num_class = num_class;
+    o->tree_per_rounds = 1;
+    bool grouped = o->objective == "multi:softprob" || o->objective == "multi:softmax" ||
+                   o->objective == "binary:logistic";
+    if (grouped) {
+        group_label(o->y, o->label);
+        o->num_class = (int)o->label.size();
+        if (o->num_class > 2) o->tree_per_rounds = o->num_class;
+    } else if (o->objective.find("reg:") != std::string::npos) {
+        o->num_class = 1;
+    }
+    return o;
+}
+
+void orc_destroy(void *h) { delete (Oracle *)h; }
+
+void orc_set_debug(void *h, int keep_debug, int shadow64) {
+    Oracle *o = (Oracle *)h;
+    o->keep_debug = keep_debug;
+    o->shadow64 = shadow64;
+}
+
+// HistTreeBuilder_single::init (:783-844) + Booster::init (booster.h:36-74)
+void orc_prepare(void *h) {
+    Oracle &o = *(Oracle *)h;
+    o.n_bins = cut_points(o.F, o.nnz, o.val.data(), o.col.data(), o.max_num_bin, o.cut_val, o.cut_row_ptr, o.cut_fid);
+    o.bin_id.resize(o.nnz);
+#pragma omp parallel for
+    for (long i = 0; i < o.nnz; ++i) o.bin_id[i] = bin_of(o.cut_val.data(), o.cut_row_ptr.data(), o.col[i], o.val[i]);
+    long n_out = (long)o.num_class * o.n;
+    if (o.num_class == 2) n_out = o.n;
+    o.y_pred.assign(n_out, 0.f);
+    o.gh.assign((long)o.num_class * o.n, GH{0, 0});
+    o.nid.assign(o.n, 0);
+    init_base_score(o);
+}
+
+void orc_boost(void *h, int rounds) {
+    Oracle &o = *(Oracle *)h;
+    for (int r = 0; r < rounds; ++r) boost_round(o);
+}
+
+// step-wise driving for lock-step tests
+void orc_compute_gradient(void *h) {
+    Oracle &o = *(Oracle *)h;
+    gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+}
+void orc_tree_init(void *h, int k) { tree_init(*(Oracle *)h, k); }
+void orc_find_split(void *h, int level) { find_split(*(Oracle *)h, level); }
+void orc_update_tree(void *h) { update_tree(*(Oracle *)h); }
+int orc_update_ins2node(void *h) { return update_ins2node(*(Oracle *)h); }
+int orc_prune(void *h) {
+    Oracle &o = *(Oracle *)h;
+    return prune(o.nodes, o.gamma);
+}
+void orc_predict_in_training(void *h, int k) { predict_in_training(*(Oracle *)h, k); }
+void orc_build_tree(void *h, int k) { build_tree(*(Oracle *)h, k); }
+float orc_metric(void *h) {
+    Oracle &o = *(Oracle *)h;
+    return metric(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data());
+}
+
+// getters / setters
+int orc_n_features(void *h) { return ((Oracle *)h)->F; }
+int orc_n_bins(void *h) { return ((Oracle *)h)->n_bins; }
+int orc_num_class(void *h) { return ((Oracle *)h)->num_class; }
+int orc_tree_per_rounds(void *h) { return ((Oracle *)h)->tree_per_rounds; }
+int orc_n_labels(void *h) { return (int)((Oracle *)h)->label.size(); }
+float orc_base_score(void *h) { return ((Oracle *)h)->base_score; }
+int orc_n_nodes(void *h) { return (1 << (((Oracle *)h)->depth + 1)) - 1; }
+long orc_rows_built(void *h) { return ((Oracle *)h)->rows_built_total; }
+void orc_get_labels(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.label.begin(), o.label.end(), out);
+}
+void orc_get_y(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.y.begin(), o.y.end(), out);
+}
+void orc_get_cuts(void *h, float *cut_val, int *cut_row_ptr, int *cut_fid) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.cut_val.begin(), o.cut_val.end(), cut_val);
+    std::copy(o.cut_row_ptr.begin(), o.cut_row_ptr.end(), cut_row_ptr);
+    std::copy(o.cut_fid.begin(), o.cut_fid.end(), cut_fid);
+}
+void orc_get_bin_ids(void *h, int *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.bin_id.begin(), o.bin_id.end(), out);
+}
+long orc_y_pred_size(void *h) { return (long)((Oracle *)h)->y_pred.size(); }
+void orc_get_y_pred(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.y_pred.begin(), o.y_pred.end(), out);
+}
+void orc_set_y_pred(void *h, const float *in) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(in, in + o.y_pred.size(), o.y_pred.begin());
+}
+void orc_get_gh(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(out, o.gh.data(), o.gh.size() * sizeof(GH));
+}
+void orc_set_gh(void *h, const float *in) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(o.gh.data(), in, o.gh.size() * sizeof(GH));
+}
+void orc_get_nid(void *h, int *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.nid.begin(), o.nid.end(), out);
+}
+void orc_set_nid(void *h, const int *in) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(in, in + o.n, o.nid.begin());
+}
+void orc_get_nodes(void *h, void *out) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(out, o.nodes.data(), o.nodes.size() * sizeof(Node));
+}
+void orc_set_nodes(void *h, const void *in) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(o.nodes.data(), in, o.nodes.size() * sizeof(Node));
+}
+int orc_get_splits(void *h, void *out) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(out, o.sp.data(), o.sp.size() * sizeof(Split));
+    return (int)o.sp.size();
+}
+// raw histogram of node `node_in_level` of the level last passed to orc_find_split
+void orc_get_level_hist(void *h, int node_in_level, float *out, double *out64) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(out, o.hist_cur.data() + (size_t)node_in_level * o.n_bins, o.n_bins * sizeof(GH));
+    if (out64 && o.shadow64)
+        std::memcpy(out64, o.hist64_cur.data() + (size_t)node_in_level * o.n_bins * 2, o.n_bins * 2 * sizeof(double));
+}
+// debug views of the current tree (need orc_set_debug(keep_debug=1) before orc_tree_init)
+void orc_get_tree_scores(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.dbg_score.begin(), o.dbg_score.end(), out);
+}
+void orc_get_tree_hists(void *h, float *out, double *out64, int *built) {
+    Oracle &o = *(Oracle *)h;
+    std::memcpy(out, o.dbg_hist.data(), o.dbg_hist.size() * sizeof(GH));
+    if (out64 && o.shadow64) std::copy(o.dbg_hist64.begin(), o.dbg_hist64.end(), out64);
+    if (built) std::copy(o.dbg_built.begin(), o.dbg_built.end(), built);
+}
+int orc_model_size(void *h) { return (int)((Oracle *)h)->model.size(); }
+void orc_get_model(void *h, void *out) {
+    Oracle &o = *(Oracle *)h;
+    char *p = (char *)out;
+    for (auto &r : o.model) {
+        std::memcpy(p, r.data(), r.size() * sizeof(Node));
+        p += r.size() * sizeof(Node);
+    }
+}
+int orc_get_metric_log(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.metric_log.begin(), o.metric_log.end(), out);
+    return (int)o.metric_log.size();
+}
+int orc_get_rows_built_level(void *h, long *out, int cap) {
+    Oracle &o = *(Oracle *)h;
+    int m = std::min<int>(cap, (int)o.rows_built_level.size());
+    std::copy(o.rows_built_level.begin(), o.rows_built_level.begin() + m, out);
+    return m;
+}
+
+// ---- stateless entry points ------------------------------------------------------------------
+int orc_cut_points(int F, long nnz, const float *val, const int *col, int max_bin, float *cut_val, int *cut_row_ptr,
+                   int *cut_fid) {
+    std::vector<float> cv;
+    std::vector<int> crp, cf;
+    int nb = cut_points(F, nnz, val, col, max_bin, cv, crp, cf);
+    std::copy(cv.begin(), cv.end(), cut_val);
+    std::copy(crp.begin(), crp.end(), cut_row_ptr);
+    std::copy(cf.begin(), cf.end(), cut_fid);
+    return nb;
+}
+void orc_bin_ids(long nnz, const float *val, const int *col, const float *cut_val, const int *cut_row_ptr, int *out) {
+#pragma omp parallel for
+    for (long i = 0; i < nnz; ++i) out[i] = bin_of(cut_val, cut_row_ptr, col[i], val[i]);
+}
+void orc_gradient(const char *objective, int n, int num_class, const float *y, const float *yp, float *gh) {
+    gradient(objective, n, num_class, y, yp, (GH *)gh);
+}
+float orc_metric_score(const char *objective, int n, int num_class, const float *y, const float *yp) {
+    return metric(objective, n, num_class, y, yp);
+}
+int orc_prune_nodes(void *nodes, int n_nodes, float gamma) {
+    std::vector<Node> v((Node *)nodes, (Node *)nodes + n_nodes);
+    int np = prune(v, gamma);
+    std::memcpy(nodes, v.data(), n_nodes * sizeof(Node));
+    return np;
+}
+void orc_group_label(int n, float *y, float *label_out, int *n_label) {
+    std::vector<float> yy(y, y + n), lab;
+    group_label(yy, lab);
+    std::copy(yy.begin(), yy.end(), y);
+    std::copy(lab.begin(), lab.end(), label_out);
+    *n_label = (int)lab.size();
+}
+void orc_predict_raw(int n, int F, const float *val, const int *row_ptr, const int *col, const void *model,
+                     int n_iter, int n_class_trees, int n_nodes, float lr, float base_score, float *out) {
+    predict_raw(n, F, val, row_ptr, col, (const Node *)model, n_iter, n_class_trees, n_nodes, lr, base_score, out);
+}
+long orc_predict_transform(const char *objective, int n, int num_class, const float *label, float *y) {
+    return predict_transform(objective, n, num_class, label, y);
+}
+int orc_num_threads() {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+}
