@@ -1,0 +1,132 @@
+/*
+ * C ABI of libthundergbm.so (MI355X build).
+ *
+ * Part 1 is the drop-in boundary: the nine entry points that the reference's Python wrapper
+ * (python/thundergbm/thundergbm.py) binds with ctypes, with the argument order, types and
+ * ownership rules of src/thundergbm/scikit_tgbm.cpp. Where the reference declares `Tree *&model`
+ * the ABI passes the address of an 8-byte slot; it is spelled `tgbm_model **` here. The model is
+ * opaque, owned by the library and released only by model_free().
+ *
+ * Part 2 is a session API over the same trainer for callers that keep data resident in HBM between
+ * calls (the benchmark) or drive the stages one by one (the parity tests).
+ *
+ * Failures abort the process after printing a FATAL line, as the reference's CHECK macros do.
+ * The library is not re-entrant; one call trains on one GPU and blocks until done.
+ */
+#ifndef THUNDERGBM_H
+#define THUNDERGBM_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tgbm_model tgbm_model;
+
+/* ---------------------------------------------------------------- Part 1: reference boundary */
+
+/* scikit_tgbm.cpp:13-23. verbose 0 = silent, 1 = info, 2 = debug. */
+void set_logger(int verbose);
+
+/* scikit_tgbm.cpp:26-80. CSR input (float32 values, int32 indices, ascending columns per row).
+ * num_class is in/out, group_label receives the distinct labels (caller allocates one float per
+ * distinct label), tree_per_iter and *model are outputs. n_device, bagging, column_sampling_rate,
+ * n_parallel_trees, group and num_group are accepted for signature compatibility and ignored. */
+void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *label, int depth, int n_trees,
+                         int n_device, float min_child_weight, float lambda, float gamma, int max_num_bin,
+                         int verbose, float column_sampling_rate, int bagging, int n_parallel_trees,
+                         float learning_rate, char *obj_type, int *num_class, char *tree_method, tgbm_model **model,
+                         int *tree_per_iter, float *group_label, int *group, int num_group);
+
+/* scikit_tgbm.cpp:83-121. y_pred: row_size floats, or row_size * num_class (class-major) for
+ * multi:softprob. As in the reference the base score is not part of this path. */
+void sparse_predict_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *y_pred, tgbm_model **model,
+                           int n_trees, int trees_per_iter, char *objective, int num_class, float learning_rate,
+                           float *group_label, int *group, int num_group, int verbose);
+
+/* scikit_tgbm.cpp:123-147 / parser.cpp:146-171: raw binary model file. */
+void save(char *model_path, char *objective, float learning_rate, int num_class, int n_trees, int trees_per_iter,
+          tgbm_model **model, float *group_label);
+
+/* scikit_tgbm.cpp:148-172 / parser.cpp:102-145. */
+void load_model(char *model_path, float *learning_rate, int *num_class, int *n_trees, int *trees_per_iter,
+                tgbm_model **model);
+
+/* scikit_tgbm.cpp:173-182: the label table of a model file. */
+void load_config(char *model_path, float *group_label);
+
+/* scikit_tgbm.cpp:184-197: node count of every tree (all 2^(depth+1)-1 heap slots). */
+void get_n_nodes(tgbm_model **model, int *n_nodes, int n_trees, int tree_per_iter);
+
+/* scikit_tgbm.cpp:199-248: one tree as parallel arrays in heap order. */
+void get_a_tree(tgbm_model **model, int tree_id, int n_nodes, int *children_left, int *children_right,
+                int *children_default, int *features, float *thresholds, float *values,
+                float *node_sample_weights);
+
+/* scikit_tgbm.cpp:250-254. */
+void model_free(tgbm_model **model);
+
+/* ------------------------------------------------------------------- Part 2: session API */
+
+typedef struct tgbm_trainer tgbm_trainer;
+
+/* DataSet::load_from_sparse + HistTreeBuilder_single::init + Booster::init
+ * (dataset.cpp:20-63, hist_tree_builder_single.cu:783-844, booster.h:36-74): copies the CSR input
+ * to the GPU, builds cut points, the bin matrix and the base score. */
+tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
+                                  const float *label, int depth, int n_trees, float min_child_weight, float lambda,
+                                  float gamma, int max_num_bin, float learning_rate, const char *objective,
+                                  int num_class, int verbose);
+void tgbm_trainer_destroy(tgbm_trainer *t);
+
+/* `rounds` iterations of Booster::boost (booster.h:76-93); returns after the GPU finished. */
+void tgbm_trainer_boost(tgbm_trainer *t, int rounds);
+
+/* Stage-wise driving; each call returns after enqueueing (tgbm_trainer_get synchronises).
+ * gradient = ObjectiveFunction::get_gradient; tree_init = Tree::init2; find_split = find_split +
+ * update_tree of the level; partition = update_ins2node_id; finish_tree = prune_self +
+ * predict_in_training. */
+void tgbm_trainer_gradient(tgbm_trainer *t);
+void tgbm_trainer_tree_init(tgbm_trainer *t, int class_id);
+void tgbm_trainer_find_split(tgbm_trainer *t, int level);
+void tgbm_trainer_partition(tgbm_trainer *t, int level);
+void tgbm_trainer_finish_tree(tgbm_trainer *t, int class_id);
+float tgbm_trainer_metric(tgbm_trainer *t);
+
+/* Integer facts: n, n_features, n_bins, num_class, tree_per_rounds, n_nodes, dense_W,
+ * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems. */
+int tgbm_trainer_info(tgbm_trainer *t, const char *key);
+float tgbm_trainer_base_score(tgbm_trainer *t);
+
+/* Copies a device buffer to `out` when `cap` is large enough; always returns its size in bytes.
+ * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist0, hist1, ctl,
+ * seg, ridx0, ridx1, model, metric_log. */
+size_t tgbm_trainer_get(tgbm_trainer *t, const char *name, void *out, size_t cap);
+/* Overwrites gh or y_pred (lock-step tests feed both implementations the same state). */
+void tgbm_trainer_set(tgbm_trainer *t, const char *name, const void *in, size_t bytes);
+
+/* Histogram-build timing with HIP events on the trainer's stream. get_profile fills
+ * out[0] = summed kernel milliseconds, out[1] = launches, out[2] = rows visited,
+ * out[3] = algorithmic bytes (rows x (features + 8 [+4 below the root])). */
+void tgbm_trainer_set_profiling(tgbm_trainer *t, int on);
+void tgbm_trainer_get_profile(tgbm_trainer *t, double *out4);
+
+/* Moves the trees built so far into a model handle usable with the Part 1 functions. */
+tgbm_model *tgbm_trainer_export_model(tgbm_trainer *t);
+
+/* Predictor::predict_raw (predictor.cu:32-189) with an explicit base score: class-major raw scores,
+ * row_size * trees_per_iter floats. */
+void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const int *col_ptr, tgbm_model *model,
+                      int n_trees, int trees_per_iter, float learning_rate, float base_score, float *out);
+
+/* Cut points and global bin ids of a CSR matrix (HistCut::get_cut_points_single, hist_cut.cu:232-286;
+ * get_bin_ids, hist_tree_builder_single.cu:49-130), computed on the GPU. cut_val / cut_fid need one
+ * slot per stored value at most (row_ptr[row_size]); returns the number of cut points. */
+int tgbm_cut_points(int row_size, int n_features, const float *val, const int *row_ptr, const int *col_ptr,
+                    int max_num_bin, float *cut_val, int *cut_row_ptr, int *cut_fid, int *bin_id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THUNDERGBM_H */

@@ -453,12 +453,11 @@ void find_split(Oracle &o, int level) {
             int nl = ptr[a + 1] - ptr[a], nr = ptr[b + 1] - ptr[b];
             if (std::max(nl, nr) == 0) {
                 // :454-465. Both siblings empty: invalid nodes are flagged. A valid pair without rows
-                // cannot occur (a split with an empty side has zero gain); it is flagged too instead
-                // of reproducing the reference's zero-initialised SplitPoint (which addresses node 0).
-                for (int j = 0; j < 2; ++j) {
-                    o.sp[2 * p + j].nid = -1;
-                    o.sp[2 * p + j].fid = -1;
-                }
+                // cannot occur (a split with an empty side has zero gain); instead of reproducing the
+                // reference's zero-initialised SplitPoint (which would address node 0) such a node is
+                // evaluated on an all-zero histogram and therefore becomes a leaf.
+                for (int j = 0; j < 2; ++j)
+                    evaluate_node(o, off + 2 * p + j, o.hist_cur.data() + (size_t)(2 * p + j) * B, o.sp[2 * p + j]);
                 continue;
             }
             if (nl > nr) std::swap(a, b);  // build the one with fewer rows, ties build the left one

@@ -27,7 +27,13 @@ def read_libsvm(path):
 
 
 def dense_to_csr(X):
+    """Dense -> CSR with the reference wrapper's rule: exact zeros are dropped (they become missing)."""
     X = np.asarray(X, dtype=np.float32)
+    n, F = X.shape
+    if np.count_nonzero(X) == X.size:  # nothing to drop: skip the index gymnastics on big matrices
+        row_ptr = (np.arange(n + 1, dtype=np.int64) * F).astype(np.int32)
+        col = np.tile(np.arange(F, dtype=np.int32), n)
+        return np.ascontiguousarray(X).reshape(-1), row_ptr, col
     mask = X != 0
     row_ptr = np.zeros(X.shape[0] + 1, dtype=np.int32)
     np.cumsum(mask.sum(axis=1), out=row_ptr[1:])

@@ -1,0 +1,102 @@
+"""Comparators shared by the GPU parity tests.
+
+Tolerances (north-star statement): cut points, bin ids and node assignments bit-exact; histogram
+sums, gains and predictions within 1e-5 relative in an fp64-accumulated comparison; tree structure
+identical wherever the gap between competing split gains exceeds that tolerance.
+"""
+import numpy as np
+
+REL = 1e-5
+
+
+def abs_hist(bins, rows, gh, n_bins):
+    """Per-bin sum of |g| and |h| over all stored entries: the scale a relative error refers to."""
+    out = np.zeros((n_bins, 2))
+    np.add.at(out, bins, np.abs(gh[rows].astype(np.float64)))
+    return out
+
+
+def assert_hist_close(got, ref64, scale, what="", rel=REL):
+    """|got - ref64| <= rel * scale, scale = per-bin sum of absolute contributions."""
+    err = np.abs(got.astype(np.float64) - ref64)
+    tol = rel * scale + 1e-30
+    bad = err > tol
+    assert not bad.any(), "%s: %d bins off, worst err/scale %.3g" % (
+        what, int(bad.sum()), float((err / np.maximum(scale, 1e-30)).max()))
+
+
+def gain_scale(node_sum, left_sum, lam):
+    """Magnitude of the three terms whose difference is the gain."""
+    fg, fh = node_sum
+    lg, lh = left_sum
+    rg, rh = fg - lg, fh - lh
+    return lg * lg / (lh + lam) + rg * rg / (rh + lam) + fg * fg / (fh + lam)
+
+
+class TreeDiff:
+    def __init__(self):
+        self.compared = 0
+        self.near_ties = []  # (node, oracle best |gain|, oracle |gain| of the GPU's choice)
+
+    def __repr__(self):
+        return "TreeDiff(compared=%d, near_ties=%r)" % (self.compared, self.near_ties)
+
+
+def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, feature_has_missing=None, rel=REL):
+    """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
+
+    Where both trees split on the same candidate everything must agree: threshold and bin exactly,
+    gain / child sums / weights to `rel` of their scale. Where the choice differs, the oracle's own
+    gain of the GPU's candidate must be within tolerance of the oracle's best (a near tie); the
+    subtree below such a node is not compared. `default_right` is only compared for features that
+    have missing values (for dense features the reference decides it by float32 round-off).
+    orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle (None forbids any mismatch);
+    crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
+    """
+    diff = TreeDiff()
+    slack = 10 * rel
+    stack = [0]
+    while stack:
+        x = stack.pop()
+        g, o = gpu[x], orc[x]
+        assert bool(g["is_valid"]) == bool(o["is_valid"]), "node %d validity differs" % x
+        if not o["is_valid"]:
+            continue
+        diff.compared += 1
+        S = (float(o["sum_g"]), float(o["sum_h"]))
+        sum_scale = max(1.0, abs(S[0]) + abs(S[1]))
+        assert abs(g["sum_g"] - o["sum_g"]) <= slack * sum_scale and abs(g["sum_h"] - o["sum_h"]) <= slack * sum_scale, \
+            "node %d sum differs: gpu (%g,%g) oracle (%g,%g)" % (x, g["sum_g"], g["sum_h"], o["sum_g"], o["sum_h"])
+        assert abs(g["base_weight"] - o["base_weight"]) <= slack * max(1.0, abs(o["base_weight"])), \
+            "node %d weight differs: %g vs %g" % (x, g["base_weight"], o["base_weight"])
+        split_g, split_o = g["split_fid"] >= 0, o["split_fid"] >= 0
+        if not split_g and not split_o:
+            continue
+        if split_g and split_o and g["split_fid"] == o["split_fid"] and g["split_bid"] == o["split_bid"]:
+            assert g["split_value"] == o["split_value"], "node %d threshold differs" % x
+            lch = orc[o["lch"]]
+            sc = max(1.0, abs(float(o["gain"])), gain_scale(S, (float(lch["sum_g"]), float(lch["sum_h"])), lam))
+            assert abs(g["gain"] - o["gain"]) <= slack * sc, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
+            if feature_has_missing is not None and feature_has_missing[o["split_fid"]]:
+                assert g["default_right"] == o["default_right"], "node %d default direction differs" % x
+            stack.extend([int(o["lch"]), int(o["rch"])])
+            continue
+        assert orc_scores is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (
+            x, g["split_fid"], g["split_bid"], o["split_fid"], o["split_bid"])
+        sc = orc_scores[x]
+        best = float(np.abs(sc).max())
+        scale = max(1.0, best, S[0] * S[0] / (S[1] + lam))
+        if split_g:
+            alt = abs(float(sc[int(crp[g["split_fid"]]) + int(g["split_bid"])]))
+            assert best - alt <= slack * scale, \
+                "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d)" % (
+                    x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"])
+        else:
+            alt = 0.0  # gpu made a leaf where the oracle split: the gain must sit at the rt_eps edge
+            assert best <= 1e-6 + slack * scale, "node %d: gpu leaf, oracle split gain %g" % (x, best)
+        diff.near_ties.append((x, best, alt))
+    if not diff.near_ties:
+        for key in ("is_leaf", "is_pruned", "final_id", "lch", "rch", "parent"):
+            valid = orc["is_valid"] == 1
+            assert np.array_equal(gpu[key][valid], orc[key][valid]), "field %s differs" % key
+    return diff

@@ -1,0 +1,452 @@
+"""GPU parity tests: the HIP library (through its C ABI) against the CPU oracle on the same seeded
+inputs. Run on the MI355X box with `pytest -m gpu`."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import datasets as D
+import oracle_lib as O
+import parity as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def T():
+    import thundergbm_amd
+    thundergbm_amd.load()
+    return thundergbm_amd
+
+
+def _missing_dataset(n, F, seed, frac=0.3, round_to=1):
+    rng = np.random.default_rng(seed)
+    X = np.round(rng.standard_normal((n, F)) * 2, round_to).astype(np.float32)
+    X[X == 0] = 0.5
+    miss = rng.random((n, F)) < frac
+    miss[:, 0] = False
+    X[miss] = 0
+    y = (X[:, 0] * 1.5 - X[:, 1] + rng.standard_normal(n) * 0.3).astype(np.float32)
+    return X, y
+
+
+def _cases():
+    X1, y1 = D.config1(10000, 8, seed=0)
+    X2, y2 = _missing_dataset(6000, 11, 3)
+    X3, y3 = D.config2(20000, seed=1)
+    X5, y5 = D.config5(8000, seed=4)
+    return {
+        "c1_regression": (D.dense_to_csr(X1), y1, dict(objective="reg:linear", depth=6, max_num_bin=255)),
+        "missing_regression": (D.dense_to_csr(X2), y2, dict(objective="reg:linear", depth=5, max_num_bin=16)),
+        "c2_binary": (D.dense_to_csr(X3), y3, dict(objective="binary:logistic", depth=6, max_num_bin=255)),
+        "c5_softmax": (D.dense_to_csr(X5), y5, dict(objective="multi:softmax", depth=4, max_num_bin=255)),
+    }
+
+
+CASES = None
+
+
+def case(name):
+    global CASES
+    if CASES is None:
+        CASES = _cases()
+    return CASES[name]
+
+
+CASE_NAMES = ["c1_regression", "missing_regression", "c2_binary", "c5_softmax"]
+
+
+# ----------------------------------------------------------------------- cuts and bin ids (exact)
+def _cut_points_gpu(T, val, rp, col, F, max_bin):
+    L = T.load()
+    val = np.ascontiguousarray(val, np.float32)
+    rp = np.ascontiguousarray(rp, np.int32)
+    col = np.ascontiguousarray(col, np.int32)
+    cap = max(len(val), 1)
+    cv = np.zeros(cap, np.float32)
+    cf = np.zeros(cap, np.int32)
+    crp = np.zeros(F + 1, np.int32)
+    bins = np.zeros(cap, np.int32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    nb = L.tgbm_cut_points(len(rp) - 1, F, p(val), p(rp), p(col), max_bin, p(cv), p(crp), p(cf), p(bins))
+    return cv[:nb], crp, cf[:nb], bins[: len(val)]
+
+
+@pytest.mark.parametrize("max_bin", [2, 16, 63, 255])
+def test_cut_points_and_bins_exact(T, max_bin):
+    rng = np.random.default_rng(max_bin)
+    n, F = 30000, 13
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[:, 1] = np.round(X[:, 1], 1)            # few uniques (< 255)
+    X[:, 2] = rng.integers(0, 255, n)          # exactly around max_bin uniques, zeros become missing
+    X[:, 3] = rng.integers(0, 2, n)            # one unique stored value
+    X[:, 4] = 0                                # feature without any stored value
+    X[:, 5] = -np.abs(X[:, 5])                 # all negative
+    X[:, 6] = rng.integers(-300, 300, n) * 0.5
+    X[rng.random((n, F)) < 0.2] = 0
+    val, rp, col = D.dense_to_csr(X)
+    ocv, ocrp, ocf = O.cut_points(val, col, F, max_bin)
+    obins = O.bin_ids(val, col, ocv, ocrp)
+    cv, crp, cf, bins = _cut_points_gpu(T, val, rp, col, F, max_bin)
+    assert np.array_equal(crp, ocrp)
+    assert np.array_equal(cv.view(np.uint32), ocv.view(np.uint32))
+    assert np.array_equal(cf, ocf)
+    assert np.array_equal(bins, obins)
+
+
+def test_cut_points_ragged_and_empty_rows(T):
+    rng = np.random.default_rng(9)
+    n, F = 5000, 300
+    lens = rng.integers(0, 12, n)
+    lens[:10] = 0
+    rp = np.zeros(n + 1, np.int32)
+    np.cumsum(lens, out=rp[1:])
+    col = np.concatenate([np.sort(rng.choice(F, size=l, replace=False)) for l in lens]).astype(np.int32)
+    val = rng.lognormal(0, 1, len(col)).astype(np.float32)
+    ocv, ocrp, ocf = O.cut_points(val, col, F, 63)
+    cv, crp, cf, bins = _cut_points_gpu(T, val, rp, col, F, 63)
+    assert np.array_equal(crp, ocrp) and np.array_equal(cv, ocv) and np.array_equal(cf, ocf)
+    assert np.array_equal(bins, O.bin_ids(val, col, ocv, ocrp))
+
+
+def test_cut_points_a1a_fixture(T):
+    val, rp, col, y = D.read_libsvm(D.A1A)
+    cv, crp, cf, bins = _cut_points_gpu(T, val, rp, col, 119, 255)
+    assert np.all(cv == 1.0) and np.array_equal(cf, np.unique(col))
+    assert np.array_equal(bins, crp[col])  # single cut per feature -> local bin 0
+
+
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_session_cuts_bins_base_score(T, name):
+    (val, rp, col), y, kw = case(name)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    cv, crp, cf = s.cuts()
+    ocv, ocrp, ocf = o.cuts()
+    assert np.array_equal(cv, ocv) and np.array_equal(crp, ocrp) and np.array_equal(cf, ocf)
+    gb, local = s.global_bin_ids(rp, col)
+    assert np.array_equal(gb, o.bin_ids())
+    # every (row, feature) without a stored value is the missing sentinel
+    m = s.binmat()
+    W = s.info("dense_W")
+    stored = np.zeros((s.n, m.shape[0] * W), bool)
+    stored[np.repeat(np.arange(s.n), np.diff(rp)), col] = True
+    flat = m.transpose(1, 0, 2).reshape(s.n, -1)
+    assert np.all(flat[~stored] == 255)
+    assert s.num_class == o.num_class and s.tree_per_rounds == o.tree_per_rounds
+    assert np.array_equal(s.labels(), o.labels())
+    assert np.array_equal(s.y(), o.y())
+    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(s.y_pred(), o.y_pred(), rtol=1e-5, atol=1e-7)
+    s.close()
+
+
+# ------------------------------------------------------------------------------------- gradients
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_gradients(T, name):
+    (val, rp, col), y, kw = case(name)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    rng = np.random.default_rng(5)
+    yp = (rng.standard_normal(len(o.y_pred())) * 2).astype(np.float32)
+    s.set("y_pred", yp)
+    o.set_y_pred(yp)
+    s.gradient()
+    o.compute_gradient()
+    g, og = s.gh(), o.gh()
+    if kw["objective"] == "reg:linear":
+        assert np.array_equal(g, og)
+    else:
+        np.testing.assert_allclose(g[:, 0], og[:, 0], rtol=1e-5, atol=2e-7)
+        np.testing.assert_allclose(g[:, 1], og[:, 1], rtol=1e-5, atol=2e-7)
+    s.close()
+
+
+# ------------------------------------------------------------ one tree in lock step, level by level
+@pytest.mark.parametrize("name", CASE_NAMES)
+def test_tree_lockstep(T, name):
+    (val, rp, col), y, kw = case(name)
+    kw = dict(kw, gamma=0.5)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, debug=True, shadow64=True, **kw).prepare()
+    n, nb, depth = s.n, s.n_bins, kw["depth"]
+    _, crp, cf = s.cuts()
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    gbins = o.bin_ids()
+    s.gradient()
+    gh_all = s.gh()
+    o.set_gh(gh_all)  # both sides build from bit-identical gradients
+    lam = 1.0
+    for k in range(s.tree_per_rounds):
+        gh = gh_all[k * n:(k + 1) * n]
+        scale_root = P.abs_hist(gbins, rows, gh, nb)
+        s.tree_init(k)
+        o.tree_init(k)
+        diverged = False
+        for level in range(depth):
+            s.find_split(level)
+            o.find_split(level)
+            o.update_tree()
+            gh_level = s.level_hist(level)
+            onodes = o.nodes()
+            gnodes = s.nodes()
+            off = (1 << level) - 1
+            sp_g, sp_o = s.splits(level), o.splits()
+            for x in range(1 << level):
+                if not onodes[off + x]["is_valid"]:
+                    assert sp_g[x]["nid"] == -1 and sp_o[x]["nid"] == -1
+                    continue
+                _, h64 = o.level_hist(x)
+                P.assert_hist_close(gh_level[x], h64, scale_root, "tree %d level %d node %d" % (k, level, x))
+                a, b = sp_g[x], sp_o[x]
+                if a["best_index"] != b["best_index"]:
+                    sc = o.tree_scores()[off + x]
+                    best = abs(sc).max()
+                    assert best - abs(sc[a["best_index"]]) <= 1e-4 * max(1.0, best), \
+                        "level %d node %d picks %d vs %d" % (level, x, a["best_index"], b["best_index"])
+                    diverged = True
+                    continue
+                assert a["fid"] == b["fid"] and a["bid"] == b["bid"] and a["fval"] == b["fval"]
+                S = (float(onodes[off + x]["sum_g"]), float(onodes[off + x]["sum_h"]))
+                gs = max(1.0, P.gain_scale(S, (float(b["lch_g"]), float(b["lch_h"])), lam))
+                assert abs(a["gain"] - b["gain"]) <= 1e-4 * gs
+                nsc = max(1.0, abs(S[0]) + abs(S[1]))
+                for key in ("lch_g", "lch_h", "miss_g", "miss_h"):
+                    assert abs(a[key] - b[key]) <= 1e-4 * nsc, (key, a[key], b[key])
+            if diverged:
+                break
+            # same splits -> node arrays agree and the partition must be bit-identical
+            for key in ("is_valid", "is_leaf", "split_fid", "split_bid"):
+                assert np.array_equal(gnodes[key], onodes[key]), key
+            assert np.array_equal(gnodes["split_value"], onodes["split_value"])
+            # default direction matters only where values are missing; force agreement for the rest
+            # by copying the GPU's nodes into the oracle (sums differ in the last ulps only)
+            np.testing.assert_allclose(gnodes["sum_g"], onodes["sum_g"], rtol=0, atol=1e-4 * max(1, abs(gh[:, 0]).sum()))
+            o.set_nodes(gnodes)
+            s.partition(level)
+            has = o.update_ins2node()
+            assert np.array_equal(s.nid(), o.nid()), "node assignment differs at level %d" % level
+            # row lists: every node's segment holds exactly its rows in ascending order
+            seg = s.get("seg", np.int32, (-1, 2))
+            ridx = s.get("ridx%d" % ((level + 1) & 1), np.int32)
+            nid = s.nid()
+            for x in range((2 << level) - 1, (4 << level) - 1):
+                b, e = seg[x]
+                mine = np.flatnonzero(nid == x)
+                if gnodes[(x - 1) // 2]["split_fid"] >= 0 and not gnodes[(x - 1) // 2]["is_leaf"]:
+                    assert np.array_equal(ridx[b:e], mine), "row list of node %d" % x
+                else:
+                    assert e - b == 0
+            if not has:
+                break
+        if diverged:
+            continue
+        s.finish_tree(k)
+        o.prune()
+        o.predict_in_training(k)
+        d = P.compare_trees(s.nodes(), o.nodes(), lam, crp=crp, orc_scores=o.tree_scores())
+        assert not d.near_ties
+        np.testing.assert_allclose(s.y_pred(), o.y_pred(), rtol=1e-5, atol=1e-6)
+    s.close()
+
+
+# -------------------------------------------------------------------- boosting, tree by tree
+@pytest.mark.parametrize("name,rounds", [("c1_regression", 40), ("missing_regression", 10), ("c2_binary", 10),
+                                         ("c5_softmax", 3)])
+def test_boosting_teacher_forced(T, name, rounds):
+    """Each round both sides start from the GPU's predictions, so every tree is compared on its own."""
+    (val, rp, col), y, kw = case(name)
+    kw = dict(kw, n_trees=rounds, learning_rate=0.1 if name == "c1_regression" else 0.3)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    _, crp, _ = s.cuts()
+    X_has_missing = np.bincount(col, minlength=s.F) < s.n
+    n = s.n
+    total_ties = 0
+    for r in range(rounds):
+        yp = s.y_pred()
+        o.set_y_pred(yp)
+        s.boost(1)
+        model = s.model()
+        o.compute_gradient()
+        gh, ogh = s.gh(), o.gh()  # the gradients this round was built from
+        np.testing.assert_allclose(gh, ogh, rtol=1e-5, atol=2e-7)
+        o.set_gh(gh)
+        ok_round = True
+        for k in range(s.tree_per_rounds):
+            o.build_tree(k)
+            d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(),
+                                feature_has_missing=X_has_missing)
+            total_ties += len(d.near_ties)
+            ok_round &= not d.near_ties
+        if ok_round:
+            np.testing.assert_allclose(s.y_pred(), o.y_pred(), rtol=1e-5, atol=2e-6)
+            np.testing.assert_allclose(s.metric_log()[-1], o.metric(), rtol=1e-5, atol=1e-6)
+    assert total_ties <= max(2, rounds * s.tree_per_rounds // 5), "too many near ties: %d" % total_ties
+    s.close()
+
+
+def test_free_running_c1_matches_oracle(T):
+    """BASELINE config 1 end to end (10 000 x 8, 40 trees, depth 6, lr 0.1) without teacher forcing."""
+    X, y = D.config1(10000, 8, seed=0)
+    val, rp, col = D.dense_to_csr(X)
+    kw = dict(depth=6, n_trees=40, learning_rate=0.1, max_num_bin=255)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    s.boost(40)
+    o.boost(40)
+    ml, oml = s.metric_log(), o.metric_log()
+    assert np.all(np.diff(ml) < 0)
+    np.testing.assert_allclose(ml, oml, rtol=2e-3)
+    np.testing.assert_allclose(ml[:5], oml[:5], rtol=1e-5)
+    s.close()
+
+
+# -------------------------------------------------------------------------- prediction and C ABI
+@pytest.mark.parametrize("objective", ["reg:linear", "binary:logistic", "multi:softmax", "multi:softprob"])
+def test_estimator_fit_predict_save_load(T, objective, tmp_path):
+    n, F = 3000, 9
+    X, y = _missing_dataset(n, F, 17)
+    if objective == "binary:logistic":
+        y = np.where(y > 0, 1.0, -1.0).astype(np.float32)
+    elif objective.startswith("multi:"):
+        y = (np.digitize(y, np.quantile(y, [0.25, 0.5, 0.75])) * 2 + 1).astype(np.float32)
+    cls = T.TGBMRegressor if objective == "reg:linear" else T.TGBMClassifier
+    m = cls(depth=4, n_trees=5, learning_rate=0.5, objective=objective, verbose=0, max_num_bin=32)
+    m.fit(X, y)
+    pred = m.predict(X)
+    # the oracle on the same CSR input
+    val, rp, col = D.dense_to_csr(X)
+    o = O.Oracle(val, rp, col, y, depth=4, n_trees=5, learning_rate=0.5, objective=objective, max_num_bin=32,
+                 num_class=2).prepare()
+    o.boost(5)
+    # the C-API predict path carries no base score (reference quirk): raw = sum of trees only
+    raw = O.predict_raw(val, rp, col, F, o.model(), 0.5, 0.0)
+    labels = o.labels() if objective != "reg:linear" else np.zeros(1, np.float32)
+    exp = O.predict_transform(objective, raw, n, o.num_class, labels)
+    assert m.num_class == o.num_class and m.tree_per_iter == o.tree_per_rounds
+    if objective == "reg:linear" or objective == "multi:softprob":
+        np.testing.assert_allclose(pred.ravel(), exp, rtol=1e-4, atol=1e-5)
+    else:
+        assert np.mean(pred == exp) > 0.995
+    # tree export
+    trees = m.get_trees()
+    assert len(trees) == 5 * m.tree_per_iter and len(trees[0]["feature"]) == 31
+    om = o.model().reshape(-1, 31)
+    leaf = om[0]["is_leaf"] == 1
+    assert np.array_equal(trees[0]["children_left"][leaf], -np.ones(leaf.sum(), np.int32))
+    # save / load round trip gives identical predictions
+    path = str(tmp_path / "m.model")
+    m.save_model(path)
+    m2 = cls(objective=objective, verbose=0)
+    m2.load_model(path)
+    pred2 = m2.predict(X)
+    assert np.array_equal(np.asarray(pred), np.asarray(pred2))
+    assert m2.group_label == m.group_label or objective == "reg:linear"
+
+
+def test_predict_raw_equals_training_prediction(T):
+    (val, rp, col), y, kw = case("c2_binary")
+    s = T.Session(val, rp, col, y, n_trees=8, learning_rate=0.3, **kw)
+    s.boost(8)
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    out = np.zeros(s.n, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    L.tgbm_predict_raw(s.n, p(val), p(rp), p(col), model, 8, 1, 0.3, s.base_score, p(out))
+    np.testing.assert_allclose(out, s.y_pred(), rtol=1e-5, atol=1e-6)
+    # and against the oracle's predictor on the GPU's model
+    ref = O.predict_raw(val, rp, col, s.F, s.model(), 0.3, s.base_score)
+    np.testing.assert_allclose(out, ref, rtol=1e-6, atol=1e-6)
+    L.model_free(C.byref(model))
+    s.close()
+
+
+def test_predict_wide_float_path_and_unseen_rows(T):
+    # F > 96 takes the reference's float accumulation path; unseen rows exercise default directions
+    rng = np.random.default_rng(3)
+    n, F = 4000, 130
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.5] = 0
+    y = (X[:, 0] - X[:, 5] + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    s = T.Session(val, rp, col, y, depth=5, n_trees=6, learning_rate=0.4, max_num_bin=64)
+    s.boost(6)
+    Xt = rng.standard_normal((1000, F)).astype(np.float32)
+    Xt[rng.random((1000, F)) < 0.5] = 0
+    tv, trp, tc = D.dense_to_csr(Xt)
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    out = np.zeros(1000, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    L.tgbm_predict_raw(1000, p(tv), p(trp), p(tc), model, 6, 1, 0.4, s.base_score, p(out))
+    ref = O.predict_raw(tv, trp, tc, F, s.model(), 0.4, s.base_score)
+    np.testing.assert_allclose(out, ref, rtol=1e-6, atol=1e-6)
+    L.model_free(C.byref(model))
+    s.close()
+
+
+def test_a1a_quickstart_known_answer(T):
+    # README.md:76-80 of the reference: RMSE = 0.489562 (zero initial prediction, see the oracle test)
+    val, rp, col, y = D.read_libsvm(D.A1A)
+    s = T.Session(val, rp, col, y, depth=6, n_trees=40, learning_rate=1.0)
+    s.set("y_pred", np.zeros(len(y), np.float32))
+    s.boost(40)
+    assert abs(float(s.metric_log()[-1]) - 0.489562) < 5e-5
+    s.close()
+
+
+# --------------------------------------------- size-independent properties at the benchmark shape
+def test_full_size_properties_config2(T):
+    n = int(os.environ.get("TGBM_TEST_FULL_ROWS", "10000000"))
+    X, y = D.config2(n, seed=1)
+    val, rp, col = D.dense_to_csr(X)
+    del X
+    s = T.Session(val, rp, col, y, depth=8, n_trees=2, objective="binary:logistic", learning_rate=0.3)
+    _, crp, cf = s.cuts()
+    # cut invariants
+    cv = s.cuts()[0]
+    for f in range(s.F):
+        seg = cv[crp[f]:crp[f + 1]]
+        assert len(seg) <= 255 and np.all(np.diff(seg) > 0)
+    s.gradient()
+    s.tree_init(0)
+    gh = s.gh()[:n].astype(np.float64)
+    for level in range(8):
+        s.find_split(level)
+        hist = s.level_hist(level).astype(np.float64)
+        nodes = s.nodes()
+        off = (1 << level) - 1
+        for x in range(1 << level):
+            nd = nodes[off + x]
+            if not nd["is_valid"]:
+                continue
+            for f in (0, 13, 27):  # dense features: every row lands in exactly one bin of the feature
+                tot = hist[x, crp[f]:crp[f + 1]].sum(axis=0)
+                sc = max(1.0, np.abs(gh[:, 0]).sum() / (1 << level))
+                assert abs(tot[0] - nd["sum_g"]) <= 2e-4 * sc and abs(tot[1] - nd["sum_h"]) <= 2e-4 * sc
+        s.partition(level)
+    nid = s.nid()
+    nodes = s.nodes()
+    cnt = np.bincount(nid, minlength=len(nodes))
+    # rows only sit in valid nodes; child hessian sums match the rows that arrived (fp64 recount)
+    assert np.all(nodes["is_valid"][cnt > 0] == 1)
+    hs = np.bincount(nid, weights=gh[:, 1], minlength=len(nodes))
+    gs = np.bincount(nid, weights=gh[:, 0], minlength=len(nodes))
+    occupied = np.flatnonzero(cnt > 0)
+    np.testing.assert_allclose(nodes["sum_h"][occupied], hs[occupied], rtol=2e-4, atol=1e-2)
+    np.testing.assert_allclose(nodes["sum_g"][occupied], gs[occupied], rtol=0, atol=2e-4 * np.abs(gh[:, 0]).sum() / 16)
+    s.finish_tree(0)
+    # training-time prediction == predictor on a sample of the training rows
+    yp = s.y_pred()
+    sub = slice(0, 200000)
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    out = np.zeros(200000, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    srp = rp[: 200001].copy()
+    L.tgbm_predict_raw(200000, p(val), p(srp), p(col), model, 1, 1, 0.3, s.base_score, p(out))
+    np.testing.assert_allclose(out, yp[sub], rtol=1e-5, atol=1e-6)
+    L.model_free(C.byref(model))
+    s.close()

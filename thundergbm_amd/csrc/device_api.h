@@ -1,0 +1,117 @@
+// Host-callable launchers of the HIP kernels (gfx950). All launches are stream-ordered and never
+// synchronise; sizes are validated by the callers in trainer.hip / predictor.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+#define HIP_CHECK(expr)                                                                              \
+    do {                                                                                             \
+        hipError_t e_ = (expr);                                                                      \
+        if (e_ != hipSuccess) ::tgbm::fatal("%s:%d HIP error %s: %s", __FILE__, __LINE__, #expr,     \
+                                            hipGetErrorString(e_));                                  \
+    } while (0)
+
+namespace tgbm {
+
+constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
+constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
+constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
+
+// Per-level control block written by the planning kernels and read by the worker kernels.
+struct LevelCtl {
+    int hchunk;      // rows per histogram work item
+    int n_hitems;    // histogram work items of the level
+    int n_pitems;    // partition work items of the level
+    int rows_built;  // rows visited by the histogram build of the level
+};
+
+// Candidate produced by one wavefront of the split finder.
+struct SplitCand {
+    float score;  // signed gain: > 0 missing goes left, <= 0 missing goes right
+    int index;    // global bin index
+    GHPair miss;
+    GHPair left;  // sum of the bins strictly below the candidate, within its feature
+    int pad[2];
+};
+
+// Dense column-blocked bin matrix: block b holds features [b*W, (b+1)*W) as n rows of W bytes.
+struct DenseBins {
+    const uint8_t *data = nullptr;
+    int W = 0;          // bytes (features) per row of a block, multiple of 4
+    int n_blocks = 0;
+    size_t block_stride = 0;  // bytes between blocks = n * W
+};
+
+struct TreeBuffers {
+    int n = 0, n_bins = 0, F = 0, depth = 0, n_nodes = 0;
+    TreeNode *nodes = nullptr;     // [n_nodes]
+    int2 *seg = nullptr;           // [n_nodes] row-list segment [x, y) of every node
+    int *nid = nullptr;            // [n]
+    int *ridx[2] = {nullptr, nullptr};  // [n] row lists, ping-pong by level parity
+    uint8_t *goes_right = nullptr; // [n]
+    GHPair *hist[2] = {nullptr, nullptr};  // [max_level_nodes * n_bins] raw histograms by level parity
+    GHPair *partial = nullptr;     // [max_hitems * n_bins]
+    int max_hitems = 0, target_hitems = 0, max_pitems = 0;
+    int *hpair_begin = nullptr;    // [max_pairs + 1] first histogram item of every sibling pair
+    int *hpair_built = nullptr;    // [max_pairs] heap id of the node built from rows, -1 = inactive pair
+    int *pitem_begin = nullptr;    // [max_level_nodes + 1]
+    int *pitem_nleft = nullptr;    // [max_pitems]
+    int *pitem_loff = nullptr;     // [max_pitems]
+    int *node_nleft = nullptr;     // [max_level_nodes]
+    LevelCtl *ctl = nullptr;       // [depth + 1]
+    SplitPoint *sp = nullptr;      // [max_level_nodes]
+    SplitCand *cand = nullptr;     // [max_level_nodes * n_packs]
+    GHPair *root_partial = nullptr;  // [num_class * n_grad_blocks] block sums of the gradient kernel
+    int n_grad_blocks = 0;
+    // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1])
+    const int *pack_begin = nullptr;
+    int n_packs = 0;
+    const int *cut_row_ptr = nullptr;
+    const int *cut_fid = nullptr;
+    const float *cut_val = nullptr;
+    // dense block tables
+    const int *blk_bin_begin = nullptr;  // [n_blocks + 1] first global bin of every block
+    const int *feat_lds_off = nullptr;   // [n_blocks * W] bin offset of a feature inside its block
+    int max_block_bins = 0;
+};
+
+// objective codes
+enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
+
+void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
+                     GHPair *block_sums, int n_blocks);
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *class_block_sums, float lambda);
+void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
+void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);
+void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda);
+void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level);
+void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma);
+void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, float *yp_class, float lr);
+void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
+                   double *scratch, float *out);
+void launch_fill_f32(hipStream_t s, float *p, float v, size_t n);
+void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
+
+// data preparation
+void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
+                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride);
+void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
+                    const int *cut_row_ptr, int *bin_id);
+// cut points on device: returns the device arrays through out parameters allocated by the callee
+struct DeviceCuts {
+    float *cut_val = nullptr;
+    int *cut_row_ptr = nullptr;
+    int *cut_fid = nullptr;
+    int n_bins = 0;
+};
+DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, const int *d_col, int max_num_bin);
+
+// prediction
+void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
+                    const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
+                    float *out);
+void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y);
+
+}  // namespace tgbm

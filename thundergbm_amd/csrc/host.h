@@ -1,0 +1,57 @@
+// Host-side pieces that mirror the reference's DataSet, Parser, TreeTrainer and Predictor.
+#pragma once
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace tgbm {
+
+// Host CSR dataset (the reference's DataSet, include/thundergbm/dataset.h).
+struct DataSet {
+    std::vector<float> csr_val;
+    std::vector<int> csr_row_ptr;
+    std::vector<int> csr_col_idx;
+    std::vector<float> y;
+    std::vector<float> label;  // distinct class labels, ascending
+    std::vector<int> group;
+    size_t n_features_ = 0;
+
+    size_t n_features() const { return n_features_; }
+    size_t n_instances() const { return y.size(); }
+
+    // src/thundergbm/dataset.cpp:20-63
+    void load_from_sparse(int n_instances, const float *csr_val, const int *csr_row_ptr, const int *csr_col_idx,
+                          const float *y, const int *group, int num_group, GBMParam &param);
+    // src/thundergbm/dataset.cpp:170-320 (LIBSVM text, 1-based feature ids)
+    void load_from_file(const std::string &file_name, GBMParam &param);
+    // src/thundergbm/dataset.cpp:83-101
+    void group_label();
+};
+
+bool objective_needs_group_label(const std::string &objective);
+bool objective_supported(const std::string &objective);
+
+// Parameter parsing and the raw binary model format (src/thundergbm/parser.cpp).
+struct Parser {
+    static void parse_param(GBMParam &param, int argc, char **argv);
+    static void load_model(const std::string &path, GBMParam &param, std::vector<std::vector<Tree>> &model,
+                           DataSet &dataset);
+    static void save_model(const std::string &path, const GBMParam &param,
+                           const std::vector<std::vector<Tree>> &model, const DataSet &dataset);
+};
+
+class Trainer;  // device trainer, trainer.hip
+
+// src/thundergbm/trainer.cu:18-57
+std::vector<std::vector<Tree>> train(GBMParam &param, const DataSet &dataset);
+
+// src/thundergbm/predictor.cu:11-30 / :32-189. Returns class-major raw scores (predict_raw) or the
+// transformed predictions (predict).
+std::vector<float> predict_raw(const GBMParam &param, const std::vector<std::vector<Tree>> &model,
+                               const DataSet &dataset);
+std::vector<float> predict(const GBMParam &param, const std::vector<std::vector<Tree>> &model,
+                           const DataSet &dataset, bool log_metric);
+
+}  // namespace tgbm

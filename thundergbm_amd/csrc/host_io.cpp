@@ -1,0 +1,253 @@
+// Host-side I/O: logging, CSR ingestion with label grouping, LIBSVM text loading, key=value
+// parameter parsing and the raw binary model file. No device code here.
+#include <algorithm>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <sstream>
+
+#include "host.h"
+
+namespace tgbm {
+
+int g_verbose = 1;
+
+void log_info(const char *fmt, ...) {
+    if (g_verbose < 1) return;
+    va_list ap;
+    va_start(ap, fmt);
+    std::fputs("INFO  ", stdout);
+    std::vprintf(fmt, ap);
+    std::fputc('\n', stdout);
+    std::fflush(stdout);
+    va_end(ap);
+}
+
+void log_debug(const char *fmt, ...) {
+    if (g_verbose < 2) return;
+    va_list ap;
+    va_start(ap, fmt);
+    std::fputs("DEBUG ", stdout);
+    std::vprintf(fmt, ap);
+    std::fputc('\n', stdout);
+    std::fflush(stdout);
+    va_end(ap);
+}
+
+void fatal(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    std::fputs("FATAL ", stderr);
+    std::vfprintf(stderr, fmt, ap);
+    std::fputc('\n', stderr);
+    std::fflush(stderr);
+    va_end(ap);
+    std::abort();
+}
+
+bool objective_needs_group_label(const std::string &o) {
+    return o == "multi:softprob" || o == "multi:softmax" || o == "binary:logistic";
+}
+
+bool objective_supported(const std::string &o) {
+    return o == "reg:linear" || o == "reg:logistic" || o == "binary:logistic" || o == "multi:softprob" ||
+           o == "multi:softmax";
+}
+
+void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr, const int *col_idx,
+                               const float *labels, const int *grp, int num_group, GBMParam &param) {
+    n_features_ = 0;
+    y.clear();
+    label.clear();
+    group.clear();
+    const int nnz = row_ptr[n_rows];
+    y.assign(n_rows, 0.f);
+    if (labels != nullptr) std::copy(labels, labels + n_rows, y.begin());
+    csr_val.assign(val, val + nnz);
+    csr_col_idx.assign(col_idx, col_idx + nnz);
+    csr_row_ptr.assign(row_ptr, row_ptr + n_rows + 1);
+    int max_col = 0;
+    for (int i = 0; i < nnz; ++i) max_col = std::max(max_col, col_idx[i]);
+    n_features_ = (size_t)max_col + 1;
+    log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
+    if (labels != nullptr && objective_needs_group_label(param.objective)) {
+        group_label();
+        param.num_class = (int)label.size();
+    }
+    (void)grp;
+    (void)num_group;  // query groups belong to the ranking objectives, which this library does not train
+}
+
+void DataSet::group_label() {
+    std::vector<int> distinct(y.begin(), y.end());  // labels are truncated to int for the label set
+    std::sort(distinct.begin(), distinct.end());
+    distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
+    std::map<float, int> index_of;
+    label.clear();
+    for (int v : distinct) {
+        index_of[(float)v] = (int)label.size();
+        label.push_back((float)v);
+    }
+    for (float &v : y) {
+        auto it = index_of.find(v);
+        v = it == index_of.end() ? 0.f : (float)it->second;  // unknown keys read as class 0
+    }
+}
+
+void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {
+    log_info("loading LIBSVM dataset from file ## %s ##", file_name.c_str());
+    std::ifstream ifs(file_name, std::ifstream::binary);
+    TGBM_CHECK(ifs.is_open(), "file ## %s ## not found. ", file_name.c_str());
+    y.clear();
+    label.clear();
+    csr_val.clear();
+    csr_col_idx.clear();
+    csr_row_ptr.assign(1, 0);
+    n_features_ = 0;
+    std::string line;
+    while (std::getline(ifs, line)) {
+        const char *p = line.c_str();
+        while (*p == ' ' || *p == '\t') ++p;
+        if (*p == '\0' || *p == '#' || *p == '\r') continue;
+        char *end = nullptr;
+        float lab = std::strtof(p, &end);
+        if (end == p) continue;
+        y.push_back(lab);
+        p = end;
+        for (;;) {
+            while (*p == ' ' || *p == '\t' || *p == '\r') ++p;
+            if (*p == '\0' || *p == '#') break;
+            long fid = std::strtol(p, &end, 10);
+            if (end == p || *end != ':') break;
+            p = end + 1;
+            float v = std::strtof(p, &end);
+            if (end == p) break;
+            p = end;
+            csr_col_idx.push_back((int)fid - 1);
+            csr_val.push_back(v);
+            if ((size_t)fid > n_features_) n_features_ = (size_t)fid;
+        }
+        csr_row_ptr.push_back((int)csr_val.size());
+    }
+    label = y;  // the reference keeps a copy of all labels here (dataset.cpp:290-291) ...
+    log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
+    if (objective_needs_group_label(param.objective)) {
+        group_label();  // ... which grouping replaces by the distinct ones
+        param.num_class = (int)label.size();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+void Parser::parse_param(GBMParam &p, int argc, char **argv) {
+    p = GBMParam();  // defaults of src/thundergbm/parser.cpp:10-28
+    if (argc < 2) {
+        std::printf("Usage: <config>\n");
+        std::exit(0);
+    }
+    auto parse_value = [&](const char *name_val) {
+        char name[256], val[256];
+        if (std::sscanf(name_val, "%255[^=]=%255s", name, val) == 2) {
+            std::string k(name);
+            if (k == "max_depth" || k == "depth") p.depth = std::atoi(val);
+            else if (k == "num_round" || k == "n_trees") p.n_trees = std::atoi(val);
+            else if (k == "n_gpus") p.n_device = std::atoi(val);
+            else if (k == "verbosity" || k == "verbose") p.verbose = std::atoi(val);
+            else if (k == "profiling") p.profiling = std::atoi(val);
+            else if (k == "data") p.path = val;
+            else if (k == "max_bin" || k == "max_num_bin") p.max_num_bin = std::atoi(val);
+            else if (k == "colsample" || k == "column_sampling_rate") p.column_sampling_rate = (float)std::atof(val);
+            else if (k == "bagging") p.bagging = std::atoi(val);
+            else if (k == "num_parallel_tree" || k == "n_parallel_trees") p.n_parallel_trees = std::atoi(val);
+            else if (k == "eta" || k == "learning_rate") p.learning_rate = (float)std::atof(val);
+            else if (k == "objective") p.objective = val;
+            else if (k == "num_class") p.num_class = std::atoi(val);
+            else if (k == "min_child_weight") p.min_child_weight = (float)std::atoi(val);  // atoi, as parser.cpp:67
+            else if (k == "lambda" || k == "lambda_tgbm") p.lambda = (float)std::atof(val);
+            else if (k == "gamma" || k == "min_split_loss") p.gamma = (float)std::atof(val);
+            else if (k == "tree_method") p.tree_method = val;
+            else log_info("\"%s\" is unknown option!", name);
+        } else if (std::string(name_val) == "-help") {
+            std::printf("please refer to \"docs/parameters.md\" in the GitHub repository for more information "
+                        "about setting the options\n");
+            std::exit(0);
+        }
+    };
+    std::ifstream conf(argv[1]);
+    std::string line;
+    while (std::getline(conf, line)) parse_value(line.c_str());
+    for (int i = 0; i < argc; ++i) parse_value(argv[i]);
+}
+
+// Model file (src/thundergbm/parser.cpp:102-171), little endian, no header:
+// i32 len | objective | f32 lr | i32 num_class | i32 n_trees | f32 base_score | i32 n_label |
+// f32 label[] | i32 n_iter | per iter { i32 n_trees_in_iter | per tree { u64 n_nodes | TreeNode[] } }
+void Parser::save_model(const std::string &path, const GBMParam &param, const std::vector<std::vector<Tree>> &model,
+                        const DataSet &dataset) {
+    std::ofstream out(path, std::ios::binary);
+    TGBM_CHECK(out.is_open(), "cannot open %s for writing", path.c_str());
+    auto put = [&](const void *p, size_t n) { out.write(static_cast<const char *>(p), (std::streamsize)n); };
+    int len = (int)param.objective.size();
+    put(&len, 4);
+    put(param.objective.data(), (size_t)len);
+    put(&param.learning_rate, 4);
+    put(&param.num_class, 4);
+    put(&param.n_trees, 4);
+    put(&param.base_score, 4);
+    int n_label = (int)dataset.label.size();
+    put(&n_label, 4);
+    put(dataset.label.data(), sizeof(float) * (size_t)n_label);
+    int n_iter = (int)model.size();
+    put(&n_iter, 4);
+    for (const auto &iter : model) {
+        int n_in = (int)iter.size();
+        put(&n_in, 4);
+        for (const Tree &t : iter) {
+            uint64_t n_nodes = t.nodes.size();
+            put(&n_nodes, 8);
+            put(t.nodes.data(), sizeof(TreeNode) * t.nodes.size());
+        }
+    }
+}
+
+void Parser::load_model(const std::string &path, GBMParam &param, std::vector<std::vector<Tree>> &model,
+                        DataSet &dataset) {
+    std::ifstream in(path, std::ios::binary);
+    TGBM_CHECK(in.is_open(), "cannot open model file %s", path.c_str());
+    auto get = [&](void *p, size_t n) {
+        in.read(static_cast<char *>(p), (std::streamsize)n);
+        TGBM_CHECK((size_t)in.gcount() == n, "model file %s is truncated", path.c_str());
+    };
+    int len = 0;
+    get(&len, 4);
+    TGBM_CHECK(len >= 0 && len < 4096, "model file %s: bad objective length", path.c_str());
+    std::string obj((size_t)len, '\0');
+    get(&obj[0], (size_t)len);
+    param.objective = obj;
+    get(&param.learning_rate, 4);
+    get(&param.num_class, 4);
+    get(&param.n_trees, 4);
+    get(&param.base_score, 4);
+    int n_label = 0;
+    get(&n_label, 4);
+    TGBM_CHECK(n_label >= 0, "model file %s: bad label count", path.c_str());
+    dataset.label.assign((size_t)n_label, 0.f);
+    get(dataset.label.data(), sizeof(float) * (size_t)n_label);
+    int n_iter = 0;
+    get(&n_iter, 4);
+    model.clear();
+    for (int i = 0; i < n_iter; ++i) {
+        int n_in = 0;
+        get(&n_in, 4);
+        std::vector<Tree> iter((size_t)n_in);
+        for (Tree &t : iter) {
+            uint64_t n_nodes = 0;
+            get(&n_nodes, 8);
+            TGBM_CHECK(n_nodes < (1ull << 28), "model file %s: bad node count", path.c_str());
+            t.nodes.resize((size_t)n_nodes);
+            get(t.nodes.data(), sizeof(TreeNode) * (size_t)n_nodes);
+        }
+        model.push_back(std::move(iter));
+    }
+}
+
+}  // namespace tgbm

@@ -1,0 +1,123 @@
+// Tree-traversal prediction (the reference's Predictor::predict_raw, src/thundergbm/predictor.cu:32-189)
+// and the objectives' predict_transform.
+#include "device_api.h"
+
+namespace tgbm {
+namespace {
+
+constexpr int kBlock = 256;
+
+// Value of feature `f` in a CSR row with ascending column indices; `missing` when not stored.
+__device__ __forceinline__ float row_value(const int *__restrict__ ci, const float *__restrict__ cv, int len, int f,
+                                           bool *missing) {
+    int lo = 0, hi = len;
+    while (lo < hi) {
+        int mid = lo + (hi - lo) / 2;
+        int c = ci[mid];
+        if (c == f) {
+            *missing = false;
+            return cv[mid];
+        }
+        if (c > f)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    *missing = true;
+    return 0.f;
+}
+
+// One thread per row; the model (all trees, 48-byte nodes) is read through the caches. ACC is
+// double where the reference takes its shared-memory path (n_features * 128 * 4 <= 48 KB, :85) and
+// float otherwise (:166); in the double path a stored +inf counts as missing (:96-118).
+template <typename ACC, bool INF_IS_MISSING>
+__global__ __launch_bounds__(kBlock) void k_predict(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
+                                                   const float *__restrict__ val, const TreeNode *__restrict__ model,
+                                                   int n_iter, int n_class_trees, int n_nodes, float lr,
+                                                   float base_score, float *__restrict__ out) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int rb = row_ptr[i];
+    const int len = row_ptr[i + 1] - rb;
+    const int *ci = col + rb;
+    const float *cv = val + rb;
+    for (int t = 0; t < n_class_trees; ++t) {
+        ACC sum = base_score;
+        for (int it = 0; it < n_iter; ++it) {
+            const TreeNode *nd = model + ((size_t)it * n_class_trees + t) * n_nodes;
+            int cur = 0;
+            while (!nd[cur].is_leaf) {
+                const TreeNode &c = nd[cur];
+                bool missing;
+                float v = row_value(ci, cv, len, c.split_feature_id, &missing);
+                if (INF_IS_MISSING && !(v < INFINITY)) missing = true;
+                if (!missing)
+                    cur = v < c.split_value ? c.lch_index : c.rch_index;
+                else
+                    cur = c.default_right ? c.rch_index : c.lch_index;
+            }
+            sum += lr * nd[cur].base_weight;
+        }
+        out[(size_t)t * n + i] += (float)sum;
+    }
+}
+
+// kind 1: binary label lookup, 2: arg-max label lookup, 3: softmax probabilities in place,
+// 4: sigmoid (reg:logistic). regression_obj.h:27-32,76-92 and multiclass_obj.cu:44-88 of the reference.
+__global__ void k_predict_transform(int kind, int n, int K, const float *__restrict__ label, float *__restrict__ y) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        if (kind == 1) {
+            y[i] = label[y[i] > 0 ? 1 : 0];
+        } else if (kind == 2) {
+            int nc = K == 2 ? 1 : K;
+            int mk = 0;
+            float mp = y[i];
+            for (int k = 1; k < nc; ++k) {
+                float v = y[(size_t)k * n + i];
+                if (mp < v) {
+                    mp = v;
+                    mk = k;
+                }
+            }
+            y[i] = label[mk];
+        } else if (kind == 3) {
+            float mx = y[i];
+            for (int k = 1; k < K; ++k) mx = fmaxf(mx, y[(size_t)k * n + i]);
+            float sum = 0;
+            for (int k = 0; k < K; ++k) {
+                float e = expf(y[(size_t)k * n + i] - mx);
+                y[(size_t)k * n + i] = e;
+                sum += e;
+            }
+            for (int k = 0; k < K; ++k) y[(size_t)k * n + i] /= sum;
+        } else if (kind == 4) {
+            y[i] = 1.f / (1.f + expf(-y[i]));
+        }
+    }
+}
+
+}  // namespace
+
+void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
+                    const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
+                    float *out) {
+    if (n == 0) return;
+    if (n_class_trees > 1) base_score = 0;  // predictor.cu:81-83
+    const bool dense_path = (size_t)F * 128 * sizeof(float) <= 48 * 1024;
+    int grid = (n + kBlock - 1) / kBlock;
+    if (dense_path)
+        k_predict<double, true><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr,
+                                                       base_score, out);
+    else
+        k_predict<float, false><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr,
+                                                       base_score, out);
+}
+
+void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y) {
+    if (n == 0 || kind == 0) return;
+    int grid = (n + kBlock - 1) / kBlock;
+    if (grid > 4096) grid = 4096;
+    k_predict_transform<<<grid, kBlock, 0, s>>>(kind, n, num_class, label, y);
+}
+
+}  // namespace tgbm

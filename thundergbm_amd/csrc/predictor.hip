@@ -1,0 +1,115 @@
+// Host side of prediction: the reference's Predictor (src/thundergbm/predictor.cu:11-86).
+#include <cstring>
+
+#include "device_api.h"
+#include "host.h"
+
+namespace tgbm {
+
+static int transform_kind(const std::string &objective) {
+    if (objective == "binary:logistic") return 1;
+    if (objective == "multi:softmax") return 2;
+    if (objective == "multi:softprob") return 3;
+    if (objective == "reg:logistic") return 4;
+    return 0;
+}
+
+// Runs the traversal kernel and, if asked, the objective's transform and the training metric.
+static std::vector<float> run_predict(const GBMParam &param, const std::vector<std::vector<Tree>> &model,
+                                      const DataSet &ds, bool transform, bool log_metric) {
+    int n_dev = 0;
+    hipError_t e = hipGetDeviceCount(&n_dev);
+    TGBM_CHECK(e == hipSuccess && n_dev >= 1, "no HIP device available: this library has no CPU path");
+    const int n = (int)ds.n_instances();
+    const int F = (int)ds.n_features();
+    const long nnz = (long)ds.csr_val.size();
+    TGBM_CHECK(!model.empty() && !model.front().empty(), "empty model");
+    const int n_iter = (int)model.size();
+    const int nct = (int)model.front().size();
+    const int n_nodes = (int)model[0][0].nodes.size();
+    std::vector<TreeNode> flat((size_t)n_iter * nct * n_nodes);
+    size_t t = 0;
+    for (const auto &iter : model) {
+        TGBM_CHECK((int)iter.size() == nct, "ragged model");
+        for (const Tree &tr : iter) {
+            TGBM_CHECK((int)tr.nodes.size() == n_nodes, "trees of different size in one model");
+            std::memcpy(flat.data() + t * n_nodes, tr.nodes.data(), sizeof(TreeNode) * (size_t)n_nodes);
+            ++t;
+        }
+    }
+    hipStream_t s;
+    HIP_CHECK(hipStreamCreate(&s));
+    float *d_val = nullptr, *d_out = nullptr, *d_label = nullptr;
+    int *d_col = nullptr, *d_row_ptr = nullptr;
+    TreeNode *d_model = nullptr;
+    const size_t n_out = (size_t)n * nct;
+    HIP_CHECK(hipMalloc(&d_val, sizeof(float) * (size_t)std::max(nnz, 1l)));
+    HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz, 1l)));
+    HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n + 1)));
+    HIP_CHECK(hipMalloc(&d_model, sizeof(TreeNode) * flat.size()));
+    HIP_CHECK(hipMalloc(&d_out, sizeof(float) * std::max(n_out, (size_t)1)));
+    if (nnz) {
+        HIP_CHECK(hipMemcpyAsync(d_val, ds.csr_val.data(), sizeof(float) * (size_t)nnz, hipMemcpyHostToDevice, s));
+        HIP_CHECK(hipMemcpyAsync(d_col, ds.csr_col_idx.data(), sizeof(int) * (size_t)nnz, hipMemcpyHostToDevice, s));
+    }
+    HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.csr_row_ptr.data(), sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
+    HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));
+    launch_fill_f32(s, d_out, 0.f, n_out);
+    launch_predict(s, n, F, d_row_ptr, d_col, d_val, d_model, n_iter, nct, n_nodes, param.learning_rate,
+                   param.base_score, d_out);
+    size_t n_ret = n_out;
+    if (log_metric && (int)ds.y.size() == n && n > 0) {
+        int kind = 0;
+        if (param.objective == "binary:logistic") kind = 1;
+        if (param.objective.find("multi:") == 0) kind = 2;
+        static const char *names[] = {"RMSE", "test error", "multi-class accuracy"};
+        float *d_y = nullptr, *d_m = nullptr;
+        double *d_scratch = nullptr;
+        HIP_CHECK(hipMalloc(&d_y, sizeof(float) * (size_t)n));
+        HIP_CHECK(hipMalloc(&d_m, sizeof(float)));
+        HIP_CHECK(hipMalloc(&d_scratch, sizeof(double) * 1024));
+        HIP_CHECK(hipMemcpyAsync(d_y, ds.y.data(), sizeof(float) * (size_t)n, hipMemcpyHostToDevice, s));
+        launch_metric(s, kind, n, nct, d_y, d_out, d_scratch, d_m);
+        float v = 0;
+        HIP_CHECK(hipMemcpyAsync(&v, d_m, sizeof(float), hipMemcpyDeviceToHost, s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        log_info("%s = %g", names[kind], v);
+        HIP_CHECK(hipFree(d_y));
+        HIP_CHECK(hipFree(d_m));
+        HIP_CHECK(hipFree(d_scratch));
+    }
+    if (transform) {
+        const int kind = transform_kind(param.objective);
+        if (kind == 1 || kind == 2) {
+            const size_t need = kind == 1 ? 2 : (size_t)std::max(param.num_class, 1);
+            TGBM_CHECK(ds.label.size() >= need, "predict: %zu class labels given, %zu needed", ds.label.size(), need);
+            HIP_CHECK(hipMalloc(&d_label, sizeof(float) * ds.label.size()));
+            HIP_CHECK(hipMemcpyAsync(d_label, ds.label.data(), sizeof(float) * ds.label.size(), hipMemcpyHostToDevice, s));
+        }
+        launch_predict_transform(s, kind, n, kind == 2 || kind == 3 ? nct : param.num_class, d_label, d_out);
+        if (kind == 1 || kind == 2) n_ret = (size_t)n;
+    }
+    std::vector<float> out(n_ret);
+    if (n_ret) HIP_CHECK(hipMemcpyAsync(out.data(), d_out, sizeof(float) * n_ret, hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipFree(d_val));
+    HIP_CHECK(hipFree(d_col));
+    HIP_CHECK(hipFree(d_row_ptr));
+    HIP_CHECK(hipFree(d_model));
+    HIP_CHECK(hipFree(d_out));
+    if (d_label) HIP_CHECK(hipFree(d_label));
+    HIP_CHECK(hipStreamDestroy(s));
+    return out;
+}
+
+std::vector<float> predict_raw(const GBMParam &param, const std::vector<std::vector<Tree>> &model,
+                               const DataSet &dataset) {
+    return run_predict(param, model, dataset, false, false);
+}
+
+std::vector<float> predict(const GBMParam &param, const std::vector<std::vector<Tree>> &model, const DataSet &dataset,
+                           bool log_metric) {
+    return run_predict(param, model, dataset, true, log_metric);
+}
+
+}  // namespace tgbm

@@ -1,0 +1,357 @@
+// One-off data preparation on the device: quantile cut points (a stable LSD radix sort of
+// (feature, value) keys, run-length flags, exclusive scan, strided selection) and the dense
+// column-blocked bin matrix. Runs once per training call, outside the boosting loop.
+#include <algorithm>
+#include <vector>
+
+#include "device_api.h"
+
+namespace tgbm {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / 64;
+constexpr int kSortRounds = 64;               // keys per lane and tile
+constexpr int kSortTile = 64 * kSortRounds;   // keys per wavefront tile
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kBlock * kScanItems;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+__device__ __forceinline__ int lanes_below(unsigned long long mask) {
+    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
+}
+
+// Order-preserving map float -> uint32 (-0.0 is folded into +0.0 so that == duplicates share a key).
+__device__ __forceinline__ unsigned float_key(float v) {
+    if (v == 0.f) v = 0.f;
+    unsigned u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(unsigned k) {
+    unsigned u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+    return __uint_as_float(u);
+}
+
+__global__ void k_make_keys(long n, const float *__restrict__ val, const int *__restrict__ col,
+                            unsigned long long *__restrict__ keys) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        keys[i] = ((unsigned long long)(unsigned)col[i] << 32) | float_key(val[i]);
+}
+
+// ---- radix sort, 8 bits per pass; every wavefront owns one tile of kSortTile consecutive keys ----
+__global__ __launch_bounds__(kBlock) void k_radix_count(const unsigned long long *__restrict__ keys, long n, int shift,
+                                                       long n_tiles, unsigned *__restrict__ counts) {
+    __shared__ unsigned cnt[kWaves][256];
+    const int w = wave_id(), lane = lane_id();
+    const long tile = (long)blockIdx.x * kWaves + w;
+    for (int d = lane; d < 256; d += 64) cnt[w][d] = 0;
+    __syncthreads();
+    if (tile < n_tiles) {
+        const long base = tile * kSortTile;
+        for (int r = 0; r < kSortRounds; ++r) {
+            long i = base + (long)r * 64 + lane;
+            if (i < n) atomicAdd(&cnt[w][(unsigned)(keys[i] >> shift) & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    if (tile < n_tiles)
+        for (int d = lane; d < 256; d += 64) counts[(size_t)d * n_tiles + tile] = cnt[w][d];
+}
+
+__global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long long *__restrict__ in,
+                                                         unsigned long long *__restrict__ out, long n, int shift,
+                                                         long n_tiles, const unsigned *__restrict__ offsets) {
+    __shared__ unsigned run[kWaves][256];
+    const int w = wave_id(), lane = lane_id();
+    const long tile = (long)blockIdx.x * kWaves + w;
+    const bool live = tile < n_tiles;
+    if (live)
+        for (int d = lane; d < 256; d += 64) run[w][d] = offsets[(size_t)d * n_tiles + tile];
+    __syncthreads();
+    const long base = tile * kSortTile;
+    for (int r = 0; r < kSortRounds; ++r) {
+        long i = base + (long)r * 64 + lane;
+        bool valid = live && i < n;
+        unsigned long long key = valid ? in[i] : 0ull;
+        unsigned d = (unsigned)(key >> shift) & 255u;
+        // lanes holding the same digit (match-any built from eight ballots)
+        unsigned long long mask = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            bool bit = (d >> b) & 1u;
+            unsigned long long m = __ballot(bit);
+            mask &= bit ? m : ~m;
+        }
+        unsigned first = valid ? run[w][d] : 0u;
+        int rank = lanes_below(mask);
+        __syncthreads();
+        if (valid) {
+            out[(size_t)first + rank] = key;
+            if (rank == 0) run[w][d] = first + (unsigned)__popcll(mask);
+        }
+        __syncthreads();
+    }
+}
+
+// ---- exclusive scan of 32-bit counters (tile scan + recursive scan of tile sums + add) ----------
+template <bool FROM_KEYS>
+__device__ __forceinline__ unsigned scan_load(const void *in, long i) {
+    if (FROM_KEYS) {
+        const unsigned long long *k = static_cast<const unsigned long long *>(in);
+        return (i == 0 || k[i] != k[i - 1]) ? 1u : 0u;  // 1 at the first entry of every (feature, value) run
+    }
+    return static_cast<const unsigned *>(in)[i];
+}
+
+template <bool FROM_KEYS>
+__global__ __launch_bounds__(kBlock) void k_scan_tiles(const void *__restrict__ in, unsigned *__restrict__ out, long n,
+                                                      unsigned *__restrict__ tile_sums) {
+    __shared__ unsigned ws[kWaves];
+    const long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
+    unsigned v[kScanItems];
+    unsigned local = 0;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+        long i = base + j;
+        v[j] = i < n ? scan_load<FROM_KEYS>(in, i) : 0u;
+        local += v[j];
+    }
+    unsigned inc = local;
+    const int lane = lane_id(), w = wave_id();
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        unsigned t = __shfl_up(inc, d);
+        if (lane >= d) inc += t;
+    }
+    if (lane == 63) ws[w] = inc;
+    __syncthreads();
+    unsigned wbase = 0, tot = 0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) {
+        if (i < w) wbase += ws[i];
+        tot += ws[i];
+    }
+    unsigned run = wbase + inc - local;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+        long i = base + j;
+        if (i < n) out[i] = run;
+        run += v[j];
+    }
+    if (threadIdx.x == 0) tile_sums[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(kBlock) void k_scan_add(unsigned *__restrict__ out, long n,
+                                                    const unsigned *__restrict__ tile_offsets) {
+    const unsigned add = tile_offsets[blockIdx.x];
+    const long base = (long)blockIdx.x * kScanTile;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+        long i = base + (long)j * kBlock + threadIdx.x;
+        if (i < n) out[i] += add;
+    }
+}
+
+// out[i] = sum of in[0..i); returns nothing, the total is written to *d_total (device).
+template <bool FROM_KEYS>
+void exclusive_scan(hipStream_t s, const void *in, unsigned *out, long n, unsigned *d_total,
+                    std::vector<void *> &scratch) {
+    long tiles = (n + kScanTile - 1) / kScanTile;
+    unsigned *sums = nullptr;
+    HIP_CHECK(hipMalloc(&sums, sizeof(unsigned) * (size_t)(tiles + 1)));
+    scratch.push_back(sums);
+    k_scan_tiles<FROM_KEYS><<<(unsigned)tiles, kBlock, 0, s>>>(in, out, n, sums);
+    if (tiles > 1) {
+        unsigned *sums_scanned = nullptr;
+        HIP_CHECK(hipMalloc(&sums_scanned, sizeof(unsigned) * (size_t)(tiles + 1)));
+        scratch.push_back(sums_scanned);
+        exclusive_scan<false>(s, sums, sums_scanned, tiles, d_total, scratch);
+        k_scan_add<<<(unsigned)tiles, kBlock, 0, s>>>(out, n, sums_scanned);
+    } else {
+        HIP_CHECK(hipMemcpyAsync(d_total, sums, sizeof(unsigned), hipMemcpyDeviceToDevice, s));
+    }
+}
+
+// First sorted entry of every feature (binary search of f << 32), estart[F] = nnz.
+__global__ void k_feature_starts(const unsigned long long *__restrict__ keys, long n, int F, long *__restrict__ estart) {
+    for (int f = blockIdx.x * blockDim.x + threadIdx.x; f <= F; f += gridDim.x * blockDim.x) {
+        unsigned long long target = (unsigned long long)(unsigned)f << 32;
+        long lo = 0, hi = n;
+        while (lo < hi) {
+            long mid = lo + (hi - lo) / 2;
+            if (keys[mid] < target)
+                lo = mid + 1;
+            else
+                hi = mid;
+        }
+        estart[f] = lo;
+    }
+}
+
+// ustart[f] = number of distinct (feature, value) pairs of features < f.
+__global__ void k_unique_starts(const long *__restrict__ estart, const unsigned *__restrict__ uidx, long n, int F,
+                                const unsigned *__restrict__ d_total, unsigned *__restrict__ ustart) {
+    for (int f = blockIdx.x * blockDim.x + threadIdx.x; f <= F; f += gridDim.x * blockDim.x) {
+        long e = estart[f];
+        ustart[f] = e < n ? uidx[e] : *d_total;
+    }
+}
+
+// Strided selection of the reference (hist_cut.cu:259-265): with m distinct values and
+// step = m / max_bin, keep all of them if step == 0, else the values at ranks 0, step, 2 step, ...
+// (max_bin of them).
+__global__ void k_emit_cuts(const unsigned long long *__restrict__ keys, const unsigned *__restrict__ uidx, long n,
+                            const unsigned *__restrict__ ustart, const int *__restrict__ cut_row_ptr, int max_bin,
+                            float *__restrict__ cut_val, int *__restrict__ cut_fid) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        unsigned long long k = keys[i];
+        if (i != 0 && k == keys[i - 1]) continue;
+        int f = (int)(k >> 32);
+        unsigned j = uidx[i] - ustart[f];
+        unsigned m = ustart[f + 1] - ustart[f];
+        unsigned step = m / (unsigned)max_bin;
+        int out = -1;
+        if (step == 0)
+            out = cut_row_ptr[f] + (int)j;
+        else if (j % step == 0 && j / step < (unsigned)max_bin)
+            out = cut_row_ptr[f] + (int)(j / step);
+        if (out >= 0) {
+            cut_val[out] = key_float((unsigned)k);
+            cut_fid[out] = f;
+        }
+    }
+}
+
+// Bin of a stored value (the reference's clamped upper bound, hist_tree_builder_single.cu:81-119):
+// min(#cuts <= v, k - 1), as a local (per-feature) bin id.
+__device__ __forceinline__ int local_bin(const float *__restrict__ cuts, int k, float v) {
+    int left = 0, right = k - 1;
+    while (left < right) {
+        int mid = left + (right - left) / 2;
+        if (cuts[mid] <= v)
+            left = mid + 1;
+        else
+            right = mid;
+    }
+    return left;
+}
+
+__global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
+                            const float *__restrict__ val, const float *__restrict__ cut_val,
+                            const int *__restrict__ cut_row_ptr, uint8_t *__restrict__ binmat, int W,
+                            size_t block_stride) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        for (int e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
+            int f = col[e];
+            int cb = cut_row_ptr[f];
+            int k = cut_row_ptr[f + 1] - cb;
+            int b = local_bin(cut_val + cb, k, val[e]);
+            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (uint8_t)b;
+        }
+    }
+}
+
+__global__ void k_bin_csr(long nnz, const int *__restrict__ col, const float *__restrict__ val,
+                          const float *__restrict__ cut_val, const int *__restrict__ cut_row_ptr,
+                          int *__restrict__ bin_id) {
+    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (long)gridDim.x * blockDim.x) {
+        int f = col[e];
+        int cb = cut_row_ptr[f];
+        int k = cut_row_ptr[f + 1] - cb;
+        bin_id[e] = cb + local_bin(cut_val + cb, k, val[e]);
+    }
+}
+
+int grid_for(size_t n, int cap = 8192) {
+    size_t b = (n + kBlock - 1) / kBlock;
+    if (b < 1) b = 1;
+    if (b > (size_t)cap) b = cap;
+    return (int)b;
+}
+
+}  // namespace
+
+// Cut points of the reference's HistCut::get_cut_points_single (src/thundergbm/hist_cut.cu:232-286).
+DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, const int *d_col, int max_num_bin) {
+    DeviceCuts out;
+    HIP_CHECK(hipMalloc(&out.cut_row_ptr, sizeof(int) * (size_t)(F + 1)));
+    if (nnz == 0) {
+        HIP_CHECK(hipMemsetAsync(out.cut_row_ptr, 0, sizeof(int) * (size_t)(F + 1), s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        return out;
+    }
+    std::vector<void *> scratch;
+    unsigned long long *keys[2];
+    HIP_CHECK(hipMalloc(&keys[0], sizeof(unsigned long long) * (size_t)nnz));
+    HIP_CHECK(hipMalloc(&keys[1], sizeof(unsigned long long) * (size_t)nnz));
+    k_make_keys<<<grid_for(nnz), kBlock, 0, s>>>(nnz, d_val, d_col, keys[0]);
+
+    int fid_bits = 0;
+    while ((1ll << fid_bits) < (long long)F) ++fid_bits;
+    const int passes = (32 + fid_bits + 7) / 8;
+    const long n_tiles = (nnz + kSortTile - 1) / kSortTile;
+    const size_t n_counts = (size_t)256 * n_tiles;
+    unsigned *counts = nullptr, *offsets = nullptr, *d_total = nullptr;
+    HIP_CHECK(hipMalloc(&counts, sizeof(unsigned) * n_counts));
+    HIP_CHECK(hipMalloc(&offsets, sizeof(unsigned) * (n_counts + 1)));
+    HIP_CHECK(hipMalloc(&d_total, sizeof(unsigned)));
+    const unsigned sort_grid = (unsigned)((n_tiles + kWaves - 1) / kWaves);
+    int cur = 0;
+    for (int p = 0; p < passes; ++p) {
+        const int shift = 8 * p;
+        k_radix_count<<<sort_grid, kBlock, 0, s>>>(keys[cur], nnz, shift, n_tiles, counts);
+        exclusive_scan<false>(s, counts, offsets, (long)n_counts, d_total, scratch);
+        k_radix_scatter<<<sort_grid, kBlock, 0, s>>>(keys[cur], keys[cur ^ 1], nnz, shift, n_tiles, offsets);
+        cur ^= 1;
+    }
+    const unsigned long long *sorted = keys[cur];
+    unsigned *uidx = nullptr;
+    HIP_CHECK(hipMalloc(&uidx, sizeof(unsigned) * (size_t)nnz));
+    exclusive_scan<true>(s, sorted, uidx, nnz, d_total, scratch);
+    long *estart = nullptr;
+    unsigned *ustart = nullptr;
+    HIP_CHECK(hipMalloc(&estart, sizeof(long) * (size_t)(F + 1)));
+    HIP_CHECK(hipMalloc(&ustart, sizeof(unsigned) * (size_t)(F + 1)));
+    k_feature_starts<<<grid_for(F + 1), kBlock, 0, s>>>(sorted, nnz, F, estart);
+    k_unique_starts<<<grid_for(F + 1), kBlock, 0, s>>>(estart, uidx, nnz, F, d_total, ustart);
+    std::vector<unsigned> h_ustart(F + 1);
+    HIP_CHECK(hipMemcpyAsync(h_ustart.data(), ustart, sizeof(unsigned) * (size_t)(F + 1), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    std::vector<int> h_crp(F + 1, 0);
+    for (int f = 0; f < F; ++f) {
+        unsigned m = h_ustart[f + 1] - h_ustart[f];
+        unsigned k = (m / (unsigned)max_num_bin == 0) ? m : (unsigned)max_num_bin;
+        h_crp[f + 1] = h_crp[f] + (int)k;
+    }
+    out.n_bins = h_crp[F];
+    HIP_CHECK(hipMemcpyAsync(out.cut_row_ptr, h_crp.data(), sizeof(int) * (size_t)(F + 1), hipMemcpyHostToDevice, s));
+    HIP_CHECK(hipMalloc(&out.cut_val, sizeof(float) * (size_t)std::max(out.n_bins, 1)));
+    HIP_CHECK(hipMalloc(&out.cut_fid, sizeof(int) * (size_t)std::max(out.n_bins, 1)));
+    k_emit_cuts<<<grid_for(nnz), kBlock, 0, s>>>(sorted, uidx, nnz, ustart, out.cut_row_ptr, max_num_bin, out.cut_val,
+                                               out.cut_fid);
+    HIP_CHECK(hipStreamSynchronize(s));
+    for (void *p : scratch) HIP_CHECK(hipFree(p));
+    HIP_CHECK(hipFree(keys[0]));
+    HIP_CHECK(hipFree(keys[1]));
+    HIP_CHECK(hipFree(counts));
+    HIP_CHECK(hipFree(offsets));
+    HIP_CHECK(hipFree(d_total));
+    HIP_CHECK(hipFree(uidx));
+    HIP_CHECK(hipFree(estart));
+    HIP_CHECK(hipFree(ustart));
+    return out;
+}
+
+void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
+                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride) {
+    k_bin_dense<<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride);
+}
+
+void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
+                    const int *cut_row_ptr, int *bin_id) {
+    if (nnz == 0) return;
+    k_bin_csr<<<grid_for(nnz), kBlock, 0, s>>>(nnz, col, val, cut_val, cut_row_ptr, bin_id);
+}
+
+}  // namespace tgbm

@@ -1,0 +1,91 @@
+// Device trainer: owns every HBM buffer of a training session and drives the kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "device_api.h"
+#include "host.h"
+
+namespace tgbm {
+
+struct HistProfile {
+    double hist_ms = 0;          // summed duration of the histogram-build launches
+    long long hist_launches = 0;
+    long long rows_built = 0;    // rows visited by those launches
+    long long hist_bytes = 0;    // algorithmic bytes of those launches
+};
+
+class Trainer {
+   public:
+    // Uploads the dataset, builds cut points and bin ids on the device and initialises the base
+    // score (HistTreeBuilder_single::init + Booster::init of the reference).
+    Trainer(const DataSet &dataset, GBMParam &param);
+    ~Trainer();
+    Trainer(const Trainer &) = delete;
+    Trainer &operator=(const Trainer &) = delete;
+
+    // One call = `rounds` iterations of Booster::boost: gradients, tree_per_rounds trees, metric.
+    void boost(int rounds);
+    // step-wise driving (used by parity tests)
+    void compute_gradient();
+    void tree_init(int k);
+    void find_split(int level);  // histogram, merge/subtract, split search, update_tree
+    void partition(int level);   // update_ins2node_id + next level's row lists
+    void finish_tree(int k);     // prune, prediction update, append the tree to the model
+    float metric();
+    void sync();
+
+    // results
+    std::vector<std::vector<Tree>> model_to_host();
+    std::vector<float> metric_log();
+    const GBMParam &param() const { return param_; }
+    int info(const std::string &key) const;
+    size_t get(const std::string &name, void *out, size_t cap);  // returns bytes, copies if cap suffices
+    void set(const std::string &name, const void *in, size_t bytes);
+    void set_profiling(bool on);
+    HistProfile profile();
+
+   private:
+    void build_level(int level);
+    void alloc_tree_buffers();
+    template <typename T>
+    T *dalloc(size_t count);
+
+    GBMParam param_;
+    hipStream_t stream_ = nullptr;
+    int n_ = 0, F_ = 0, n_bins_ = 0;
+    long nnz_ = 0;
+    int objective_ = OBJ_SQUARE, metric_kind_ = 0;
+    std::vector<void *> allocs_;
+    // dataset
+    float *d_y_ = nullptr;
+    float *d_yp_ = nullptr;
+    long n_yp_ = 0;
+    GHPair *d_gh_ = nullptr;
+    DeviceCuts cuts_;
+    std::vector<int> h_cut_row_ptr_;
+    uint8_t *d_binmat_ = nullptr;
+    DenseBins bins_;
+    TreeBuffers tb_;
+    // model
+    TreeNode *d_model_ = nullptr;
+    int trees_built_ = 0, rounds_done_ = 0, model_cap_trees_ = 0;
+    float *d_metric_ = nullptr;
+    double *d_metric_scratch_ = nullptr;
+    int cur_class_ = 0;
+    // profiling
+    bool profiling_ = false;
+    struct HistEvent {
+        hipEvent_t start, stop;
+        int level;
+        int tree;
+    };
+    std::vector<HistEvent> events_;
+    std::vector<LevelCtl> ctl_log_;  // per tree, depth + 1 entries (copied at tree end when profiling)
+    HistProfile prof_;
+};
+
+}  // namespace tgbm

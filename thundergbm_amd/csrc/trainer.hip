@@ -1,0 +1,468 @@
+// Host orchestration of a training session on one MI355X: Booster::init / Booster::boost /
+// TreeBuilder::build_approximate of the reference (include/thundergbm/booster.h:36-93,
+// src/thundergbm/builder/tree_builder.cu:147-194), restructured so that a whole tree is a
+// stream-ordered chain of level-wide launches without host synchronisation.
+#include "trainer.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+
+namespace tgbm {
+
+template <typename T>
+T *Trainer::dalloc(size_t count) {
+    void *p = nullptr;
+    if (count == 0) count = 1;
+    HIP_CHECK(hipMalloc(&p, count * sizeof(T)));
+    allocs_.push_back(p);
+    return static_cast<T *>(p);
+}
+
+template <typename T>
+static T *upload(hipStream_t s, T *dst, const T *src, size_t count) {
+    if (count) HIP_CHECK(hipMemcpyAsync(dst, src, count * sizeof(T), hipMemcpyHostToDevice, s));
+    return dst;
+}
+
+Trainer::Trainer(const DataSet &ds, GBMParam &param) {
+    int n_dev = 0;
+    hipError_t e = hipGetDeviceCount(&n_dev);
+    TGBM_CHECK(e == hipSuccess && n_dev >= 1, "no HIP device available: this library has no CPU path");
+    HIP_CHECK(hipStreamCreate(&stream_));
+    n_ = (int)ds.n_instances();
+    F_ = (int)ds.n_features();
+    nnz_ = (long)ds.csr_val.size();
+    TGBM_CHECK(n_ > 0, "empty dataset");
+    TGBM_CHECK(param.depth >= 1 && param.depth <= 14, "depth %d out of the supported range 1..14", param.depth);
+    TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 255,
+               "max_num_bin %d out of the supported range 2..255", param.max_num_bin);
+    TGBM_CHECK(objective_supported(param.objective), "undefined objective %s", param.objective.c_str());
+    if (param.bagging || param.column_sampling_rate < 1.f)
+        log_info("bagging / column sampling are not part of this build and are ignored");
+    // class bookkeeping of TreeTrainer::train (src/thundergbm/trainer.cu:24-37)
+    if (param.objective.find("multi:") != std::string::npos || param.objective.find("binary:") != std::string::npos) {
+        int nc = (int)ds.label.size();
+        if (param.num_class != nc) {
+            log_info("updating number of classes from %d to %d", param.num_class, nc);
+            param.num_class = nc;
+        }
+        if (param.num_class > 2) param.tree_per_rounds = param.num_class;
+    } else if (param.objective.find("reg:") != std::string::npos) {
+        param.num_class = 1;
+    }
+    if (param.objective == "reg:linear") {
+        objective_ = OBJ_SQUARE;
+        metric_kind_ = 0;
+    } else if (param.objective == "reg:logistic") {
+        objective_ = OBJ_LOGISTIC;
+        metric_kind_ = 0;
+    } else if (param.objective == "binary:logistic") {
+        objective_ = OBJ_LOGISTIC;
+        metric_kind_ = 1;
+        TGBM_CHECK(ds.label.size() == 2, "binary:logistic needs exactly two distinct labels, got %zu",
+                   ds.label.size());
+    } else {
+        objective_ = OBJ_SOFTMAX;
+        metric_kind_ = 2;
+        // the reference aborts here as well (tree_builder.cu:87-90 vs multiclass_obj.cu:8)
+        TGBM_CHECK(param.num_class != 2, "multi:softmax/softprob with two classes is not supported; use binary:logistic");
+    }
+    param_ = param;
+
+    // ---- upload CSR, cut points, bin matrix --------------------------------------------------
+    float *d_val = nullptr;
+    int *d_col = nullptr, *d_row_ptr = nullptr;
+    HIP_CHECK(hipMalloc(&d_val, sizeof(float) * (size_t)std::max(nnz_, 1l)));
+    HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz_, 1l)));
+    HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n_ + 1)));
+    upload(stream_, d_val, ds.csr_val.data(), (size_t)nnz_);
+    upload(stream_, d_col, ds.csr_col_idx.data(), (size_t)nnz_);
+    upload(stream_, d_row_ptr, ds.csr_row_ptr.data(), (size_t)n_ + 1);
+    log_info("Fast getting cut points...");
+    cuts_ = build_cut_points(stream_, F_, nnz_, d_val, d_col, param_.max_num_bin);
+    n_bins_ = cuts_.n_bins;
+    allocs_.push_back(cuts_.cut_row_ptr);
+    if (cuts_.cut_val) allocs_.push_back(cuts_.cut_val);
+    if (cuts_.cut_fid) allocs_.push_back(cuts_.cut_fid);
+    log_info("TOTAL CP:%d", n_bins_);
+    log_info("NNZ: %ld", nnz_);
+    TGBM_CHECK(n_bins_ > 0, "the dataset has no stored feature value");
+    h_cut_row_ptr_.resize(F_ + 1);
+    HIP_CHECK(hipMemcpyAsync(h_cut_row_ptr_.data(), cuts_.cut_row_ptr, sizeof(int) * (size_t)(F_ + 1),
+                             hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+
+    // dense column-blocked layout: blocks of W features, each block n rows x W bytes
+    int W;
+    if (F_ <= 32) {
+        W = 4;
+        while (W < F_) W *= 2;
+    } else if (F_ <= 64 && n_bins_ <= 12288) {
+        W = 64;
+    } else {
+        W = 32;
+    }
+    const int n_blocks = (F_ + W - 1) / W;
+    const size_t mat_bytes = (size_t)n_ * W * n_blocks;
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    TGBM_CHECK(mat_bytes < free_b / 2,
+               "dense bin matrix of %zu bytes does not fit (free %zu); the sparse histogram path is not built yet",
+               mat_bytes, free_b);
+    d_binmat_ = dalloc<uint8_t>(mat_bytes);
+    launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);
+    launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
+                     (size_t)n_ * W);
+    bins_.data = d_binmat_;
+    bins_.W = W;
+    bins_.n_blocks = n_blocks;
+    bins_.block_stride = (size_t)n_ * W;
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    HIP_CHECK(hipFree(d_val));
+    HIP_CHECK(hipFree(d_col));
+    HIP_CHECK(hipFree(d_row_ptr));
+
+    // ---- labels, predictions, gradients (Booster::init) --------------------------------------
+    d_y_ = dalloc<float>(n_);
+    upload(stream_, d_y_, ds.y.data(), (size_t)n_);
+    n_yp_ = (long)param_.num_class * n_;
+    if (param_.num_class == 2) n_yp_ = n_;
+    d_yp_ = dalloc<float>((size_t)n_yp_);
+    launch_fill_f32(stream_, d_yp_, 0.f, (size_t)n_yp_);
+    d_gh_ = dalloc<GHPair>((size_t)param_.num_class * n_);
+    launch_fill_f32(stream_, reinterpret_cast<float *>(d_gh_), 0.f, (size_t)param_.num_class * n_ * 2);
+    alloc_tree_buffers();
+
+    // base score (regression_obj.h:35-53, :95-114; only for squared / logistic objectives)
+    if (objective_ != OBJ_SOFTMAX) {
+        launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
+        launch_tree_init(stream_, tb_, d_gh_, param_.lambda);  // reuses the root-sum reduction
+        TreeNode root;
+        HIP_CHECK(hipMemcpyAsync(&root, tb_.nodes, sizeof(TreeNode), hipMemcpyDeviceToHost, stream_));
+        HIP_CHECK(hipStreamSynchronize(stream_));
+        float weight = (float)(-root.sum_gh_pair.g / std::fmax((double)root.sum_gh_pair.h, 1e-6));
+        float base = weight;
+        if (param_.objective == "binary:logistic") {
+            weight = 1 / (1 + expf(-weight));
+            base = -logf(1.0f / weight - 1.0f);
+        }
+        log_info("base_score %g", base);
+        param_.base_score = base;
+        launch_fill_f32(stream_, d_yp_, base, (size_t)n_yp_);
+    } else {
+        param_.base_score = 0;
+    }
+    param.base_score = param_.base_score;
+    HIP_CHECK(hipStreamSynchronize(stream_));
+}
+
+void Trainer::alloc_tree_buffers() {
+    TreeBuffers &tb = tb_;
+    const int depth = param_.depth;
+    tb.n = n_;
+    tb.n_bins = n_bins_;
+    tb.F = F_;
+    tb.depth = depth;
+    tb.n_nodes = (1 << (depth + 1)) - 1;
+    const int max_level_nodes = 1 << (depth - 1 > 0 ? depth - 1 : 0);
+    const int max_pairs = std::max(1, max_level_nodes / 2);
+    tb.nodes = dalloc<TreeNode>(tb.n_nodes);
+    tb.seg = dalloc<int2>(tb.n_nodes);
+    tb.nid = dalloc<int>(n_);
+    tb.ridx[0] = dalloc<int>(n_);
+    tb.ridx[1] = dalloc<int>(n_);
+    tb.goes_right = dalloc<uint8_t>((size_t)n_ + 4);
+    tb.hist[0] = dalloc<GHPair>((size_t)max_level_nodes * n_bins_);
+    tb.hist[1] = dalloc<GHPair>((size_t)max_level_nodes * n_bins_);
+    tb.target_hitems = std::min(1024, std::max(4, 1024 / bins_.n_blocks));
+    tb.max_hitems = tb.target_hitems + max_pairs + 1;
+    tb.partial = dalloc<GHPair>((size_t)tb.max_hitems * n_bins_);
+    tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
+    // the planning kernel of the last level also writes the (unused) plan of level `depth`
+    tb.hpair_begin = dalloc<int>((size_t)max_level_nodes + 1);
+    tb.hpair_built = dalloc<int>((size_t)max_level_nodes);
+    tb.pitem_begin = dalloc<int>((size_t)max_level_nodes + 1);
+    tb.pitem_nleft = dalloc<int>((size_t)tb.max_pitems + 1);
+    tb.pitem_loff = dalloc<int>((size_t)tb.max_pitems + 1);
+    tb.node_nleft = dalloc<int>((size_t)max_level_nodes);
+    tb.ctl = dalloc<LevelCtl>((size_t)depth + 2);
+    tb.sp = dalloc<SplitPoint>((size_t)max_level_nodes);
+    tb.n_grad_blocks = std::min(1024, (n_ + 255) / 256);
+    tb.root_partial = dalloc<GHPair>((size_t)tb.n_grad_blocks);
+    tb.cut_row_ptr = cuts_.cut_row_ptr;
+    tb.cut_fid = cuts_.cut_fid;
+    tb.cut_val = cuts_.cut_val;
+
+    // split-finder packs: whole features, at most kEvalPackBins bins per wavefront
+    std::vector<int> pack_begin;
+    pack_begin.push_back(0);
+    int cur = 0;
+    for (int f = 0; f < F_; ++f) {
+        int k = h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f];
+        if (k == 0) continue;
+        TGBM_CHECK(k <= kEvalPackBins, "feature %d has %d cut points, more than %d", f, k, kEvalPackBins);
+        if (cur + k > kEvalPackBins) {
+            pack_begin.push_back(h_cut_row_ptr_[f]);
+            cur = 0;
+        }
+        cur += k;
+    }
+    pack_begin.push_back(n_bins_);
+    tb.n_packs = (int)pack_begin.size() - 1;
+    int *d_pack = dalloc<int>(pack_begin.size());
+    upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
+    tb.pack_begin = d_pack;
+    tb.cand = dalloc<SplitCand>((size_t)max_level_nodes * tb.n_packs);
+
+    // dense block tables
+    const int W = bins_.W, nb = bins_.n_blocks;
+    std::vector<int> blk_begin(nb + 1), feat_off((size_t)nb * W, 0);
+    int max_block_bins = 0;
+    for (int b = 0; b <= nb; ++b) blk_begin[b] = h_cut_row_ptr_[std::min(b * W, F_)];
+    for (int b = 0; b < nb; ++b) {
+        max_block_bins = std::max(max_block_bins, blk_begin[b + 1] - blk_begin[b]);
+        for (int j = 0; j < W; ++j) {
+            int f = b * W + j;
+            feat_off[(size_t)b * W + j] = f < F_ ? h_cut_row_ptr_[f] - blk_begin[b] : 0;
+        }
+    }
+    TGBM_CHECK((size_t)max_block_bins * 8 <= 160 * 1024, "feature block histogram exceeds the LDS");
+    tb.max_block_bins = max_block_bins;
+    int *d_blk = dalloc<int>(blk_begin.size());
+    int *d_off = dalloc<int>(feat_off.size());
+    upload(stream_, d_blk, blk_begin.data(), blk_begin.size());
+    upload(stream_, d_off, feat_off.data(), feat_off.size());
+    tb.blk_bin_begin = d_blk;
+    tb.feat_lds_off = d_off;
+    HIP_CHECK(hipStreamSynchronize(stream_));  // the host vectors above go out of scope
+
+    model_cap_trees_ = std::max(1, param_.n_trees) * param_.tree_per_rounds;
+    d_model_ = dalloc<TreeNode>((size_t)model_cap_trees_ * tb.n_nodes);
+    d_metric_ = dalloc<float>((size_t)std::max(1, param_.n_trees));
+    d_metric_scratch_ = dalloc<double>(1024);
+}
+
+Trainer::~Trainer() {
+    if (stream_) (void)hipStreamSynchronize(stream_);
+    for (auto &ev : events_) {
+        (void)hipEventDestroy(ev.start);
+        (void)hipEventDestroy(ev.stop);
+    }
+    for (void *p : allocs_) (void)hipFree(p);
+    if (stream_) (void)hipStreamDestroy(stream_);
+}
+
+void Trainer::sync() { HIP_CHECK(hipStreamSynchronize(stream_)); }
+
+void Trainer::compute_gradient() {
+    launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
+}
+
+void Trainer::tree_init(int k) {
+    cur_class_ = k;
+    launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda);
+}
+
+void Trainer::find_split(int level) {
+    const GHPair *gh = d_gh_ + (size_t)cur_class_ * n_;
+    if (profiling_) {
+        HistEvent ev;
+        HIP_CHECK(hipEventCreate(&ev.start));
+        HIP_CHECK(hipEventCreate(&ev.stop));
+        ev.level = level;
+        ev.tree = trees_built_;
+        HIP_CHECK(hipEventRecord(ev.start, stream_));
+        launch_hist_dense(stream_, tb_, bins_, gh, level);
+        HIP_CHECK(hipEventRecord(ev.stop, stream_));
+        events_.push_back(ev);
+    } else {
+        launch_hist_dense(stream_, tb_, bins_, gh, level);
+    }
+    launch_hist_merge(stream_, tb_, level);
+    launch_eval_split(stream_, tb_, level, param_.min_child_weight, param_.lambda);
+    launch_best_update(stream_, tb_, level, param_.rt_eps, param_.lambda);
+}
+
+void Trainer::partition(int level) { launch_partition_dense(stream_, tb_, bins_, level); }
+
+void Trainer::finish_tree(int k) {
+    launch_prune(stream_, tb_, param_.gamma);
+    launch_predict_in_training(stream_, tb_, d_yp_ + (size_t)k * n_, param_.learning_rate);
+    TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
+    HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb_.n_nodes, tb_.nodes,
+                             sizeof(TreeNode) * (size_t)tb_.n_nodes, hipMemcpyDeviceToDevice, stream_));
+    if (profiling_) {
+        size_t off = ctl_log_.size();
+        ctl_log_.resize(off + param_.depth + 1);
+        HIP_CHECK(hipMemcpyAsync(ctl_log_.data() + off, tb_.ctl, sizeof(LevelCtl) * (size_t)(param_.depth + 1),
+                                 hipMemcpyDeviceToHost, stream_));
+        HIP_CHECK(hipStreamSynchronize(stream_));
+    }
+    ++trees_built_;
+}
+
+float Trainer::metric() {
+    float *slot = d_metric_ + std::min(rounds_done_, std::max(1, param_.n_trees) - 1);
+    launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+    float v = 0;
+    HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    return v;
+}
+
+void Trainer::boost(int rounds) {
+    static const char *names[] = {"RMSE", "test error", "multi-class accuracy"};
+    for (int r = 0; r < rounds; ++r) {
+        TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
+        compute_gradient();
+        for (int k = 0; k < param_.tree_per_rounds; ++k) {
+            tree_init(k);
+            // The reference leaves the level loop when no row sits in a node that was split
+            // (tree_builder.cu:174-181). Running the remaining levels is a no-op on every output
+            // (no valid node, no work item), so the loop is not cut short and needs no readback.
+            for (int level = 0; level < param_.depth; ++level) {
+                find_split(level);
+                partition(level);
+            }
+            finish_tree(k);
+        }
+        float *slot = d_metric_ + rounds_done_;
+        launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+        if (g_verbose >= 1) {
+            float v = 0;
+            HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
+            HIP_CHECK(hipStreamSynchronize(stream_));
+            log_info("[%d/%d] %s = %g", rounds_done_ + 1, param_.n_trees, names[metric_kind_], v);
+        }
+        ++rounds_done_;
+    }
+}
+
+std::vector<std::vector<Tree>> Trainer::model_to_host() {
+    sync();
+    std::vector<TreeNode> flat((size_t)trees_built_ * tb_.n_nodes);
+    if (!flat.empty())
+        HIP_CHECK(hipMemcpy(flat.data(), d_model_, flat.size() * sizeof(TreeNode), hipMemcpyDeviceToHost));
+    std::vector<std::vector<Tree>> out;
+    const int tpr = param_.tree_per_rounds;
+    for (int t = 0; t < trees_built_; ++t) {
+        if (t % tpr == 0) out.emplace_back();
+        Tree tr;
+        tr.nodes.assign(flat.begin() + (size_t)t * tb_.n_nodes, flat.begin() + (size_t)(t + 1) * tb_.n_nodes);
+        out.back().push_back(std::move(tr));
+    }
+    return out;
+}
+
+std::vector<float> Trainer::metric_log() {
+    sync();
+    std::vector<float> v((size_t)rounds_done_);
+    if (!v.empty()) HIP_CHECK(hipMemcpy(v.data(), d_metric_, v.size() * sizeof(float), hipMemcpyDeviceToHost));
+    return v;
+}
+
+void Trainer::set_profiling(bool on) {
+    sync();
+    profiling_ = on;
+}
+
+HistProfile Trainer::profile() {
+    sync();
+    HistProfile p;
+    const int W = bins_.W;
+    for (size_t i = 0; i < events_.size(); ++i) {
+        float ms = 0;
+        HIP_CHECK(hipEventElapsedTime(&ms, events_[i].start, events_[i].stop));
+        p.hist_ms += ms;
+        p.hist_launches++;
+    }
+    // algorithmic bytes: every visited row reads its bin bytes (one per feature), its gradient pair
+    // and, below the root, its row index; every launch writes the level's built histograms once.
+    const int per_tree = param_.depth + 1;
+    for (size_t t = 0; t * per_tree < ctl_log_.size(); ++t) {
+        for (int level = 0; level < param_.depth; ++level) {
+            const LevelCtl &c = ctl_log_[t * per_tree + level];
+            p.rows_built += c.rows_built;
+            p.hist_bytes += (long long)c.rows_built * (F_ + 8 + (level > 0 ? 4 : 0));
+        }
+    }
+    (void)W;
+    return p;
+}
+
+int Trainer::info(const std::string &key) const {
+    if (key == "n") return n_;
+    if (key == "n_features") return F_;
+    if (key == "n_bins") return n_bins_;
+    if (key == "num_class") return param_.num_class;
+    if (key == "tree_per_rounds") return param_.tree_per_rounds;
+    if (key == "n_nodes") return tb_.n_nodes;
+    if (key == "dense_W") return bins_.W;
+    if (key == "dense_blocks") return bins_.n_blocks;
+    if (key == "trees_built") return trees_built_;
+    if (key == "rounds_done") return rounds_done_;
+    if (key == "n_packs") return tb_.n_packs;
+    if (key == "depth") return param_.depth;
+    if (key == "y_pred_size") return (int)n_yp_;
+    if (key == "max_hitems") return tb_.max_hitems;
+    fatal("unknown info key %s", key.c_str());
+}
+
+size_t Trainer::get(const std::string &name, void *out, size_t cap) {
+    sync();
+    const void *src = nullptr;
+    size_t bytes = 0;
+    const int max_level_nodes = 1 << (param_.depth - 1 > 0 ? param_.depth - 1 : 0);
+    if (name == "cut_val") src = cuts_.cut_val, bytes = sizeof(float) * (size_t)n_bins_;
+    else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
+    else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
+    else if (name == "binmat") src = d_binmat_, bytes = (size_t)n_ * bins_.W * bins_.n_blocks;
+    else if (name == "nid") src = tb_.nid, bytes = sizeof(int) * (size_t)n_;
+    else if (name == "gh") src = d_gh_, bytes = sizeof(GHPair) * (size_t)param_.num_class * n_;
+    else if (name == "y_pred") src = d_yp_, bytes = sizeof(float) * (size_t)n_yp_;
+    else if (name == "y") src = d_y_, bytes = sizeof(float) * (size_t)n_;
+    else if (name == "nodes") src = tb_.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
+    else if (name == "sp") src = tb_.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
+    else if (name == "hist0") src = tb_.hist[0], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "hist1") src = tb_.hist[1], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "ctl") src = tb_.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
+    else if (name == "seg") src = tb_.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;
+    else if (name == "ridx0") src = tb_.ridx[0], bytes = sizeof(int) * (size_t)n_;
+    else if (name == "ridx1") src = tb_.ridx[1], bytes = sizeof(int) * (size_t)n_;
+    else if (name == "model") src = d_model_, bytes = sizeof(TreeNode) * (size_t)trees_built_ * tb_.n_nodes;
+    else if (name == "metric_log") src = d_metric_, bytes = sizeof(float) * (size_t)rounds_done_;
+    else fatal("unknown buffer %s", name.c_str());
+    if (out != nullptr && cap >= bytes && bytes > 0) HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
+    return bytes;
+}
+
+void Trainer::set(const std::string &name, const void *in, size_t bytes) {
+    sync();
+    void *dst = nullptr;
+    size_t want = 0;
+    if (name == "gh") dst = d_gh_, want = sizeof(GHPair) * (size_t)param_.num_class * n_;
+    else if (name == "y_pred") dst = d_yp_, want = sizeof(float) * (size_t)n_yp_;
+    else fatal("buffer %s cannot be set", name.c_str());
+    TGBM_CHECK(bytes == want, "set %s: got %zu bytes, expected %zu", name.c_str(), bytes, want);
+    HIP_CHECK(hipMemcpy(dst, in, bytes, hipMemcpyHostToDevice));
+}
+
+// ---------------------------------------------------------------------------------------------
+// TreeTrainer::train (src/thundergbm/trainer.cu:18-57)
+std::vector<std::vector<Tree>> train(GBMParam &param, const DataSet &dataset) {
+    if (param.tree_method == "auto") param.tree_method = "hist";  // this build has the histogram method only
+    TGBM_CHECK(param.tree_method == "hist", "tree_method %s is not part of this build (hist only)",
+               param.tree_method.c_str());
+    if (param.n_device != 1) log_info("n_gpus=%d requested; this build trains on one GPU", param.n_device);
+    Trainer trainer(dataset, param);
+    auto start = std::chrono::high_resolution_clock::now();
+    trainer.boost(param.n_trees);
+    trainer.sync();
+    auto stop = std::chrono::high_resolution_clock::now();
+    log_info("training time = %g", std::chrono::duration<float>(stop - start).count());
+    return trainer.model_to_host();
+}
+
+}  // namespace tgbm

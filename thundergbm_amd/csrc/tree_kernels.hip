@@ -1,0 +1,1002 @@
+// Tree-building kernels for gfx950 (wave64): gradients, LDS-privatised histograms, merge + sibling
+// subtraction, wavefront segmented-scan split finding, ballot/popcount row partition, pruning and the
+// in-training prediction update. Every stage of a level is one launch over all nodes of the level;
+// work lists are planned on the device so the host never waits inside a tree.
+#include "device_api.h"
+
+namespace tgbm {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / 64;
+constexpr int kHistMinChunk = 1024;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+__device__ __forceinline__ int lanes_below(unsigned long long mask) {
+    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
+}
+
+// Exclusive scan of one int per thread over a 256-thread block; lds needs kWaves ints.
+__device__ int block_excl_scan(int v, int *lds, int *total) {
+    int lane = lane_id(), w = wave_id();
+    int inc = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int t = __shfl_up(inc, d);
+        if (lane >= d) inc += t;
+    }
+    if (lane == 63) lds[w] = inc;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) {
+        int c = lds[i];
+        if (i < w) base += c;
+        tot += c;
+    }
+    *total = tot;
+    __syncthreads();
+    return base + inc - v;
+}
+
+__device__ int block_sum(int v, int *lds) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    if (lane_id() == 0) lds[wave_id()] = v;
+    __syncthreads();
+    int tot = 0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) tot += lds[i];
+    __syncthreads();
+    return tot;
+}
+
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    return v;
+}
+
+// Largest p in [0, n) with begin[p] <= item (begin is non-decreasing, begin[0] <= item < begin[n]).
+__device__ int find_owner(const int *begin, int n, int item) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (begin[mid] <= item)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+// ------------------------------------------------------------------------------------ fills
+__global__ void k_fill_f32(float *p, float v, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+__global__ void k_fill_u32(unsigned *p, unsigned v, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// -------------------------------------------------------------------------------- gradients
+// Squared / logistic: include/thundergbm/objective/regression_obj.h:130-154 of the reference.
+__global__ void k_gradient_pointwise(int objective, int n, const float *__restrict__ y, const float *__restrict__ yp,
+                                     GHPair *__restrict__ gh) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        float p = yp[i];
+        GHPair o;
+        if (objective == OBJ_SQUARE) {
+            o.g = p - y[i];
+            o.h = 1.f;
+        } else {
+            float s = 1.f / (1.f + expf(-p));
+            o.g = s - y[i];
+            o.h = fmaxf(s * (1.f - s), 1e-16f);
+        }
+        gh[i] = o;
+    }
+}
+
+// Softmax: src/thundergbm/objective/multiclass_obj.cu:6-35 (class-major predictions and gradients,
+// hessian 2p(1-p)).
+__global__ void k_gradient_softmax(int n, int K, const float *__restrict__ y, const float *__restrict__ yp,
+                                   GHPair *__restrict__ gh) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        float mx = yp[i];
+        for (int k = 1; k < K; ++k) mx = fmaxf(mx, yp[(size_t)k * n + i]);
+        float sum = 0;
+        for (int k = 0; k < K; ++k) sum += expf(yp[(size_t)k * n + i] - mx);
+        float yi = y[i];
+        for (int k = 0; k < K; ++k) {
+            float p = expf(yp[(size_t)k * n + i] - mx) / sum;
+            GHPair o;
+            o.g = (k == yi) ? (p - 1.f) : p;
+            o.h = fmaxf(2.f * p * (1.f - p), 1e-16f);
+            gh[(size_t)k * n + i] = o;
+        }
+    }
+}
+
+// Block sums of (g,h) for the root node of a tree; fixed grid and fixed reduction order.
+__global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GHPair *__restrict__ out) {
+    __shared__ float sg[kWaves], sh[kWaves];
+    float g = 0, h = 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        GHPair v = gh[i];
+        g += v.g;
+        h += v.h;
+    }
+    g = wave_sum_f(g);
+    h = wave_sum_f(h);
+    if (lane_id() == 0) {
+        sg[wave_id()] = g;
+        sh[wave_id()] = h;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        GHPair o{0, 0};
+        for (int i = 0; i < kWaves; ++i) {
+            o.g += sg[i];
+            o.h += sh[i];
+        }
+        out[blockIdx.x] = o;
+    }
+}
+
+// ------------------------------------------------------------------------------- tree init
+// Node array initialisation of the reference's Tree::init2 (src/thundergbm/tree.cu:8-39), root sum
+// from the block partials, root segment and the histogram plan of level 0. One workgroup.
+__global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const GHPair *__restrict__ block_sums,
+                                                     float lambda) {
+    __shared__ float sg[kWaves], sh[kWaves];
+    const int nn = tb.n_nodes;
+    for (int i = threadIdx.x; i < nn; i += kBlock) {
+        TreeNode nd;
+        nd.final_id = i;
+        nd.parent_index = i == 0 ? -1 : (i - 1) / 2;
+        nd.gain = 0;
+        nd.base_weight = 0;
+        nd.split_feature_id = -1;
+        nd.split_value = 0;
+        nd.split_bid = 0;
+        nd.default_right = false;
+        nd.is_valid = false;
+        nd.is_pruned = false;
+        nd.sum_gh_pair = GHPair{0, 0};
+        if (i < nn / 2) {
+            nd.is_leaf = false;
+            nd.lch_index = 2 * i + 1;
+            nd.rch_index = 2 * i + 2;
+        } else {
+            nd.is_leaf = true;
+            nd.lch_index = -1;
+            nd.rch_index = -1;
+        }
+        // zero the padding bytes too: nodes are written raw into model files
+        unsigned *raw = reinterpret_cast<unsigned *>(&nd);
+        raw[9] &= 0x000000ffu;  // bytes 37..39 are padding (byte 36 = is_pruned)
+        tb.nodes[i] = nd;
+        tb.seg[i] = make_int2(0, 0);
+    }
+    float g = 0, h = 0;
+    for (int i = threadIdx.x; i < tb.n_grad_blocks; i += kBlock) {
+        g += block_sums[i].g;
+        h += block_sums[i].h;
+    }
+    g = wave_sum_f(g);
+    h = wave_sum_f(h);
+    if (lane_id() == 0) {
+        sg[wave_id()] = g;
+        sh[wave_id()] = h;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        GHPair s{0, 0};
+        for (int i = 0; i < kWaves; ++i) {
+            s.g += sg[i];
+            s.h += sh[i];
+        }
+        TreeNode &root = tb.nodes[0];
+        root.sum_gh_pair = s;
+        root.is_valid = true;
+        root.base_weight = -s.g / (s.h + lambda);
+        tb.seg[0] = make_int2(0, tb.n);
+        int chunk = (tb.n + tb.target_hitems - 1) / tb.target_hitems;
+        chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
+        int items = (tb.n + chunk - 1) / chunk;
+        tb.hpair_begin[0] = 0;
+        tb.hpair_begin[1] = items;
+        tb.hpair_built[0] = 0;
+        LevelCtl c;
+        c.hchunk = chunk;
+        c.n_hitems = items;
+        c.n_pitems = 0;
+        c.rows_built = tb.n;
+        tb.ctl[0] = c;
+    }
+}
+
+// ------------------------------------------------------------------------- dense histogram
+// One workgroup = one work item (a run of rows of one node) x one feature block. The block's
+// gradient / hessian histogram lives in LDS (g in the first half, h in the second) and is updated
+// with LDS float atomics; the finished private histogram is stored to the item's slot of `partial`.
+// LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
+// instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
+template <int LPR, bool DIRECT>
+__global__ __launch_bounds__(kBlock) void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
+                                                      const int *__restrict__ ridx, const int2 *__restrict__ seg,
+                                                      const int *__restrict__ hpair_begin,
+                                                      const int *__restrict__ hpair_built, int n_pairs,
+                                                      const LevelCtl *__restrict__ ctl,
+                                                      const int *__restrict__ blk_bin_begin,
+                                                      const int *__restrict__ feat_lds_off,
+                                                      GHPair *__restrict__ partial, int n_bins) {
+    extern __shared__ float lds[];
+    __shared__ int s_range[2];
+    const LevelCtl c = *ctl;
+    const int item = blockIdx.x;
+    if (item >= c.n_hitems) return;
+    const int fb = blockIdx.y;
+    const int bin0 = blk_bin_begin[fb];
+    const int nb = blk_bin_begin[fb + 1] - bin0;
+    if (nb == 0) return;
+    if (threadIdx.x == 0) {
+        int p = find_owner(hpair_begin, n_pairs, item);
+        int node = hpair_built[p];
+        int2 sg = seg[node];
+        int b = sg.x + (item - hpair_begin[p]) * c.hchunk;
+        s_range[0] = b;
+        s_range[1] = min(sg.y, b + c.hchunk);
+    }
+    for (int i = threadIdx.x; i < 2 * nb; i += kBlock) lds[i] = 0.f;
+    __syncthreads();
+    const int begin = s_range[0], end = s_range[1];
+    constexpr int RPS = kBlock / LPR;  // rows per step of the whole block
+    const int q = threadIdx.x % LPR;
+    const int rsub = threadIdx.x / LPR;
+    const int W = LPR * 4;
+    const int *fo = feat_lds_off + fb * W + q * 4;
+    const int o0 = fo[0], o1 = fo[1], o2 = fo[2], o3 = fo[3];
+    float *lg = lds;
+    float *lh = lds + nb;
+    const uint8_t *blk = bins.data + (size_t)fb * bins.block_stride + q * 4;
+    constexpr int U = 4;
+    for (int pos0 = begin + rsub; pos0 < end; pos0 += RPS * U) {
+        unsigned pk[U];
+        GHPair s[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int pos = pos0 + u * RPS;
+            ok[u] = pos < end;
+            int r = 0;
+            if (ok[u]) r = DIRECT ? pos : ridx[pos];
+            pk[u] = ok[u] ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
+            s[u] = ok[u] ? gh[r] : GHPair{0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            unsigned v = pk[u];
+            unsigned b0 = v & 0xff, b1 = (v >> 8) & 0xff, b2 = (v >> 16) & 0xff, b3 = v >> 24;
+            if (b0 != kMissingBin) {
+                unsafeAtomicAdd(lg + o0 + b0, s[u].g);
+                unsafeAtomicAdd(lh + o0 + b0, s[u].h);
+            }
+            if (b1 != kMissingBin) {
+                unsafeAtomicAdd(lg + o1 + b1, s[u].g);
+                unsafeAtomicAdd(lh + o1 + b1, s[u].h);
+            }
+            if (b2 != kMissingBin) {
+                unsafeAtomicAdd(lg + o2 + b2, s[u].g);
+                unsafeAtomicAdd(lh + o2 + b2, s[u].h);
+            }
+            if (b3 != kMissingBin) {
+                unsafeAtomicAdd(lg + o3 + b3, s[u].g);
+                unsafeAtomicAdd(lh + o3 + b3, s[u].h);
+            }
+        }
+    }
+    __syncthreads();
+    GHPair *out = partial + (size_t)item * n_bins + bin0;
+    for (int i = threadIdx.x; i < nb; i += kBlock) out[i] = GHPair{lg[i], lh[i]};
+}
+
+// Sum the private histograms of the node that was built from rows and derive its sibling as
+// parent - built (the reference's subtraction trick, hist_tree_builder_single.cu:526-540).
+__global__ __launch_bounds__(kBlock) void k_hist_merge(const float *__restrict__ partial, float *__restrict__ cur,
+                                                      const float *__restrict__ prev,
+                                                      const int *__restrict__ hpair_begin,
+                                                      const int *__restrict__ hpair_built, int level, int n_bins) {
+    const int p = blockIdx.y;
+    const int built = hpair_built[p];
+    if (built < 0) return;
+    const int j = blockIdx.x * kBlock + threadIdx.x;
+    const size_t stride = (size_t)2 * n_bins;
+    if (j >= (int)stride) return;
+    const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
+    float s = 0.f;
+    for (int it = ib; it < ie; ++it) s += partial[(size_t)it * stride + j];
+    const int off = (1 << level) - 1;
+    cur[(size_t)(built - off) * stride + j] = s;
+    if (level > 0) {
+        const int sib = (built & 1) ? built + 1 : built - 1;
+        cur[(size_t)(sib - off) * stride + j] = prev[(size_t)p * stride + j] - s;
+    }
+}
+
+// ------------------------------------------------------------------------ split finding
+__device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float lambda) {
+    GHPair r{f.g - l.g, f.h - l.h};
+    float gain = 0.f;
+    if (l.h >= mcw && r.h >= mcw)
+        gain = (l.g * l.g) / (l.h + lambda) + (r.g * r.g) / (r.h + lambda) - (f.g * f.g) / (f.h + lambda);
+    return fmaxf(0.f, gain);
+}
+
+// One wavefront scans one pack of whole features (at most 256 bins, 4 consecutive bins per lane):
+// segmented inclusive prefix sums per feature, missing = node sum - feature total, gain of every
+// candidate with missing values sent right and left, and the wavefront's best candidate (largest
+// |gain|, ties to the smaller bin index). Follows hist_tree_builder_single.cu:257-347 / :614-704.
+__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const GHPair *__restrict__ hist, int level,
+                                                      float mcw, float lambda) {
+    __shared__ GHPair s_miss[kWaves][kEvalPackBins];
+    const int lane = lane_id(), w = wave_id();
+    const int pack = blockIdx.x * kWaves + w;
+    const int x_in = blockIdx.y;
+    const int x = (1 << level) - 1 + x_in;
+    const TreeNode nd = tb.nodes[x];
+    const bool active = pack < tb.n_packs && nd.is_valid;
+    int b_begin = 0, b_end = 0;
+    if (active) {
+        b_begin = tb.pack_begin[pack];
+        b_end = tb.pack_begin[pack + 1];
+    }
+    const GHPair S = nd.sum_gh_pair;
+    const GHPair *h = hist + (size_t)x_in * tb.n_bins;
+
+    GHPair inc[4];
+    int lastb[4];  // pack-relative index of the last bin of the element's feature
+    bool valid[4], head[4], last[4];
+    GHPair run{0, 0};
+    bool any_head = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int b = b_begin + lane * 4 + j;
+        valid[j] = b < b_end;
+        lastb[j] = 0;
+        head[j] = false;
+        last[j] = false;
+        inc[j] = GHPair{0, 0};
+        if (valid[j]) {
+            GHPair v = h[b];
+            const int f = tb.cut_fid[b];
+            const int fend = tb.cut_row_ptr[f + 1];
+            head[j] = tb.cut_row_ptr[f] == b;
+            last[j] = fend == b + 1;
+            lastb[j] = fend - 1 - b_begin;
+            if (head[j]) {
+                run = v;
+                any_head = true;
+            } else {
+                run.g += v.g;
+                run.h += v.h;
+            }
+            inc[j] = run;
+        }
+    }
+    // wavefront segmented inclusive scan of the lane aggregates
+    GHPair agg = run;
+    int flag = any_head ? 1 : 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        float pg = __shfl_up(agg.g, d);
+        float ph = __shfl_up(agg.h, d);
+        int pf = __shfl_up(flag, d);
+        if (lane >= d) {
+            if (!flag) {
+                agg.g = pg + agg.g;
+                agg.h = ph + agg.h;
+            }
+            flag |= pf;
+        }
+    }
+    GHPair carry;
+    carry.g = __shfl_up(agg.g, 1);
+    carry.h = __shfl_up(agg.h, 1);
+    if (lane == 0) carry = GHPair{0, 0};
+    bool seen = false;
+    GHPair excl[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (valid[j]) {
+            if (head[j]) seen = true;
+            if (!seen) {
+                inc[j].g = carry.g + inc[j].g;
+                inc[j].h = carry.h + inc[j].h;
+            }
+        }
+        if (head[j])
+            excl[j] = GHPair{0, 0};
+        else
+            excl[j] = (j == 0) ? carry : inc[j - 1];
+        if (valid[j] && last[j]) s_miss[w][lastb[j]] = GHPair{S.g - inc[j].g, S.h - inc[j].h};
+    }
+    __syncthreads();
+    float best = -1.f;  // |score| of the lane's best candidate
+    float best_score = 0.f;
+    int best_idx = 0x7fffffff;
+    GHPair best_miss{0, 0}, best_left{0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (valid[j]) {
+            GHPair m = s_miss[w][lastb[j]];
+            GHPair l = excl[j];
+            float gr = split_gain(S, l, mcw, lambda);
+            GHPair l2{l.g + m.g, l.h + m.h};
+            float gl = split_gain(S, l2, mcw, lambda);
+            float score = (gl > gr) ? gl : -gr;
+            float a = fabsf(score);
+            if (a > best) {
+                best = a;
+                best_score = score;
+                best_idx = b_begin + lane * 4 + j;
+                best_miss = m;
+                best_left = l;
+            }
+        }
+    }
+    // wavefront arg-max: larger |score| wins, ties go to the smaller bin index
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        float oa = __shfl_xor(best, d);
+        float os = __shfl_xor(best_score, d);
+        int oi = __shfl_xor(best_idx, d);
+        float omg = __shfl_xor(best_miss.g, d), omh = __shfl_xor(best_miss.h, d);
+        float olg = __shfl_xor(best_left.g, d), olh = __shfl_xor(best_left.h, d);
+        if (oa > best || (oa == best && oi < best_idx)) {
+            best = oa;
+            best_score = os;
+            best_idx = oi;
+            best_miss = GHPair{omg, omh};
+            best_left = GHPair{olg, olh};
+        }
+    }
+    if (active && lane == 0) {
+        SplitCand c;
+        c.score = best_score;
+        c.index = best_idx;
+        c.miss = best_miss;
+        c.left = best_left;
+        c.pad[0] = c.pad[1] = 0;
+        tb.cand[(size_t)x_in * tb.n_packs + pack] = c;
+    }
+}
+
+// Per node: reduce the wavefront candidates, fill the split record (hist_tree_builder_single.cu
+// :365-389) and apply it to the tree (update_tree, :860-899). One workgroup per node of the level.
+__global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb, int level, float rt_eps, float lambda) {
+    __shared__ float s_abs[kWaves];
+    __shared__ int s_idx[kWaves];
+    __shared__ int s_pack[kWaves];
+    const int x_in = blockIdx.x;
+    const int x = (1 << level) - 1 + x_in;
+    TreeNode &node = tb.nodes[x];
+    SplitPoint &sp = tb.sp[x_in];
+    if (!node.is_valid) {
+        if (threadIdx.x == 0) {
+            SplitPoint z{};
+            z.nid = -1;
+            z.split_fea_id = -1;
+            sp = z;
+        }
+        return;
+    }
+    float best = -1.f;
+    int best_idx = 0x7fffffff, best_pack = -1;
+    for (int p = threadIdx.x; p < tb.n_packs; p += kBlock) {
+        const SplitCand &c = tb.cand[(size_t)x_in * tb.n_packs + p];
+        float a = fabsf(c.score);
+        if (a > best || (a == best && c.index < best_idx)) {
+            best = a;
+            best_idx = c.index;
+            best_pack = p;
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        float oa = __shfl_xor(best, d);
+        int oi = __shfl_xor(best_idx, d);
+        int op = __shfl_xor(best_pack, d);
+        if (oa > best || (oa == best && oi < best_idx)) {
+            best = oa;
+            best_idx = oi;
+            best_pack = op;
+        }
+    }
+    if (lane_id() == 0) {
+        s_abs[wave_id()] = best;
+        s_idx[wave_id()] = best_idx;
+        s_pack[wave_id()] = best_pack;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    for (int i = 0; i < kWaves; ++i) {
+        if (s_abs[i] > best || (s_abs[i] == best && s_idx[i] < best_idx)) {
+            best = s_abs[i];
+            best_idx = s_idx[i];
+            best_pack = s_pack[i];
+        }
+    }
+    const SplitCand c = tb.cand[(size_t)x_in * tb.n_packs + best_pack];
+    const int f = tb.cut_fid[c.index];
+    const int fbegin = tb.cut_row_ptr[f];
+    SplitPoint s{};
+    s.split_fea_id = f;
+    s.nid = x;
+    s.gain = fabsf(c.score);
+    s.split_bid = (int)(unsigned char)(c.index - fbegin);
+    s.fea_missing_gh = c.miss;
+    s.default_right = c.score < 0;
+    s.best_index = c.index;
+    if (c.index != fbegin) {
+        s.lch_sum_gh = c.left;
+        s.fval = tb.cut_val[c.index - 1];
+    } else {
+        s.lch_sum_gh = GHPair{0, 0};
+        float c0 = tb.cut_val[fbegin];
+        s.fval = (float)((double)(c0 - fabsf(c0)) - 1e-5);
+    }
+    sp = s;
+    if (s.gain > rt_eps) {
+        node.gain = s.gain;
+        TreeNode &l = tb.nodes[node.lch_index];
+        TreeNode &r = tb.nodes[node.rch_index];
+        l.is_valid = true;
+        r.is_valid = true;
+        node.split_feature_id = f;
+        node.split_value = s.fval;
+        node.split_bid = (unsigned char)s.split_bid;
+        GHPair ls = s.lch_sum_gh;
+        if (!s.default_right) {
+            ls.g += s.fea_missing_gh.g;
+            ls.h += s.fea_missing_gh.h;
+            node.default_right = false;
+        } else {
+            node.default_right = true;
+        }
+        GHPair rs{node.sum_gh_pair.g - ls.g, node.sum_gh_pair.h - ls.h};
+        l.sum_gh_pair = ls;
+        r.sum_gh_pair = rs;
+        l.base_weight = -ls.g / (ls.h + lambda);
+        r.base_weight = -rs.g / (rs.h + lambda);
+    } else {
+        node.is_leaf = true;
+        tb.nodes[node.lch_index].is_valid = false;
+        tb.nodes[node.rch_index].is_valid = false;
+    }
+}
+
+// ------------------------------------------------------------------------------ partition
+__device__ __forceinline__ bool node_splits(const TreeNode &nd) {
+    return nd.is_valid && !nd.is_leaf && nd.split_feature_id >= 0;
+}
+
+// Partition work items: every node of the level that was split gets ceil(rows / kPartChunk) items.
+__global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb, int level) {
+    __shared__ int lds[kWaves];
+    const int nl = 1 << level, off = nl - 1;
+    int carry = 0;
+    for (int base = 0; base < nl; base += kBlock) {
+        int x_in = base + threadIdx.x;
+        int cnt = 0;
+        if (x_in < nl) {
+            const TreeNode &nd = tb.nodes[off + x_in];
+            int2 sg = tb.seg[off + x_in];
+            if (node_splits(nd)) cnt = (sg.y - sg.x + kPartChunk - 1) / kPartChunk;
+        }
+        int tot;
+        int ex = block_excl_scan(cnt, lds, &tot);
+        if (x_in < nl) tb.pitem_begin[x_in] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) {
+        tb.pitem_begin[nl] = carry;
+        tb.ctl[level].n_pitems = carry;
+    }
+}
+
+// Decide left/right for every row of a work item from the split feature's byte of the bin matrix
+// (missing -> default direction, else right iff bin >= split bin; the reference's rule at
+// hist_tree_builder_single.cu:986-1011) and count the rows that go left.
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb, DenseBins bins,
+                                                            const int *__restrict__ ridx, int level) {
+    __shared__ int lds[kWaves];
+    __shared__ int s_x;
+    const int item = blockIdx.x;
+    if (item >= tb.ctl[level].n_pitems) return;
+    const int nl = 1 << level, off = nl - 1;
+    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    __syncthreads();
+    const int x_in = s_x;
+    const TreeNode &nd = tb.nodes[off + x_in];
+    const int2 sg = tb.seg[off + x_in];
+    const int pb = sg.x + (item - tb.pitem_begin[x_in]) * kPartChunk;
+    const int pe = min(sg.y, pb + kPartChunk);
+    const int f = nd.split_feature_id;
+    const int sbid = nd.split_bid;
+    const bool dr = nd.default_right;
+    const uint8_t *blk = bins.data + (size_t)(f / bins.W) * bins.block_stride + (f % bins.W);
+    int nleft = 0;
+#pragma unroll
+    for (int k = 0; k < kPartChunk / kBlock; ++k) {
+        int pos = pb + k * kBlock + threadIdx.x;
+        if (pos < pe) {
+            int row = DIRECT ? pos : ridx[pos];
+            int b = blk[(size_t)row * bins.W];
+            bool right = (b == kMissingBin) ? dr : (b >= sbid);
+            tb.goes_right[pos] = right ? 1 : 0;
+            nleft += right ? 0 : 1;
+        }
+    }
+    int tot = block_sum(nleft, lds);
+    if (threadIdx.x == 0) tb.pitem_nleft[item] = tot;
+}
+
+// Scan the per-item left counts, publish the children's row segments and plan the histogram work
+// of the next level: per sibling pair the child with fewer rows is built (ties: the left one, as
+// hist_tree_builder_single.cu:466-467), the other one comes from subtraction. One workgroup.
+__global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb, int level) {
+    __shared__ int lds[kWaves];
+    const int nl = 1 << level, off = nl - 1;
+    const int n_p = tb.ctl[level].n_pitems;
+    int carry = 0;
+    for (int base = 0; base < n_p; base += kBlock) {
+        int i = base + threadIdx.x;
+        int v = i < n_p ? tb.pitem_nleft[i] : 0;
+        int tot;
+        int ex = block_excl_scan(v, lds, &tot);
+        if (i < n_p) tb.pitem_loff[i] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) tb.pitem_loff[n_p] = carry;
+    __syncthreads();
+    // children segments + rows of the built child of every pair
+    int rows_sum = 0;
+    for (int x_in = threadIdx.x; x_in < nl; x_in += kBlock) {
+        const TreeNode &nd = tb.nodes[off + x_in];
+        const int2 sg = tb.seg[off + x_in];
+        int built = -1;
+        if (node_splits(nd)) {
+            int nleft = tb.pitem_loff[tb.pitem_begin[x_in + 1]] - tb.pitem_loff[tb.pitem_begin[x_in]];
+            int nright = (sg.y - sg.x) - nleft;
+            tb.node_nleft[x_in] = nleft;
+            tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
+            tb.seg[nd.rch_index] = make_int2(sg.x + nleft, sg.y);
+            built = (nleft <= nright) ? nd.lch_index : nd.rch_index;
+            rows_sum += min(nleft, nright);
+        } else {
+            tb.node_nleft[x_in] = 0;
+            tb.seg[nd.lch_index] = make_int2(0, 0);
+            tb.seg[nd.rch_index] = make_int2(0, 0);
+        }
+        tb.hpair_built[x_in] = built;
+    }
+    const int total_rows = block_sum(rows_sum, lds);
+    int chunk = (total_rows + tb.target_hitems - 1) / tb.target_hitems;
+    chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
+    carry = 0;
+    for (int base = 0; base < nl; base += kBlock) {
+        int x_in = base + threadIdx.x;
+        int cnt = 0;
+        if (x_in < nl) {
+            int built = tb.hpair_built[x_in];
+            if (built >= 0) {
+                int2 sg = tb.seg[built];
+                cnt = (sg.y - sg.x + chunk - 1) / chunk;
+            }
+        }
+        int tot;
+        int ex = block_excl_scan(cnt, lds, &tot);
+        if (x_in < nl) tb.hpair_begin[x_in] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) {
+        tb.hpair_begin[nl] = carry;
+        LevelCtl c;
+        c.hchunk = chunk;
+        c.n_hitems = carry;
+        c.n_pitems = 0;
+        c.rows_built = total_rows;
+        tb.ctl[level + 1] = c;
+    }
+}
+
+// Stable two-way compaction of a work item's rows into the children's segments with wavefront
+// ballots and popcounts; also records the new node of every moved row.
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const int *__restrict__ ridx_cur,
+                                                        int *__restrict__ ridx_next, int level) {
+    __shared__ int s_x;
+    __shared__ int s_cnt[2][kWaves];
+    const int item = blockIdx.x;
+    if (item >= tb.ctl[level].n_pitems) return;
+    const int nl = 1 << level, off = nl - 1;
+    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    __syncthreads();
+    const int x_in = s_x;
+    const TreeNode &nd = tb.nodes[off + x_in];
+    const int lch = nd.lch_index, rch = nd.rch_index;
+    const int2 sg = tb.seg[off + x_in];
+    const int first_item = tb.pitem_begin[x_in];
+    const int pb = sg.x + (item - first_item) * kPartChunk;
+    const int pe = min(sg.y, pb + kPartChunk);
+    const int loff = tb.pitem_loff[item] - tb.pitem_loff[first_item];
+    int left_base = sg.x + loff;
+    int right_base = sg.x + tb.node_nleft[x_in] + ((pb - sg.x) - loff);
+    const int lane = lane_id(), w = wave_id();
+    for (int k = 0; k < kPartChunk / kBlock; ++k) {
+        int pos = pb + k * kBlock + threadIdx.x;
+        bool valid = pos < pe;
+        int row = 0;
+        bool right = false;
+        if (valid) {
+            row = DIRECT ? pos : ridx_cur[pos];
+            right = tb.goes_right[pos] != 0;
+        }
+        unsigned long long mL = __ballot(valid && !right);
+        unsigned long long mR = __ballot(valid && right);
+        if (lane == 0) {
+            s_cnt[0][w] = __popcll(mL);
+            s_cnt[1][w] = __popcll(mR);
+        }
+        __syncthreads();
+        int bL = 0, bR = 0, tL = 0, tR = 0;
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) {
+            int cl = s_cnt[0][i], cr = s_cnt[1][i];
+            if (i < w) {
+                bL += cl;
+                bR += cr;
+            }
+            tL += cl;
+            tR += cr;
+        }
+        if (valid) {
+            int dest = right ? right_base + bR + lanes_below(mR) : left_base + bL + lanes_below(mL);
+            ridx_next[dest] = row;
+            tb.nid[row] = right ? rch : lch;
+        }
+        left_base += tL;
+        right_base += tR;
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------------- prune
+// Bottom-up, level-parallel form of the reference's Tree::prune_self (src/thundergbm/tree.cu:96-128):
+// a node whose two children are valid leaves and whose gain is below gamma becomes a leaf and its
+// children are marked pruned; then final ids are renumbered over valid, unpruned nodes.
+__global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb, float gamma) {
+    __shared__ int lds[kWaves];
+    for (int level = tb.depth - 1; level >= 0; --level) {
+        const int nl = 1 << level, off = nl - 1;
+        for (int x_in = threadIdx.x; x_in < nl; x_in += kBlock) {
+            TreeNode &p = tb.nodes[off + x_in];
+            if (p.is_valid && !p.is_leaf) {
+                TreeNode &l = tb.nodes[p.lch_index];
+                TreeNode &r = tb.nodes[p.rch_index];
+                if (l.is_valid && l.is_leaf && r.is_valid && r.is_leaf && p.gain < gamma) {
+                    l.is_pruned = true;
+                    r.is_pruned = true;
+                    p.is_leaf = true;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    int carry = 0;
+    for (int base = 0; base < tb.n_nodes; base += kBlock) {
+        int i = base + threadIdx.x;
+        int keep = 0;
+        if (i < tb.n_nodes) keep = (tb.nodes[i].is_valid && !tb.nodes[i].is_pruned) ? 1 : 0;
+        int tot;
+        int ex = block_excl_scan(keep, lds, &tot);
+        if (keep) tb.nodes[i].final_id = carry + ex;
+        carry += tot;
+    }
+}
+
+// y_pred += lr * weight of the (unpruned) leaf the row ended in (tree_builder.cu:62-74).
+__global__ void k_predict_in_training(int n, const int *__restrict__ nid, const TreeNode *__restrict__ nodes,
+                                      float *__restrict__ yp, float lr) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        int x = nid[i];
+        while (x != -1 && nodes[x].is_pruned) x = nodes[x].parent_index;
+        yp[i] += lr * nodes[x].base_weight;
+    }
+}
+
+// ---------------------------------------------------------------------------------- metric
+// kind 0: sum of squared errors; 1: correct binary decisions (sigmoid > 0.5 in double, like
+// multiclass_metric.cu:40); 2: correct arg-max decisions (first maximum wins, :17-29).
+__global__ __launch_bounds__(kBlock) void k_metric_partial(int kind, int n, int K, const float *__restrict__ y,
+                                                          const float *__restrict__ yp, double *__restrict__ out) {
+    __shared__ double sd[kWaves];
+    double acc = 0;
+    float accf = 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        if (kind == 0) {
+            float e = yp[i] - y[i];
+            accf += e * e;
+        } else if (kind == 1) {
+            int k = (1.0 / (1.0 + exp(-(double)yp[i])) > 0.5) ? 1 : 0;
+            acc += (k == y[i]) ? 1 : 0;
+        } else {
+            int mk = 0;
+            float mp = yp[i];
+            for (int k = 1; k < K; ++k) {
+                float v = yp[(size_t)k * n + i];
+                if (v > mp) {
+                    mp = v;
+                    mk = k;
+                }
+            }
+            acc += (mk == y[i]) ? 1 : 0;
+        }
+    }
+    acc += (double)accf;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
+    if (lane_id() == 0) sd[wave_id()] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double s = 0;
+        for (int i = 0; i < kWaves; ++i) s += sd[i];
+        out[blockIdx.x] = s;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_metric_final(int kind, int n, int n_blocks, const double *__restrict__ in,
+                                                        float *__restrict__ out) {
+    __shared__ double sd[kWaves];
+    double acc = 0;
+    for (int i = threadIdx.x; i < n_blocks; i += kBlock) acc += in[i];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
+    if (lane_id() == 0) sd[wave_id()] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double s = 0;
+        for (int i = 0; i < kWaves; ++i) s += sd[i];
+        if (kind == 0) {
+            out[0] = sqrtf((float)s / n);
+        } else {
+            float a = (float)s / (float)n;
+            out[0] = kind == 1 ? 1.f - a : a;
+        }
+    }
+}
+
+constexpr int kMetricBlocks = 1024;
+
+int grid_for(size_t n, int cap = 4096) {
+    size_t b = (n + kBlock - 1) / kBlock;
+    if (b < 1) b = 1;
+    if (b > (size_t)cap) b = cap;
+    return (int)b;
+}
+
+}  // namespace
+
+// =================================================================================== launchers
+void launch_fill_f32(hipStream_t s, float *p, float v, size_t n) {
+    if (n == 0) return;
+    k_fill_f32<<<grid_for(n), kBlock, 0, s>>>(p, v, n);
+}
+
+void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n) {
+    // n must be a multiple of 4 (all users allocate padded buffers)
+    if (n == 0) return;
+    unsigned w = v * 0x01010101u;
+    k_fill_u32<<<grid_for(n / 4), kBlock, 0, s>>>(reinterpret_cast<unsigned *>(p), w, n / 4);
+}
+
+void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
+                     GHPair *, int) {
+    if (objective == OBJ_SOFTMAX)
+        k_gradient_softmax<<<grid_for(n), kBlock, 0, s>>>(n, num_class, y, yp, gh);
+    else
+        k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
+}
+
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda) {
+    k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
+    k_fill_u32<<<grid_for(tb.n), kBlock, 0, s>>>(reinterpret_cast<unsigned *>(tb.nid), 0u, (size_t)tb.n);
+    k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
+}
+
+template <int LPR>
+static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
+                                int level) {
+    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    dim3 grid(tb.max_hitems, bins.n_blocks);
+    size_t lds = (size_t)tb.max_block_bins * 2 * sizeof(float);
+    if (level == 0) {
+        static bool attr_done = false;
+        if (!attr_done) {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            attr_done = true;
+        }
+        k_hist_dense<LPR, true><<<grid, kBlock, lds, s>>>(bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built,
+                                                         n_pairs, tb.ctl + level, tb.blk_bin_begin, tb.feat_lds_off,
+                                                         tb.partial, tb.n_bins);
+    } else {
+        k_hist_dense<LPR, false><<<grid, kBlock, lds, s>>>(bins, gh, tb.ridx[level & 1], tb.seg, tb.hpair_begin,
+                                                          tb.hpair_built, n_pairs, tb.ctl + level, tb.blk_bin_begin,
+                                                          tb.feat_lds_off, tb.partial, tb.n_bins);
+    }
+}
+
+void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level) {
+    switch (bins.W / 4) {
+        case 1: hist_dense_dispatch<1>(s, tb, bins, gh, level); break;
+        case 2: hist_dense_dispatch<2>(s, tb, bins, gh, level); break;
+        case 4: hist_dense_dispatch<4>(s, tb, bins, gh, level); break;
+        case 8: hist_dense_dispatch<8>(s, tb, bins, gh, level); break;
+        case 16: hist_dense_dispatch<16>(s, tb, bins, gh, level); break;
+        default: fatal("unsupported dense block width %d", bins.W);
+    }
+}
+
+void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level) {
+    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    dim3 grid((2 * tb.n_bins + kBlock - 1) / kBlock, n_pairs);
+    k_hist_merge<<<grid, kBlock, 0, s>>>(reinterpret_cast<const float *>(tb.partial),
+                                        reinterpret_cast<float *>(tb.hist[level & 1]),
+                                        reinterpret_cast<const float *>(tb.hist[(level + 1) & 1]), tb.hpair_begin,
+                                        tb.hpair_built, level, tb.n_bins);
+}
+
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
+    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level);
+    k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist[level & 1], level, mcw, lambda);
+}
+
+void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda) {
+    k_best_update<<<1 << level, kBlock, 0, s>>>(tb, level, rt_eps, lambda);
+}
+
+void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level) {
+    k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
+    const int *cur = tb.ridx[level & 1];
+    int *next = tb.ridx[(level + 1) & 1];
+    if (level == 0) {
+        k_part_count_dense<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
+        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+    } else {
+        k_part_count_dense<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
+        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+    }
+}
+
+void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma) { k_prune<<<1, kBlock, 0, s>>>(tb, gamma); }
+
+void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, float *yp_class, float lr) {
+    k_predict_in_training<<<grid_for(tb.n), kBlock, 0, s>>>(tb.n, tb.nid, tb.nodes, yp_class, lr);
+}
+
+void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
+                   float *out) {
+    int blocks = grid_for(n, kMetricBlocks);
+    k_metric_partial<<<blocks, kBlock, 0, s>>>(kind, n, num_class, y, yp, scratch);
+    k_metric_final<<<1, kBlock, 0, s>>>(kind, n, blocks, scratch, out);
+}
+
+}  // namespace tgbm

@@ -1,0 +1,177 @@
+"""scikit-learn style estimators over the C ABI, with the constructor arguments, method names and
+data handling of the reference wrapper (python/thundergbm/thundergbm.py): dense inputs lose their
+exact zeros on the way to CSR (zeros are missing values), values go in as float32 with ascending
+column indices, classifier predictions come back as the original labels."""
+import ctypes as C
+
+import numpy as np
+import scipy.sparse as sp
+from sklearn.base import BaseEstimator, ClassifierMixin, RegressorMixin
+
+from . import _lib
+
+_PARAMS = ("depth", "n_trees", "n_gpus", "min_child_weight", "lambda_tgbm", "gamma", "max_num_bin", "verbose",
+           "column_sampling_rate", "bagging", "n_parallel_trees", "learning_rate", "objective", "num_class",
+           "tree_method")
+
+
+def _csr(X):
+    X = X.tocsr(copy=True) if sp.issparse(X) else sp.csr_matrix(np.asarray(X))
+    X.data = np.ascontiguousarray(X.data, dtype=np.float32)
+    X.sort_indices()
+    return X
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class TGBMModel(BaseEstimator):
+    def __init__(self, depth=6, n_trees=40, n_gpus=1, min_child_weight=1.0, lambda_tgbm=1.0, gamma=1.0,
+                 max_num_bin=255, verbose=1, column_sampling_rate=1.0, bagging=0, n_parallel_trees=1,
+                 learning_rate=1.0, objective="reg:linear", num_class=1, tree_method="auto"):
+        for name in _PARAMS:
+            setattr(self, name, locals()[name])
+        self.model = None
+        self.tree_per_iter = -1
+        self.group_label = None
+
+    def __del__(self):
+        self._release()
+
+    def _release(self):
+        if getattr(self, "model", None) is not None:
+            _lib.load().model_free(C.byref(self.model))
+            self.model = None
+
+    def fit(self, X, y, groups=None):
+        lib = _lib.load()
+        self._release()
+        X = _csr(X)
+        y = np.ascontiguousarray(y, dtype=np.float32)
+        if X.shape[0] != len(y):
+            raise ValueError("X and y have different numbers of rows")
+        indptr = np.ascontiguousarray(X.indptr, dtype=np.int32)
+        indices = np.ascontiguousarray(X.indices, dtype=np.int32)
+        n_labels = len(set(y.tolist()))
+        group_label = (C.c_float * max(n_labels, 1))()
+        n_class = (C.c_int * 1)(self.num_class)
+        per_iter = (C.c_int * 1)(0)
+        self.model = C.c_void_p(None)
+        grp = None if groups is None else np.ascontiguousarray(groups, dtype=np.int32)
+        lib.sparse_train_scikit(X.shape[0], _ptr(X.data), _ptr(indptr), _ptr(indices), _ptr(y), self.depth,
+                                self.n_trees, self.n_gpus, self.min_child_weight, self.lambda_tgbm, self.gamma,
+                                self.max_num_bin, self.verbose, self.column_sampling_rate, int(self.bagging),
+                                self.n_parallel_trees, self.learning_rate, self.objective.encode("utf-8"),
+                                C.cast(n_class, C.c_void_p), self.tree_method.encode("utf-8"),
+                                C.cast(C.byref(self.model), C.c_void_p), C.cast(per_iter, C.c_void_p),
+                                C.cast(group_label, C.c_void_p), None if grp is None else _ptr(grp),
+                                0 if grp is None else len(grp))
+        self.num_class = n_class[0]
+        self.tree_per_iter = per_iter[0]
+        self.group_label = [group_label[i] for i in range(n_labels)]
+        if not self.model:
+            raise RuntimeError("The model returned is empty!")
+        return self
+
+    def predict(self, X, groups=None):
+        if not self.model:
+            raise ValueError("Please train the model first or load model from file!")
+        lib = _lib.load()
+        X = _csr(X)
+        indptr = np.ascontiguousarray(X.indptr, dtype=np.int32)
+        indices = np.ascontiguousarray(X.indices, dtype=np.int32)
+        n = X.shape[0]
+        n_out = n * self.num_class if self.objective == "multi:softprob" else n
+        out = np.zeros(max(n_out, n * max(self.tree_per_iter, 1)), dtype=np.float32)
+        labels = np.asarray(self.group_label if self.group_label else [0.0], dtype=np.float32)
+        lib.sparse_predict_scikit(n, _ptr(X.data), _ptr(indptr), _ptr(indices), _ptr(out),
+                                  C.cast(C.byref(self.model), C.c_void_p), self.n_trees, self.tree_per_iter,
+                                  self.objective.encode("utf-8"), self.num_class, self.learning_rate, _ptr(labels),
+                                  None, 0, self.verbose)
+        if self.objective == "multi:softprob":
+            # the library returns class-major probabilities; the reference wrapper reshapes them as
+            # [-1, num_class] without transposing (thundergbm.py:169-171) and so does this one
+            self.predict_label = out[:n_out].reshape([-1, self.num_class])
+        else:
+            self.predict_label = out[:n].copy()
+        return self.predict_label
+
+    def predict_proba_class_major(self, X):
+        """multi:softprob probabilities as [num_class, n_rows] (the layout the library produces)."""
+        p = self.predict(X)
+        return p.reshape(self.num_class, -1)
+
+    def save_model(self, model_path):
+        if not self.model:
+            raise ValueError("Please train the model first or load model from file!")
+        labels = np.asarray(self.group_label if self.group_label else [0.0], dtype=np.float32)
+        _lib.load().save(model_path.encode("utf-8"), self.objective.encode("utf-8"), self.learning_rate,
+                         self.num_class, self.n_trees, self.tree_per_iter, C.cast(C.byref(self.model), C.c_void_p),
+                         _ptr(labels))
+
+    def load_model(self, model_path):
+        lib = _lib.load()
+        self._release()
+        self.model = C.c_void_p(None)
+        lr = (C.c_float * 1)()
+        n_class = (C.c_int * 1)()
+        n_trees = (C.c_int * 1)()
+        per_iter = (C.c_int * 1)()
+        lib.load_model(model_path.encode("utf-8"), C.cast(lr, C.c_void_p), C.cast(n_class, C.c_void_p),
+                       C.cast(n_trees, C.c_void_p), C.cast(per_iter, C.c_void_p),
+                       C.cast(C.byref(self.model), C.c_void_p))
+        if not self.model:
+            raise ValueError("Model is None.")
+        self.learning_rate = lr[0]
+        self.num_class = n_class[0]
+        self.n_trees = n_trees[0]
+        self.tree_per_iter = per_iter[0]
+        labels = (C.c_float * max(self.num_class, 1))()
+        lib.load_config(model_path.encode("utf-8"), C.cast(labels, C.c_void_p))
+        self.group_label = [labels[i] for i in range(self.num_class)]
+
+    def get_trees(self):
+        """Every tree as parallel heap-ordered arrays (the dictionaries the reference hands to shap)."""
+        if not self.model:
+            raise ValueError("Please train the model first or load model from file!")
+        lib = _lib.load()
+        total = self.n_trees * self.tree_per_iter
+        n_nodes = np.zeros(total, dtype=np.int32)
+        mp = C.cast(C.byref(self.model), C.c_void_p)
+        lib.get_n_nodes(mp, _ptr(n_nodes), self.n_trees, self.tree_per_iter)
+        trees = []
+        for t in range(total):
+            nn = int(n_nodes[t])
+            d = {"children_left": np.empty(nn, np.int32), "children_right": np.empty(nn, np.int32),
+                 "children_default": np.empty(nn, np.int32), "feature": np.empty(nn, np.int32),
+                 "threshold": np.empty(nn, np.float32), "value": np.empty(nn, np.float32),
+                 "node_sample_weight": np.empty(nn, np.float32)}
+            lib.get_a_tree(mp, t, nn, _ptr(d["children_left"]), _ptr(d["children_right"]),
+                           _ptr(d["children_default"]), _ptr(d["feature"]), _ptr(d["threshold"]), _ptr(d["value"]),
+                           _ptr(d["node_sample_weight"]))
+            d["value"] = d["value"].reshape(-1, 1)
+            trees.append(d)
+        return trees
+
+
+class TGBMClassifier(TGBMModel, ClassifierMixin):
+    _impl = "classifier"
+
+    def __init__(self, depth=6, n_trees=40, n_gpus=1, min_child_weight=1.0, lambda_tgbm=1.0, gamma=1.0,
+                 max_num_bin=255, verbose=1, column_sampling_rate=1.0, bagging=0, n_parallel_trees=1,
+                 learning_rate=1.0, objective="multi:softmax", num_class=2, tree_method="auto"):
+        super().__init__(depth, n_trees, n_gpus, min_child_weight, lambda_tgbm, gamma, max_num_bin, verbose,
+                         column_sampling_rate, bagging, n_parallel_trees, learning_rate, objective, num_class,
+                         tree_method)
+
+
+class TGBMRegressor(TGBMModel, RegressorMixin):
+    _impl = "regressor"
+
+    def __init__(self, depth=6, n_trees=40, n_gpus=1, min_child_weight=1.0, lambda_tgbm=1.0, gamma=1.0,
+                 max_num_bin=255, verbose=1, column_sampling_rate=1.0, bagging=0, n_parallel_trees=1,
+                 learning_rate=1.0, objective="reg:linear", num_class=1, tree_method="auto"):
+        super().__init__(depth, n_trees, n_gpus, min_child_weight, lambda_tgbm, gamma, max_num_bin, verbose,
+                         column_sampling_rate, bagging, n_parallel_trees, learning_rate, objective, num_class,
+                         tree_method)
