@@ -223,6 +223,36 @@ void group_label(std::vector<float> &y, std::vector<float> &label) {
     for (float &v : y) v = (float)m[v];
 }
 
+
+// fp32 sum of (g,h) in a tree order: 256-element sequential leaves, then pairwise. The reference uses
+// thrust::reduce (src/thundergbm/tree.cu:31, regression_obj.h:41,101), whose order is unspecified
+// but tree-shaped; a long sequential float32 sum of near-constant hessians would drift by more than
+// the comparison tolerance.
+GH sum_gh(const GH *g, long n) {
+    const long CH = 256;
+    long nch = (n + CH - 1) / CH;
+    std::vector<GH> part((size_t)std::max<long>(nch, 1), GH{0, 0});
+#pragma omp parallel for
+    for (long c = 0; c < nch; ++c) {
+        float a = 0, b = 0;
+        long e = std::min<long>(n, (c + 1) * CH);
+        for (long i = c * CH; i < e; ++i) {
+            a += g[i].g;
+            b += g[i].h;
+        }
+        part[c] = GH{a, b};
+    }
+    for (long m = nch; m > 1;) {
+        long half = (m + 1) / 2;
+        for (long i = 0; i + half < m; ++i) {
+            part[i].g += part[i + half].g;
+            part[i].h += part[i + half].h;
+        }
+        m = half;
+    }
+    return part[0];
+}
+
 // a4  Tree::init2, src/thundergbm/tree.cu:8-39
 void tree_init(Oracle &o, int k) {
     o.cur_class = k;
@@ -244,29 +274,8 @@ void tree_init(Oracle &o, int k) {
             nd.lch = nd.rch = -1;
         }
     }
-    const GH *g = o.gh.data() + (long)k * o.n;
-    // fp32 reduction (the reference's thrust::reduce order is unspecified; pairwise per thread chunk)
-    double sg = 0, sh = 0;
-    float fg = 0, fh = 0;
-    const int CH = 4096;
-    long nch = (o.n + CH - 1) / CH;
-    std::vector<GH> part(nch);
-#pragma omp parallel for
-    for (long c = 0; c < nch; ++c) {
-        float a = 0, b = 0;
-        long e = std::min<long>(o.n, (c + 1) * CH);
-        for (long i = c * CH; i < e; ++i) {
-            a += g[i].g;
-            b += g[i].h;
-        }
-        part[c] = GH{a, b};
-    }
-    for (long c = 0; c < nch; ++c) {
-        fg += part[c].g;
-        fh += part[c].h;
-    }
-    (void)sg;
-    (void)sh;
+    const GH rs = sum_gh(o.gh.data() + (long)k * o.n, o.n);
+    const float fg = rs.g, fh = rs.h;
     Node &root = o.nodes[0];
     root.sum = GH{fg, fh};
     root.is_valid = true;
@@ -633,17 +642,8 @@ float metric(const std::string &obj, int n, int num_class, const float *y, const
 void init_base_score(Oracle &o) {
     if (o.objective == "reg:linear" || o.objective == "reg:logistic" || o.objective == "binary:logistic") {
         gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
-        float sg = 0, sh = 0;
-        const int CH = 4096;
-        for (long c = 0; c < o.n; c += CH) {
-            float a = 0, b = 0;
-            for (long i = c; i < std::min<long>(o.n, c + CH); ++i) {
-                a += o.gh[i].g;
-                b += o.gh[i].h;
-            }
-            sg += a;
-            sh += b;
-        }
+        const GH bs = sum_gh(o.gh.data(), o.n);
+        const float sg = bs.g, sh = bs.h;
         float w = (float)(-sg / fmax((double)sh, 1e-6));
         if (o.objective == "binary:logistic") {
             w = 1 / (1 + expf(-w));

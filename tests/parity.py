@@ -42,20 +42,46 @@ class TreeDiff:
         return "TreeDiff(compared=%d, near_ties=%r)" % (self.compared, self.near_ties)
 
 
-def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, feature_has_missing=None, rel=REL):
+def rows_in_node(final_nid, x):
+    """Mask of the rows whose path from the root passes through heap node x."""
+    cur = np.asarray(final_nid).copy()
+    while True:
+        above = cur > x
+        if not above.any():
+            break
+        cur[above] = (cur[above] - 1) // 2
+    return cur == x
+
+
+def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL):
     """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
 
     Where both trees split on the same candidate everything must agree: threshold and bin exactly,
-    gain / child sums / weights to `rel` of their scale. Where the choice differs, the oracle's own
-    gain of the GPU's candidate must be within tolerance of the oracle's best (a near tie); the
-    subtree below such a node is not compared. `default_right` is only compared for features that
-    have missing values (for dense features the reference decides it by float32 round-off).
+    gain / child sums / weights to tolerance. Where the choice differs, the oracle's own gain of the
+    GPU's candidate must be within tolerance of the oracle's best (a near tie); the subtree below
+    such a node is not compared. `default_right` is only compared where
+    missing_rows(node, feature) > 0: without missing rows in the node the reference decides it by
+    float32 round-off of node_sum - feature_total.
+
+    Tolerance: node sums are float32 results of a chain of histogram subtractions that starts at the
+    root, so their error is relative to the root-level sums of |g| and |h| (abs_scale = (Ag, Ah)):
+    |dG| <= rel * Ag, |dH| <= rel * Ah. Weights and gains get the first-order propagation of those
+    two bounds (w = -G/(H+lam); d gain/dG = -2w, d gain/dH = -w^2 per term).
     orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle (None forbids any mismatch);
     crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
     """
     diff = TreeDiff()
-    slack = 10 * rel
     stack = [0]
+    if abs_scale is None:
+        abs_scale = (max(1.0, abs(float(orc[0]["sum_g"])) + float(orc[0]["sum_h"])),) * 2
+    dG, dH = rel * abs_scale[0] + 1e-7, rel * abs_scale[1] + 1e-7
+
+    def gain_tol(x, o):
+        ws = [float(orc[x]["base_weight"])]
+        if o["lch"] >= 0:
+            ws += [float(orc[o["lch"]]["base_weight"]), float(orc[o["rch"]]["base_weight"])]
+        return sum(2 * abs(w) * dG + w * w * dH for w in ws) + rel * max(1.0, abs(float(o["gain"])))
+
     while stack:
         x = stack.pop()
         g, o = gpu[x], orc[x]
@@ -64,20 +90,18 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, feature_has_missing=
             continue
         diff.compared += 1
         S = (float(o["sum_g"]), float(o["sum_h"]))
-        sum_scale = max(1.0, abs(S[0]) + abs(S[1]))
-        assert abs(g["sum_g"] - o["sum_g"]) <= slack * sum_scale and abs(g["sum_h"] - o["sum_h"]) <= slack * sum_scale, \
+        assert abs(g["sum_g"] - o["sum_g"]) <= dG and abs(g["sum_h"] - o["sum_h"]) <= dH, \
             "node %d sum differs: gpu (%g,%g) oracle (%g,%g)" % (x, g["sum_g"], g["sum_h"], o["sum_g"], o["sum_h"])
-        assert abs(g["base_weight"] - o["base_weight"]) <= slack * max(1.0, abs(o["base_weight"])), \
-            "node %d weight differs: %g vs %g" % (x, g["base_weight"], o["base_weight"])
+        w = float(o["base_weight"])
+        assert abs(g["base_weight"] - w) <= (dG + abs(w) * dH) / (S[1] + lam) + rel * max(1.0, abs(w)), \
+            "node %d weight differs: %g vs %g" % (x, g["base_weight"], w)
         split_g, split_o = g["split_fid"] >= 0, o["split_fid"] >= 0
         if not split_g and not split_o:
             continue
         if split_g and split_o and g["split_fid"] == o["split_fid"] and g["split_bid"] == o["split_bid"]:
             assert g["split_value"] == o["split_value"], "node %d threshold differs" % x
-            lch = orc[o["lch"]]
-            sc = max(1.0, abs(float(o["gain"])), gain_scale(S, (float(lch["sum_g"]), float(lch["sum_h"])), lam))
-            assert abs(g["gain"] - o["gain"]) <= slack * sc, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
-            if feature_has_missing is not None and feature_has_missing[o["split_fid"]]:
+            assert abs(g["gain"] - o["gain"]) <= gain_tol(x, o), "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
+            if missing_rows is not None and missing_rows(x, int(o["split_fid"])) > 0:
                 assert g["default_right"] == o["default_right"], "node %d default direction differs" % x
             stack.extend([int(o["lch"]), int(o["rch"])])
             continue
@@ -85,18 +109,37 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, feature_has_missing=
             x, g["split_fid"], g["split_bid"], o["split_fid"], o["split_bid"])
         sc = orc_scores[x]
         best = float(np.abs(sc).max())
-        scale = max(1.0, best, S[0] * S[0] / (S[1] + lam))
+        tol = 2 * gain_tol(x, o)
         if split_g:
             alt = abs(float(sc[int(crp[g["split_fid"]]) + int(g["split_bid"])]))
-            assert best - alt <= slack * scale, \
-                "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d)" % (
-                    x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"])
+            assert best - alt <= tol, \
+                "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d), tol %g" % (
+                    x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"], tol)
         else:
             alt = 0.0  # gpu made a leaf where the oracle split: the gain must sit at the rt_eps edge
-            assert best <= 1e-6 + slack * scale, "node %d: gpu leaf, oracle split gain %g" % (x, best)
+            assert best <= 1e-6 + tol, "node %d: gpu leaf, oracle split gain %g" % (x, best)
         diff.near_ties.append((x, best, alt))
     if not diff.near_ties:
         for key in ("is_leaf", "is_pruned", "final_id", "lch", "rch", "parent"):
             valid = orc["is_valid"] == 1
             assert np.array_equal(gpu[key][valid], orc[key][valid]), "field %s differs" % key
     return diff
+
+
+def leaf_of(nodes, nid):
+    """Unpruned leaf of every row (climbs pruned nodes, like predict_in_training)."""
+    cur = np.asarray(nid).copy()
+    while True:
+        pr = nodes["is_pruned"][cur] == 1
+        if not pr.any():
+            return cur
+        cur[pr] = nodes["parent"][cur[pr]]
+
+
+def pred_tolerance(nodes, nid, lr, lam, abs_scale, y_pred, rel=REL):
+    """Per-row bound on the prediction update lr * w(leaf) given the node-sum bounds of compare_trees."""
+    leaf = leaf_of(nodes, nid)
+    w = np.abs(nodes["base_weight"][leaf].astype(np.float64))
+    H = nodes["sum_h"][leaf].astype(np.float64)
+    dG, dH = rel * abs_scale[0] + 1e-7, rel * abs_scale[1] + 1e-7
+    return lr * ((dG + w * dH) / (H + lam) + rel * np.maximum(1.0, w)) + rel * np.abs(y_pred) + 1e-6

@@ -16,7 +16,6 @@ namespace tgbm {
 
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
 constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
-constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
 
 // Per-level control block written by the planning kernels and read by the worker kernels.
 struct LevelCtl {
@@ -64,8 +63,8 @@ struct TreeBuffers {
     SplitCand *cand = nullptr;     // [max_level_nodes * n_packs]
     GHPair *root_partial = nullptr;  // [num_class * n_grad_blocks] block sums of the gradient kernel
     int n_grad_blocks = 0;
-    // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1])
-    const int *pack_begin = nullptr;
+    // split finder: wavefront w of a node covers features [64 w, 64 w + 64)
+    const int *pack_begin = nullptr;  // unused
     int n_packs = 0;
     const int *cut_row_ptr = nullptr;
     const int *cut_fid = nullptr;

@@ -195,25 +195,9 @@ void Trainer::alloc_tree_buffers() {
     tb.cut_fid = cuts_.cut_fid;
     tb.cut_val = cuts_.cut_val;
 
-    // split-finder packs: whole features, at most kEvalPackBins bins per wavefront
-    std::vector<int> pack_begin;
-    pack_begin.push_back(0);
-    int cur = 0;
-    for (int f = 0; f < F_; ++f) {
-        int k = h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f];
-        if (k == 0) continue;
-        TGBM_CHECK(k <= kEvalPackBins, "feature %d has %d cut points, more than %d", f, k, kEvalPackBins);
-        if (cur + k > kEvalPackBins) {
-            pack_begin.push_back(h_cut_row_ptr_[f]);
-            cur = 0;
-        }
-        cur += k;
-    }
-    pack_begin.push_back(n_bins_);
-    tb.n_packs = (int)pack_begin.size() - 1;
-    int *d_pack = dalloc<int>(pack_begin.size());
-    upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
-    tb.pack_begin = d_pack;
+    // split finder: one lane per feature, one candidate record per wavefront of 64 features
+    tb.n_packs = (F_ + 63) / 64;
+    tb.pack_begin = nullptr;
     tb.cand = dalloc<SplitCand>((size_t)max_level_nodes * tb.n_packs);
 
     // dense block tables

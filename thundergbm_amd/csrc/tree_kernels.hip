@@ -327,6 +327,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(const float *__restrict__
 
 // ------------------------------------------------------------------------ split finding
 __device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float lambda) {
+#pragma clang fp contract(off)
     GHPair r{f.g - l.g, f.h - l.h};
     float gain = 0.f;
     if (l.h >= mcw && r.h >= mcw)
@@ -334,119 +335,60 @@ __device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float
     return fmaxf(0.f, gain);
 }
 
-// One wavefront scans one pack of whole features (at most 256 bins, 4 consecutive bins per lane):
-// segmented inclusive prefix sums per feature, missing = node sum - feature total, gain of every
-// candidate with missing values sent right and left, and the wavefront's best candidate (largest
-// |gain|, ties to the smaller bin index). Follows hist_tree_builder_single.cu:257-347 / :614-704.
+// Split search of one node: every lane owns one feature and walks its bins in ascending order,
+// keeping the running prefix sum in registers, so prefix sums (and therefore exact ties between
+// candidates separated by empty bins) are those of a sequential float32 scan. Pass 1 yields the
+// feature total and missing = node sum - total; pass 2 evaluates every candidate with missing
+// values sent right and left (hist_tree_builder_single.cu:257-325 / :614-681 of the reference).
+// The wavefront then reduces to its best candidate: largest |gain|, ties to the smaller bin index
+// (:330-335). A feature has at most 256 bins, so the walk is a few hundred dependent adds.
 __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const GHPair *__restrict__ hist, int level,
                                                       float mcw, float lambda) {
-    __shared__ GHPair s_miss[kWaves][kEvalPackBins];
-    const int lane = lane_id(), w = wave_id();
-    const int pack = blockIdx.x * kWaves + w;
+#pragma clang fp contract(off)
+    const int lane = lane_id();
+    const int f = blockIdx.x * kBlock + threadIdx.x;
+    const int pack = blockIdx.x * kWaves + wave_id();
     const int x_in = blockIdx.y;
     const int x = (1 << level) - 1 + x_in;
     const TreeNode nd = tb.nodes[x];
-    const bool active = pack < tb.n_packs && nd.is_valid;
-    int b_begin = 0, b_end = 0;
+    const bool active = f < tb.F && nd.is_valid;
+    int b0 = 0, b1 = 0;
     if (active) {
-        b_begin = tb.pack_begin[pack];
-        b_end = tb.pack_begin[pack + 1];
+        b0 = tb.cut_row_ptr[f];
+        b1 = tb.cut_row_ptr[f + 1];
     }
     const GHPair S = nd.sum_gh_pair;
     const GHPair *h = hist + (size_t)x_in * tb.n_bins;
-
-    GHPair inc[4];
-    int lastb[4];  // pack-relative index of the last bin of the element's feature
-    bool valid[4], head[4], last[4];
-    GHPair run{0, 0};
-    bool any_head = false;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int b = b_begin + lane * 4 + j;
-        valid[j] = b < b_end;
-        lastb[j] = 0;
-        head[j] = false;
-        last[j] = false;
-        inc[j] = GHPair{0, 0};
-        if (valid[j]) {
-            GHPair v = h[b];
-            const int f = tb.cut_fid[b];
-            const int fend = tb.cut_row_ptr[f + 1];
-            head[j] = tb.cut_row_ptr[f] == b;
-            last[j] = fend == b + 1;
-            lastb[j] = fend - 1 - b_begin;
-            if (head[j]) {
-                run = v;
-                any_head = true;
-            } else {
-                run.g += v.g;
-                run.h += v.h;
-            }
-            inc[j] = run;
-        }
+    float tg = 0.f, th = 0.f;
+    for (int b = b0; b < b1; ++b) {
+        GHPair v = h[b];
+        tg += v.g;
+        th += v.h;
     }
-    // wavefront segmented inclusive scan of the lane aggregates
-    GHPair agg = run;
-    int flag = any_head ? 1 : 0;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        float pg = __shfl_up(agg.g, d);
-        float ph = __shfl_up(agg.h, d);
-        int pf = __shfl_up(flag, d);
-        if (lane >= d) {
-            if (!flag) {
-                agg.g = pg + agg.g;
-                agg.h = ph + agg.h;
-            }
-            flag |= pf;
-        }
-    }
-    GHPair carry;
-    carry.g = __shfl_up(agg.g, 1);
-    carry.h = __shfl_up(agg.h, 1);
-    if (lane == 0) carry = GHPair{0, 0};
-    bool seen = false;
-    GHPair excl[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (valid[j]) {
-            if (head[j]) seen = true;
-            if (!seen) {
-                inc[j].g = carry.g + inc[j].g;
-                inc[j].h = carry.h + inc[j].h;
-            }
-        }
-        if (head[j])
-            excl[j] = GHPair{0, 0};
-        else
-            excl[j] = (j == 0) ? carry : inc[j - 1];
-        if (valid[j] && last[j]) s_miss[w][lastb[j]] = GHPair{S.g - inc[j].g, S.h - inc[j].h};
-    }
-    __syncthreads();
+    GHPair miss{0.f, 0.f};
+    if (b1 > b0) miss = GHPair{S.g - tg, S.h - th};
     float best = -1.f;  // |score| of the lane's best candidate
     float best_score = 0.f;
     int best_idx = 0x7fffffff;
-    GHPair best_miss{0, 0}, best_left{0, 0};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (valid[j]) {
-            GHPair m = s_miss[w][lastb[j]];
-            GHPair l = excl[j];
-            float gr = split_gain(S, l, mcw, lambda);
-            GHPair l2{l.g + m.g, l.h + m.h};
-            float gl = split_gain(S, l2, mcw, lambda);
-            float score = (gl > gr) ? gl : -gr;
-            float a = fabsf(score);
-            if (a > best) {
-                best = a;
-                best_score = score;
-                best_idx = b_begin + lane * 4 + j;
-                best_miss = m;
-                best_left = l;
-            }
+    GHPair best_left{0.f, 0.f};
+    GHPair run{0.f, 0.f};
+    for (int b = b0; b < b1; ++b) {
+        float gr = split_gain(S, run, mcw, lambda);
+        GHPair l2{run.g + miss.g, run.h + miss.h};
+        float gl = split_gain(S, l2, mcw, lambda);
+        float score = (gl > gr) ? gl : -gr;
+        float a = fabsf(score);
+        if (a > best) {
+            best = a;
+            best_score = score;
+            best_idx = b;
+            best_left = run;
         }
+        GHPair v = h[b];
+        run.g += v.g;
+        run.h += v.h;
     }
-    // wavefront arg-max: larger |score| wins, ties go to the smaller bin index
+    GHPair best_miss = miss;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
         float oa = __shfl_xor(best, d);
@@ -462,10 +404,10 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const GHP
             best_left = GHPair{olg, olh};
         }
     }
-    if (active && lane == 0) {
+    if (lane == 0 && pack < tb.n_packs && nd.is_valid) {
         SplitCand c;
         c.score = best_score;
-        c.index = best_idx;
+        c.index = best_idx;  // 0x7fffffff when none of the wavefront's features has a bin
         c.miss = best_miss;
         c.left = best_left;
         c.pad[0] = c.pad[1] = 0;
@@ -496,6 +438,7 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb, int leve
     int best_idx = 0x7fffffff, best_pack = -1;
     for (int p = threadIdx.x; p < tb.n_packs; p += kBlock) {
         const SplitCand &c = tb.cand[(size_t)x_in * tb.n_packs + p];
+        if (c.index == 0x7fffffff) continue;  // a wavefront whose features have no bins
         float a = fabsf(c.score);
         if (a > best || (a == best && c.index < best_idx)) {
             best = a;
@@ -923,15 +866,18 @@ static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const Dens
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
     dim3 grid(tb.max_hitems, bins.n_blocks);
     size_t lds = (size_t)tb.max_block_bins * 2 * sizeof(float);
-    if (level == 0) {
-        static bool attr_done = false;
-        if (!attr_done) {
+    if (lds > 64 * 1024) {
+        // more than the default dynamic LDS window: opt in once per kernel instance and size
+        static size_t opted = 0;
+        if (lds > opted) {
             HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, true>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, false>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            attr_done = true;
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            opted = lds;
         }
+    }
+    if (level == 0) {
         k_hist_dense<LPR, true><<<grid, kBlock, lds, s>>>(bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built,
                                                          n_pairs, tb.ctl + level, tb.blk_bin_begin, tb.feat_lds_off,
                                                          tb.partial, tb.n_bins);
@@ -963,7 +909,7 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level) {
 }
 
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
-    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level);
+    dim3 grid((tb.F + kBlock - 1) / kBlock, 1 << level);
     k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist[level & 1], level, mcw, lambda);
 }
 
