@@ -423,6 +423,7 @@ def test_full_size_properties_config2(T):
     s.gradient()
     s.tree_init(0)
     gh = s.gh()[:n].astype(np.float64)
+    Ag, Ah = np.abs(gh[:, 0]).sum(), np.abs(gh[:, 1]).sum()
     for level in range(8):
         s.find_split(level)
         hist = s.level_hist(level).astype(np.float64)
@@ -445,8 +446,8 @@ def test_full_size_properties_config2(T):
     hs = np.bincount(nid, weights=gh[:, 1], minlength=len(nodes))
     gs = np.bincount(nid, weights=gh[:, 0], minlength=len(nodes))
     occupied = np.flatnonzero(cnt > 0)
-    np.testing.assert_allclose(nodes["sum_h"][occupied], hs[occupied], rtol=2e-4, atol=1e-2)
-    np.testing.assert_allclose(nodes["sum_g"][occupied], gs[occupied], rtol=0, atol=2e-4 * np.abs(gh[:, 0]).sum() / 16)
+    np.testing.assert_allclose(nodes["sum_h"][occupied], hs[occupied], rtol=0, atol=1e-5 * Ah)
+    np.testing.assert_allclose(nodes["sum_g"][occupied], gs[occupied], rtol=0, atol=1e-5 * Ag)
     s.finish_tree(0)
     # training-time prediction == predictor on a sample of the training rows
     yp = s.y_pred()

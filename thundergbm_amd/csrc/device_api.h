@@ -25,6 +25,22 @@ struct LevelCtl {
     int rows_built;  // rows visited by the histogram build of the level
 };
 
+// Fixed-point scales of one tree. Gradients and hessians are accumulated in LDS as one packed
+// 64-bit integer per bin (gradient in the high, hessian in the low 32 bits) because gfx950 executes
+// 64-bit integer LDS atomics about 15x faster than float ones; scales are powers of two chosen so
+// that a work item's sums cannot leave their 32-bit fields. Sums are merged in 64-bit integers, so
+// histograms (and sibling subtraction) are exact in the quantised values and bit-reproducible.
+struct QuantCtl {
+    float scale_g, scale_h;  // value -> integer
+    float inv_g, inv_h;      // integer -> value
+};
+
+// Block result of the per-tree gradient reduction.
+struct GradStats {
+    float g, h;        // sums
+    float gmax, hmax;  // max |g|, max h
+};
+
 // Candidate produced by one wavefront of the split finder.
 struct SplitCand {
     float score;  // signed gain: > 0 missing goes left, <= 0 missing goes right
@@ -50,7 +66,9 @@ struct TreeBuffers {
     int *ridx[2] = {nullptr, nullptr};  // [n] row lists, ping-pong by level parity
     uint8_t *goes_right = nullptr; // [n]
     GHPair *hist[2] = {nullptr, nullptr};  // [max_level_nodes * n_bins] raw histograms by level parity
-    GHPair *partial = nullptr;     // [max_hitems * n_bins]
+    longlong2 *hist_q[2] = {nullptr, nullptr};  // same shape, exact fixed-point sums (g, h)
+    int2 *partial = nullptr;       // [max_hitems * n_bins] per-item fixed-point sums (g signed, h unsigned)
+    QuantCtl *quant = nullptr;     // scales of the current tree
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
     int *hpair_begin = nullptr;    // [max_pairs + 1] first histogram item of every sibling pair
     int *hpair_built = nullptr;    // [max_pairs] heap id of the node built from rows, -1 = inactive pair
@@ -61,7 +79,7 @@ struct TreeBuffers {
     LevelCtl *ctl = nullptr;       // [depth + 1]
     SplitPoint *sp = nullptr;      // [max_level_nodes]
     SplitCand *cand = nullptr;     // [max_level_nodes * n_packs]
-    GHPair *root_partial = nullptr;  // [num_class * n_grad_blocks] block sums of the gradient kernel
+    GradStats *root_partial = nullptr;  // [n_grad_blocks] block results of the per-tree gradient reduction
     int n_grad_blocks = 0;
     // split finder: wavefront w of a node covers features [64 w, 64 w + 64)
     const int *pack_begin = nullptr;  // unused
@@ -80,7 +98,7 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *class_block_sums, float lambda);
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);

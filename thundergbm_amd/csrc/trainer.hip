@@ -178,7 +178,10 @@ void Trainer::alloc_tree_buffers() {
     tb.hist[1] = dalloc<GHPair>((size_t)max_level_nodes * n_bins_);
     tb.target_hitems = std::min(1024, std::max(4, 1024 / bins_.n_blocks));
     tb.max_hitems = tb.target_hitems + max_pairs + 1;
-    tb.partial = dalloc<GHPair>((size_t)tb.max_hitems * n_bins_);
+    tb.hist_q[0] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
+    tb.hist_q[1] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
+    tb.partial = dalloc<int2>((size_t)tb.max_hitems * n_bins_);
+    tb.quant = dalloc<QuantCtl>(1);
     tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
     // the planning kernel of the last level also writes the (unused) plan of level `depth`
     tb.hpair_begin = dalloc<int>((size_t)max_level_nodes + 1);
@@ -190,7 +193,7 @@ void Trainer::alloc_tree_buffers() {
     tb.ctl = dalloc<LevelCtl>((size_t)depth + 2);
     tb.sp = dalloc<SplitPoint>((size_t)max_level_nodes);
     tb.n_grad_blocks = std::min(1024, (n_ + 255) / 256);
-    tb.root_partial = dalloc<GHPair>((size_t)tb.n_grad_blocks);
+    tb.root_partial = dalloc<GradStats>((size_t)tb.n_grad_blocks);
     tb.cut_row_ptr = cuts_.cut_row_ptr;
     tb.cut_fid = cuts_.cut_fid;
     tb.cut_val = cuts_.cut_val;
@@ -411,6 +414,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "sp") src = tb_.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
     else if (name == "hist0") src = tb_.hist[0], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
     else if (name == "hist1") src = tb_.hist[1], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "quant") src = tb_.quant, bytes = sizeof(QuantCtl);
     else if (name == "ctl") src = tb_.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
     else if (name == "seg") src = tb_.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;
     else if (name == "ridx0") src = tb_.ridx[0], bytes = sizeof(int) * (size_t)n_;
