@@ -28,6 +28,8 @@ def main():
     ap.add_argument("--depth", type=int, default=8)
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--cpu-steps", type=int, default=2, help="boosting iterations of the CPU baseline (0 = skip)")
+    ap.add_argument("--calibration-copy-mb", type=int, default=0,
+                    help="also run 3 launches of a plain copy kernel of this many MiB (profiler counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU baseline sample (0 = all rows)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -80,6 +82,8 @@ def main():
                         "rows_built_per_tree": prof["rows_built"] // args.profile_steps}
     metric_log = s.metric_log()
     s.close()
+    if args.calibration_copy_mb > 0:
+        T.load().tgbm_calibration_copy(args.calibration_copy_mb << 20, 3)
 
     cpu = None
     if args.cpu_steps > 0:

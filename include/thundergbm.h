@@ -100,8 +100,8 @@ int tgbm_trainer_info(tgbm_trainer *t, const char *key);
 float tgbm_trainer_base_score(tgbm_trainer *t);
 
 /* Copies a device buffer to `out` when `cap` is large enough; always returns its size in bytes.
- * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist0, hist1, ctl,
- * seg, ridx0, ridx1, model, metric_log. */
+ * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist_q0, hist_q1,
+ * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels. */
 size_t tgbm_trainer_get(tgbm_trainer *t, const char *name, void *out, size_t cap);
 /* Overwrites gh or y_pred (lock-step tests feed both implementations the same state). */
 void tgbm_trainer_set(tgbm_trainer *t, const char *name, const void *in, size_t bytes);
@@ -125,6 +125,11 @@ void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const 
  * slot per stored value at most (row_ptr[row_size]); returns the number of cut points. */
 int tgbm_cut_points(int row_size, int n_features, const float *val, const int *row_ptr, const int *col_ptr,
                     int max_num_bin, float *cut_val, int *cut_row_ptr, int *cut_fid, int *bin_id);
+
+/* Runs `repeats` launches of a plain streaming copy kernel (k_calibration_copy) over `bytes` bytes.
+ * It has no counterpart in the reference: it exists to calibrate a profiler's HBM byte counters
+ * (FETCH_SIZE / WRITE_SIZE) against a transfer of known size. */
+void tgbm_calibration_copy(size_t bytes, int repeats);
 
 #ifdef __cplusplus
 }

@@ -435,8 +435,9 @@ def test_full_size_properties_config2(T):
                 continue
             for f in (0, 13, 27):  # dense features: every row lands in exactly one bin of the feature
                 tot = hist[x, crp[f]:crp[f + 1]].sum(axis=0)
-                sc = max(1.0, np.abs(gh[:, 0]).sum() / (1 << level))
-                assert abs(tot[0] - nd["sum_g"]) <= 2e-4 * sc and abs(tot[1] - nd["sum_h"]) <= 2e-4 * sc
+                # node sums come from float32 prefix sums of ancestors' histograms, so their error
+                # is relative to the root-level magnitude, not to the node's own
+                assert abs(tot[0] - nd["sum_g"]) <= 1e-5 * Ag and abs(tot[1] - nd["sum_h"]) <= 1e-5 * Ah
         s.partition(level)
     nid = s.nid()
     nodes = s.nodes()

@@ -16,6 +16,7 @@ namespace tgbm {
 
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
 constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
+constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
 
 // Per-level control block written by the planning kernels and read by the worker kernels.
 struct LevelCtl {
@@ -28,7 +29,8 @@ struct LevelCtl {
 // Fixed-point scales of one tree. Gradients and hessians are accumulated in LDS as one packed
 // 64-bit integer per bin (gradient in the high, hessian in the low 32 bits) because gfx950 executes
 // 64-bit integer LDS atomics about 15x faster than float ones; scales are powers of two chosen so
-// that a work item's sums cannot leave their 32-bit fields. Sums are merged in 64-bit integers, so
+// that the sums of a few thousand rows cannot leave their 32-bit fields; the LDS bins are drained
+// into 64-bit integers before that many rows were added. All further sums are 64-bit integers, so
 // histograms (and sibling subtraction) are exact in the quantised values and bit-reproducible.
 struct QuantCtl {
     float scale_g, scale_h;  // value -> integer
@@ -56,6 +58,10 @@ struct DenseBins {
     int W = 0;          // bytes (features) per row of a block, multiple of 4
     int n_blocks = 0;
     size_t block_stride = 0;  // bytes between blocks = n * W
+    // Column-major copy (feature f = n consecutive bytes at col + f * col_stride): the partition reads
+    // one feature of many rows, which costs one byte per row here instead of one sector per row.
+    const uint8_t *col = nullptr;
+    size_t col_stride = 0;
 };
 
 struct TreeBuffers {
@@ -65,9 +71,9 @@ struct TreeBuffers {
     int *nid = nullptr;            // [n]
     int *ridx[2] = {nullptr, nullptr};  // [n] row lists, ping-pong by level parity
     uint8_t *goes_right = nullptr; // [n]
-    GHPair *hist[2] = {nullptr, nullptr};  // [max_level_nodes * n_bins] raw histograms by level parity
-    longlong2 *hist_q[2] = {nullptr, nullptr};  // same shape, exact fixed-point sums (g, h)
-    int2 *partial = nullptr;       // [max_hitems * n_bins] per-item fixed-point sums (g signed, h unsigned)
+    longlong2 *hist_q[2] = {nullptr, nullptr};  // [max_level_nodes * n_bins] exact fixed-point histograms (g, h)
+                                                // of the nodes of a level, ping-pong by level parity
+    longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
     QuantCtl *quant = nullptr;     // scales of the current tree
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
     int *hpair_begin = nullptr;    // [max_pairs + 1] first histogram item of every sibling pair
@@ -81,9 +87,11 @@ struct TreeBuffers {
     SplitCand *cand = nullptr;     // [max_level_nodes * n_packs]
     GradStats *root_partial = nullptr;  // [n_grad_blocks] block results of the per-tree gradient reduction
     int n_grad_blocks = 0;
-    // split finder: wavefront w of a node covers features [64 w, 64 w + 64)
-    const int *pack_begin = nullptr;  // unused
+    // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1]) (whole features)
+    const int *pack_begin = nullptr;
     int n_packs = 0;
+    int *fitem_begin = nullptr;    // [n_nodes + 1] work items of the row -> node rebuild
+    int max_fitems = 0;
     const int *cut_row_ptr = nullptr;
     const int *cut_fid = nullptr;
     const float *cut_val = nullptr;
@@ -104,16 +112,19 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level);
+void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb);
 void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma);
 void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, float *yp_class, float lr);
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);
 void launch_fill_f32(hipStream_t s, float *p, float v, size_t n);
+void launch_calibration_copy(hipStream_t s, const void *src, void *dst, size_t bytes);
 void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 
 // data preparation
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
-                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride);
+                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
+                      size_t col_stride);
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id);
 // cut points on device: returns the device arrays through out parameters allocated by the callee

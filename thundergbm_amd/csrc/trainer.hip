@@ -108,13 +108,18 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     const size_t mat_bytes = (size_t)n_ * W * n_blocks;
     size_t free_b = 0, total_b = 0;
     HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-    TGBM_CHECK(mat_bytes < free_b / 2,
+    TGBM_CHECK(mat_bytes + (size_t)n_ * F_ < free_b / 2,
                "dense bin matrix of %zu bytes does not fit (free %zu); the sparse histogram path is not built yet",
                mat_bytes, free_b);
     d_binmat_ = dalloc<uint8_t>(mat_bytes);
     launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);
+    const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
+    uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_);
+    launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_);
     launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                     (size_t)n_ * W);
+                     (size_t)n_ * W, d_colmat, col_stride);
+    bins_.col = d_colmat;
+    bins_.col_stride = col_stride;
     bins_.data = d_binmat_;
     bins_.W = W;
     bins_.n_blocks = n_blocks;
@@ -174,13 +179,11 @@ void Trainer::alloc_tree_buffers() {
     tb.ridx[0] = dalloc<int>(n_);
     tb.ridx[1] = dalloc<int>(n_);
     tb.goes_right = dalloc<uint8_t>((size_t)n_ + 4);
-    tb.hist[0] = dalloc<GHPair>((size_t)max_level_nodes * n_bins_);
-    tb.hist[1] = dalloc<GHPair>((size_t)max_level_nodes * n_bins_);
-    tb.target_hitems = std::min(1024, std::max(4, 1024 / bins_.n_blocks));
+    tb.target_hitems = std::min(512, std::max(4, 512 / bins_.n_blocks));  // ~2 resident workgroups per CU
     tb.max_hitems = tb.target_hitems + max_pairs + 1;
     tb.hist_q[0] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
     tb.hist_q[1] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
-    tb.partial = dalloc<int2>((size_t)tb.max_hitems * n_bins_);
+    tb.partial = dalloc<longlong2>((size_t)tb.max_hitems * n_bins_);
     tb.quant = dalloc<QuantCtl>(1);
     tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
     // the planning kernel of the last level also writes the (unused) plan of level `depth`
@@ -198,10 +201,28 @@ void Trainer::alloc_tree_buffers() {
     tb.cut_fid = cuts_.cut_fid;
     tb.cut_val = cuts_.cut_val;
 
-    // split finder: one lane per feature, one candidate record per wavefront of 64 features
-    tb.n_packs = (F_ + 63) / 64;
-    tb.pack_begin = nullptr;
+    // split-finder packs: whole features, at most kEvalPackBins bins per wavefront
+    std::vector<int> pack_begin;
+    pack_begin.push_back(0);
+    int cur = 0;
+    for (int f = 0; f < F_; ++f) {
+        int k = h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f];
+        if (k == 0) continue;
+        TGBM_CHECK(k <= kEvalPackBins, "feature %d has %d cut points, more than %d", f, k, kEvalPackBins);
+        if (cur + k > kEvalPackBins) {
+            pack_begin.push_back(h_cut_row_ptr_[f]);
+            cur = 0;
+        }
+        cur += k;
+    }
+    pack_begin.push_back(n_bins_);
+    tb.n_packs = (int)pack_begin.size() - 1;
+    int *d_pack = dalloc<int>(pack_begin.size());
+    upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
+    tb.pack_begin = d_pack;
     tb.cand = dalloc<SplitCand>((size_t)max_level_nodes * tb.n_packs);
+    tb.fitem_begin = dalloc<int>((size_t)tb.n_nodes + 1);
+    tb.max_fitems = n_ / kPartChunk + tb.n_nodes + 1;
 
     // dense block tables
     const int W = bins_.W, nb = bins_.n_blocks;
@@ -276,6 +297,7 @@ void Trainer::partition(int level) { launch_partition_dense(stream_, tb_, bins_,
 
 void Trainer::finish_tree(int k) {
     launch_prune(stream_, tb_, param_.gamma);
+    launch_nid_rebuild(stream_, tb_);
     launch_predict_in_training(stream_, tb_, d_yp_ + (size_t)k * n_, param_.learning_rate);
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb_.n_nodes, tb_.nodes,
@@ -406,14 +428,18 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
     else if (name == "binmat") src = d_binmat_, bytes = (size_t)n_ * bins_.W * bins_.n_blocks;
-    else if (name == "nid") src = tb_.nid, bytes = sizeof(int) * (size_t)n_;
+    else if (name == "nid") {
+        launch_nid_rebuild(stream_, tb_);  // the map is kept as row lists; materialise it on demand
+        sync();
+        src = tb_.nid, bytes = sizeof(int) * (size_t)n_;
+    }
     else if (name == "gh") src = d_gh_, bytes = sizeof(GHPair) * (size_t)param_.num_class * n_;
     else if (name == "y_pred") src = d_yp_, bytes = sizeof(float) * (size_t)n_yp_;
     else if (name == "y") src = d_y_, bytes = sizeof(float) * (size_t)n_;
     else if (name == "nodes") src = tb_.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
     else if (name == "sp") src = tb_.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
-    else if (name == "hist0") src = tb_.hist[0], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
-    else if (name == "hist1") src = tb_.hist[1], bytes = sizeof(GHPair) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "hist_q0") src = tb_.hist_q[0], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "hist_q1") src = tb_.hist_q[1], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
     else if (name == "quant") src = tb_.quant, bytes = sizeof(QuantCtl);
     else if (name == "ctl") src = tb_.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
     else if (name == "seg") src = tb_.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;

@@ -10,6 +10,15 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / 64;
 constexpr int kHistMinChunk = 1024;
+#ifndef TGBM_HIST_BLOCK
+#define TGBM_HIST_BLOCK 1024
+#endif
+constexpr int kHistBlock = TGBM_HIST_BLOCK;  // threads per histogram workgroup (they share one LDS histogram)
+#ifndef TGBM_FLUSH_EVERY
+#define TGBM_FLUSH_EVERY 8192
+#endif
+constexpr int kHistFlushEvery = TGBM_FLUSH_EVERY;  // timing experiments only; must equal kHistFlushRows
+constexpr int kHistFlushRows = 8192;         // rows a packed 32+32-bit LDS bin may absorb before it is drained
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
@@ -69,6 +78,12 @@ __device__ int find_owner(const int *begin, int n, int item) {
             hi = mid;
     }
     return lo;
+}
+
+// Plain streaming copy of 16-byte words; used to calibrate the profiler's HBM byte counters.
+__global__ void k_calibration_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
 }
 
 // ------------------------------------------------------------------------------------ fills
@@ -248,12 +263,12 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
         c.n_pitems = 0;
         c.rows_built = tb.n;
         tb.ctl[0] = c;
-        // No level has larger work items than the root (their chunk is derived from at most n rows),
-        // so one pair of scales serves the whole tree: a work item's gradient sum stays inside a
-        // signed and its hessian sum inside an unsigned 32-bit field.
+        // One pair of scales serves the whole tree: between two drains of the LDS histogram at most
+        // kHistFlushRows rows are added, which keeps a bin's gradient sum inside a signed and its
+        // hessian sum inside an unsigned 32-bit field.
         QuantCtl q;
-        q.scale_g = pow2_scale(gm, chunk, 1073741824.f);
-        q.scale_h = pow2_scale(hm, chunk, 2147483648.f);
+        q.scale_g = pow2_scale(gm, kHistFlushRows, 2147483520.f);  // largest float below 2^31
+        q.scale_h = pow2_scale(hm, kHistFlushRows, 4294967040.f);  // largest float below 2^32
         q.inv_g = 1.f / q.scale_g;
         q.inv_h = 1.f / q.scale_h;
         *tb.quant = q;
@@ -264,20 +279,23 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
 // One workgroup = one work item (a run of rows of one node) x one feature block. The block's
 // histogram lives in LDS as one 64-bit integer per bin holding the fixed-point gradient sum in the
 // high and the hessian sum in the low half; a row contributes with a single ds_add_u64 per feature
-// (float LDS atomics run at ~0.3 lanes/clk/CU on gfx950, 64-bit integer ones at ~5). The finished
-// private histogram is stored to the item's slot of `partial`.
+// (float LDS atomics run at ~0.3 lanes/clk/CU on gfx950, 64-bit integer ones at ~5). The 32-bit
+// fields are safe for kHistFlushRows rows (that bound sets the fixed-point scales), so after at most
+// that many rows every thread drains the bins it owns into 64-bit register accumulators and clears
+// them; at the end the registers go to the item's slot of `partial`.
 // LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
 // instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
-template <int LPR, bool DIRECT>
-__global__ __launch_bounds__(kBlock) void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
-                                                      const int *__restrict__ ridx, const int2 *__restrict__ seg,
-                                                      const int *__restrict__ hpair_begin,
-                                                      const int *__restrict__ hpair_built, int n_pairs,
-                                                      const LevelCtl *__restrict__ ctl,
-                                                      const QuantCtl *__restrict__ quant,
-                                                      const int *__restrict__ blk_bin_begin,
-                                                      const int *__restrict__ feat_lds_off,
-                                                      int2 *__restrict__ partial, int n_bins) {
+template <int LPR, bool DIRECT, int BLK, int SLOTS>
+__global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
+void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
+                                                    const int *__restrict__ ridx, const int2 *__restrict__ seg,
+                                                    const int *__restrict__ hpair_begin,
+                                                    const int *__restrict__ hpair_built, int n_pairs,
+                                                    const LevelCtl *__restrict__ ctl,
+                                                    const QuantCtl *__restrict__ quant,
+                                                    const int *__restrict__ blk_bin_begin,
+                                                    const int *__restrict__ feat_lds_off,
+                                                    longlong2 *__restrict__ partial, int n_bins) {
     extern __shared__ unsigned long long lds[];
     __shared__ int s_range[2];
     const LevelCtl c = *ctl;
@@ -295,30 +313,58 @@ __global__ __launch_bounds__(kBlock) void k_hist_dense(DenseBins bins, const GHP
         s_range[0] = b;
         s_range[1] = min(sg.y, b + c.hchunk);
     }
-    for (int i = threadIdx.x; i < nb; i += kBlock) lds[i] = 0ull;
+    for (int i = threadIdx.x; i < nb; i += BLK) lds[i] = 0ull;
     __syncthreads();
     const int begin = s_range[0], end = s_range[1];
     const float scale_g = quant->scale_g, scale_h = quant->scale_h;
-    constexpr int RPS = kBlock / LPR;  // rows per step of the whole block
+    constexpr int RPS = BLK / LPR;  // rows per step of the whole block
+    constexpr int U = 4;
+    static_assert(RPS * U <= kHistFlushRows, "one iteration must not exceed the flush interval");
     const int q = threadIdx.x % LPR;
     const int rsub = threadIdx.x / LPR;
     const int W = LPR * 4;
     const int *fo = feat_lds_off + fb * W + q * 4;
     const int o0 = fo[0], o1 = fo[1], o2 = fo[2], o3 = fo[3];
     const uint8_t *blk = bins.data + (size_t)fb * bins.block_stride + q * 4;
-    constexpr int U = 4;
-    for (int pos0 = begin + rsub; pos0 < end; pos0 += RPS * U) {
-        unsigned pk[U];
-        GHPair s[U];
+    long long accg[SLOTS], acch[SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) accg[k] = acch[k] = 0;
+    int pending = 0;  // rows accumulated in LDS since the last drain (uniform across the block)
+    unsigned pk[U], pk_next[U];
+    GHPair s[U], s_next[U];
+    auto load_rows = [&](int base, unsigned(&opk)[U], GHPair(&os)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            int pos = pos0 + u * RPS;
+            int pos = base + rsub + u * RPS;
             bool ok = pos < end;
             int r = 0;
             if (ok) r = DIRECT ? pos : ridx[pos];
-            pk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
-            s[u] = ok ? gh[r] : GHPair{0, 0};
+            opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
+            os[u] = ok ? gh[r] : GHPair{0, 0};
         }
+    };
+    if (begin < end) load_rows(begin, pk, s);
+    for (int base = begin; base < end; base += RPS * U) {
+        // the next step's rows are requested before this step's atomics (and before a drain's
+        // barriers), so the memory pipeline stays busy
+        if (base + RPS * U < end) load_rows(base + RPS * U, pk_next, s_next);
+        if (pending + RPS * U > kHistFlushEvery) {
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < SLOTS; ++k) {
+                const int i = threadIdx.x + k * BLK;
+                if (i < nb) {
+                    const unsigned long long t = lds[i];
+                    lds[i] = 0ull;
+                    const unsigned lo = (unsigned)t;
+                    accg[k] += (int)((long long)(t - lo) >> 32);
+                    acch[k] += lo;
+                }
+            }
+            __syncthreads();
+            pending = 0;
+        }
+        pending += RPS * U;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const unsigned v = pk[u];
@@ -331,49 +377,67 @@ __global__ __launch_bounds__(kBlock) void k_hist_dense(DenseBins bins, const GHP
             if (b2 != kMissingBin) atomicAdd(lds + o2 + b2, add);
             if (b3 != kMissingBin) atomicAdd(lds + o3 + b3, add);
         }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            pk[u] = pk_next[u];
+            s[u] = s_next[u];
+        }
     }
     __syncthreads();
-    int2 *out = partial + (size_t)item * n_bins + bin0;
-    for (int i = threadIdx.x; i < nb; i += kBlock) {
-        const unsigned long long t = lds[i];
-        const unsigned lo = (unsigned)t;
-        const int hi = (int)((long long)(t - lo) >> 32);
-        out[i] = make_int2(hi, (int)lo);
+    longlong2 *out = partial + (size_t)item * n_bins + bin0;
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int i = threadIdx.x + k * BLK;
+        if (i < nb) {
+            const unsigned long long t = lds[i];
+            const unsigned lo = (unsigned)t;
+            out[i] = make_longlong2(accg[k] + (int)((long long)(t - lo) >> 32), acch[k] + lo);
+        }
     }
 }
 
-// Sum the private histograms of the node that was built from rows (64-bit integers, exact) and
-// derive its sibling as parent - built (the reference's subtraction trick,
-// hist_tree_builder_single.cu:526-540), then convert both to float for the split finder.
-__global__ __launch_bounds__(kBlock) void k_hist_merge(const int2 *__restrict__ partial, longlong2 *__restrict__ cur_q,
+// Sum the private histograms of the node that was built from rows (64-bit integers, exact, any
+// order gives the same bits) and derive its sibling as parent - built (the reference's subtraction
+// trick, hist_tree_builder_single.cu:526-540). A block covers 32 bins of one sibling pair; its eight
+// thread groups stride over the pair's work items and are combined through LDS.
+constexpr int kMergeBins = 32;
+constexpr int kMergeGroups = kBlock / kMergeBins;
+
+__global__ __launch_bounds__(kBlock) void k_hist_merge(const longlong2 *__restrict__ partial,
+                                                      longlong2 *__restrict__ cur_q,
                                                       const longlong2 *__restrict__ prev_q,
-                                                      GHPair *__restrict__ cur, const QuantCtl *__restrict__ quant,
                                                       const int *__restrict__ hpair_begin,
                                                       const int *__restrict__ hpair_built, int level, int n_bins) {
+    __shared__ long long s_g[kMergeGroups][kMergeBins], s_h[kMergeGroups][kMergeBins];
     const int p = blockIdx.y;
     const int built = hpair_built[p];
     if (built < 0) return;
-    const int j = blockIdx.x * kBlock + threadIdx.x;
-    if (j >= n_bins) return;
+    const int jl = threadIdx.x % kMergeBins, ig = threadIdx.x / kMergeBins;
+    const int j = blockIdx.x * kMergeBins + jl;
     const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
     long long sg = 0, sh = 0;
-    for (int it = ib; it < ie; ++it) {
-        int2 v = partial[(size_t)it * n_bins + j];
-        sg += v.x;
-        sh += (unsigned)v.y;
+    if (j < n_bins) {
+        for (int it = ib + ig; it < ie; it += kMergeGroups) {
+            longlong2 v = partial[(size_t)it * n_bins + j];
+            sg += v.x;
+            sh += v.y;
+        }
     }
-    const double inv_g = quant->inv_g, inv_h = quant->inv_h;
+    s_g[ig][jl] = sg;
+    s_h[ig][jl] = sh;
+    __syncthreads();
+    if (ig != 0 || j >= n_bins) return;
+#pragma unroll
+    for (int k = 1; k < kMergeGroups; ++k) {
+        sg += s_g[k][jl];
+        sh += s_h[k][jl];
+    }
     const int off = (1 << level) - 1;
-    const size_t bi = (size_t)(built - off) * n_bins + j;
-    cur_q[bi] = make_longlong2(sg, sh);
-    cur[bi] = GHPair{(float)((double)sg * inv_g), (float)((double)sh * inv_h)};
+    cur_q[(size_t)(built - off) * n_bins + j] = make_longlong2(sg, sh);
     if (level > 0) {
         const int sib = (built & 1) ? built + 1 : built - 1;
-        const size_t si = (size_t)(sib - off) * n_bins + j;
         const longlong2 par = prev_q[(size_t)p * n_bins + j];
-        const long long rg = par.x - sg, rh = par.y - sh;
-        cur_q[si] = make_longlong2(rg, rh);
-        cur[si] = GHPair{(float)((double)rg * inv_g), (float)((double)rh * inv_h)};
+        cur_q[(size_t)(sib - off) * n_bins + j] = make_longlong2(par.x - sg, par.y - sh);
     }
 }
 
@@ -387,60 +451,135 @@ __device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float
     return fmaxf(0.f, gain);
 }
 
-// Split search of one node: every lane owns one feature and walks its bins in ascending order,
-// keeping the running prefix sum in registers, so prefix sums (and therefore exact ties between
-// candidates separated by empty bins) are those of a sequential float32 scan. Pass 1 yields the
-// feature total and missing = node sum - total; pass 2 evaluates every candidate with missing
-// values sent right and left (hist_tree_builder_single.cu:257-325 / :614-681 of the reference).
-// The wavefront then reduces to its best candidate: largest |gain|, ties to the smaller bin index
-// (:330-335). A feature has at most 256 bins, so the walk is a few hundred dependent adds.
-__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const GHPair *__restrict__ hist, int level,
+__device__ __forceinline__ long long shfl_up_ll(long long v, int d) {
+    int lo = __shfl_up((int)(unsigned)(unsigned long long)v, d);
+    int hi = __shfl_up((int)((unsigned long long)v >> 32), d);
+    return (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
+// Split search. One wavefront scans one pack of whole features (at most 256 bins, 4 consecutive bins
+// per lane) of one node with a segmented inclusive prefix sum over the exact 64-bit fixed-point
+// histogram: integer sums are associative, so the parallel scan returns bit-for-bit what a
+// sequential one would, and candidates separated only by empty bins tie exactly. Per candidate:
+// left = sum of the feature's bins below it, missing = node sum - feature total, gain with missing
+// values sent right and left (hist_tree_builder_single.cu:257-325 / :614-681 of the reference);
+// the wavefront keeps its best candidate: largest |gain|, ties to the smaller bin index (:330-335).
+__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const longlong2 *__restrict__ hist_q, int level,
                                                       float mcw, float lambda) {
 #pragma clang fp contract(off)
-    const int lane = lane_id();
-    const int f = blockIdx.x * kBlock + threadIdx.x;
-    const int pack = blockIdx.x * kWaves + wave_id();
+    __shared__ GHPair s_miss[kWaves][kEvalPackBins];
+    const int lane = lane_id(), w = wave_id();
+    const int pack = blockIdx.x * kWaves + w;
     const int x_in = blockIdx.y;
     const int x = (1 << level) - 1 + x_in;
     const TreeNode nd = tb.nodes[x];
-    const bool active = f < tb.F && nd.is_valid;
-    int b0 = 0, b1 = 0;
+    const bool active = pack < tb.n_packs && nd.is_valid;
+    int b_begin = 0, b_end = 0;
     if (active) {
-        b0 = tb.cut_row_ptr[f];
-        b1 = tb.cut_row_ptr[f + 1];
+        b_begin = tb.pack_begin[pack];
+        b_end = tb.pack_begin[pack + 1];
     }
     const GHPair S = nd.sum_gh_pair;
-    const GHPair *h = hist + (size_t)x_in * tb.n_bins;
-    float tg = 0.f, th = 0.f;
-    for (int b = b0; b < b1; ++b) {
-        GHPair v = h[b];
-        tg += v.g;
-        th += v.h;
+    const longlong2 *h = hist_q + (size_t)x_in * tb.n_bins;
+    const double inv_g = tb.quant->inv_g, inv_h = tb.quant->inv_h;
+
+    long long incg[4], inch[4];
+    int lastb[4];  // pack-relative index of the last bin of the element's feature
+    bool valid[4], head[4], last[4];
+    long long rung = 0, runh = 0;
+    bool any_head = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int b = b_begin + lane * 4 + j;
+        valid[j] = b < b_end;
+        lastb[j] = 0;
+        head[j] = false;
+        last[j] = false;
+        incg[j] = inch[j] = 0;
+        if (valid[j]) {
+            longlong2 v = h[b];
+            const int f = tb.cut_fid[b];
+            const int fend = tb.cut_row_ptr[f + 1];
+            head[j] = tb.cut_row_ptr[f] == b;
+            last[j] = fend == b + 1;
+            lastb[j] = fend - 1 - b_begin;
+            if (head[j]) {
+                rung = v.x;
+                runh = v.y;
+                any_head = true;
+            } else {
+                rung += v.x;
+                runh += v.y;
+            }
+            incg[j] = rung;
+            inch[j] = runh;
+        }
     }
-    GHPair miss{0.f, 0.f};
-    if (b1 > b0) miss = GHPair{S.g - tg, S.h - th};
+    // wavefront segmented inclusive scan of the lane aggregates
+    long long aggg = rung, aggh = runh;
+    int flag = any_head ? 1 : 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        long long pg = shfl_up_ll(aggg, d);
+        long long ph = shfl_up_ll(aggh, d);
+        int pf = __shfl_up(flag, d);
+        if (lane >= d) {
+            if (!flag) {
+                aggg += pg;
+                aggh += ph;
+            }
+            flag |= pf;
+        }
+    }
+    long long carryg = shfl_up_ll(aggg, 1), carryh = shfl_up_ll(aggh, 1);
+    if (lane == 0) carryg = carryh = 0;
+    bool seen = false;
+    long long exg[4], exh[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (valid[j]) {
+            if (head[j]) seen = true;
+            if (!seen) {
+                incg[j] += carryg;
+                inch[j] += carryh;
+            }
+        }
+        if (head[j]) {
+            exg[j] = exh[j] = 0;
+        } else {
+            exg[j] = (j == 0) ? carryg : incg[j > 0 ? j - 1 : 0];
+            exh[j] = (j == 0) ? carryh : inch[j > 0 ? j - 1 : 0];
+        }
+        if (valid[j] && last[j]) {
+            const float tg = (float)((double)incg[j] * inv_g), th = (float)((double)inch[j] * inv_h);
+            s_miss[w][lastb[j]] = GHPair{S.g - tg, S.h - th};
+        }
+    }
+    __syncthreads();
     float best = -1.f;  // |score| of the lane's best candidate
     float best_score = 0.f;
     int best_idx = 0x7fffffff;
-    GHPair best_left{0.f, 0.f};
-    GHPair run{0.f, 0.f};
-    for (int b = b0; b < b1; ++b) {
-        float gr = split_gain(S, run, mcw, lambda);
-        GHPair l2{run.g + miss.g, run.h + miss.h};
-        float gl = split_gain(S, l2, mcw, lambda);
-        float score = (gl > gr) ? gl : -gr;
-        float a = fabsf(score);
-        if (a > best) {
-            best = a;
-            best_score = score;
-            best_idx = b;
-            best_left = run;
+    GHPair best_miss{0, 0}, best_left{0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (valid[j]) {
+            const GHPair m = s_miss[w][lastb[j]];
+            const GHPair l{(float)((double)exg[j] * inv_g), (float)((double)exh[j] * inv_h)};
+            float gr = split_gain(S, l, mcw, lambda);
+            GHPair l2{l.g + m.g, l.h + m.h};
+            float gl = split_gain(S, l2, mcw, lambda);
+            float score = (gl > gr) ? gl : -gr;
+            float a = fabsf(score);
+            if (a > best) {
+                best = a;
+                best_score = score;
+                best_idx = b_begin + lane * 4 + j;
+                best_miss = m;
+                best_left = l;
+            }
         }
-        GHPair v = h[b];
-        run.g += v.g;
-        run.h += v.h;
     }
-    GHPair best_miss = miss;
+    // wavefront arg-max: larger |score| wins, ties go to the smaller bin index
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
         float oa = __shfl_xor(best, d);
@@ -456,10 +595,10 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const GHP
             best_left = GHPair{olg, olh};
         }
     }
-    if (lane == 0 && pack < tb.n_packs && nd.is_valid) {
+    if (active && lane == 0) {
         SplitCand c;
         c.score = best_score;
-        c.index = best_idx;  // 0x7fffffff when none of the wavefront's features has a bin
+        c.index = best_idx;
         c.miss = best_miss;
         c.left = best_left;
         c.pad[0] = c.pad[1] = 0;
@@ -601,7 +740,7 @@ __global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb, int level)
     }
 }
 
-// Decide left/right for every row of a work item from the split feature's byte of the bin matrix
+// Decide left/right for every row of a work item from the split feature's column of the bin matrix
 // (missing -> default direction, else right iff bin >= split bin; the reference's rule at
 // hist_tree_builder_single.cu:986-1011) and count the rows that go left.
 template <bool DIRECT>
@@ -622,14 +761,14 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb, Den
     const int f = nd.split_feature_id;
     const int sbid = nd.split_bid;
     const bool dr = nd.default_right;
-    const uint8_t *blk = bins.data + (size_t)(f / bins.W) * bins.block_stride + (f % bins.W);
+    const uint8_t *column = bins.col + (size_t)f * bins.col_stride;
     int nleft = 0;
 #pragma unroll
     for (int k = 0; k < kPartChunk / kBlock; ++k) {
         int pos = pb + k * kBlock + threadIdx.x;
         if (pos < pe) {
             int row = DIRECT ? pos : ridx[pos];
-            int b = blk[(size_t)row * bins.W];
+            int b = column[row];
             bool right = (b == kMissingBin) ? dr : (b >= sbid);
             tb.goes_right[pos] = right ? 1 : 0;
             nleft += right ? 0 : 1;
@@ -709,7 +848,9 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb, int l
 }
 
 // Stable two-way compaction of a work item's rows into the children's segments with wavefront
-// ballots and popcounts; also records the new node of every moved row.
+// ballots and popcounts. (Moving the gradient pairs along with the row ids was measured: it makes
+// the histogram's gradient reads sequential but costs more in this kernel than it saves there.) The row -> node map is not touched here; it is rebuilt from the segments
+// when it is needed (k_nid_plan / k_nid_write).
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const int *__restrict__ ridx_cur,
                                                         int *__restrict__ ridx_next, int level) {
@@ -721,8 +862,6 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const i
     if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
     __syncthreads();
     const int x_in = s_x;
-    const TreeNode &nd = tb.nodes[off + x_in];
-    const int lch = nd.lch_index, rch = nd.rch_index;
     const int2 sg = tb.seg[off + x_in];
     const int first_item = tb.pitem_begin[x_in];
     const int pb = sg.x + (item - first_item) * kPartChunk;
@@ -761,11 +900,50 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const i
         if (valid) {
             int dest = right ? right_base + bR + lanes_below(mR) : left_base + bL + lanes_below(mL);
             ridx_next[dest] = row;
-            tb.nid[row] = right ? rch : lch;
         }
         left_base += tL;
         right_base += tR;
         __syncthreads();
+    }
+}
+
+// Row -> node map (the reference's ins2node_id) from the row lists: a node holds rows iff it is valid
+// and was not split; its rows are its segment of the row list of its level's parity. Planning is one
+// workgroup over all nodes, writing is one workgroup per kPartChunk rows.
+__global__ __launch_bounds__(kBlock) void k_nid_plan(TreeBuffers tb) {
+    __shared__ int lds[kWaves];
+    int carry = 0;
+    for (int base = 0; base < tb.n_nodes; base += kBlock) {
+        int x = base + threadIdx.x;
+        int cnt = 0;
+        if (x < tb.n_nodes) {
+            const TreeNode &nd = tb.nodes[x];
+            int2 sg = tb.seg[x];
+            if (nd.is_valid && nd.split_feature_id < 0) cnt = (sg.y - sg.x + kPartChunk - 1) / kPartChunk;
+        }
+        int tot;
+        int ex = block_excl_scan(cnt, lds, &tot);
+        if (x < tb.n_nodes) tb.fitem_begin[x] = carry + ex;
+        carry += tot;
+    }
+    if (threadIdx.x == 0) tb.fitem_begin[tb.n_nodes] = carry;
+}
+
+__global__ __launch_bounds__(kBlock) void k_nid_write(TreeBuffers tb) {
+    __shared__ int s_x;
+    const int item = blockIdx.x;
+    if (item >= tb.fitem_begin[tb.n_nodes]) return;
+    if (threadIdx.x == 0) s_x = find_owner(tb.fitem_begin, tb.n_nodes, item);
+    __syncthreads();
+    const int x = s_x;
+    const int level = 31 - __clz(x + 1);
+    const int2 sg = tb.seg[x];
+    const int pb = sg.x + (item - tb.fitem_begin[x]) * kPartChunk;
+    const int pe = min(sg.y, pb + kPartChunk);
+    const int *ridx = tb.ridx[level & 1];
+    for (int pos = pb + threadIdx.x; pos < pe; pos += kBlock) {
+        int row = level == 0 ? pos : ridx[pos];
+        tb.nid[row] = x;
     }
 }
 
@@ -886,6 +1064,12 @@ int grid_for(size_t n, int cap = 4096) {
 }  // namespace
 
 // =================================================================================== launchers
+void launch_calibration_copy(hipStream_t s, const void *src, void *dst, size_t bytes) {
+    size_t n = bytes / 16;
+    if (n == 0) return;
+    k_calibration_copy<<<grid_for(n, 16384), kBlock, 0, s>>>(static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n);
+}
+
 void launch_fill_f32(hipStream_t s, float *p, float v, size_t n) {
     if (n == 0) return;
     k_fill_f32<<<grid_for(n), kBlock, 0, s>>>(p, v, n);
@@ -908,13 +1092,12 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
 
 void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda) {
     k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
-    k_fill_u32<<<grid_for(tb.n), kBlock, 0, s>>>(reinterpret_cast<unsigned *>(tb.nid), 0u, (size_t)tb.n);
     k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
 }
 
-template <int LPR>
-static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
-                                int level) {
+template <int LPR, int SLOTS>
+static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
+                              int level) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
     dim3 grid(tb.max_hitems, bins.n_blocks);
     size_t lds = (size_t)tb.max_block_bins * sizeof(unsigned long long);
@@ -922,22 +1105,34 @@ static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const Dens
         // more than the default dynamic LDS window: opt in once per kernel instance and size
         static size_t opted = 0;
         if (lds > opted) {
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, true>),
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, false>),
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             opted = lds;
         }
     }
     if (level == 0) {
-        k_hist_dense<LPR, true><<<grid, kBlock, lds, s>>>(bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built,
-                                                         n_pairs, tb.ctl + level, tb.quant, tb.blk_bin_begin,
-                                                         tb.feat_lds_off, tb.partial, tb.n_bins);
+        k_hist_dense<LPR, true, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
+            bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
+            tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
     } else {
-        k_hist_dense<LPR, false><<<grid, kBlock, lds, s>>>(bins, gh, tb.ridx[level & 1], tb.seg, tb.hpair_begin,
-                                                          tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
-                                                          tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
+        k_hist_dense<LPR, false, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
+            bins, gh, tb.ridx[level & 1], tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
+            tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
     }
+}
+
+template <int LPR>
+static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
+                                int level) {
+    const int slots = (tb.max_block_bins + kHistBlock - 1) / kHistBlock;  // bins drained per thread
+    if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level);
+    else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level);
+    else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level);
+    else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level);
+    else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level);
+    else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
 }
 
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level) {
@@ -953,15 +1148,14 @@ void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bi
 
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
-    dim3 grid((tb.n_bins + kBlock - 1) / kBlock, n_pairs);
-    k_hist_merge<<<grid, kBlock, 0, s>>>(tb.partial, tb.hist_q[level & 1], tb.hist_q[(level + 1) & 1],
-                                        tb.hist[level & 1], tb.quant, tb.hpair_begin, tb.hpair_built, level,
-                                        tb.n_bins);
+    dim3 grid((tb.n_bins + kMergeBins - 1) / kMergeBins, n_pairs);
+    k_hist_merge<<<grid, kBlock, 0, s>>>(tb.partial, tb.hist_q[level & 1], tb.hist_q[(level + 1) & 1], tb.hpair_begin,
+                                        tb.hpair_built, level, tb.n_bins);
 }
 
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
-    dim3 grid((tb.F + kBlock - 1) / kBlock, 1 << level);
-    k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist[level & 1], level, mcw, lambda);
+    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level);
+    k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist_q[level & 1], level, mcw, lambda);
 }
 
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda) {
@@ -981,6 +1175,11 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
         k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
         k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
     }
+}
+
+void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb) {
+    k_nid_plan<<<1, kBlock, 0, s>>>(tb);
+    k_nid_write<<<tb.max_fitems, kBlock, 0, s>>>(tb);
 }
 
 void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma) { k_prune<<<1, kBlock, 0, s>>>(tb, gamma); }

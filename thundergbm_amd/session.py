@@ -135,9 +135,11 @@ class Session:
         return self.get("sp", SPLIT_DTYPE)[: 1 << level]
 
     def level_hist(self, level):
-        """Raw histograms of the nodes of `level`: [2^level, n_bins, 2]."""
-        h = self.get("hist%d" % (level & 1), np.float32)
-        return h[: (1 << level) * self.n_bins * 2].reshape(1 << level, self.n_bins, 2)
+        """Raw histograms of the nodes of `level`: [2^level, n_bins, 2] (exact fixed-point sums as float32)."""
+        q = self.get("hist_q%d" % (level & 1), np.int64)
+        q = q[: (1 << level) * self.n_bins * 2].reshape(1 << level, self.n_bins, 2)
+        sc = self.get("quant", np.float32)  # scale_g, scale_h, inv_g, inv_h
+        return (q.astype(np.float64) * sc[2:4].astype(np.float64)).astype(np.float32)
 
     def ctl(self):
         return self.get("ctl", CTL_DTYPE)
