@@ -13,6 +13,13 @@ import parity as P
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _default_layout():
+    os.environ.pop("TGBM_LAYOUT", None)  # the library picks the layout itself unless a case forces one
+    yield
+    os.environ.pop("TGBM_LAYOUT", None)
+
+
 @pytest.fixture(scope="module")
 def T():
     import thundergbm_amd
@@ -36,7 +43,9 @@ def _cases():
     X2, y2 = _missing_dataset(6000, 11, 3)
     X3, y3 = D.config2(20000, seed=1)
     X5, y5 = D.config5(8000, seed=4)
+    v4, rp4, c4, y4 = D.config4(n=20000, F=3000, nnz_per_row=20, seed=3)
     return {
+        "c4_sparse": ((v4, rp4, c4), y4, dict(objective="binary:logistic", depth=6, max_num_bin=63)),
         "c1_regression": (D.dense_to_csr(X1), y1, dict(objective="reg:linear", depth=6, max_num_bin=255)),
         "missing_regression": (D.dense_to_csr(X2), y2, dict(objective="reg:linear", depth=5, max_num_bin=16)),
         "c2_binary": (D.dense_to_csr(X3), y3, dict(objective="binary:logistic", depth=6, max_num_bin=255)),
@@ -48,13 +57,16 @@ CASES = None
 
 
 def case(name):
+    """Returns (csr, y, kwargs). Names ending in @sparse run the same data through the CSR layout."""
     global CASES
     if CASES is None:
         CASES = _cases()
-    return CASES[name]
+    os.environ["TGBM_LAYOUT"] = "sparse" if name.endswith("@sparse") or name.startswith("c4") else "dense"
+    return CASES[name.split("@")[0]]
 
 
-CASE_NAMES = ["c1_regression", "missing_regression", "c2_binary", "c5_softmax"]
+CASE_NAMES = ["c1_regression", "missing_regression", "c2_binary", "c5_softmax", "c4_sparse", "missing_regression@sparse",
+              "c5_softmax@sparse"]
 
 
 # ----------------------------------------------------------------------- cuts and bin ids (exact)
@@ -127,13 +139,15 @@ def test_session_cuts_bins_base_score(T, name):
     assert np.array_equal(cv, ocv) and np.array_equal(crp, ocrp) and np.array_equal(cf, ocf)
     gb, local = s.global_bin_ids(rp, col)
     assert np.array_equal(gb, o.bin_ids())
-    # every (row, feature) without a stored value is the missing sentinel
-    m = s.binmat()
-    W = s.info("dense_W")
-    stored = np.zeros((s.n, m.shape[0] * W), bool)
-    stored[np.repeat(np.arange(s.n), np.diff(rp)), col] = True
-    flat = m.transpose(1, 0, 2).reshape(s.n, -1)
-    assert np.all(flat[~stored] == 255)
+    assert s.info("sparse") == (1 if os.environ["TGBM_LAYOUT"] == "sparse" else 0)
+    if not s.info("sparse"):
+        # every (row, feature) without a stored value is the missing sentinel
+        m = s.binmat()
+        W = s.info("dense_W")
+        stored = np.zeros((s.n, m.shape[0] * W), bool)
+        stored[np.repeat(np.arange(s.n), np.diff(rp)), col] = True
+        flat = m.transpose(1, 0, 2).reshape(s.n, -1)
+        assert np.all(flat[~stored] == 255)
     assert s.num_class == o.num_class and s.tree_per_rounds == o.tree_per_rounds
     assert np.array_equal(s.labels(), o.labels())
     assert np.array_equal(s.y(), o.y())
@@ -256,7 +270,8 @@ def test_tree_lockstep(T, name):
 
 # -------------------------------------------------------------------- boosting, tree by tree
 @pytest.mark.parametrize("name,rounds", [("c1_regression", 40), ("missing_regression", 10), ("c2_binary", 10),
-                                         ("c5_softmax", 3)])
+                                         ("c5_softmax", 3), ("c4_sparse", 10), ("missing_regression@sparse", 10),
+                                         ("c1_regression@sparse", 5)])
 def test_boosting_teacher_forced(T, name, rounds):
     """Each round both sides start from the GPU's predictions, so every tree is compared on its own."""
     (val, rp, col), y, kw = case(name)
@@ -397,8 +412,10 @@ def test_predict_wide_float_path_and_unseen_rows(T):
     s.close()
 
 
-def test_a1a_quickstart_known_answer(T):
+@pytest.mark.parametrize("layout", ["dense", "sparse"])
+def test_a1a_quickstart_known_answer(T, layout):
     # README.md:76-80 of the reference: RMSE = 0.489562 (zero initial prediction, see the oracle test)
+    os.environ["TGBM_LAYOUT"] = layout
     val, rp, col, y = D.read_libsvm(D.A1A)
     s = T.Session(val, rp, col, y, depth=6, n_trees=40, learning_rate=1.0)
     s.set("y_pred", np.zeros(len(y), np.float32))

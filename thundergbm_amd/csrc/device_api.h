@@ -64,8 +64,16 @@ struct DenseBins {
     size_t col_stride = 0;
 };
 
+// Sparse layout for wide, mostly-missing data: the reference's own representation, CSR rows of global
+// bin ids (hist_tree_builder_single.cu:49-130).
+struct CsrBins {
+    const int *row_ptr = nullptr;  // [n + 1]
+    const int *bin = nullptr;      // [nnz] global bin id, ascending within a row
+};
+
 struct TreeBuffers {
     int n = 0, n_bins = 0, F = 0, depth = 0, n_nodes = 0;
+    int sparse = 0;                // 1: CSR layout, histograms accumulated directly in hist_q
     TreeNode *nodes = nullptr;     // [n_nodes]
     int2 *seg = nullptr;           // [n_nodes] row-list segment [x, y) of every node
     int *nid = nullptr;            // [n]
@@ -109,6 +117,8 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
 void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
+void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);
+void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level);
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level);

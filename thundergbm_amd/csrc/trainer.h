@@ -49,7 +49,7 @@ class Trainer {
     HistProfile profile();
 
    private:
-    void build_level(int level);
+    void build_level_hist(int level, const GHPair *gh);
     void alloc_tree_buffers();
     template <typename T>
     T *dalloc(size_t count);
@@ -69,6 +69,8 @@ class Trainer {
     std::vector<int> h_cut_row_ptr_;
     uint8_t *d_binmat_ = nullptr;
     DenseBins bins_;
+    bool sparse_ = false;
+    CsrBins csr_;
     TreeBuffers tb_;
     // model
     TreeNode *d_model_ = nullptr;

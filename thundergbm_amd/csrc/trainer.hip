@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 
 namespace tgbm {
@@ -94,40 +95,60 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
                              hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
 
-    // dense column-blocked layout: blocks of W features, each block n rows x W bytes
-    int W;
-    if (F_ <= 32) {
-        W = 4;
-        while (W < F_) W *= 2;
-    } else if (F_ <= 64 && n_bins_ <= 12288) {
-        W = 64;
-    } else {
-        W = 32;
-    }
-    const int n_blocks = (F_ + W - 1) / W;
-    const size_t mat_bytes = (size_t)n_ * W * n_blocks;
+    // Layout choice. Dense: column-blocked uint8 matrix (needs max_num_bin <= 255 and room for
+    // n x F bytes twice). Sparse: CSR rows of global bin ids, for wide data whose rows store few values.
+    const double density = (double)nnz_ / ((double)n_ * (double)F_);
     size_t free_b = 0, total_b = 0;
     HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-    TGBM_CHECK(mat_bytes + (size_t)n_ * F_ < free_b / 2,
-               "dense bin matrix of %zu bytes does not fit (free %zu); the sparse histogram path is not built yet",
-               mat_bytes, free_b);
-    d_binmat_ = dalloc<uint8_t>(mat_bytes);
-    launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);
-    const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
-    uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_);
-    launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_);
-    launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                     (size_t)n_ * W, d_colmat, col_stride);
-    bins_.col = d_colmat;
-    bins_.col_stride = col_stride;
-    bins_.data = d_binmat_;
-    bins_.W = W;
-    bins_.n_blocks = n_blocks;
-    bins_.block_stride = (size_t)n_ * W;
-    HIP_CHECK(hipStreamSynchronize(stream_));
-    HIP_CHECK(hipFree(d_val));
-    HIP_CHECK(hipFree(d_col));
-    HIP_CHECK(hipFree(d_row_ptr));
+    const char *force = std::getenv("TGBM_LAYOUT");  // "dense" / "sparse" override the heuristic (tests)
+    sparse_ = (F_ > 4096 && density < 0.05) || (size_t)n_ * F_ * 2 > free_b / 2;
+    if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
+    if (force != nullptr && std::string(force) == "dense") sparse_ = false;
+    log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
+    if (sparse_) {
+        int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
+        launch_bin_csr(stream_, nnz_, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_bin);
+        allocs_.push_back(d_row_ptr);  // kept for the whole session
+        csr_.row_ptr = d_row_ptr;
+        csr_.bin = d_bin;
+        bins_.W = 4;
+        bins_.n_blocks = 1;
+        HIP_CHECK(hipStreamSynchronize(stream_));
+        HIP_CHECK(hipFree(d_val));
+        HIP_CHECK(hipFree(d_col));
+    } else {
+        // dense column-blocked layout: blocks of W features, each block n rows x W bytes
+        int W;
+        if (F_ <= 32) {
+            W = 4;
+            while (W < F_) W *= 2;
+        } else if (F_ <= 64 && n_bins_ <= 8192) {
+            W = 64;
+        } else {
+            W = 32;
+        }
+        const int n_blocks = (F_ + W - 1) / W;
+        const size_t mat_bytes = (size_t)n_ * W * n_blocks;
+        TGBM_CHECK(mat_bytes + (size_t)n_ * F_ < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
+                   mat_bytes, free_b);
+        d_binmat_ = dalloc<uint8_t>(mat_bytes);
+        launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);
+        const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
+        uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_);
+        launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_);
+        launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
+                         (size_t)n_ * W, d_colmat, col_stride);
+        bins_.col = d_colmat;
+        bins_.col_stride = col_stride;
+        bins_.data = d_binmat_;
+        bins_.W = W;
+        bins_.n_blocks = n_blocks;
+        bins_.block_stride = (size_t)n_ * W;
+        HIP_CHECK(hipStreamSynchronize(stream_));
+        HIP_CHECK(hipFree(d_val));
+        HIP_CHECK(hipFree(d_col));
+        HIP_CHECK(hipFree(d_row_ptr));
+    }
 
     // ---- labels, predictions, gradients (Booster::init) --------------------------------------
     d_y_ = dalloc<float>(n_);
@@ -168,6 +189,7 @@ void Trainer::alloc_tree_buffers() {
     const int depth = param_.depth;
     tb.n = n_;
     tb.n_bins = n_bins_;
+    tb.sparse = sparse_ ? 1 : 0;
     tb.F = F_;
     tb.depth = depth;
     tb.n_nodes = (1 << (depth + 1)) - 1;
@@ -183,7 +205,7 @@ void Trainer::alloc_tree_buffers() {
     tb.max_hitems = tb.target_hitems + max_pairs + 1;
     tb.hist_q[0] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
     tb.hist_q[1] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
-    tb.partial = dalloc<longlong2>((size_t)tb.max_hitems * n_bins_);
+    tb.partial = dalloc<longlong2>(sparse_ ? 1 : (size_t)tb.max_hitems * n_bins_);
     tb.quant = dalloc<QuantCtl>(1);
     tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
     // the planning kernel of the last level also writes the (unused) plan of level `depth`
@@ -236,7 +258,7 @@ void Trainer::alloc_tree_buffers() {
             feat_off[(size_t)b * W + j] = f < F_ ? h_cut_row_ptr_[f] - blk_begin[b] : 0;
         }
     }
-    TGBM_CHECK((size_t)max_block_bins * 8 <= 160 * 1024, "feature block histogram exceeds the LDS");
+    TGBM_CHECK(sparse_ || (size_t)max_block_bins * 8 <= 160 * 1024, "feature block histogram exceeds the LDS");
     tb.max_block_bins = max_block_bins;
     int *d_blk = dalloc<int>(blk_begin.size());
     int *d_off = dalloc<int>(feat_off.size());
@@ -282,18 +304,30 @@ void Trainer::find_split(int level) {
         ev.level = level;
         ev.tree = trees_built_;
         HIP_CHECK(hipEventRecord(ev.start, stream_));
-        launch_hist_dense(stream_, tb_, bins_, gh, level);
+        build_level_hist(level, gh);
         HIP_CHECK(hipEventRecord(ev.stop, stream_));
         events_.push_back(ev);
     } else {
-        launch_hist_dense(stream_, tb_, bins_, gh, level);
+        build_level_hist(level, gh);
     }
-    launch_hist_merge(stream_, tb_, level);
+    if (!sparse_) launch_hist_merge(stream_, tb_, level);
     launch_eval_split(stream_, tb_, level, param_.min_child_weight, param_.lambda);
     launch_best_update(stream_, tb_, level, param_.rt_eps, param_.lambda);
 }
 
-void Trainer::partition(int level) { launch_partition_dense(stream_, tb_, bins_, level); }
+void Trainer::build_level_hist(int level, const GHPair *gh) {
+    if (sparse_)
+        launch_hist_csr(stream_, tb_, csr_, gh, level);
+    else
+        launch_hist_dense(stream_, tb_, bins_, gh, level);
+}
+
+void Trainer::partition(int level) {
+    if (sparse_)
+        launch_partition_csr(stream_, tb_, csr_, level);
+    else
+        launch_partition_dense(stream_, tb_, bins_, level);
+}
 
 void Trainer::finish_tree(int k) {
     launch_prune(stream_, tb_, param_.gamma);
@@ -394,7 +428,10 @@ HistProfile Trainer::profile() {
         for (int level = 0; level < param_.depth; ++level) {
             const LevelCtl &c = ctl_log_[t * per_tree + level];
             p.rows_built += c.rows_built;
-            p.hist_bytes += (long long)c.rows_built * (F_ + 8 + (level > 0 ? 4 : 0));
+            if (sparse_)  // CSR: 4-byte bin id per stored value + row pointer, gradient pair and row index per row
+                p.hist_bytes += (long long)((double)c.rows_built * ((double)nnz_ / n_ * 4 + 8 + 8 + (level > 0 ? 4 : 0)));
+            else
+                p.hist_bytes += (long long)c.rows_built * (F_ + 8 + (level > 0 ? 4 : 0));
         }
     }
     (void)W;
@@ -408,6 +445,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "num_class") return param_.num_class;
     if (key == "tree_per_rounds") return param_.tree_per_rounds;
     if (key == "n_nodes") return tb_.n_nodes;
+    if (key == "sparse") return sparse_ ? 1 : 0;
     if (key == "dense_W") return bins_.W;
     if (key == "dense_blocks") return bins_.n_blocks;
     if (key == "trees_built") return trees_built_;
@@ -427,7 +465,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     if (name == "cut_val") src = cuts_.cut_val, bytes = sizeof(float) * (size_t)n_bins_;
     else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
-    else if (name == "binmat") src = d_binmat_, bytes = (size_t)n_ * bins_.W * bins_.n_blocks;
+    else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
+    else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
         launch_nid_rebuild(stream_, tb_);  // the map is kept as row lists; materialise it on demand
         sync();

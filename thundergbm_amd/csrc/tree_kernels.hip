@@ -2,6 +2,8 @@
 // subtraction, wavefront segmented-scan split finding, ballot/popcount row partition, pruning and the
 // in-training prediction update. Every stage of a level is one launch over all nodes of the level;
 // work lists are planned on the device so the host never waits inside a tree.
+#include <algorithm>
+
 #include "device_api.h"
 
 namespace tgbm {
@@ -267,8 +269,14 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
         // kHistFlushRows rows are added, which keeps a bin's gradient sum inside a signed and its
         // hessian sum inside an unsigned 32-bit field.
         QuantCtl q;
-        q.scale_g = pow2_scale(gm, kHistFlushRows, 2147483520.f);  // largest float below 2^31
-        q.scale_h = pow2_scale(hm, kHistFlushRows, 4294967040.f);  // largest float below 2^32
+        if (tb.sparse) {
+            // sums go straight into 64-bit integers: the whole dataset must fit below 2^62
+            q.scale_g = pow2_scale(gm, tb.n, 4.6e18f);
+            q.scale_h = pow2_scale(hm, tb.n, 4.6e18f);
+        } else {
+            q.scale_g = pow2_scale(gm, kHistFlushRows, 2147483520.f);  // largest float below 2^31
+            q.scale_h = pow2_scale(hm, kHistFlushRows, 4294967040.f);  // largest float below 2^32
+        }
         q.inv_g = 1.f / q.scale_g;
         q.inv_h = 1.f / q.scale_h;
         *tb.quant = q;
@@ -439,6 +447,124 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(const longlong2 *__restri
         const longlong2 par = prev_q[(size_t)p * n_bins + j];
         cur_q[(size_t)(sib - off) * n_bins + j] = make_longlong2(par.x - sg, par.y - sh);
     }
+}
+
+// --------------------------------------------------------------------------- sparse histogram
+// CSR rows of global bin ids: the histogram is too large for LDS (one slot per cut point of every
+// feature), so every stored value adds its row's fixed-point gradient pair to the node's histogram
+// in HBM with two 64-bit integer atomics (exact and order-independent, unlike the float atomics of
+// hist_tree_builder_single.cu:203-216 / :485-505). One wavefront walks one row at a time.
+__global__ __launch_bounds__(kBlock) void k_hist_zero_built(longlong2 *__restrict__ cur_q,
+                                                           const int *__restrict__ hpair_built, int level,
+                                                           int n_bins) {
+    const int built = hpair_built[blockIdx.y];
+    if (built < 0) return;
+    const int off = (1 << level) - 1;
+    longlong2 *h = cur_q + (size_t)(built - off) * n_bins;
+    for (int j = blockIdx.x * kBlock + threadIdx.x; j < n_bins; j += gridDim.x * kBlock) h[j] = make_longlong2(0, 0);
+}
+
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb, CsrBins bins, const GHPair *__restrict__ gh,
+                                                    const int *__restrict__ ridx, longlong2 *__restrict__ cur_q,
+                                                    int n_pairs, int level) {
+    __shared__ int s_info[3];
+    const LevelCtl c = tb.ctl[level];
+    const int item = blockIdx.x;
+    if (item >= c.n_hitems) return;
+    if (threadIdx.x == 0) {
+        int p = find_owner(tb.hpair_begin, n_pairs, item);
+        int node = tb.hpair_built[p];
+        int2 sg = tb.seg[node];
+        int b = sg.x + (item - tb.hpair_begin[p]) * c.hchunk;
+        s_info[0] = b;
+        s_info[1] = min(sg.y, b + c.hchunk);
+        s_info[2] = node - ((1 << level) - 1);
+    }
+    __syncthreads();
+    const int begin = s_info[0], end = s_info[1];
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(cur_q + (size_t)s_info[2] * tb.n_bins);
+    const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
+    const int lane = lane_id(), w = wave_id();
+    for (int pos = begin + w; pos < end; pos += kWaves) {
+        const int r = DIRECT ? pos : ridx[pos];
+        const GHPair s = gh[r];
+        const long long gq = __float2ll_rn(s.g * scale_g);
+        const long long hq = __float2ll_rn(s.h * scale_h);
+        const int e0 = bins.row_ptr[r], e1 = bins.row_ptr[r + 1];
+        for (int e = e0 + lane; e < e1; e += 64) {
+            const int b = bins.bin[e];
+            atomicAdd(h + 2 * (size_t)b, (unsigned long long)gq);
+            atomicAdd(h + 2 * (size_t)b + 1, (unsigned long long)hq);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_hist_sub_csr(longlong2 *__restrict__ cur_q,
+                                                        const longlong2 *__restrict__ prev_q,
+                                                        const int *__restrict__ hpair_built, int level, int n_bins) {
+    const int p = blockIdx.y;
+    const int built = hpair_built[p];
+    if (built < 0) return;
+    const int off = (1 << level) - 1;
+    const int sib = (built & 1) ? built + 1 : built - 1;
+    const longlong2 *b = cur_q + (size_t)(built - off) * n_bins;
+    longlong2 *sq = cur_q + (size_t)(sib - off) * n_bins;
+    const longlong2 *par = prev_q + (size_t)p * n_bins;
+    for (int j = blockIdx.x * kBlock + threadIdx.x; j < n_bins; j += gridDim.x * kBlock) {
+        longlong2 pv = par[j], bv = b[j];
+        sq[j] = make_longlong2(pv.x - bv.x, pv.y - bv.y);
+    }
+}
+
+// Left/right decision of the sparse layout: binary search of the row's bin ids for the one inside
+// the split feature's bin range (absent = missing), hist_tree_builder_single.cu:941-1011.
+template <bool DIRECT>
+__global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb, CsrBins bins, const int *__restrict__ ridx,
+                                                          int level) {
+    __shared__ int lds[kWaves];
+    __shared__ int s_x;
+    const int item = blockIdx.x;
+    if (item >= tb.ctl[level].n_pitems) return;
+    const int nl = 1 << level, off = nl - 1;
+    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    __syncthreads();
+    const int x_in = s_x;
+    const TreeNode &nd = tb.nodes[off + x_in];
+    const int2 sg = tb.seg[off + x_in];
+    const int pb = sg.x + (item - tb.pitem_begin[x_in]) * kPartChunk;
+    const int pe = min(sg.y, pb + kPartChunk);
+    const int f = nd.split_feature_id;
+    const int cb = tb.cut_row_ptr[f], ce = tb.cut_row_ptr[f + 1];
+    const int sbid = cb + nd.split_bid;
+    const bool dr = nd.default_right;
+    int nleft = 0;
+#pragma unroll
+    for (int k = 0; k < kPartChunk / kBlock; ++k) {
+        int pos = pb + k * kBlock + threadIdx.x;
+        if (pos < pe) {
+            int row = DIRECT ? pos : ridx[pos];
+            int lo = bins.row_ptr[row], hi = bins.row_ptr[row + 1];
+            int found = -1;
+            while (lo < hi) {
+                int mid = lo + (hi - lo) / 2;
+                int b = bins.bin[mid];
+                if (b >= cb && b < ce) {
+                    found = b;
+                    break;
+                }
+                if (b < cb)
+                    lo = mid + 1;
+                else
+                    hi = mid;
+            }
+            bool right = found < 0 ? dr : (found >= sbid);
+            tb.goes_right[pos] = right ? 1 : 0;
+            nleft += right ? 0 : 1;
+        }
+    }
+    int tot = block_sum(nleft, lds);
+    if (threadIdx.x == 0) tb.pitem_nleft[item] = tot;
 }
 
 // ------------------------------------------------------------------------ split finding
@@ -1153,6 +1279,20 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level) {
                                         tb.hpair_built, level, tb.n_bins);
 }
 
+void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level) {
+    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    const int zgrid = std::min(1024, (tb.n_bins + kBlock - 1) / kBlock);
+    longlong2 *cur = tb.hist_q[level & 1];
+    k_hist_zero_built<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hpair_built, level, tb.n_bins);
+    if (level == 0) {
+        k_hist_csr<true><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, nullptr, cur, n_pairs, level);
+    } else {
+        k_hist_csr<false><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, tb.ridx[level & 1], cur, n_pairs, level);
+        k_hist_sub_csr<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hist_q[(level + 1) & 1], tb.hpair_built, level,
+                                                              tb.n_bins);
+    }
+}
+
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
     dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level);
     k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist_q[level & 1], level, mcw, lambda);
@@ -1172,6 +1312,21 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
         k_part_scatter<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
     } else {
         k_part_count_dense<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
+        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+    }
+}
+
+void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level) {
+    k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
+    const int *cur = tb.ridx[level & 1];
+    int *next = tb.ridx[(level + 1) & 1];
+    if (level == 0) {
+        k_part_count_csr<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
+        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+    } else {
+        k_part_count_csr<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
         k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
         k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
     }

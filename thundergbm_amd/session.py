@@ -105,7 +105,11 @@ class Session:
         return self.get("binmat", np.uint8, (nb, self.n, W))
 
     def global_bin_ids(self, row_ptr, col):
-        """Global bin id of every stored value (the reference's csr_bin_id) from the dense matrix."""
+        """Global bin id of every stored value (the reference's csr_bin_id) and its local bin id."""
+        if self.info("sparse"):
+            gb = self.get("csr_bin", np.int32)
+            _, crp, _ = self.cuts()
+            return gb, gb - crp[col]
         W = self.info("dense_W")
         m = self.binmat()
         _, crp, _ = self.cuts()
