@@ -1,0 +1,81 @@
+// Microbenchmark of LDS atomic throughput on gfx950: float vs 32/64-bit integer adds, random vs
+// conflict-free vs same-address, 256/512/1024-thread groups. It is the measurement behind the
+// fixed-point histogram of tree_kernels.hip; built as bin/bench_lds_atomics, not linked into the library.
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <vector>
+#define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("err %s line %d\n", hipGetErrorString(e), __LINE__); return 1; } } while (0)
+constexpr int NBINS = 14336;  // floats (56 KB)
+constexpr int ITERS = 2048;
+
+template <int MODE>
+__global__ __launch_bounds__(1024) void k(float *out, int iters) {
+    extern __shared__ float lds[];
+    for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lds[i] = 0.f;
+    __syncthreads();
+    unsigned s = (blockIdx.x * blockDim.x + threadIdx.x) * 2654435761u + 12345u;
+    unsigned lane = threadIdx.x & 63;
+    float v = 1.0f + lane * 1e-3f;
+    for (int it = 0; it < iters; ++it) {
+        s = s * 1664525u + 1013904223u;
+        unsigned r = (s >> 8) % NBINS;
+        if (MODE == 0) unsafeAtomicAdd(&lds[r], v);                              // float, random
+        if (MODE == 1) atomicAdd((unsigned *)&lds[r], 1u);                       // uint, random
+        if (MODE == 2) unsafeAtomicAdd(&lds[(it * 64 + lane) % NBINS], v);       // float, conflict free
+        if (MODE == 3) atomicAdd((unsigned *)&lds[(it * 64 + lane) % NBINS], 1u);// uint, conflict free
+        if (MODE == 4) unsafeAtomicAdd(&lds[it % NBINS], v);                     // float, same address
+        if (MODE == 5) { float o = atomicAdd(&lds[r], v); v += o * 1e-30f; }     // float with return
+        if (MODE == 6) atomicAdd((unsigned long long *)&lds[(r & ~1u)], 1ull);   // u64 random
+        if (MODE == 7) lds[r] = v;                                               // plain store random
+        if (MODE == 8) v += lds[r];                                              // plain load random
+        if (MODE == 9) { lds[r] += v; }                                          // non-atomic rmw random
+        if (MODE == 10) unsafeAtomicAdd(&lds[(r & ~31u) | (lane & 31)], v);      // float, random rows, bank = lane%32 (2-way)
+        if (MODE == 11) atomicAdd((int *)&lds[r], 3);                            // int add random
+        if (MODE == 12) atomicAdd((unsigned long long *)&lds[((it * 64 + lane) * 2) % NBINS], 1ull);  // u64 conflict free
+    }
+    __syncthreads();
+    float acc = v;
+    for (int i = threadIdx.x; i < NBINS; i += blockDim.x) acc += lds[i];
+    if (acc == 123.456f) out[0] = acc;
+}
+
+template <int MODE>
+int run(const char *name, float *d_out, int block = 256) {
+    hipEvent_t a, b;
+    CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+    const int grid = 2048 * 256 / block;
+    k<MODE><<<grid, block, NBINS * 4>>>(d_out, 16);
+    CK(hipDeviceSynchronize());
+    CK(hipEventRecord(a));
+    k<MODE><<<grid, block, NBINS * 4>>>(d_out, ITERS);
+    CK(hipEventRecord(b));
+    CK(hipEventSynchronize(b));
+    float ms; CK(hipEventElapsedTime(&ms, a, b));
+    double ops = (double)grid * block * ITERS;
+    printf("%-40s %8.3f ms  %8.1f G lane-ops/s  %.2f lane-ops/clk/CU (2.4GHz, 256 CU)\n", name, ms, ops / ms / 1e6,
+           ops / (ms * 1e-3) / 256 / 2.4e9);
+    return 0;
+}
+
+int main() {
+    float *d; CK(hipMalloc(&d, 64));
+    run<0>("float add, random", d);
+    run<1>("uint add, random", d);
+    run<2>("float add, conflict free", d);
+    run<3>("uint add, conflict free", d);
+    run<4>("float add, same address", d);
+    run<5>("float add rtn, random", d);
+    run<6>("u64 add, random", d);
+    run<7>("plain store, random", d);
+    run<8>("plain load, random", d);
+    run<9>("non-atomic rmw, random", d);
+    run<10>("float add, 2-way bank", d);
+    run<11>("int add, random", d);
+    run<12>("u64 add, conflict free", d);
+    run<6>("u64 add, random, block 512", d, 512);
+    run<6>("u64 add, random, block 1024", d, 1024);
+    run<12>("u64 add, conflict free, block 1024", d, 1024);
+    run<1>("uint add, random, block 1024", d, 1024);
+    run<0>("float add, random, block 1024", d, 1024);
+    return 0;
+}
