@@ -58,6 +58,12 @@ struct DenseBins {
     int W = 0;          // bytes (features) per row of a block, multiple of 4
     int n_blocks = 0;
     size_t block_stride = 0;  // bytes between blocks = n * W
+    // Record mode (one feature block, W <= 32): a row's bins and its gradient pair of the current tree
+    // share one record, rec_per_line records per 128-byte line, so a gathered row costs one line
+    // instead of two. rec_size == 0 selects the plain rows above with gradients read from their array.
+    int rec_size = 0;
+    int rec_per_line = 0;
+    int gh_off = 0;  // byte offset of (g,h) inside a record
     // Column-major copy (feature f = n consecutive bytes at col + f * col_stride): the partition reads
     // one feature of many rows, which costs one byte per row here instead of one sector per row.
     const uint8_t *col = nullptr;
@@ -70,6 +76,11 @@ struct CsrBins {
     const int *row_ptr = nullptr;  // [n + 1]
     const int *bin = nullptr;      // [nnz] global bin id, ascending within a row
 };
+
+__host__ __device__ inline size_t dense_row_offset(const DenseBins &b, int r) {
+    if (b.rec_size == 0) return (size_t)r * b.W;
+    return (size_t)(r / b.rec_per_line) * 128 + (size_t)(r % b.rec_per_line) * b.rec_size;
+}
 
 struct TreeBuffers {
     int n = 0, n_bins = 0, F = 0, depth = 0, n_nodes = 0;
@@ -114,7 +125,10 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda);
+// bins.rec_size != 0: the gradient pairs are also written into the row records
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh_class,
+                      float lambda);
+void launch_unpack_records(hipStream_t s, const DenseBins &bins, int n, uint8_t *out);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);
@@ -133,7 +147,7 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 
 // data preparation
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
-                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
+                      const int *cut_row_ptr, uint8_t *binmat, const DenseBins &layout, uint8_t *colmat,
                       size_t col_stride);
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id);
