@@ -58,12 +58,13 @@ struct DenseBins {
     int W = 0;          // bytes (features) per row of a block, multiple of 4
     int n_blocks = 0;
     size_t block_stride = 0;  // bytes between blocks = n * W
-    // Record mode (one feature block, W <= 32): a row's bins and its gradient pair of the current tree
-    // share one record, rec_per_line records per 128-byte line, so a gathered row costs one line
-    // instead of two. rec_size == 0 selects the plain rows above with gradients read from their array.
-    int rec_size = 0;
-    int rec_per_line = 0;
-    int gh_off = 0;  // byte offset of (g,h) inside a record
+    // Record mode (one feature block, W <= 32): a 128-byte line holds the bins of rec_per_line rows
+    // followed by those rows' gradient pairs of the current tree, so a gathered row costs one line
+    // instead of two and the per-tree gradient refresh writes one contiguous run per line.
+    // rec_size == 0 selects the plain rows above with gradients read from their array.
+    int rec_size = 0;      // != 0 selects record mode; bytes of one row's bins inside a line (= W)
+    int rec_per_line = 0;  // rows per 128-byte line
+    int gh_off = 0;        // byte offset of the line's gradient pairs (rec_per_line x 8 bytes, contiguous)
     // Column-major copy (feature f = n consecutive bytes at col + f * col_stride): the partition reads
     // one feature of many rows, which costs one byte per row here instead of one sector per row.
     const uint8_t *col = nullptr;
@@ -80,6 +81,10 @@ struct CsrBins {
 __host__ __device__ inline size_t dense_row_offset(const DenseBins &b, int r) {
     if (b.rec_size == 0) return (size_t)r * b.W;
     return (size_t)(r / b.rec_per_line) * 128 + (size_t)(r % b.rec_per_line) * b.rec_size;
+}
+// record mode: byte offset of row r's gradient pair
+__host__ __device__ inline size_t dense_gh_offset(const DenseBins &b, int r) {
+    return (size_t)(r / b.rec_per_line) * 128 + b.gh_off + (size_t)(r % b.rec_per_line) * 8;
 }
 
 struct TreeBuffers {

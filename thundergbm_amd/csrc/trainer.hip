@@ -132,9 +132,9 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         bins_.n_blocks = n_blocks;
         const char *rec_env = std::getenv("TGBM_ROW_RECORDS");  // "0" keeps plain rows (tests of both layouts)
         if (n_blocks == 1 && W <= 32 && !(rec_env != nullptr && rec_env[0] == '0')) {
-            bins_.gh_off = (W + 7) / 8 * 8;
-            bins_.rec_size = bins_.gh_off + 8;
-            bins_.rec_per_line = 128 / bins_.rec_size;
+            bins_.rec_size = W;
+            bins_.rec_per_line = 128 / (W + 8);
+            bins_.gh_off = (bins_.rec_per_line * W + 7) / 8 * 8;
         }
         const size_t mat_bytes = bins_.rec_size != 0
                                      ? ((size_t)n_ + bins_.rec_per_line - 1) / bins_.rec_per_line * 128

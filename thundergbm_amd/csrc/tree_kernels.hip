@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restri
     uint8_t *rec = const_cast<uint8_t *>(bins.data);
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         GHPair v = gh[i];
-        if (bins.rec_size != 0) *reinterpret_cast<GHPair *>(rec + dense_row_offset(bins, i) + bins.gh_off) = v;
+        if (bins.rec_size != 0) *reinterpret_cast<GHPair *>(rec + dense_gh_offset(bins, i)) = v;
         g += v.g;
         h += v.h;
         gm = fmaxf(gm, fabsf(v.g));
@@ -353,9 +353,8 @@ void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
             int r = 0;
             if (ok) r = DIRECT ? pos : ridx[pos];
             if (REC) {
-                const uint8_t *row = blk + dense_row_offset(bins, r);
-                opk[u] = ok ? *reinterpret_cast<const unsigned *>(row) : 0xffffffffu;
-                os[u] = ok ? *reinterpret_cast<const GHPair *>(row - q * 4 + bins.gh_off) : GHPair{0, 0};
+                opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + dense_row_offset(bins, r)) : 0xffffffffu;
+                os[u] = ok ? *reinterpret_cast<const GHPair *>(bins.data + dense_gh_offset(bins, r)) : GHPair{0, 0};
             } else {
                 opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
                 os[u] = ok ? gh[r] : GHPair{0, 0};
