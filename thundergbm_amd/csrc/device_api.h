@@ -58,13 +58,6 @@ struct DenseBins {
     int W = 0;          // bytes (features) per row of a block, multiple of 4
     int n_blocks = 0;
     size_t block_stride = 0;  // bytes between blocks = n * W
-    // Record mode (one feature block, W <= 32): a 128-byte line holds the bins of rec_per_line rows
-    // followed by those rows' gradient pairs of the current tree, so a gathered row costs one line
-    // instead of two and the per-tree gradient refresh writes one contiguous run per line.
-    // rec_size == 0 selects the plain rows above with gradients read from their array.
-    int rec_size = 0;      // != 0 selects record mode; bytes of one row's bins inside a line (= W)
-    int rec_per_line = 0;  // rows per 128-byte line
-    int gh_off = 0;        // byte offset of the line's gradient pairs (rec_per_line x 8 bytes, contiguous)
     // Column-major copy (feature f = n consecutive bytes at col + f * col_stride): the partition reads
     // one feature of many rows, which costs one byte per row here instead of one sector per row.
     const uint8_t *col = nullptr;
@@ -77,15 +70,6 @@ struct CsrBins {
     const int *row_ptr = nullptr;  // [n + 1]
     const int *bin = nullptr;      // [nnz] global bin id, ascending within a row
 };
-
-__host__ __device__ inline size_t dense_row_offset(const DenseBins &b, int r) {
-    if (b.rec_size == 0) return (size_t)r * b.W;
-    return (size_t)(r / b.rec_per_line) * 128 + (size_t)(r % b.rec_per_line) * b.rec_size;
-}
-// record mode: byte offset of row r's gradient pair
-__host__ __device__ inline size_t dense_gh_offset(const DenseBins &b, int r) {
-    return (size_t)(r / b.rec_per_line) * 128 + b.gh_off + (size_t)(r % b.rec_per_line) * 8;
-}
 
 struct TreeBuffers {
     int n = 0, n_bins = 0, F = 0, depth = 0, n_nodes = 0;
@@ -130,10 +114,7 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
-// bins.rec_size != 0: the gradient pairs are also written into the row records
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh_class,
-                      float lambda);
-void launch_unpack_records(hipStream_t s, const DenseBins &bins, int n, uint8_t *out);
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);
@@ -152,7 +133,7 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 
 // data preparation
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
-                      const int *cut_row_ptr, uint8_t *binmat, const DenseBins &layout, uint8_t *colmat,
+                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
                       size_t col_stride);
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id);

@@ -239,15 +239,15 @@ __device__ __forceinline__ int local_bin(const float *__restrict__ cuts, int k, 
 
 __global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
                             const float *__restrict__ val, const float *__restrict__ cut_val,
-                            const int *__restrict__ cut_row_ptr, uint8_t *__restrict__ binmat, DenseBins lay,
-                            uint8_t *__restrict__ colmat, size_t col_stride) {
+                            const int *__restrict__ cut_row_ptr, uint8_t *__restrict__ binmat, int W,
+                            size_t block_stride, uint8_t *__restrict__ colmat, size_t col_stride) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         for (int e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
             int f = col[e];
             int cb = cut_row_ptr[f];
             int k = cut_row_ptr[f + 1] - cb;
             int b = local_bin(cut_val + cb, k, val[e]);
-            binmat[(size_t)(f / lay.W) * lay.block_stride + dense_row_offset(lay, i) + (f % lay.W)] = (uint8_t)b;
+            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (uint8_t)b;
             colmat[(size_t)f * col_stride + i] = (uint8_t)b;
         }
     }
@@ -345,10 +345,10 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
 }
 
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
-                      const int *cut_row_ptr, uint8_t *binmat, const DenseBins &layout, uint8_t *colmat,
+                      const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
                       size_t col_stride) {
-    k_bin_dense<<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, layout, colmat,
-                                              col_stride);
+    k_bin_dense<<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride,
+                                              colmat, col_stride);
 }
 
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,

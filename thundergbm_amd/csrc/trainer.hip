@@ -130,16 +130,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         const int n_blocks = (F_ + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;
-        const char *rec_env = std::getenv("TGBM_ROW_RECORDS");  // "0" keeps plain rows (tests of both layouts)
-        if (n_blocks == 1 && W <= 32 && !(rec_env != nullptr && rec_env[0] == '0')) {
-            bins_.rec_size = W;
-            bins_.rec_per_line = 128 / (W + 8);
-            bins_.gh_off = (bins_.rec_per_line * W + 7) / 8 * 8;
-        }
-        const size_t mat_bytes = bins_.rec_size != 0
-                                     ? ((size_t)n_ + bins_.rec_per_line - 1) / bins_.rec_per_line * 128
-                                     : (size_t)n_ * W * n_blocks;
-        bins_.block_stride = bins_.rec_size != 0 ? mat_bytes : (size_t)n_ * W;
+        const size_t mat_bytes = (size_t)n_ * W * n_blocks;
+        bins_.block_stride = (size_t)n_ * W;
         TGBM_CHECK(mat_bytes + (size_t)n_ * F_ < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
                    mat_bytes, free_b);
         d_binmat_ = dalloc<uint8_t>(mat_bytes);
@@ -147,8 +139,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
         uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_);
         launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_);
-        launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, bins_,
-                         d_colmat, col_stride);
+        launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
+                         bins_.block_stride, d_colmat, col_stride);
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
@@ -172,7 +164,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     // base score (regression_obj.h:35-53, :95-114; only for squared / logistic objectives)
     if (objective_ != OBJ_SOFTMAX) {
         launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
-        launch_tree_init(stream_, tb_, bins_, d_gh_, param_.lambda);  // reuses the root-sum reduction
+        launch_tree_init(stream_, tb_, d_gh_, param_.lambda);  // reuses the root-sum reduction
         TreeNode root;
         HIP_CHECK(hipMemcpyAsync(&root, tb_.nodes, sizeof(TreeNode), hipMemcpyDeviceToHost, stream_));
         HIP_CHECK(hipStreamSynchronize(stream_));
@@ -300,7 +292,7 @@ void Trainer::compute_gradient() {
 
 void Trainer::tree_init(int k) {
     cur_class_ = k;
-    launch_tree_init(stream_, tb_, bins_, d_gh_ + (size_t)k * n_, param_.lambda);
+    launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda);
 }
 
 void Trainer::find_split(int level) {
@@ -454,7 +446,6 @@ int Trainer::info(const std::string &key) const {
     if (key == "tree_per_rounds") return param_.tree_per_rounds;
     if (key == "n_nodes") return tb_.n_nodes;
     if (key == "sparse") return sparse_ ? 1 : 0;
-    if (key == "row_records") return bins_.rec_size;
     if (key == "dense_W") return bins_.W;
     if (key == "dense_blocks") return bins_.n_blocks;
     if (key == "trees_built") return trees_built_;
@@ -474,19 +465,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     if (name == "cut_val") src = cuts_.cut_val, bytes = sizeof(float) * (size_t)n_bins_;
     else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
-    else if (name == "binmat") {
-        bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
-        src = d_binmat_;
-        if (!sparse_ && bins_.rec_size != 0) {  // hand out plain rows
-            uint8_t *tmp = nullptr;
-            HIP_CHECK(hipMalloc(&tmp, bytes));
-            launch_unpack_records(stream_, bins_, n_, tmp);
-            sync();
-            if (out != nullptr && cap >= bytes && bytes > 0) HIP_CHECK(hipMemcpy(out, tmp, bytes, hipMemcpyDeviceToHost));
-            HIP_CHECK(hipFree(tmp));
-            return bytes;
-        }
-    }
+    else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
         launch_nid_rebuild(stream_, tb_);  // the map is kept as row lists; materialise it on demand

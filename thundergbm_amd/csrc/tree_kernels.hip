@@ -136,15 +136,11 @@ __global__ void k_gradient_softmax(int n, int K, const float *__restrict__ y, co
 }
 
 // Block sums of (g,h) and block maxima of |g|, h for one tree; fixed grid and fixed reduction order.
-// In record mode the same pass drops every row's pair into its row record.
-__global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out,
-                                                  DenseBins bins) {
+__global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out) {
     __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
     float g = 0, h = 0, gm = 0, hm = 0;
-    uint8_t *rec = const_cast<uint8_t *>(bins.data);
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         GHPair v = gh[i];
-        if (bins.rec_size != 0) *reinterpret_cast<GHPair *>(rec + dense_gh_offset(bins, i)) = v;
         g += v.g;
         h += v.h;
         gm = fmaxf(gm, fabsf(v.g));
@@ -297,8 +293,10 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
 // them; at the end the registers go to the item's slot of `partial`.
 // LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
 // instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
-// REC: rows are records that also hold the row's gradient pair (one 128-byte line per gathered row).
-template <int LPR, bool DIRECT, int BLK, int SLOTS, bool REC>
+// (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
+// instead of two was measured: it halves the fetched bytes below the root, but the per-tree refresh of
+// the pairs costs what the gathers save.)
+template <int LPR, bool DIRECT, int BLK, int SLOTS>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
                                                     const int *__restrict__ ridx, const int2 *__restrict__ seg,
@@ -352,13 +350,8 @@ void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
             bool ok = pos < end;
             int r = 0;
             if (ok) r = DIRECT ? pos : ridx[pos];
-            if (REC) {
-                opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + dense_row_offset(bins, r)) : 0xffffffffu;
-                os[u] = ok ? *reinterpret_cast<const GHPair *>(bins.data + dense_gh_offset(bins, r)) : GHPair{0, 0};
-            } else {
-                opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
-                os[u] = ok ? gh[r] : GHPair{0, 0};
-            }
+            opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
+            os[u] = ok ? gh[r] : GHPair{0, 0};
         }
     };
     if (begin < end) load_rows(begin, pk, s);
@@ -1239,25 +1232,12 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
 }
 
-__global__ void k_unpack_records(DenseBins bins, int n, uint8_t *__restrict__ out) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < (size_t)n * bins.W;
-         i += (size_t)gridDim.x * blockDim.x) {
-        int r = (int)(i / bins.W), j = (int)(i % bins.W);
-        out[i] = bins.data[dense_row_offset(bins, r) + j];
-    }
-}
-
-void launch_unpack_records(hipStream_t s, const DenseBins &bins, int n, uint8_t *out) {
-    k_unpack_records<<<grid_for((size_t)n * bins.W), kBlock, 0, s>>>(bins, n, out);
-}
-
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh_class,
-                      float lambda) {
-    k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial, bins);
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda) {
+    k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
     k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
 }
 
-template <int LPR, int SLOTS, bool REC>
+template <int LPR, int SLOTS>
 static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                               int level) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
@@ -1268,43 +1248,34 @@ static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseB
         static size_t opted = 0;
         if (lds > opted) {
             HIP_CHECK(hipFuncSetAttribute(
-                reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS, REC>),
+                reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS>),
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             HIP_CHECK(hipFuncSetAttribute(
-                reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS, REC>),
+                reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS>),
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             opted = lds;
         }
     }
     if (level == 0) {
-        k_hist_dense<LPR, true, kHistBlock, SLOTS, REC><<<grid, kHistBlock, lds, s>>>(
+        k_hist_dense<LPR, true, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
             bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
             tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
     } else {
-        k_hist_dense<LPR, false, kHistBlock, SLOTS, REC><<<grid, kHistBlock, lds, s>>>(
+        k_hist_dense<LPR, false, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
             bins, gh, tb.ridx[level & 1], tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
             tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
     }
-}
-
-template <int LPR, int SLOTS>
-static void hist_dense_launch_layout(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
-                                     int level) {
-    if (bins.rec_size != 0)
-        hist_dense_launch<LPR, SLOTS, true>(s, tb, bins, gh, level);
-    else
-        hist_dense_launch<LPR, SLOTS, false>(s, tb, bins, gh, level);
 }
 
 template <int LPR>
 static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                                 int level) {
     const int slots = (tb.max_block_bins + kHistBlock - 1) / kHistBlock;  // bins drained per thread
-    if (slots <= 1) hist_dense_launch_layout<LPR, 1>(s, tb, bins, gh, level);
-    else if (slots <= 2) hist_dense_launch_layout<LPR, 2>(s, tb, bins, gh, level);
-    else if (slots <= 4) hist_dense_launch_layout<LPR, 4>(s, tb, bins, gh, level);
-    else if (slots <= 8) hist_dense_launch_layout<LPR, 8>(s, tb, bins, gh, level);
-    else if (slots <= 20) hist_dense_launch_layout<LPR, 20>(s, tb, bins, gh, level);
+    if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level);
+    else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level);
+    else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level);
+    else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level);
+    else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level);
     else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
 }
 
