@@ -19,6 +19,19 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 import numpy as np  # noqa: E402
 
 
+def measured_traffic_per_launch():
+    """HBM bytes per k_hist_dense launch from the committed rocprofv3 --pmc summary (FETCH_SIZE and
+    WRITE_SIZE runs, calibrated against a plain copy kernel); None when the summary is absent."""
+    path = os.path.join(ROOT, "profiles", "k_hist_dense_config2_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,7 +88,8 @@ def main():
         if prof["launches"] > 0 and prof["hist_ms"] > 0:
             achieved = prof["bytes"] / (prof["hist_ms"] * 1e-3) / 1e9
             roofline = {"bound": "hbm", "kernel": "k_hist_dense", "achieved": round(achieved, 2), "peak": 8000.0,
-                        "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": None,
+                        "unit": "GB/s", "frac": round(achieved / 8000.0, 4),
+                        "traffic": measured_traffic_per_launch() if args.rows == 10_000_000 else None,
                         "bytes_per_launch": round(prof["bytes"] / prof["launches"], 1),
                         "avg_launch_us": round(prof["hist_ms"] * 1e3 / prof["launches"], 2),
                         "hist_ms_per_tree": round(prof["hist_ms"] / args.profile_steps, 4),
