@@ -1,0 +1,154 @@
+"""GPU parity on edge shapes: tiny and ragged inputs, empty rows, one feature, extreme depths and bin
+counts, every objective. Each case boosts a few rounds with the oracle restarted from the GPU's
+predictions (teacher forcing) and compares every tree."""
+import os
+
+import numpy as np
+import pytest
+
+import datasets as D
+import oracle_lib as O
+import parity as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def T():
+    import thundergbm_amd
+    thundergbm_amd.load()
+    return thundergbm_amd
+
+
+@pytest.fixture(autouse=True)
+def _default_layout():
+    os.environ.pop("TGBM_LAYOUT", None)
+    yield
+    os.environ.pop("TGBM_LAYOUT", None)
+
+
+def _ragged(n, F, seed, max_len):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, max_len + 1, n)
+    lens[: max(1, n // 50)] = 0  # some completely empty rows
+    rp = np.zeros(n + 1, np.int32)
+    np.cumsum(lens, out=rp[1:])
+    col = np.concatenate([np.sort(rng.choice(F, size=l, replace=False)) for l in lens] + [np.zeros(0, np.int64)])
+    col = col.astype(np.int32)
+    val = np.round(rng.standard_normal(len(col)) * 3, 1).astype(np.float32)
+    val[val == 0] = 1.5
+    if len(col) and col.max() != F - 1:  # make sure the feature count is what the case says
+        col[-1] = F - 1
+    return val, rp, col
+
+
+def _target(val, rp, col, n, F, seed, kind):
+    rng = np.random.default_rng(seed + 100)
+    w = rng.standard_normal(F)
+    s = np.zeros(n)
+    rows = np.repeat(np.arange(n), np.diff(rp))
+    np.add.at(s, rows, w[col] * val)
+    s += 0.3 * rng.standard_normal(n)
+    if kind == "reg":
+        return s.astype(np.float32)
+    if kind == "bin":
+        return np.where(s > np.median(s), 5.0, 2.0).astype(np.float32)  # arbitrary label values
+    if kind == "prob":
+        return (1 / (1 + np.exp(-s))).astype(np.float32)
+    q = np.quantile(s, [0.2, 0.5, 0.8])
+    return (np.digitize(s, q) * 10 - 7).astype(np.float32)  # labels -7, 3, 13, 23
+
+
+CASES = {
+    # name: (n, F, max row length, objective, target kind, kwargs, layout)
+    "tiny": (37, 5, 5, "reg:linear", "reg", dict(depth=3, max_num_bin=8), None),
+    "one_feature": (500, 1, 1, "reg:linear", "reg", dict(depth=4, max_num_bin=16), None),
+    "depth1": (800, 6, 6, "binary:logistic", "bin", dict(depth=1, max_num_bin=32), None),
+    "depth10": (3000, 7, 7, "reg:linear", "reg", dict(depth=10, max_num_bin=64, gamma=0.0), None),
+    "two_bins": (1000, 9, 9, "binary:logistic", "bin", dict(depth=4, max_num_bin=2), None),
+    "reg_logistic": (1200, 8, 8, "reg:logistic", "prob", dict(depth=4, max_num_bin=32), None),
+    "softprob": (1500, 10, 8, "multi:softprob", "multi", dict(depth=3, max_num_bin=32), None),
+    "wide_dense_blocks": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense"),
+    "wide_sparse": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse"),
+    "lambda0_mcw5": (900, 6, 6, "reg:linear", "reg", dict(depth=4, max_num_bin=32, lambda_=0.0, min_child_weight=5.0),
+                     None),
+    "gamma_prunes_all": (600, 5, 5, "reg:linear", "reg", dict(depth=4, max_num_bin=16, gamma=1e9), None),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_edge_case_matches_oracle(T, name):
+    n, F, max_len, objective, kind, kw, layout = CASES[name]
+    if layout:
+        os.environ["TGBM_LAYOUT"] = layout
+    val, rp, col = _ragged(n, F, hash(name) % 1000, max_len)
+    y = _target(val, rp, col, n, F, hash(name) % 1000, kind)
+    rounds = 4
+    kw = dict(kw, objective=objective, n_trees=rounds, learning_rate=0.5)
+    lam = kw.get("lambda_", 1.0)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    # data preparation: exact
+    cv, crp, cf = s.cuts()
+    ocv, ocrp, ocf = o.cuts()
+    assert np.array_equal(cv, ocv) and np.array_equal(crp, ocrp) and np.array_equal(cf, ocf)
+    gb, _ = s.global_bin_ids(rp, col)
+    assert np.array_equal(gb, o.bin_ids())
+    assert np.array_equal(s.y(), o.y()) and np.array_equal(s.labels(), o.labels())
+    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7)
+    present = np.zeros((n, s.F), bool)
+    present[np.repeat(np.arange(n), np.diff(rp)), col] = True
+    for r in range(rounds):
+        o.set_y_pred(s.y_pred())
+        s.boost(1)
+        o.compute_gradient()
+        gh = s.gh()
+        np.testing.assert_allclose(gh, o.gh(), rtol=1e-5, atol=2e-7)
+        o.set_gh(gh)
+        model = s.model()
+        tol = np.zeros(len(o.y_pred()))
+        clean = True
+        for k in range(s.tree_per_rounds):
+            o.build_tree(k)
+            final_nid = o.nid()
+            ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
+            d = P.compare_trees(model[r, k], o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(),
+                                missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
+                                abs_scale=(ghk[0], ghk[1]))
+            clean &= not d.near_ties
+            sl = slice(k * n, (k + 1) * n)
+            tol[sl] = P.pred_tolerance(o.nodes(), final_nid, 0.5, lam, (ghk[0], ghk[1]), o.y_pred()[sl])
+        if clean:
+            assert np.all(np.abs(s.y_pred().astype(np.float64) - o.y_pred()) <= tol)
+            assert np.array_equal(s.nid(), o.nid())
+            np.testing.assert_allclose(s.metric_log()[-1], o.metric(), rtol=1e-4, atol=1e-5)
+    if name == "gamma_prunes_all":
+        assert all(t[0]["is_leaf"] for rnd in s.model() for t in rnd)  # every tree collapsed into its root
+    s.close()
+
+
+def test_predict_transforms_through_the_c_abi(T):
+    """sparse_predict_scikit for every objective against the oracle's predictor + transform on unseen rows."""
+    n, F = 1500, 7
+    val, rp, col = _ragged(n, F, 5, 7)
+    tv, trp, tc = _ragged(400, F, 6, 7)
+    for objective, kind, cls in (("reg:linear", "reg", "r"), ("reg:logistic", "prob", "r"),
+                                 ("binary:logistic", "bin", "c"), ("multi:softmax", "multi", "c"),
+                                 ("multi:softprob", "multi", "c")):
+        y = _target(val, rp, col, n, F, 5, kind)
+        import scipy.sparse as sp
+        X = sp.csr_matrix((val, col, rp), shape=(n, F))
+        Xt = sp.csr_matrix((tv, tc, trp), shape=(400, F))
+        Est = T.TGBMRegressor if cls == "r" else T.TGBMClassifier
+        m = Est(depth=4, n_trees=6, learning_rate=0.4, objective=objective, verbose=0, max_num_bin=32).fit(X, y)
+        got = np.asarray(m.predict(Xt)).ravel()
+        o = O.Oracle(val, rp, col, y, depth=4, n_trees=6, learning_rate=0.4, objective=objective, max_num_bin=32,
+                     num_class=2).prepare()
+        o.boost(6)
+        raw = O.predict_raw(tv, trp, tc, F, o.model(), 0.4, 0.0)  # the C-API path has no base score
+        labels = o.labels() if cls == "c" else np.zeros(1, np.float32)
+        exp = O.predict_transform(objective, raw, 400, o.num_class, labels)
+        if objective in ("binary:logistic", "multi:softmax"):
+            assert np.mean(got == exp) > 0.99
+        else:
+            np.testing.assert_allclose(got, exp, rtol=1e-4, atol=1e-5)
