@@ -101,7 +101,8 @@ float tgbm_trainer_base_score(tgbm_trainer *t);
 
 /* Copies a device buffer to `out` when `cap` is large enough; always returns its size in bytes.
  * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist_q0, hist_q1,
- * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels. */
+ * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels. After tgbm_trainer_boost `gh` may already
+ * hold the gradients of the next round (single-tree objectives compute them in the round's last pass). */
 size_t tgbm_trainer_get(tgbm_trainer *t, const char *name, void *out, size_t cap);
 /* Overwrites gh or y_pred (lock-step tests feed both implementations the same state). */
 void tgbm_trainer_set(tgbm_trainer *t, const char *name, const void *in, size_t bytes);

@@ -100,9 +100,10 @@ def test_edge_case_matches_oracle(T, name):
     present[np.repeat(np.arange(n), np.diff(rp)), col] = True
     for r in range(rounds):
         o.set_y_pred(s.y_pred())
+        s.gradient()
+        gh = s.gh()  # the gradients this round is built from (boost recomputes the same values)
         s.boost(1)
         o.compute_gradient()
-        gh = s.gh()
         np.testing.assert_allclose(gh, o.gh(), rtol=1e-5, atol=2e-7)
         o.set_gh(gh)
         model = s.model()
@@ -125,6 +126,39 @@ def test_edge_case_matches_oracle(T, name):
     if name == "gamma_prunes_all":
         assert all(t[0]["is_leaf"] for rnd in s.model() for t in rnd)  # every tree collapsed into its root
     s.close()
+
+
+@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin"),
+                                            ("reg:logistic", "prob")])
+def test_one_boost_call_equals_round_by_round(T, objective, kind):
+    """boost(6) ends every round with one fused pass (prediction update, metric, next gradients and their
+    block statistics); the stage-wise calls run the separate kernels.
+    Both must give the same bits."""
+    n, F = 6000, 9
+    val, rp, col = _ragged(n, F, 7, F)
+    y = _target(val, rp, col, n, F, 7, kind)
+    kw = dict(objective=objective, n_trees=6, depth=5, max_num_bin=32, learning_rate=0.3)
+    a = T.Session(val, rp, col, y, **kw)
+    a.boost(6)
+    b = T.Session(val, rp, col, y, **kw)
+    metrics = []
+    for _ in range(6):
+        b.gradient()
+        b.tree_init(0)
+        for level in range(5):
+            b.find_split(level)
+            b.partition(level)
+        b.finish_tree(0)
+        metrics.append(b.metric())
+    assert a.model().tobytes() == b.model().tobytes()
+    assert np.array_equal(a.y_pred(), b.y_pred())
+    assert np.array_equal(a.metric_log(), np.array(metrics, np.float32))
+    # the gradients left behind by the fused pass are those of the next round
+    g_next = a.gh()
+    b.gradient()
+    assert np.array_equal(g_next, b.gh())
+    a.close()
+    b.close()
 
 
 def test_predict_transforms_through_the_c_abi(T):

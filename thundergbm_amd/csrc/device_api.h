@@ -114,7 +114,11 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda);
+// stats_ready: tb.root_partial already holds the block statistics of gh_class (fused round end)
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda,
+                      bool stats_ready = false);
+void launch_round_end_fused(hipStream_t s, const TreeBuffers &tb, int objective, int metric_kind, const float *y,
+                            float *yp, float lr, GHPair *gh, double *metric_scratch, float *metric_out);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);

@@ -34,7 +34,9 @@ class Trainer {
     void tree_init(int k);
     void find_split(int level);  // histogram, merge/subtract, split search, update_tree
     void partition(int level);   // update_ins2node_id + next level's row lists
-    void finish_tree(int k);     // prune, prediction update, append the tree to the model
+    // prune, prediction update, append the tree to the model; fuse_round_end also computes the metric and
+    // the next round's gradients in the same pass (single-tree objectives inside boost())
+    void finish_tree(int k, bool fuse_round_end = false);
     float metric();
     void sync();
 
@@ -78,6 +80,7 @@ class Trainer {
     float *d_metric_ = nullptr;
     double *d_metric_scratch_ = nullptr;
     int cur_class_ = 0;
+    bool next_round_ready_ = false;  // d_gh_ and the root statistics already belong to the next round
     // profiling
     bool profiling_ = false;
     struct HistEvent {

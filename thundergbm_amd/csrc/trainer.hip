@@ -287,12 +287,14 @@ Trainer::~Trainer() {
 void Trainer::sync() { HIP_CHECK(hipStreamSynchronize(stream_)); }
 
 void Trainer::compute_gradient() {
+    next_round_ready_ = false;
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
 }
 
 void Trainer::tree_init(int k) {
     cur_class_ = k;
-    launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda);
+    launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
+    next_round_ready_ = false;
 }
 
 void Trainer::find_split(int level) {
@@ -329,10 +331,17 @@ void Trainer::partition(int level) {
         launch_partition_dense(stream_, tb_, bins_, level);
 }
 
-void Trainer::finish_tree(int k) {
+void Trainer::finish_tree(int k, bool fuse_round_end) {
     launch_prune(stream_, tb_, param_.gamma);
     launch_nid_rebuild(stream_, tb_);
-    launch_predict_in_training(stream_, tb_, d_yp_ + (size_t)k * n_, param_.learning_rate);
+    if (fuse_round_end) {
+        // one tree per round: prediction update + metric + next gradients + their statistics in one pass
+        launch_round_end_fused(stream_, tb_, objective_, metric_kind_, d_y_, d_yp_, param_.learning_rate, d_gh_,
+                               d_metric_scratch_, d_metric_ + rounds_done_);
+        next_round_ready_ = true;
+    } else {
+        launch_predict_in_training(stream_, tb_, d_yp_ + (size_t)k * n_, param_.learning_rate);
+    }
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb_.n_nodes, tb_.nodes,
                              sizeof(TreeNode) * (size_t)tb_.n_nodes, hipMemcpyDeviceToDevice, stream_));
@@ -359,7 +368,8 @@ void Trainer::boost(int rounds) {
     static const char *names[] = {"RMSE", "test error", "multi-class accuracy"};
     for (int r = 0; r < rounds; ++r) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
-        compute_gradient();
+        const bool fuse = objective_ != OBJ_SOFTMAX && param_.tree_per_rounds == 1;
+        if (!next_round_ready_) compute_gradient();
         for (int k = 0; k < param_.tree_per_rounds; ++k) {
             tree_init(k);
             // The reference leaves the level loop when no row sits in a node that was split
@@ -369,10 +379,10 @@ void Trainer::boost(int rounds) {
                 find_split(level);
                 partition(level);
             }
-            finish_tree(k);
+            finish_tree(k, fuse);
         }
         float *slot = d_metric_ + rounds_done_;
-        launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+        if (!fuse) launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
         if (g_verbose >= 1) {
             float v = 0;
             HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
@@ -493,6 +503,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
 
 void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     sync();
+    next_round_ready_ = false;
     void *dst = nullptr;
     size_t want = 0;
     if (name == "gh") dst = d_gh_, want = sizeof(GHPair) * (size_t)param_.num_class * n_;

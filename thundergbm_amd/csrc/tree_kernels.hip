@@ -1133,6 +1133,86 @@ __global__ void k_predict_in_training(int n, const int *__restrict__ nid, const 
     }
 }
 
+// ------------------------------------------------------------------- fused end of a round
+// For objectives with one tree per round: the in-training prediction update (tree_builder.cu:62-74),
+// the training metric partials (pointwise_metric.cu:13-20 / multiclass_metric.cu:39-44), the next
+// round's gradients (regression_obj.h:130-154) and their block statistics for the next tree's root
+// in one pass over the rows. Same grids, loops and arithmetic as k_predict_in_training,
+// k_metric_partial, k_gradient_pointwise and k_sum_gh, so the results are bit-identical to running
+// those four kernels.
+__global__ __launch_bounds__(kBlock) void k_round_end_fused(int n, int objective, int metric_kind,
+                                                           const int *__restrict__ nid,
+                                                           const TreeNode *__restrict__ nodes,
+                                                           const float *__restrict__ y, float *__restrict__ yp,
+                                                           float lr, GHPair *__restrict__ gh,
+                                                           GradStats *__restrict__ stats,
+                                                           double *__restrict__ metric_out) {
+    __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
+    __shared__ double sd[kWaves];
+    float g = 0, h = 0, gm = 0, hm = 0;
+    double acc = 0;
+    float accf = 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+        int x = nid[i];
+        while (x != -1 && nodes[x].is_pruned) x = nodes[x].parent_index;
+        float p = yp[i];
+        p += lr * nodes[x].base_weight;
+        yp[i] = p;
+        const float yi = y[i];
+        if (metric_kind == 0) {
+            float e = p - yi;
+            accf += e * e;
+        } else {
+            int k = (1.0 / (1.0 + exp(-(double)p)) > 0.5) ? 1 : 0;
+            acc += (k == yi) ? 1 : 0;
+        }
+        GHPair o;
+        if (objective == OBJ_SQUARE) {
+            o.g = p - yi;
+            o.h = 1.f;
+        } else {
+            float sgm = 1.f / (1.f + expf(-p));
+            o.g = sgm - yi;
+            o.h = fmaxf(sgm * (1.f - sgm), 1e-16f);
+        }
+        gh[i] = o;
+        g += o.g;
+        h += o.h;
+        gm = fmaxf(gm, fabsf(o.g));
+        hm = fmaxf(hm, o.h);
+    }
+    acc += (double)accf;
+    g = wave_sum_f(g);
+    h = wave_sum_f(h);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        gm = fmaxf(gm, __shfl_xor(gm, d));
+        hm = fmaxf(hm, __shfl_xor(hm, d));
+        acc += __shfl_xor(acc, d);
+    }
+    if (lane_id() == 0) {
+        sg[wave_id()] = g;
+        sh[wave_id()] = h;
+        mg[wave_id()] = gm;
+        mh[wave_id()] = hm;
+        sd[wave_id()] = acc;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        GradStats o{0, 0, 0, 0};
+        double s = 0;
+        for (int i = 0; i < kWaves; ++i) {
+            o.g += sg[i];
+            o.h += sh[i];
+            o.gmax = fmaxf(o.gmax, mg[i]);
+            o.hmax = fmaxf(o.hmax, mh[i]);
+            s += sd[i];
+        }
+        stats[blockIdx.x] = o;
+        metric_out[blockIdx.x] = s;
+    }
+}
+
 // ---------------------------------------------------------------------------------- metric
 // kind 0: sum of squared errors; 1: correct binary decisions (sigmoid > 0.5 in double, like
 // multiclass_metric.cu:40); 2: correct arg-max decisions (first maximum wins, :17-29).
@@ -1232,8 +1312,16 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
 }
 
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda) {
-    k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
+void launch_round_end_fused(hipStream_t s, const TreeBuffers &tb, int objective, int metric_kind, const float *y,
+                            float *yp, float lr, GHPair *gh, double *metric_scratch, float *metric_out) {
+    // grid == the grids of k_sum_gh and k_metric_partial (both min(1024, ceil(n / 256)))
+    k_round_end_fused<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, objective, metric_kind, tb.nid, tb.nodes, y, yp, lr, gh,
+                                                         tb.root_partial, metric_scratch);
+    k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, tb.n_grad_blocks, metric_scratch, metric_out);
+}
+
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, bool stats_ready) {
+    if (!stats_ready) k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
     k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
 }
 
