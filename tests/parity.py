@@ -53,7 +53,7 @@ def rows_in_node(final_nid, x):
     return cur == x
 
 
-def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL):
+def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL, mcw=1.0):
     """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
 
     Where both trees split on the same candidate everything must agree: threshold and bin exactly,
@@ -67,6 +67,10 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     root, so their error is relative to the root-level sums of |g| and |h| (abs_scale = (Ag, Ah)):
     |dG| <= rel * Ag, |dH| <= rel * Ah. Weights and gains get the first-order propagation of those
     two bounds (w = -G/(H+lam); d gain/dG = -2w, d gain/dH = -w^2 per term).
+    A choice that differs is also accepted as a near tie when one side's chosen split has a child whose
+    hessian sum sits within dH of min_child_weight (mcw): that gate (hist_tree_builder_single.cu
+    compute_gain: both children need h >= min_child_weight) flips on the last ulps of a sum, e.g. four
+    logistic rows with p = 0.5 give exactly 4 * 0.25 = 1.0 or one ulp less depending on the order.
     orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle (None forbids any mismatch);
     crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
     """
@@ -107,6 +111,14 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
             continue
         assert orc_scores is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (
             x, g["split_fid"], g["split_bid"], o["split_fid"], o["split_bid"])
+        on_gate = False
+        for t, has in ((gpu, split_g), (orc, split_o)):
+            if has:
+                hmin = min(float(t[int(t[x]["lch"])]["sum_h"]), float(t[int(t[x]["rch"])]["sum_h"]))
+                on_gate |= abs(hmin - mcw) <= dH
+        if on_gate:
+            diff.near_ties.append((x, float("nan"), float("nan")))
+            continue
         sc = orc_scores[x]
         best = float(np.abs(sc).max())
         tol = 2 * gain_tol(x, o)

@@ -2,6 +2,7 @@
 counts, every objective. Each case boosts a few rounds with the oracle restarted from the GPU's
 predictions (teacher forcing) and compares every tree."""
 import os
+import zlib
 
 import numpy as np
 import pytest
@@ -78,11 +79,15 @@ CASES = {
 
 @pytest.mark.parametrize("name", sorted(CASES))
 def test_edge_case_matches_oracle(T, name):
+    run_case(T, name, zlib.crc32(name.encode()) % 1000)
+
+
+def run_case(T, name, seed):
     n, F, max_len, objective, kind, kw, layout = CASES[name]
     if layout:
         os.environ["TGBM_LAYOUT"] = layout
-    val, rp, col = _ragged(n, F, hash(name) % 1000, max_len)
-    y = _target(val, rp, col, n, F, hash(name) % 1000, kind)
+    val, rp, col = _ragged(n, F, seed, max_len)
+    y = _target(val, rp, col, n, F, seed, kind)
     rounds = 4
     kw = dict(kw, objective=objective, n_trees=rounds, learning_rate=0.5)
     lam = kw.get("lambda_", 1.0)
@@ -115,7 +120,7 @@ def test_edge_case_matches_oracle(T, name):
             ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
             d = P.compare_trees(model[r, k], o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(),
                                 missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
-                                abs_scale=(ghk[0], ghk[1]))
+                                abs_scale=(ghk[0], ghk[1]), mcw=kw.get("min_child_weight", 1.0))
             clean &= not d.near_ties
             sl = slice(k * n, (k + 1) * n)
             tol[sl] = P.pred_tolerance(o.nodes(), final_nid, 0.5, lam, (ghk[0], ghk[1]), o.y_pred()[sl])

@@ -17,6 +17,8 @@ namespace tgbm {
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
 constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
 constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
+constexpr int kRowBlock = 4096;    // rows owned by one workgroup of the row-ordered passes and reductions
+inline int row_blocks(int n) { return n <= 0 ? 1 : (n + kRowBlock - 1) / kRowBlock; }
 
 // Per-level control block written by the planning kernels and read by the worker kernels.
 struct LevelCtl {
@@ -84,6 +86,8 @@ struct TreeBuffers {
     longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
     QuantCtl *quant = nullptr;     // scales of the current tree
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
+    float *leaf_value = nullptr;   // [n_nodes] prediction increment of a row that ended in the node (after pruning)
+    int *end_bound = nullptr;      // [(row_blocks(n) + 1) x (2^depth - 1)] list positions of the row block boundaries
     int *hpair_begin = nullptr;    // [max_pairs + 1] first histogram item of every sibling pair
     int *hpair_built = nullptr;    // [max_pairs] heap id of the node built from rows, -1 = inactive pair
     int *pitem_begin = nullptr;    // [max_level_nodes + 1]
@@ -117,8 +121,6 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
 // stats_ready: tb.root_partial already holds the block statistics of gh_class (fused round end)
 void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda,
                       bool stats_ready = false);
-void launch_round_end_fused(hipStream_t s, const TreeBuffers &tb, int objective, int metric_kind, const float *y,
-                            float *yp, float lr, GHPair *gh, double *metric_scratch, float *metric_out);
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);
@@ -126,9 +128,19 @@ void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &b
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level);
-void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb);
+// Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level
+// whose split nodes still hold their children's rows (-1: none).
+void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                        int lookup_level);
+void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                                int lookup_level, float *yp_class, float lr);
+// prediction update + metric + next gradients + their block statistics (tb.root_partial); metric_scratch
+// holds row_blocks(n) doubles
+void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                      int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
+                      GHPair *gh, double *metric_scratch, float *metric_out);
 void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma);
-void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, float *yp_class, float lr);
+// scratch: row_blocks(n) doubles
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);
 void launch_fill_f32(hipStream_t s, float *p, float v, size_t n);

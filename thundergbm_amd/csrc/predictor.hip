@@ -67,7 +67,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
         double *d_scratch = nullptr;
         HIP_CHECK(hipMalloc(&d_y, sizeof(float) * (size_t)n));
         HIP_CHECK(hipMalloc(&d_m, sizeof(float)));
-        HIP_CHECK(hipMalloc(&d_scratch, sizeof(double) * 1024));
+        HIP_CHECK(hipMalloc(&d_scratch, sizeof(double) * (size_t)row_blocks(n)));
         HIP_CHECK(hipMemcpyAsync(d_y, ds.y.data(), sizeof(float) * (size_t)n, hipMemcpyHostToDevice, s));
         launch_metric(s, kind, n, nct, d_y, d_out, d_scratch, d_m);
         float v = 0;

@@ -104,6 +104,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     sparse_ = (F_ > 4096 && density < 0.05) || (size_t)n_ * F_ * 2 > free_b / 2;
     if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
     if (force != nullptr && std::string(force) == "dense") sparse_ = false;
+    if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
     log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
     if (sparse_) {
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
@@ -210,6 +211,8 @@ void Trainer::alloc_tree_buffers() {
     tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
     // the planning kernel of the last level also writes the (unused) plan of level `depth`
     tb.hpair_begin = dalloc<int>((size_t)max_level_nodes + 1);
+    tb.leaf_value = dalloc<float>((size_t)tb.n_nodes);
+    tb.end_bound = dalloc<int>(((size_t)row_blocks(n_) + 1) * (((size_t)1 << depth) - 1));
     tb.hpair_built = dalloc<int>((size_t)max_level_nodes);
     tb.pitem_begin = dalloc<int>((size_t)max_level_nodes + 1);
     tb.pitem_nleft = dalloc<int>((size_t)tb.max_pitems + 1);
@@ -217,7 +220,7 @@ void Trainer::alloc_tree_buffers() {
     tb.node_nleft = dalloc<int>((size_t)max_level_nodes);
     tb.ctl = dalloc<LevelCtl>((size_t)depth + 2);
     tb.sp = dalloc<SplitPoint>((size_t)max_level_nodes);
-    tb.n_grad_blocks = std::min(1024, (n_ + 255) / 256);
+    tb.n_grad_blocks = row_blocks(n_);
     tb.root_partial = dalloc<GradStats>((size_t)tb.n_grad_blocks);
     tb.cut_row_ptr = cuts_.cut_row_ptr;
     tb.cut_fid = cuts_.cut_fid;
@@ -271,7 +274,7 @@ void Trainer::alloc_tree_buffers() {
     model_cap_trees_ = std::max(1, param_.n_trees) * param_.tree_per_rounds;
     d_model_ = dalloc<TreeNode>((size_t)model_cap_trees_ * tb.n_nodes);
     d_metric_ = dalloc<float>((size_t)std::max(1, param_.n_trees));
-    d_metric_scratch_ = dalloc<double>(1024);
+    d_metric_scratch_ = dalloc<double>((size_t)row_blocks(n_));
 }
 
 Trainer::~Trainer() {
@@ -295,6 +298,7 @@ void Trainer::tree_init(int k) {
     cur_class_ = k;
     launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
     next_round_ready_ = false;
+    lookup_level_ = -1;
 }
 
 void Trainer::find_split(int level) {
@@ -315,6 +319,7 @@ void Trainer::find_split(int level) {
     if (!sparse_) launch_hist_merge(stream_, tb_, level);
     launch_eval_split(stream_, tb_, level, param_.min_child_weight, param_.lambda);
     launch_best_update(stream_, tb_, level, param_.rt_eps, param_.lambda);
+    lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
 }
 
 void Trainer::build_level_hist(int level, const GHPair *gh) {
@@ -325,6 +330,8 @@ void Trainer::build_level_hist(int level, const GHPair *gh) {
 }
 
 void Trainer::partition(int level) {
+    // the last level is not partitioned: its split nodes keep their rows until the tree's final pass
+    if (level < param_.depth - 1) lookup_level_ = -1;
     if (sparse_)
         launch_partition_csr(stream_, tb_, csr_, level);
     else
@@ -333,14 +340,14 @@ void Trainer::partition(int level) {
 
 void Trainer::finish_tree(int k, bool fuse_round_end) {
     launch_prune(stream_, tb_, param_.gamma);
-    launch_nid_rebuild(stream_, tb_);
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
-        launch_round_end_fused(stream_, tb_, objective_, metric_kind_, d_y_, d_yp_, param_.learning_rate, d_gh_,
-                               d_metric_scratch_, d_metric_ + rounds_done_);
+        launch_round_end(stream_, tb_, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
+                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_);
         next_round_ready_ = true;
     } else {
-        launch_predict_in_training(stream_, tb_, d_yp_ + (size_t)k * n_, param_.learning_rate);
+        launch_predict_in_training(stream_, tb_, &bins_, &csr_, lookup_level_, d_yp_ + (size_t)k * n_,
+                                   param_.learning_rate);
     }
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb_.n_nodes, tb_.nodes,
@@ -478,7 +485,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
-        launch_nid_rebuild(stream_, tb_);  // the map is kept as row lists; materialise it on demand
+        // the map is kept as row lists; materialise it on demand
+        launch_nid_rebuild(stream_, tb_, &bins_, &csr_, lookup_level_);
         sync();
         src = tb_.nid, bytes = sizeof(int) * (size_t)n_;
     }

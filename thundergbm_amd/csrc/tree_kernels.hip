@@ -98,21 +98,23 @@ __global__ void k_fill_u32(unsigned *p, unsigned v, size_t n) {
 
 // -------------------------------------------------------------------------------- gradients
 // Squared / logistic: include/thundergbm/objective/regression_obj.h:130-154 of the reference.
+__device__ __forceinline__ GHPair pointwise_gradient(int objective, float yi, float p) {
+    GHPair o;
+    if (objective == OBJ_SQUARE) {
+        o.g = p - yi;
+        o.h = 1.f;
+    } else {
+        float s = 1.f / (1.f + expf(-p));
+        o.g = s - yi;
+        o.h = fmaxf(s * (1.f - s), 1e-16f);
+    }
+    return o;
+}
+
 __global__ void k_gradient_pointwise(int objective, int n, const float *__restrict__ y, const float *__restrict__ yp,
                                      GHPair *__restrict__ gh) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        float p = yp[i];
-        GHPair o;
-        if (objective == OBJ_SQUARE) {
-            o.g = p - y[i];
-            o.h = 1.f;
-        } else {
-            float s = 1.f / (1.f + expf(-p));
-            o.g = s - y[i];
-            o.h = fmaxf(s * (1.f - s), 1e-16f);
-        }
-        gh[i] = o;
-    }
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        gh[i] = pointwise_gradient(objective, y[i], yp[i]);
 }
 
 // Softmax: src/thundergbm/objective/multiclass_obj.cu:6-35 (class-major predictions and gradients,
@@ -135,19 +137,24 @@ __global__ void k_gradient_softmax(int n, int K, const float *__restrict__ y, co
     }
 }
 
-// Block sums of (g,h) and block maxima of |g|, h for one tree; fixed grid and fixed reduction order.
-__global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out) {
-    __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
+// Row-blocked reductions: workgroup b owns rows [b * kRowBlock, (b + 1) * kRowBlock), thread t adds its
+// rows t, t + kBlock, ... in that order, then lanes, then wavefronts. Every kernel that produces
+// gradient statistics or metric partials follows this order, so fused and separate passes give the
+// same bits.
+struct RowStats {
     float g = 0, h = 0, gm = 0, hm = 0;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        GHPair v = gh[i];
+    __device__ __forceinline__ void add(GHPair v) {
         g += v.g;
         h += v.h;
         gm = fmaxf(gm, fabsf(v.g));
         hm = fmaxf(hm, v.h);
     }
-    g = wave_sum_f(g);
-    h = wave_sum_f(h);
+};
+
+// lds: 4 * kWaves floats; every thread of the block must call
+__device__ void store_block_stats(RowStats r, float *lds, GradStats *out) {
+    float *sg = lds, *sh = lds + kWaves, *mg = lds + 2 * kWaves, *mh = lds + 3 * kWaves;
+    float g = wave_sum_f(r.g), h = wave_sum_f(r.h), gm = r.gm, hm = r.hm;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
         gm = fmaxf(gm, __shfl_xor(gm, d));
@@ -168,8 +175,30 @@ __global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restri
             o.gmax = fmaxf(o.gmax, mg[i]);
             o.hmax = fmaxf(o.hmax, mh[i]);
         }
-        out[blockIdx.x] = o;
+        *out = o;
     }
+}
+
+// lds: kWaves doubles
+__device__ void store_block_sum_d(double acc, double *lds, double *out) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
+    if (lane_id() == 0) lds[wave_id()] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0;
+        for (int i = 0; i < kWaves; ++i) t += lds[i];
+        *out = t;
+    }
+}
+
+// Block sums of (g,h) and block maxima of |g|, h for one tree.
+__global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out) {
+    __shared__ float lds[4 * kWaves];
+    const int r0 = blockIdx.x * kRowBlock, r1 = min(n, r0 + kRowBlock);
+    RowStats st;
+    for (int i = r0 + threadIdx.x; i < r1; i += kBlock) st.add(gh[i]);
+    store_block_stats(st, lds, out + blockIdx.x);
 }
 
 // Largest power of two s with rows * (vmax * s + 0.5) < limit; 1 when vmax is 0 or not finite.
@@ -265,6 +294,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
         c.n_pitems = 0;
         c.rows_built = tb.n;
         tb.ctl[0] = c;
+        tb.ctl[tb.depth] = LevelCtl{0, 0, 0, 0};  // the last level plans no further one
         // One pair of scales serves the whole tree: between two drains of the LDS histogram at most
         // kHistFlushRows rows are added, which keeps a bin's gradient sum inside a signed and its
         // hessian sum inside an unsigned 32-bit field.
@@ -524,6 +554,26 @@ __global__ __launch_bounds__(kBlock) void k_hist_sub_csr(longlong2 *__restrict__
 
 // Left/right decision of the sparse layout: binary search of the row's bin ids for the one inside
 // the split feature's bin range (absent = missing), hist_tree_builder_single.cu:941-1011.
+// Does the row go right at a split of the feature whose global bins are [cb, ce)? Binary search of the
+// row's ascending bin ids for one inside the feature's range; none = missing -> default direction.
+__device__ __forceinline__ bool csr_goes_right(const CsrBins &bins, int row, int cb, int ce, int sbid, bool dr) {
+    int lo = bins.row_ptr[row], hi = bins.row_ptr[row + 1];
+    int found = -1;
+    while (lo < hi) {
+        int mid = lo + (hi - lo) / 2;
+        int b = bins.bin[mid];
+        if (b >= cb && b < ce) {
+            found = b;
+            break;
+        }
+        if (b < cb)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    return found < 0 ? dr : (found >= sbid);
+}
+
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb, CsrBins bins, const int *__restrict__ ridx,
                                                           int level) {
@@ -549,21 +599,7 @@ __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb, CsrBi
         int pos = pb + k * kBlock + threadIdx.x;
         if (pos < pe) {
             int row = DIRECT ? pos : ridx[pos];
-            int lo = bins.row_ptr[row], hi = bins.row_ptr[row + 1];
-            int found = -1;
-            while (lo < hi) {
-                int mid = lo + (hi - lo) / 2;
-                int b = bins.bin[mid];
-                if (b >= cb && b < ce) {
-                    found = b;
-                    break;
-                }
-                if (b < cb)
-                    lo = mid + 1;
-                else
-                    hi = mid;
-            }
-            bool right = found < 0 ? dr : (found >= sbid);
+            bool right = csr_goes_right(bins, row, cb, ce, sbid, dr);
             tb.goes_right[pos] = right ? 1 : 0;
             nleft += right ? 0 : 1;
         }
@@ -1049,46 +1085,6 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const i
     }
 }
 
-// Row -> node map (the reference's ins2node_id) from the row lists: a node holds rows iff it is valid
-// and was not split; its rows are its segment of the row list of its level's parity. Planning is one
-// workgroup over all nodes, writing is one workgroup per kPartChunk rows.
-__global__ __launch_bounds__(kBlock) void k_nid_plan(TreeBuffers tb) {
-    __shared__ int lds[kWaves];
-    int carry = 0;
-    for (int base = 0; base < tb.n_nodes; base += kBlock) {
-        int x = base + threadIdx.x;
-        int cnt = 0;
-        if (x < tb.n_nodes) {
-            const TreeNode &nd = tb.nodes[x];
-            int2 sg = tb.seg[x];
-            if (nd.is_valid && nd.split_feature_id < 0) cnt = (sg.y - sg.x + kPartChunk - 1) / kPartChunk;
-        }
-        int tot;
-        int ex = block_excl_scan(cnt, lds, &tot);
-        if (x < tb.n_nodes) tb.fitem_begin[x] = carry + ex;
-        carry += tot;
-    }
-    if (threadIdx.x == 0) tb.fitem_begin[tb.n_nodes] = carry;
-}
-
-__global__ __launch_bounds__(kBlock) void k_nid_write(TreeBuffers tb) {
-    __shared__ int s_x;
-    const int item = blockIdx.x;
-    if (item >= tb.fitem_begin[tb.n_nodes]) return;
-    if (threadIdx.x == 0) s_x = find_owner(tb.fitem_begin, tb.n_nodes, item);
-    __syncthreads();
-    const int x = s_x;
-    const int level = 31 - __clz(x + 1);
-    const int2 sg = tb.seg[x];
-    const int pb = sg.x + (item - tb.fitem_begin[x]) * kPartChunk;
-    const int pe = min(sg.y, pb + kPartChunk);
-    const int *ridx = tb.ridx[level & 1];
-    for (int pos = pb + threadIdx.x; pos < pe; pos += kBlock) {
-        int row = level == 0 ? pos : ridx[pos];
-        tb.nid[row] = x;
-    }
-}
-
 // ---------------------------------------------------------------------------------- prune
 // Bottom-up, level-parallel form of the reference's Tree::prune_self (src/thundergbm/tree.cu:96-128):
 // a node whose two children are valid leaves and whose gain is below gamma becomes a leaf and its
@@ -1121,136 +1117,302 @@ __global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb, float gamma) {
         if (keep) tb.nodes[i].final_id = carry + ex;
         carry += tot;
     }
-}
-
-// y_pred += lr * weight of the (unpruned) leaf the row ended in (tree_builder.cu:62-74).
-__global__ void k_predict_in_training(int n, const int *__restrict__ nid, const TreeNode *__restrict__ nodes,
-                                      float *__restrict__ yp, float lr) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        int x = nid[i];
-        while (x != -1 && nodes[x].is_pruned) x = nodes[x].parent_index;
-        yp[i] += lr * nodes[x].base_weight;
+    // value a row adds to its prediction when it ended in node i: the weight of the first ancestor that
+    // was not pruned (what predict_in_training finds by climbing, tree_builder.cu:62-74)
+    for (int i = threadIdx.x; i < tb.n_nodes; i += kBlock) {
+        int x = i;
+        while (x != -1 && tb.nodes[x].is_pruned) x = tb.nodes[x].parent_index;
+        tb.leaf_value[i] = x >= 0 ? tb.nodes[x].base_weight : 0.f;
     }
 }
 
-// ------------------------------------------------------------------- fused end of a round
-// For objectives with one tree per round: the in-training prediction update (tree_builder.cu:62-74),
-// the training metric partials (pointwise_metric.cu:13-20 / multiclass_metric.cu:39-44), the next
-// round's gradients (regression_obj.h:130-154) and their block statistics for the next tree's root
-// in one pass over the rows. Same grids, loops and arithmetic as k_predict_in_training,
-// k_metric_partial, k_gradient_pointwise and k_sum_gh, so the results are bit-identical to running
-// those four kernels.
-__global__ __launch_bounds__(kBlock) void k_round_end_fused(int n, int objective, int metric_kind,
-                                                           const int *__restrict__ nid,
-                                                           const TreeNode *__restrict__ nodes,
-                                                           const float *__restrict__ y, float *__restrict__ yp,
-                                                           float lr, GHPair *__restrict__ gh,
-                                                           GradStats *__restrict__ stats,
-                                                           double *__restrict__ metric_out) {
-    __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
-    __shared__ double sd[kWaves];
-    float g = 0, h = 0, gm = 0, hm = 0;
-    double acc = 0;
-    float accf = 0;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        int x = nid[i];
-        while (x != -1 && nodes[x].is_pruned) x = nodes[x].parent_index;
-        float p = yp[i];
-        p += lr * nodes[x].base_weight;
-        yp[i] = p;
-        const float yi = y[i];
-        if (metric_kind == 0) {
-            float e = p - yi;
-            accf += e * e;
-        } else {
-            int k = (1.0 / (1.0 + exp(-(double)p)) > 0.5) ? 1 : 0;
-            acc += (k == yi) ? 1 : 0;
+// -------------------------------------------------------------------------- end of a tree
+// The trainer keeps rows as per-node lists; everything that happens per row after the last split
+// search wants row order: the row -> node map (the reference's ins2node_id), the prediction update
+// (tree_builder.cu:62-74), the training metric (pointwise_metric.cu:13-20, multiclass_metric.cu:39-44)
+// and the next round's gradients (regression_obj.h:130-154). Scattering node ids from the lists into
+// a row-ordered array costs one partial 128-byte line per row, so this kernel goes the other way:
+// a workgroup owns kRowBlock consecutive rows, finds for every node that still holds rows the part of
+// its (ascending) row list that falls into the block by binary search, drops the node ids into LDS
+// and then walks its rows in order with coalesced accesses only.
+//   A node holds rows if it is valid and was not split; a split node of level `lookup_level` still
+// holds the rows of its children (the last level of a tree is never partitioned into lists: nobody
+// reads those lists), each row's child follows from the split feature's bin as in
+// hist_tree_builder_single.cu:986-1011.
+// MODE 0: write the row -> node map only. 1: prediction update of one tree. 2: prediction update,
+// metric partials, next gradients and their block statistics (objectives with one tree per round;
+// same arithmetic and order as k_gradient_pointwise, k_sum_gh and k_metric_partial).
+__device__ __forceinline__ void metric_row(int kind, int n, int K, int i, float yi, const float *__restrict__ yp,
+                                           float p0, double &acc, float &accf);
+
+struct TreeEndArgs {
+    int lookup_level;
+    const float *y;
+    float *yp;
+    float lr;
+    int objective, metric_kind;
+    GHPair *gh;
+    GradStats *stats;
+    double *metric_partial;
+};
+
+constexpr int kEndInline = 8;                        // shorter sub-ranges are handled by the finding thread
+constexpr int kEndListCap = kRowBlock / kEndInline;  // so at most this many longer ones exist per block
+
+// First position p of the ascending run list[sx, sy) with list[p] >= r, given first = list[sx] < r and
+// last = list[sy - 1] >= r. A node's rows are spread roughly evenly over the matrix, so the search
+// starts at the interpolated position, brackets the answer by doubling steps and bisects the bracket:
+// a handful of probes that (unlike a bisection of the whole run) all fall into a few neighbouring lines.
+__device__ int list_lower_bound(const int *__restrict__ list, int sx, int sy, int first, int last, int r) {
+    int g = sx + (int)((long long)(r - first) * (sy - 1 - sx) / (last - first));
+    g = min(max(g, sx + 1), sy - 1);
+    int lo, hi;  // invariant: list[lo] < r <= list[hi]
+    if (list[g] < r) {
+        lo = g;
+        int step = 16;
+        while (lo + step < sy - 1 && list[lo + step] < r) {
+            lo += step;
+            step *= 2;
         }
-        GHPair o;
-        if (objective == OBJ_SQUARE) {
-            o.g = p - yi;
-            o.h = 1.f;
-        } else {
-            float sgm = 1.f / (1.f + expf(-p));
-            o.g = sgm - yi;
-            o.h = fmaxf(sgm * (1.f - sgm), 1e-16f);
+        hi = min(lo + step, sy - 1);
+    } else {
+        hi = g;
+        int step = 16;
+        while (hi - step > sx && list[hi - step] >= r) {
+            hi -= step;
+            step *= 2;
         }
-        gh[i] = o;
-        g += o.g;
-        h += o.h;
-        gm = fmaxf(gm, fabsf(o.g));
-        hm = fmaxf(hm, o.h);
+        lo = max(hi - step, sx);
     }
-    acc += (double)accf;
-    g = wave_sum_f(g);
-    h = wave_sum_f(h);
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        gm = fmaxf(gm, __shfl_xor(gm, d));
-        hm = fmaxf(hm, __shfl_xor(hm, d));
-        acc += __shfl_xor(acc, d);
+    while (hi - lo > 1) {
+        int mid = lo + (hi - lo) / 2;
+        if (list[mid] < r) lo = mid; else hi = mid;
     }
-    if (lane_id() == 0) {
-        sg[wave_id()] = g;
-        sh[wave_id()] = h;
-        mg[wave_id()] = gm;
-        mh[wave_id()] = hm;
-        sd[wave_id()] = acc;
+    return hi;
+}
+
+template <bool SPARSE>
+__device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBins &dbins, const CsrBins &cbins,
+                                            const TreeNode &nd, int row) {
+    bool right;
+    if (SPARSE) {
+        const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
+        right = csr_goes_right(cbins, row, cb, ce, cb + nd.split_bid, nd.default_right);
+    } else {
+        const int b = dbins.col[(size_t)nd.split_feature_id * dbins.col_stride + row];
+        right = (b == kMissingBin) ? nd.default_right : (b >= nd.split_bid);
+    }
+    return right ? nd.rch_index : nd.lch_index;
+}
+
+// bound[b * n_holders + x] = first position of node x's row list whose row is >= b * kRowBlock (b = 0 ..
+// n_blocks), 0 everywhere for nodes that hold no rows: row block b then owns positions [bound[b][x],
+// bound[b + 1][x]) of every list. One thread per entry; neighbouring threads search neighbouring
+// boundaries of the same list.
+__global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb, int lookup_level, int n_blocks) {
+    const int n_holders = (1 << tb.depth) - 1;
+    const size_t total = (size_t)n_holders * (n_blocks + 1);
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+        const int x = (int)(idx / (n_blocks + 1)), b = (int)(idx % (n_blocks + 1));
+        const TreeNode &nd = tb.nodes[x];
+        const int level = 31 - __clz(x + 1);
+        int pos = 0;
+        if (nd.is_valid && (nd.split_feature_id < 0 || level == lookup_level)) {
+            const int2 sg = tb.seg[x];
+            if (sg.y > sg.x) {
+                const long long r = (long long)b * kRowBlock;
+                if (level == 0) {  // the root's list is the identity
+                    pos = (int)min(max(r, (long long)sg.x), (long long)sg.y);
+                } else {
+                    const int *list = tb.ridx[level & 1];
+                    const int first = list[sg.x], last = list[sg.y - 1];
+                    pos = r <= first ? sg.x : (r > last ? sg.y : list_lower_bound(list, sg.x, sg.y, first, last, (int)r));
+                }
+            }
+        }
+        tb.end_bound[(size_t)b * n_holders + x] = pos;
+    }
+}
+
+template <int MODE, bool SPARSE>
+__global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb, DenseBins dbins, CsrBins cbins, TreeEndArgs a) {
+    __shared__ int s_leaf[kRowBlock];
+    __shared__ int s_list[kEndListCap][3];  // node, first and one-past-last list position
+    __shared__ int s_split[kEndListCap];    // -1: the rows stay in the node; else feature | bin << 16 | default_right << 24
+    __shared__ int s_off[kEndListCap];
+    __shared__ int s_scan[kWaves];
+    __shared__ int s_n;
+    __shared__ float s_f[4 * kWaves];
+    __shared__ double s_d[kWaves];
+    const int r0 = blockIdx.x * kRowBlock, r1 = min(tb.n, r0 + kRowBlock);
+    for (int i = threadIdx.x; i < kRowBlock; i += kBlock) s_leaf[i] = -1;
+    if (threadIdx.x == 0) s_n = 0;
+    __syncthreads();
+    const int n_holders = (1 << tb.depth) - 1;  // nodes of the levels that own row lists
+    const int *b_lo = tb.end_bound + (size_t)blockIdx.x * n_holders, *b_hi = b_lo + n_holders;
+    for (int x = threadIdx.x; x < n_holders; x += kBlock) {
+        const int pa = b_lo[x], pb = b_hi[x];
+        if (pb <= pa) continue;
+        const TreeNode &nd = tb.nodes[x];
+        if (pb - pa > kEndInline) {
+            int e = atomicAdd(&s_n, 1);
+            s_list[e][0] = x;
+            s_list[e][1] = pa;
+            s_list[e][2] = pb;
+            s_split[e] = nd.split_feature_id < 0
+                             ? -1
+                             : (nd.split_feature_id | (int)nd.split_bid << 16 | (nd.default_right ? 1 : 0) << 24);
+        } else {
+            const int *list = tb.ridx[(31 - __clz(x + 1)) & 1];
+            for (int p = pa; p < pb; ++p) {
+                const int row = x == 0 ? p : list[p];
+                s_leaf[row - r0] = nd.split_feature_id >= 0 ? end_child_of<SPARSE>(tb, dbins, cbins, nd, row) : x;
+            }
+        }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        GradStats o{0, 0, 0, 0};
-        double s = 0;
-        for (int i = 0; i < kWaves; ++i) {
-            o.g += sg[i];
-            o.h += sh[i];
-            o.gmax = fmaxf(o.gmax, mg[i]);
-            o.hmax = fmaxf(o.hmax, mh[i]);
-            s += sd[i];
+    // The listed sub-ranges are walked as one flat index space spread over all threads (independent
+    // loads in flight instead of one dependent chain per sub-range): s_off = exclusive scan of the lengths.
+    const int n_list = s_n;
+    int total = 0;
+    for (int base = 0; base < n_list; base += kBlock) {
+        const int e = base + threadIdx.x;
+        const int len = e < n_list ? s_list[e][2] - s_list[e][1] : 0;
+        int tot;
+        const int ex = block_excl_scan(len, s_scan, &tot);
+        if (e < n_list) s_off[e] = total + ex;
+        total += tot;
+    }
+    __syncthreads();
+    constexpr int U = 4;
+    for (int j0 = threadIdx.x; j0 < total; j0 += kBlock * U) {
+        int node[U], row[U], split[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int j = j0 + u * kBlock;
+            node[u] = -1;
+            if (j < total) {
+                int lo = 0, hi = n_list;  // last entry with s_off <= j
+                while (hi - lo > 1) {
+                    const int mid = (lo + hi) / 2;
+                    if (s_off[mid] <= j) lo = mid; else hi = mid;
+                }
+                node[u] = s_list[lo][0];
+                split[u] = s_split[lo];
+                const int p = s_list[lo][1] + (j - s_off[lo]);
+                row[u] = node[u] == 0 ? p : tb.ridx[(31 - __clz(node[u] + 1)) & 1][p];
+            }
         }
-        stats[blockIdx.x] = o;
-        metric_out[blockIdx.x] = s;
+        if (SPARSE) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (node[u] < 0) continue;
+                s_leaf[row[u] - r0] =
+                    split[u] >= 0 ? end_child_of<true>(tb, dbins, cbins, tb.nodes[node[u]], row[u]) : node[u];
+            }
+        } else {
+            int bin[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                bin[u] = (node[u] >= 0 && split[u] >= 0)
+                             ? dbins.col[(size_t)(split[u] & 0xffff) * dbins.col_stride + row[u]] : 0;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (node[u] < 0) continue;
+                int leaf = node[u];
+                if (split[u] >= 0) {
+                    const bool right = bin[u] == kMissingBin ? (split[u] >> 24) != 0 : bin[u] >= ((split[u] >> 16) & 0xff);
+                    leaf = 2 * node[u] + (right ? 2 : 1);  // heap order: children of x are 2x + 1 and 2x + 2
+                }
+                s_leaf[row[u] - r0] = leaf;
+            }
+        }
+    }
+    __syncthreads();
+    if (MODE == 0) {
+        for (int i = r0 + threadIdx.x; i < r1; i += kBlock) {
+            const int x = s_leaf[i - r0];
+            if (x >= 0) tb.nid[i] = x;
+        }
+        return;
+    }
+    // rows in order; thread t takes rows t, t + kBlock, ... (the order every row-blocked reduction uses)
+    const float *__restrict__ y = a.y;
+    float *__restrict__ yp = a.yp;
+    GHPair *__restrict__ gh = a.gh;
+    const float *__restrict__ leaf_value = tb.leaf_value;
+    RowStats st;
+    double acc = 0;
+    float accf = 0;
+    for (int i0 = r0 + threadIdx.x; i0 < r1; i0 += kBlock * U) {
+        float p[U], w[U], yi[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * kBlock;
+            ok[u] = i < r1;
+            const int x = ok[u] ? s_leaf[i - r0] : -1;
+            p[u] = ok[u] ? yp[i] : 0.f;
+            yi[u] = (MODE == 2 && ok[u]) ? y[i] : 0.f;
+            w[u] = x >= 0 ? leaf_value[x] : 0.f;
+            ok[u] = ok[u] && (MODE == 2 || x >= 0);
+            if (x >= 0) p[u] += a.lr * w[u];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!ok[u]) continue;
+            const int i = i0 + u * kBlock;
+            yp[i] = p[u];
+            if (MODE == 2) {
+                metric_row(a.metric_kind, tb.n, 1, i, yi[u], yp, p[u], acc, accf);
+                const GHPair o = pointwise_gradient(a.objective, yi[u], p[u]);
+                gh[i] = o;
+                st.add(o);
+            }
+        }
+    }
+    if (MODE == 2) {
+        store_block_stats(st, s_f, a.stats + blockIdx.x);
+        acc += (double)accf;
+        store_block_sum_d(acc, s_d, a.metric_partial + blockIdx.x);
     }
 }
 
 // ---------------------------------------------------------------------------------- metric
 // kind 0: sum of squared errors; 1: correct binary decisions (sigmoid > 0.5 in double, like
 // multiclass_metric.cu:40); 2: correct arg-max decisions (first maximum wins, :17-29).
+__device__ __forceinline__ void metric_row(int kind, int n, int K, int i, float yi, const float *__restrict__ yp,
+                                           float p0, double &acc, float &accf) {
+    if (kind == 0) {
+        float e = p0 - yi;
+        accf += e * e;
+    } else if (kind == 1) {
+        // sigmoid(p) > 0.5 evaluated in double as in the reference; away from zero that is the sign of p
+        int k = fabsf(p0) > 1e-6f ? (p0 > 0.f ? 1 : 0) : ((1.0 / (1.0 + exp(-(double)p0)) > 0.5) ? 1 : 0);
+        acc += (k == yi) ? 1 : 0;
+    } else {
+        int mk = 0;
+        float mp = p0;
+        for (int k = 1; k < K; ++k) {
+            float v = yp[(size_t)k * n + i];
+            if (v > mp) {
+                mp = v;
+                mk = k;
+            }
+        }
+        acc += (mk == yi) ? 1 : 0;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void k_metric_partial(int kind, int n, int K, const float *__restrict__ y,
                                                           const float *__restrict__ yp, double *__restrict__ out) {
     __shared__ double sd[kWaves];
     double acc = 0;
     float accf = 0;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
-        if (kind == 0) {
-            float e = yp[i] - y[i];
-            accf += e * e;
-        } else if (kind == 1) {
-            int k = (1.0 / (1.0 + exp(-(double)yp[i])) > 0.5) ? 1 : 0;
-            acc += (k == y[i]) ? 1 : 0;
-        } else {
-            int mk = 0;
-            float mp = yp[i];
-            for (int k = 1; k < K; ++k) {
-                float v = yp[(size_t)k * n + i];
-                if (v > mp) {
-                    mp = v;
-                    mk = k;
-                }
-            }
-            acc += (mk == y[i]) ? 1 : 0;
-        }
-    }
+    const int r0 = blockIdx.x * kRowBlock, r1 = min(n, r0 + kRowBlock);
+    for (int i = r0 + threadIdx.x; i < r1; i += kBlock) metric_row(kind, n, K, i, y[i], yp, yp[i], acc, accf);
     acc += (double)accf;
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
-    if (lane_id() == 0) sd[wave_id()] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        double s = 0;
-        for (int i = 0; i < kWaves; ++i) s += sd[i];
-        out[blockIdx.x] = s;
-    }
+    store_block_sum_d(acc, sd, out + blockIdx.x);
 }
 
 __global__ __launch_bounds__(kBlock) void k_metric_final(int kind, int n, int n_blocks, const double *__restrict__ in,
@@ -1273,8 +1435,6 @@ __global__ __launch_bounds__(kBlock) void k_metric_final(int kind, int n, int n_
         }
     }
 }
-
-constexpr int kMetricBlocks = 1024;
 
 int grid_for(size_t n, int cap = 4096) {
     size_t b = (n + kBlock - 1) / kBlock;
@@ -1312,16 +1472,8 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
 }
 
-void launch_round_end_fused(hipStream_t s, const TreeBuffers &tb, int objective, int metric_kind, const float *y,
-                            float *yp, float lr, GHPair *gh, double *metric_scratch, float *metric_out) {
-    // grid == the grids of k_sum_gh and k_metric_partial (both min(1024, ceil(n / 256)))
-    k_round_end_fused<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, objective, metric_kind, tb.nid, tb.nodes, y, yp, lr, gh,
-                                                         tb.root_partial, metric_scratch);
-    k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, tb.n_grad_blocks, metric_scratch, metric_out);
-}
-
 void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, bool stats_ready) {
-    if (!stats_ready) k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
+    if (!stats_ready) k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);  // n_grad_blocks == row_blocks(n)
     k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
 }
 
@@ -1410,6 +1562,7 @@ void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float r
 }
 
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level) {
+    if (level == tb.depth - 1) return;  // the last level's children never get row lists (see k_tree_end)
     k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
     const int *cur = tb.ridx[level & 1];
     int *next = tb.ridx[(level + 1) & 1];
@@ -1425,6 +1578,7 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
 }
 
 void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level) {
+    if (level == tb.depth - 1) return;
     k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
     const int *cur = tb.ridx[level & 1];
     int *next = tb.ridx[(level + 1) & 1];
@@ -1439,20 +1593,62 @@ void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &b
     }
 }
 
-void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb) {
-    k_nid_plan<<<1, kBlock, 0, s>>>(tb);
-    k_nid_write<<<tb.max_fitems, kBlock, 0, s>>>(tb);
+template <bool SPARSE>
+static void tree_end_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &d, const CsrBins &c, int mode,
+                            const TreeEndArgs &a) {
+    const int grid = row_blocks(tb.n);
+    if (mode == 0) k_tree_end<0, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
+    else if (mode == 1) k_tree_end<1, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
+    else k_tree_end<2, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
+}
+
+static void tree_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins, int mode,
+                     const TreeEndArgs &a) {
+    const int n_blocks = row_blocks(tb.n);
+    const size_t entries = (size_t)((1 << tb.depth) - 1) * (n_blocks + 1);
+    k_end_bounds<<<grid_for(entries, 8192), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
+    if (tb.sparse) tree_end_launch<true>(s, tb, DenseBins{}, *cbins, mode, a);
+    else tree_end_launch<false>(s, tb, *dbins, CsrBins{}, mode, a);
+}
+
+void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                        int lookup_level) {
+    TreeEndArgs a{};
+    a.lookup_level = lookup_level;
+    tree_end(s, tb, dbins, cbins, 0, a);
+}
+
+void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                                int lookup_level, float *yp_class, float lr) {
+    TreeEndArgs a{};
+    a.lookup_level = lookup_level;
+    a.yp = yp_class;
+    a.lr = lr;
+    tree_end(s, tb, dbins, cbins, 1, a);
+}
+
+void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
+                      int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
+                      GHPair *gh, double *metric_scratch, float *metric_out) {
+    TreeEndArgs a{};
+    a.lookup_level = lookup_level;
+    a.y = y;
+    a.yp = yp;
+    a.lr = lr;
+    a.objective = objective;
+    a.metric_kind = metric_kind;
+    a.gh = gh;
+    a.stats = tb.root_partial;
+    a.metric_partial = metric_scratch;
+    tree_end(s, tb, dbins, cbins, 2, a);
+    k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, row_blocks(tb.n), metric_scratch, metric_out);
 }
 
 void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma) { k_prune<<<1, kBlock, 0, s>>>(tb, gamma); }
 
-void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, float *yp_class, float lr) {
-    k_predict_in_training<<<grid_for(tb.n), kBlock, 0, s>>>(tb.n, tb.nid, tb.nodes, yp_class, lr);
-}
-
 void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
                    float *out) {
-    int blocks = grid_for(n, kMetricBlocks);
+    int blocks = row_blocks(n);  // scratch: one double per block
     k_metric_partial<<<blocks, kBlock, 0, s>>>(kind, n, num_class, y, yp, scratch);
     k_metric_final<<<1, kBlock, 0, s>>>(kind, n, blocks, scratch, out);
 }
