@@ -23,9 +23,11 @@ def T():
 
 @pytest.fixture(autouse=True)
 def _default_layout():
-    os.environ.pop("TGBM_LAYOUT", None)
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD"):
+        os.environ.pop(k, None)
     yield
-    os.environ.pop("TGBM_LAYOUT", None)
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD"):
+        os.environ.pop(k, None)
 
 
 def _ragged(n, F, seed, max_len):
@@ -71,6 +73,8 @@ CASES = {
     "softprob": (1500, 10, 8, "multi:softprob", "multi", dict(depth=3, max_num_bin=32), None),
     "wide_dense_blocks": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense"),
     "wide_sparse": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse"),
+    # the same through the kernel without an LDS head (every value goes to HBM atomics)
+    "wide_sparse_no_head": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse-nohead"),
     "lambda0_mcw5": (900, 6, 6, "reg:linear", "reg", dict(depth=4, max_num_bin=32, lambda_=0.0, min_child_weight=5.0),
                      None),
     "gamma_prunes_all": (600, 5, 5, "reg:linear", "reg", dict(depth=4, max_num_bin=16, gamma=1e9), None),
@@ -85,7 +89,9 @@ def test_edge_case_matches_oracle(T, name):
 def run_case(T, name, seed):
     n, F, max_len, objective, kind, kw, layout = CASES[name]
     if layout:
-        os.environ["TGBM_LAYOUT"] = layout
+        os.environ["TGBM_LAYOUT"] = layout.split("-")[0]
+        if layout.endswith("-nohead"):
+            os.environ["TGBM_CSR_HEAD"] = "0"
     val, rp, col = _ragged(n, F, seed, max_len)
     y = _target(val, rp, col, n, F, seed, kind)
     rounds = 4

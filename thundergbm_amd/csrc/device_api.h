@@ -3,6 +3,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <vector>
+
 #include "common.h"
 
 #define HIP_CHECK(expr)                                                                              \
@@ -17,6 +19,7 @@ namespace tgbm {
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
 constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
 constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
+constexpr int kCsrHeadBins = 4864;  // head slots of the sparse histogram: 2 x 8 bytes each, two workgroups per CU
 constexpr int kRowBlock = 4096;    // rows owned by one workgroup of the row-ordered passes and reductions
 inline int row_blocks(int n) { return n <= 0 ? 1 : (n + kRowBlock - 1) / kRowBlock; }
 
@@ -71,6 +74,12 @@ struct DenseBins {
 struct CsrBins {
     const int *row_ptr = nullptr;  // [n + 1]
     const int *bin = nullptr;      // [nnz] global bin id, ascending within a row
+    // Histogram addressing of the same stored values: the bins of the most frequent features (the
+    // "head", at most kCsrHeadBins of them) are accumulated in LDS. word >= 0: global bin id,
+    // word < 0: ~word is the head slot. nullptr: no head (every value goes to HBM).
+    const int *hist_word = nullptr;  // [nnz]
+    const int *head_bin = nullptr;   // [head_bins] global bin id of every head slot
+    int head_bins = 0;
 };
 
 struct TreeBuffers {
@@ -151,14 +160,16 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
                       size_t col_stride);
+// feat_slot (may be nullptr): first head slot of a feature or -1; then hist_word is written as well
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
-                    const int *cut_row_ptr, int *bin_id);
+                    const int *cut_row_ptr, int *bin_id, const int *feat_slot = nullptr, int *hist_word = nullptr);
 // cut points on device: returns the device arrays through out parameters allocated by the callee
 struct DeviceCuts {
     float *cut_val = nullptr;
     int *cut_row_ptr = nullptr;
     int *cut_fid = nullptr;
     int n_bins = 0;
+    std::vector<long> feature_nnz;  // host: stored values per feature
 };
 DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, const int *d_col, int max_num_bin);
 

@@ -255,12 +255,17 @@ __global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *_
 
 __global__ void k_bin_csr(long nnz, const int *__restrict__ col, const float *__restrict__ val,
                           const float *__restrict__ cut_val, const int *__restrict__ cut_row_ptr,
-                          int *__restrict__ bin_id) {
+                          int *__restrict__ bin_id, const int *__restrict__ feat_slot, int *__restrict__ hist_word) {
     for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (long)gridDim.x * blockDim.x) {
         int f = col[e];
         int cb = cut_row_ptr[f];
         int k = cut_row_ptr[f + 1] - cb;
-        bin_id[e] = cb + local_bin(cut_val + cb, k, val[e]);
+        int local = local_bin(cut_val + cb, k, val[e]);
+        bin_id[e] = cb + local;
+        if (hist_word != nullptr) {
+            int slot = feat_slot[f];
+            hist_word[e] = slot >= 0 ? ~(slot + local) : cb + local;
+        }
     }
 }
 
@@ -280,6 +285,7 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     if (nnz == 0) {
         HIP_CHECK(hipMemsetAsync(out.cut_row_ptr, 0, sizeof(int) * (size_t)(F + 1), s));
         HIP_CHECK(hipStreamSynchronize(s));
+        out.feature_nnz.assign(F, 0);
         return out;
     }
     std::vector<void *> scratch;
@@ -317,8 +323,12 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     k_feature_starts<<<grid_for(F + 1), kBlock, 0, s>>>(sorted, nnz, F, estart);
     k_unique_starts<<<grid_for(F + 1), kBlock, 0, s>>>(estart, uidx, nnz, F, d_total, ustart);
     std::vector<unsigned> h_ustart(F + 1);
+    std::vector<long> h_estart(F + 1);
     HIP_CHECK(hipMemcpyAsync(h_ustart.data(), ustart, sizeof(unsigned) * (size_t)(F + 1), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipMemcpyAsync(h_estart.data(), estart, sizeof(long) * (size_t)(F + 1), hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));
+    out.feature_nnz.resize(F);
+    for (int f = 0; f < F; ++f) out.feature_nnz[f] = h_estart[f + 1] - h_estart[f];
     std::vector<int> h_crp(F + 1, 0);
     for (int f = 0; f < F; ++f) {
         unsigned m = h_ustart[f + 1] - h_ustart[f];
@@ -352,9 +362,9 @@ void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, 
 }
 
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
-                    const int *cut_row_ptr, int *bin_id) {
+                    const int *cut_row_ptr, int *bin_id, const int *feat_slot, int *hist_word) {
     if (nnz == 0) return;
-    k_bin_csr<<<grid_for(nnz), kBlock, 0, s>>>(nnz, col, val, cut_val, cut_row_ptr, bin_id);
+    k_bin_csr<<<grid_for(nnz), kBlock, 0, s>>>(nnz, col, val, cut_val, cut_row_ptr, bin_id, feat_slot, hist_word);
 }
 
 }  // namespace tgbm

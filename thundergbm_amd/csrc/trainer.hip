@@ -108,7 +108,44 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
     if (sparse_) {
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
-        launch_bin_csr(stream_, nnz_, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_bin);
+        // Head of the histogram: the most frequent features whose bins fit the LDS slots. Worth it when
+        // they carry a real share of the stored values (skewed, e.g. Zipf-distributed, feature usage).
+        std::vector<int> feat_slot(F_, -1), head_bin;
+        {
+            std::vector<int> order(F_);
+            for (int f = 0; f < F_; ++f) order[f] = f;
+            std::stable_sort(order.begin(), order.end(),
+                             [&](int a, int b) { return cuts_.feature_nnz[a] > cuts_.feature_nnz[b]; });
+            long head_nnz = 0;
+            for (int f : order) {
+                const int k = h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f];
+                if (k == 0 || cuts_.feature_nnz[f] == 0) break;
+                if ((int)head_bin.size() + k > kCsrHeadBins) continue;
+                feat_slot[f] = (int)head_bin.size();
+                for (int j = 0; j < k; ++j) head_bin.push_back(h_cut_row_ptr_[f] + j);
+                head_nnz += cuts_.feature_nnz[f];
+            }
+            const char *he = std::getenv("TGBM_CSR_HEAD");  // "0" disables the head (tests of both kernels)
+            if (head_nnz * 10 < nnz_ || (he != nullptr && std::string(he) == "0")) head_bin.clear();
+            log_info("sparse histogram head: %zu bins in LDS carry %.1f%% of the stored values", head_bin.size(),
+                     nnz_ > 0 ? 100.0 * (double)head_nnz / (double)nnz_ : 0.0);
+        }
+        if (!head_bin.empty()) {
+            int *d_slot = nullptr;
+            HIP_CHECK(hipMalloc(&d_slot, sizeof(int) * (size_t)F_));
+            upload(stream_, d_slot, feat_slot.data(), (size_t)F_);
+            int *d_word = dalloc<int>((size_t)std::max(nnz_, 1l));
+            int *d_head = dalloc<int>(head_bin.size());
+            upload(stream_, d_head, head_bin.data(), head_bin.size());
+            launch_bin_csr(stream_, nnz_, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_bin, d_slot, d_word);
+            HIP_CHECK(hipStreamSynchronize(stream_));
+            HIP_CHECK(hipFree(d_slot));
+            csr_.hist_word = d_word;
+            csr_.head_bin = d_head;
+            csr_.head_bins = (int)head_bin.size();
+        } else {
+            launch_bin_csr(stream_, nnz_, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_bin);
+        }
         allocs_.push_back(d_row_ptr);  // kept for the whole session
         csr_.row_ptr = d_row_ptr;
         csr_.bin = d_bin;

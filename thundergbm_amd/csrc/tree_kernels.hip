@@ -535,6 +535,84 @@ __global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb, CsrBins bin
     }
 }
 
+// The same with the bins of the most frequent features ("head") accumulated in LDS: with a skewed feature
+// distribution most stored values hit a few thousand bins, and global atomics on those serialise (the
+// root level of a 2M x 100k Zipf matrix spent 10 ms there). Every head slot is a pair of 64-bit sums, so
+// no drain is needed; at the end the workgroup adds its non-zero slots to the node's histogram in HBM.
+// 1024 threads (16 wavefronts, one row each, the next row's header prefetched), two workgroups per CU.
+template <bool DIRECT>
+__global__ __launch_bounds__(TGBM_HIST_BLOCK) __attribute__((amdgpu_waves_per_eu(8)))
+void k_hist_csr_head(TreeBuffers tb, CsrBins bins, const GHPair *__restrict__ gh, const int *__restrict__ ridx,
+                     longlong2 *__restrict__ cur_q, int n_pairs, int level) {
+    extern __shared__ unsigned long long lds[];  // [2 * head_bins]: gradient, hessian of every slot
+    __shared__ int s_info[3];
+    const LevelCtl c = tb.ctl[level];
+    const int item = blockIdx.x;
+    if (item >= c.n_hitems) return;
+    if (threadIdx.x == 0) {
+        int p = find_owner(tb.hpair_begin, n_pairs, item);
+        int node = tb.hpair_built[p];
+        int2 sg = tb.seg[node];
+        int b = sg.x + (item - tb.hpair_begin[p]) * c.hchunk;
+        s_info[0] = b;
+        s_info[1] = min(sg.y, b + c.hchunk);
+        s_info[2] = node - ((1 << level) - 1);
+    }
+    for (int i = threadIdx.x; i < 2 * bins.head_bins; i += TGBM_HIST_BLOCK) lds[i] = 0ull;
+    __syncthreads();
+    const int begin = s_info[0], end = s_info[1];
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(cur_q + (size_t)s_info[2] * tb.n_bins);
+    const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    constexpr int NW = TGBM_HIST_BLOCK / 64;
+    int pos = begin + w;
+    GHPair s{0, 0};
+    int e0 = 0, e1 = 0;
+    if (pos < end) {
+        const int r = DIRECT ? pos : ridx[pos];
+        s = gh[r];
+        e0 = bins.row_ptr[r];
+        e1 = bins.row_ptr[r + 1];
+    }
+    while (pos < end) {
+        const int npos = pos + NW;
+        GHPair ns{0, 0};
+        int ne0 = 0, ne1 = 0;
+        if (npos < end) {  // requested before this row's atomics
+            const int r = DIRECT ? npos : ridx[npos];
+            ns = gh[r];
+            ne0 = bins.row_ptr[r];
+            ne1 = bins.row_ptr[r + 1];
+        }
+        const unsigned long long gq = (unsigned long long)__float2ll_rn(s.g * scale_g);
+        const unsigned long long hq = (unsigned long long)__float2ll_rn(s.h * scale_h);
+        for (int e = e0 + lane; e < e1; e += 64) {
+            const int word = bins.hist_word[e];
+            if (word < 0) {
+                const int slot = ~word;
+                atomicAdd(lds + 2 * slot, gq);
+                atomicAdd(lds + 2 * slot + 1, hq);
+            } else {
+                atomicAdd(h + 2 * (size_t)word, gq);
+                atomicAdd(h + 2 * (size_t)word + 1, hq);
+            }
+        }
+        pos = npos;
+        s = ns;
+        e0 = ne0;
+        e1 = ne1;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < bins.head_bins; i += TGBM_HIST_BLOCK) {
+        const unsigned long long g = lds[2 * i], hh = lds[2 * i + 1];
+        if ((g | hh) != 0ull) {
+            const size_t b = (size_t)bins.head_bin[i];
+            atomicAdd(h + 2 * b, g);
+            atomicAdd(h + 2 * b + 1, hh);
+        }
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void k_hist_sub_csr(longlong2 *__restrict__ cur_q,
                                                         const longlong2 *__restrict__ prev_q,
                                                         const int *__restrict__ hpair_built, int level, int n_bins) {
@@ -996,7 +1074,13 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb, int l
         tb.hpair_built[x_in] = built;
     }
     const int total_rows = block_sum(rows_sum, lds);
-    int chunk = (total_rows + tb.target_hitems - 1) / tb.target_hitems;
+    int n_built = 0;
+    for (int x_in = threadIdx.x; x_in < nl; x_in += kBlock) n_built += tb.hpair_built[x_in] >= 0 ? 1 : 0;
+    n_built = block_sum(n_built, lds);
+    // every built node adds up to one partly filled item: size the items so that their number stays
+    // within target_hitems (= the workgroups the chip holds at once; one more would run as a second round)
+    const int room = max(tb.target_hitems / 4, tb.target_hitems - n_built);
+    int chunk = (total_rows + room - 1) / room;
     chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
     carry = 0;
     for (int base = 0; base < nl; base += kBlock) {
@@ -1543,13 +1627,28 @@ void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, 
     const int zgrid = std::min(1024, (tb.n_bins + kBlock - 1) / kBlock);
     longlong2 *cur = tb.hist_q[level & 1];
     k_hist_zero_built<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hpair_built, level, tb.n_bins);
-    if (level == 0) {
-        k_hist_csr<true><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, nullptr, cur, n_pairs, level);
+    const size_t lds = (size_t)bins.head_bins * 2 * sizeof(unsigned long long);
+    if (bins.hist_word != nullptr && lds > 64 * 1024) {
+        static size_t opted = 0;  // more than the default dynamic LDS window: opt in once
+        if (lds > opted) {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_csr_head<true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_hist_csr_head<false>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            opted = lds;
+        }
+    }
+    const int *list = level == 0 ? nullptr : tb.ridx[level & 1];
+    if (bins.hist_word != nullptr) {
+        if (level == 0) k_hist_csr_head<true><<<tb.max_hitems, kHistBlock, lds, s>>>(tb, bins, gh, list, cur, n_pairs, level);
+        else k_hist_csr_head<false><<<tb.max_hitems, kHistBlock, lds, s>>>(tb, bins, gh, list, cur, n_pairs, level);
     } else {
-        k_hist_csr<false><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, tb.ridx[level & 1], cur, n_pairs, level);
+        if (level == 0) k_hist_csr<true><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, list, cur, n_pairs, level);
+        else k_hist_csr<false><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, list, cur, n_pairs, level);
+    }
+    if (level > 0)
         k_hist_sub_csr<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hist_q[(level + 1) & 1], tb.hpair_built, level,
                                                               tb.n_bins);
-    }
 }
 
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
