@@ -95,7 +95,8 @@ void tgbm_trainer_finish_tree(tgbm_trainer *t, int class_id);
 float tgbm_trainer_metric(tgbm_trainer *t);
 
 /* Integer facts: n, n_features, n_bins, num_class, tree_per_rounds, n_nodes, dense_W,
- * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems. */
+ * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems, n_sets (class trees
+ * of a round built by common launches). */
 int tgbm_trainer_info(tgbm_trainer *t, const char *key);
 float tgbm_trainer_base_score(tgbm_trainer *t);
 

@@ -23,10 +23,10 @@ def T():
 
 @pytest.fixture(autouse=True)
 def _default_layout():
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES"):
         os.environ.pop(k, None)
     yield
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES"):
         os.environ.pop(k, None)
 
 
@@ -170,6 +170,41 @@ def test_one_boost_call_equals_round_by_round(T, objective, kind):
     assert np.array_equal(g_next, b.gh())
     a.close()
     b.close()
+
+
+@pytest.mark.parametrize("layout", ["dense", "sparse"])
+def test_class_trees_built_together_equal_one_by_one(T, layout):
+    """The class trees of a softmax round are built by common launches (one buffer set per class); with
+    TGBM_BATCH_CLASSES=0 they are built one after the other. Same bits either way, also through the
+    stage-wise calls."""
+    os.environ["TGBM_LAYOUT"] = layout
+    n, F = 5000, 12
+    val, rp, col = _ragged(n, F, 11, F)
+    y = _target(val, rp, col, n, F, 11, "multi")
+    kw = dict(objective="multi:softprob", n_trees=3, depth=5, max_num_bin=32, learning_rate=0.4)
+    a = T.Session(val, rp, col, y, **kw)
+    assert a.info("n_sets") == 4
+    a.boost(3)
+    os.environ["TGBM_BATCH_CLASSES"] = "0"
+    b = T.Session(val, rp, col, y, **kw)
+    assert b.info("n_sets") == 1
+    b.boost(3)
+    os.environ.pop("TGBM_BATCH_CLASSES")
+    c = T.Session(val, rp, col, y, **kw)
+    for _ in range(3):
+        c.gradient()
+        for k in range(4):
+            c.tree_init(k)
+            for level in range(5):
+                c.find_split(level)
+                c.partition(level)
+            c.finish_tree(k)
+    ma = a.model().tobytes()
+    assert ma == b.model().tobytes() and ma == c.model().tobytes()
+    assert np.array_equal(a.y_pred(), b.y_pred()) and np.array_equal(a.y_pred(), c.y_pred())
+    assert np.array_equal(a.metric_log(), b.metric_log())
+    for s in (a, b, c):
+        s.close()
 
 
 def test_predict_transforms_through_the_c_abi(T):

@@ -111,8 +111,6 @@ struct TreeBuffers {
     // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1]) (whole features)
     const int *pack_begin = nullptr;
     int n_packs = 0;
-    int *fitem_begin = nullptr;    // [n_nodes + 1] work items of the row -> node rebuild
-    int max_fitems = 0;
     const int *cut_row_ptr = nullptr;
     const int *cut_fid = nullptr;
     const float *cut_val = nullptr;
@@ -120,6 +118,46 @@ struct TreeBuffers {
     const int *blk_bin_begin = nullptr;  // [n_blocks + 1] first global bin of every block
     const int *feat_lds_off = nullptr;   // [n_blocks * W] bin offset of a feature inside its block
     int max_block_bins = 0;
+    // Every per-tree array above is allocated n_sets times back to back (one set per class tree of a
+    // boosting round, so that the trees of a round can be built by the same launches, class = blockIdx.z).
+    int n_sets = 1;
+    int max_level_nodes = 0;
+    size_t n_end_bound = 0, n_partial = 0;
+
+    // Row list / histogram buffer of a level (selected without indexing an array member dynamically: a
+    // kernel's local copy of this struct would otherwise be placed in scratch memory).
+    __host__ __device__ int *list(int level) const { return (level & 1) ? ridx[1] : ridx[0]; }
+    __host__ __device__ longlong2 *hist(int level) const { return (level & 1) ? hist_q[1] : hist_q[0]; }
+
+    // The buffers of set k (k = 0: this object itself).
+    __host__ __device__ TreeBuffers for_class(int k) const {
+        TreeBuffers t = *this;
+        if (k == 0) return t;
+        const size_t K = (size_t)k;
+        t.nodes += K * n_nodes;
+        t.seg += K * n_nodes;
+        t.nid += K * n;
+        t.ridx[0] += K * n;
+        t.ridx[1] += K * n;
+        t.goes_right += K * ((size_t)n + 4);
+        t.hist_q[0] += K * max_level_nodes * n_bins;
+        t.hist_q[1] += K * max_level_nodes * n_bins;
+        t.partial += K * n_partial;
+        t.quant += K;
+        t.leaf_value += K * n_nodes;
+        t.end_bound += K * n_end_bound;
+        t.hpair_begin += K * (max_level_nodes + 1);
+        t.hpair_built += K * max_level_nodes;
+        t.pitem_begin += K * (max_level_nodes + 1);
+        t.pitem_nleft += K * ((size_t)max_pitems + 1);
+        t.pitem_loff += K * ((size_t)max_pitems + 1);
+        t.node_nleft += K * max_level_nodes;
+        t.ctl += K * (depth + 2);
+        t.sp += K * max_level_nodes;
+        t.cand += K * max_level_nodes * n_packs;
+        t.root_partial += K * n_grad_blocks;
+        return t;
+    }
 };
 
 // objective codes
@@ -127,28 +165,32 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
+// Tree-building launchers: `tb` is the first buffer set, `n_class` consecutive sets (the class trees of one
+// round) are served by one launch; gradient / prediction pointers address the first of those classes.
 // stats_ready: tb.root_partial already holds the block statistics of gh_class (fused round end)
 void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda,
-                      bool stats_ready = false);
-void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level);
-void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level);
-void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level);
-void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level);
-void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda);
-void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda);
-void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level);
+                      bool stats_ready = false, int n_class = 1);
+void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level,
+                       int n_class = 1);
+void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class = 1);
+void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
+                     int n_class = 1);
+void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class = 1);
+void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class = 1);
+void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class = 1);
 // Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level
 // whose split nodes still hold their children's rows (-1: none).
 void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                         int lookup_level);
 void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
-                                int lookup_level, float *yp_class, float lr);
+                                int lookup_level, float *yp_class, float lr, int n_class = 1);
 // prediction update + metric + next gradients + their block statistics (tb.root_partial); metric_scratch
 // holds row_blocks(n) doubles
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                       int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
                       GHPair *gh, double *metric_scratch, float *metric_out);
-void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma);
+void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma, int n_class = 1);
 // scratch: row_blocks(n) doubles
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);

@@ -51,7 +51,12 @@ class Trainer {
     HistProfile profile();
 
    private:
-    void build_level_hist(int level, const GHPair *gh);
+    TreeBuffers set_of(int k) const;
+    void find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level, int n_class);
+    void partition_sets(const TreeBuffers &tb, int level, int n_class);
+    void build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class);
+    void build_round_together();
+    void log_plan(const TreeBuffers &tb);
     void alloc_tree_buffers();
     template <typename T>
     T *dalloc(size_t count);
@@ -73,7 +78,8 @@ class Trainer {
     DenseBins bins_;
     bool sparse_ = false;
     CsrBins csr_;
-    TreeBuffers tb_;
+    TreeBuffers tb_;      // buffer set 0; set k = tb_.for_class(k)
+    int n_sets_ = 1;      // tree_per_rounds when the class trees of a round are built together, else 1
     // model
     TreeNode *d_model_ = nullptr;
     int trees_built_ = 0, rounds_done_ = 0, model_cap_trees_ = 0;

@@ -233,32 +233,45 @@ void Trainer::alloc_tree_buffers() {
     tb.n_nodes = (1 << (depth + 1)) - 1;
     const int max_level_nodes = 1 << (depth - 1 > 0 ? depth - 1 : 0);
     const int max_pairs = std::max(1, max_level_nodes / 2);
-    tb.nodes = dalloc<TreeNode>(tb.n_nodes);
-    tb.seg = dalloc<int2>(tb.n_nodes);
-    tb.nid = dalloc<int>(n_);
-    tb.ridx[0] = dalloc<int>(n_);
-    tb.ridx[1] = dalloc<int>(n_);
-    tb.goes_right = dalloc<uint8_t>((size_t)n_ + 4);
+    tb.max_level_nodes = max_level_nodes;
     tb.target_hitems = std::min(512, std::max(4, 512 / bins_.n_blocks));  // ~2 resident workgroups per CU
     tb.max_hitems = tb.target_hitems + max_pairs + 1;
-    tb.hist_q[0] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
-    tb.hist_q[1] = dalloc<longlong2>((size_t)max_level_nodes * n_bins_);
-    tb.partial = dalloc<longlong2>(sparse_ ? 1 : (size_t)tb.max_hitems * n_bins_);
-    tb.quant = dalloc<QuantCtl>(1);
     tb.max_pitems = n_ / kPartChunk + max_level_nodes + 1;
-    // the planning kernel of the last level also writes the (unused) plan of level `depth`
-    tb.hpair_begin = dalloc<int>((size_t)max_level_nodes + 1);
-    tb.leaf_value = dalloc<float>((size_t)tb.n_nodes);
-    tb.end_bound = dalloc<int>(((size_t)row_blocks(n_) + 1) * (((size_t)1 << depth) - 1));
-    tb.hpair_built = dalloc<int>((size_t)max_level_nodes);
-    tb.pitem_begin = dalloc<int>((size_t)max_level_nodes + 1);
-    tb.pitem_nleft = dalloc<int>((size_t)tb.max_pitems + 1);
-    tb.pitem_loff = dalloc<int>((size_t)tb.max_pitems + 1);
-    tb.node_nleft = dalloc<int>((size_t)max_level_nodes);
-    tb.ctl = dalloc<LevelCtl>((size_t)depth + 2);
-    tb.sp = dalloc<SplitPoint>((size_t)max_level_nodes);
+    tb.n_partial = sparse_ ? 1 : (size_t)tb.max_hitems * n_bins_;
+    tb.n_end_bound = ((size_t)row_blocks(n_) + 1) * (((size_t)1 << depth) - 1);
     tb.n_grad_blocks = row_blocks(n_);
-    tb.root_partial = dalloc<GradStats>((size_t)tb.n_grad_blocks);
+    // One set of buffers per class tree of a round when that fits comfortably: the trees of a round are
+    // independent and are then built together (class = blockIdx.z of every launch).
+    const int K = param_.tree_per_rounds;
+    const size_t set_bytes = (size_t)n_ * 13 + ((size_t)2 * max_level_nodes * n_bins_ + tb.n_partial) * sizeof(longlong2) +
+                             tb.n_end_bound * sizeof(int);
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    const char *be = std::getenv("TGBM_BATCH_CLASSES");  // "0": build the trees of a round one after the other
+    n_sets_ = (K > 1 && set_bytes * K < free_b / 2 && !(be != nullptr && std::string(be) == "0")) ? K : 1;
+    tb.n_sets = n_sets_;
+    const size_t S = (size_t)n_sets_;
+    tb.nodes = dalloc<TreeNode>(S * tb.n_nodes);
+    tb.seg = dalloc<int2>(S * tb.n_nodes);
+    tb.nid = dalloc<int>(S * n_);
+    tb.ridx[0] = dalloc<int>(S * n_);
+    tb.ridx[1] = dalloc<int>(S * n_);
+    tb.goes_right = dalloc<uint8_t>(S * ((size_t)n_ + 4));
+    tb.hist_q[0] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+    tb.hist_q[1] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+    tb.partial = dalloc<longlong2>(S * tb.n_partial);
+    tb.quant = dalloc<QuantCtl>(S);
+    tb.hpair_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
+    tb.leaf_value = dalloc<float>(S * tb.n_nodes);
+    tb.end_bound = dalloc<int>(S * tb.n_end_bound);
+    tb.hpair_built = dalloc<int>(S * max_level_nodes);
+    tb.pitem_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
+    tb.pitem_nleft = dalloc<int>(S * ((size_t)tb.max_pitems + 1));
+    tb.pitem_loff = dalloc<int>(S * ((size_t)tb.max_pitems + 1));
+    tb.node_nleft = dalloc<int>(S * max_level_nodes);
+    tb.ctl = dalloc<LevelCtl>(S * ((size_t)depth + 2));
+    tb.sp = dalloc<SplitPoint>(S * max_level_nodes);
+    tb.root_partial = dalloc<GradStats>(S * tb.n_grad_blocks);
     tb.cut_row_ptr = cuts_.cut_row_ptr;
     tb.cut_fid = cuts_.cut_fid;
     tb.cut_val = cuts_.cut_val;
@@ -282,9 +295,7 @@ void Trainer::alloc_tree_buffers() {
     int *d_pack = dalloc<int>(pack_begin.size());
     upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
     tb.pack_begin = d_pack;
-    tb.cand = dalloc<SplitCand>((size_t)max_level_nodes * tb.n_packs);
-    tb.fitem_begin = dalloc<int>((size_t)tb.n_nodes + 1);
-    tb.max_fitems = n_ / kPartChunk + tb.n_nodes + 1;
+    tb.cand = dalloc<SplitCand>(S * max_level_nodes * tb.n_packs);
 
     // dense block tables
     const int W = bins_.W, nb = bins_.n_blocks;
@@ -331,15 +342,19 @@ void Trainer::compute_gradient() {
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
 }
 
+// Buffer set of class tree k, and the first set with the item target of a whole round built at once.
+TreeBuffers Trainer::set_of(int k) const { return tb_.for_class(n_sets_ > 1 ? k : 0); }
+
 void Trainer::tree_init(int k) {
     cur_class_ = k;
-    launch_tree_init(stream_, tb_, d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
+    launch_tree_init(stream_, set_of(k), d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
     next_round_ready_ = false;
     lookup_level_ = -1;
 }
 
-void Trainer::find_split(int level) {
-    const GHPair *gh = d_gh_ + (size_t)cur_class_ * n_;
+void Trainer::find_split(int level) { find_split_sets(set_of(cur_class_), d_gh_ + (size_t)cur_class_ * n_, level, 1); }
+
+void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level, int n_class) {
     if (profiling_) {
         HistEvent ev;
         HIP_CHECK(hipEventCreate(&ev.start));
@@ -347,56 +362,85 @@ void Trainer::find_split(int level) {
         ev.level = level;
         ev.tree = trees_built_;
         HIP_CHECK(hipEventRecord(ev.start, stream_));
-        build_level_hist(level, gh);
+        build_level_hist(tb, level, gh, n_class);
         HIP_CHECK(hipEventRecord(ev.stop, stream_));
         events_.push_back(ev);
     } else {
-        build_level_hist(level, gh);
+        build_level_hist(tb, level, gh, n_class);
     }
-    if (!sparse_) launch_hist_merge(stream_, tb_, level);
-    launch_eval_split(stream_, tb_, level, param_.min_child_weight, param_.lambda);
-    launch_best_update(stream_, tb_, level, param_.rt_eps, param_.lambda);
+    if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
+    launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class);
+    launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
 }
 
-void Trainer::build_level_hist(int level, const GHPair *gh) {
+void Trainer::build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class) {
     if (sparse_)
-        launch_hist_csr(stream_, tb_, csr_, gh, level);
+        launch_hist_csr(stream_, tb, csr_, gh, level, n_class);
     else
-        launch_hist_dense(stream_, tb_, bins_, gh, level);
+        launch_hist_dense(stream_, tb, bins_, gh, level, n_class);
 }
 
-void Trainer::partition(int level) {
+void Trainer::partition(int level) { partition_sets(set_of(cur_class_), level, 1); }
+
+void Trainer::partition_sets(const TreeBuffers &tb, int level, int n_class) {
     // the last level is not partitioned: its split nodes keep their rows until the tree's final pass
     if (level < param_.depth - 1) lookup_level_ = -1;
     if (sparse_)
-        launch_partition_csr(stream_, tb_, csr_, level);
+        launch_partition_csr(stream_, tb, csr_, level, n_class);
     else
-        launch_partition_dense(stream_, tb_, bins_, level);
+        launch_partition_dense(stream_, tb, bins_, level, n_class);
+}
+
+void Trainer::log_plan(const TreeBuffers &tb) {
+    size_t off = ctl_log_.size();
+    ctl_log_.resize(off + param_.depth + 1);
+    HIP_CHECK(hipMemcpyAsync(ctl_log_.data() + off, tb.ctl, sizeof(LevelCtl) * (size_t)(param_.depth + 1),
+                             hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
 }
 
 void Trainer::finish_tree(int k, bool fuse_round_end) {
-    launch_prune(stream_, tb_, param_.gamma);
+    const TreeBuffers tb = set_of(k);
+    launch_prune(stream_, tb, param_.gamma);
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
-        launch_round_end(stream_, tb_, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
+        launch_round_end(stream_, tb, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
                          param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_);
         next_round_ready_ = true;
     } else {
-        launch_predict_in_training(stream_, tb_, &bins_, &csr_, lookup_level_, d_yp_ + (size_t)k * n_,
+        launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_ + (size_t)k * n_,
                                    param_.learning_rate);
     }
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
-    HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb_.n_nodes, tb_.nodes,
-                             sizeof(TreeNode) * (size_t)tb_.n_nodes, hipMemcpyDeviceToDevice, stream_));
-    if (profiling_) {
-        size_t off = ctl_log_.size();
-        ctl_log_.resize(off + param_.depth + 1);
-        HIP_CHECK(hipMemcpyAsync(ctl_log_.data() + off, tb_.ctl, sizeof(LevelCtl) * (size_t)(param_.depth + 1),
-                                 hipMemcpyDeviceToHost, stream_));
-        HIP_CHECK(hipStreamSynchronize(stream_));
-    }
+    HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
+                             sizeof(TreeNode) * (size_t)tb.n_nodes, hipMemcpyDeviceToDevice, stream_));
+    if (profiling_) log_plan(tb);
     ++trees_built_;
+}
+
+// All class trees of a round through the same launches (class = blockIdx.z): the trees are independent
+// given the round's gradients, and one launch over K small trees costs about what one tree costs.
+void Trainer::build_round_together() {
+    const int K = param_.tree_per_rounds;
+    TreeBuffers tb = tb_;
+    // the K classes share the chip: size every class's histogram items for its share of the workgroup slots
+    tb.target_hitems = std::max(4, tb_.target_hitems / K);
+    launch_tree_init(stream_, tb, d_gh_, param_.lambda, false, K);
+    lookup_level_ = -1;
+    for (int level = 0; level < param_.depth; ++level) {
+        find_split_sets(tb, d_gh_, level, K);
+        partition_sets(tb, level, K);
+    }
+    launch_prune(stream_, tb, param_.gamma, K);
+    launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_, param_.learning_rate, K);
+    TGBM_CHECK(trees_built_ + K <= model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
+    HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
+                             sizeof(TreeNode) * (size_t)tb.n_nodes * K, hipMemcpyDeviceToDevice, stream_));
+    if (profiling_)
+        for (int k = 0; k < K; ++k) log_plan(tb.for_class(k));
+    trees_built_ += K;
+    cur_class_ = K - 1;
 }
 
 float Trainer::metric() {
@@ -414,16 +458,20 @@ void Trainer::boost(int rounds) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
         const bool fuse = objective_ != OBJ_SOFTMAX && param_.tree_per_rounds == 1;
         if (!next_round_ready_) compute_gradient();
-        for (int k = 0; k < param_.tree_per_rounds; ++k) {
-            tree_init(k);
-            // The reference leaves the level loop when no row sits in a node that was split
-            // (tree_builder.cu:174-181). Running the remaining levels is a no-op on every output
-            // (no valid node, no work item), so the loop is not cut short and needs no readback.
-            for (int level = 0; level < param_.depth; ++level) {
-                find_split(level);
-                partition(level);
+        if (n_sets_ > 1) {
+            build_round_together();
+        } else {
+            for (int k = 0; k < param_.tree_per_rounds; ++k) {
+                tree_init(k);
+                // The reference leaves the level loop when no row sits in a node that was split
+                // (tree_builder.cu:174-181). Running the remaining levels is a no-op on every output
+                // (no valid node, no work item), so the loop is not cut short and needs no readback.
+                for (int level = 0; level < param_.depth; ++level) {
+                    find_split(level);
+                    partition(level);
+                }
+                finish_tree(k, fuse);
             }
-            finish_tree(k, fuse);
         }
         float *slot = d_metric_ + rounds_done_;
         if (!fuse) launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
@@ -499,6 +547,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "num_class") return param_.num_class;
     if (key == "tree_per_rounds") return param_.tree_per_rounds;
     if (key == "n_nodes") return tb_.n_nodes;
+    if (key == "n_sets") return n_sets_;
     if (key == "sparse") return sparse_ ? 1 : 0;
     if (key == "dense_W") return bins_.W;
     if (key == "dense_blocks") return bins_.n_blocks;
@@ -516,6 +565,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     const void *src = nullptr;
     size_t bytes = 0;
     const int max_level_nodes = 1 << (param_.depth - 1 > 0 ? param_.depth - 1 : 0);
+    const TreeBuffers cur = set_of(cur_class_);  // per-tree buffers: those of the class tree built last
     if (name == "cut_val") src = cuts_.cut_val, bytes = sizeof(float) * (size_t)n_bins_;
     else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
@@ -523,22 +573,22 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
         // the map is kept as row lists; materialise it on demand
-        launch_nid_rebuild(stream_, tb_, &bins_, &csr_, lookup_level_);
+        launch_nid_rebuild(stream_, cur, &bins_, &csr_, lookup_level_);
         sync();
-        src = tb_.nid, bytes = sizeof(int) * (size_t)n_;
+        src = cur.nid, bytes = sizeof(int) * (size_t)n_;
     }
     else if (name == "gh") src = d_gh_, bytes = sizeof(GHPair) * (size_t)param_.num_class * n_;
     else if (name == "y_pred") src = d_yp_, bytes = sizeof(float) * (size_t)n_yp_;
     else if (name == "y") src = d_y_, bytes = sizeof(float) * (size_t)n_;
-    else if (name == "nodes") src = tb_.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
-    else if (name == "sp") src = tb_.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
-    else if (name == "hist_q0") src = tb_.hist_q[0], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
-    else if (name == "hist_q1") src = tb_.hist_q[1], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
-    else if (name == "quant") src = tb_.quant, bytes = sizeof(QuantCtl);
-    else if (name == "ctl") src = tb_.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
-    else if (name == "seg") src = tb_.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;
-    else if (name == "ridx0") src = tb_.ridx[0], bytes = sizeof(int) * (size_t)n_;
-    else if (name == "ridx1") src = tb_.ridx[1], bytes = sizeof(int) * (size_t)n_;
+    else if (name == "nodes") src = cur.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
+    else if (name == "sp") src = cur.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
+    else if (name == "hist_q0") src = cur.hist_q[0], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "hist_q1") src = cur.hist_q[1], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "quant") src = cur.quant, bytes = sizeof(QuantCtl);
+    else if (name == "ctl") src = cur.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
+    else if (name == "seg") src = cur.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;
+    else if (name == "ridx0") src = cur.ridx[0], bytes = sizeof(int) * (size_t)n_;
+    else if (name == "ridx1") src = cur.ridx[1], bytes = sizeof(int) * (size_t)n_;
     else if (name == "model") src = d_model_, bytes = sizeof(TreeNode) * (size_t)trees_built_ * tb_.n_nodes;
     else if (name == "metric_log") src = d_metric_, bytes = sizeof(float) * (size_t)rounds_done_;
     else fatal("unknown buffer %s", name.c_str());

@@ -193,8 +193,11 @@ __device__ void store_block_sum_d(double acc, double *lds, double *out) {
 }
 
 // Block sums of (g,h) and block maxima of |g|, h for one tree.
+// Class trees of a round: blockIdx.z selects the class (gradients and outputs are class-major).
 __global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out) {
     __shared__ float lds[4 * kWaves];
+    gh += (size_t)blockIdx.z * n;
+    out += (size_t)blockIdx.z * gridDim.x;
     const int r0 = blockIdx.x * kRowBlock, r1 = min(n, r0 + kRowBlock);
     RowStats st;
     for (int i = r0 + threadIdx.x; i < r1; i += kBlock) st.add(gh[i]);
@@ -214,9 +217,10 @@ __device__ float pow2_scale(float vmax, int rows, float limit) {
 // ------------------------------------------------------------------------------- tree init
 // Node array initialisation of the reference's Tree::init2 (src/thundergbm/tree.cu:8-39), root sum
 // from the block partials, root segment and the histogram plan of level 0. One workgroup.
-__global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const GradStats *__restrict__ block_sums,
-                                                     float lambda) {
+__global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float lambda) {
     __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const GradStats *__restrict__ block_sums = tb.root_partial;
     const int nn = tb.n_nodes;
     for (int i = threadIdx.x; i < nn; i += kBlock) {
         TreeNode nd;
@@ -328,18 +332,21 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb, const Grad
 // the pairs costs what the gathers save.)
 template <int LPR, bool DIRECT, int BLK, int SLOTS>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
-void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
-                                                    const int *__restrict__ ridx, const int2 *__restrict__ seg,
-                                                    const int *__restrict__ hpair_begin,
-                                                    const int *__restrict__ hpair_built, int n_pairs,
-                                                    const LevelCtl *__restrict__ ctl,
-                                                    const QuantCtl *__restrict__ quant,
-                                                    const int *__restrict__ blk_bin_begin,
-                                                    const int *__restrict__ feat_lds_off,
-                                                    longlong2 *__restrict__ partial, int n_bins) {
+void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
     __shared__ int s_range[2];
-    const LevelCtl c = *ctl;
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    gh += (size_t)blockIdx.z * tb.n;
+    const int *__restrict__ ridx = tb.list(level);
+    const int2 *__restrict__ seg = tb.seg;
+    const int *__restrict__ hpair_begin = tb.hpair_begin;
+    const int *__restrict__ hpair_built = tb.hpair_built;
+    const QuantCtl *__restrict__ quant = tb.quant;
+    const int *__restrict__ blk_bin_begin = tb.blk_bin_begin;
+    const int *__restrict__ feat_lds_off = tb.feat_lds_off;
+    longlong2 *__restrict__ partial = tb.partial;
+    const int n_bins = tb.n_bins;
+    const LevelCtl c = tb.ctl[level];
     const int item = blockIdx.x;
     if (item >= c.n_hitems) return;
     const int fb = blockIdx.y;
@@ -446,12 +453,15 @@ void k_hist_dense(DenseBins bins, const GHPair *__restrict__ gh,
 constexpr int kMergeBins = 32;
 constexpr int kMergeGroups = kBlock / kMergeBins;
 
-__global__ __launch_bounds__(kBlock) void k_hist_merge(const longlong2 *__restrict__ partial,
-                                                      longlong2 *__restrict__ cur_q,
-                                                      const longlong2 *__restrict__ prev_q,
-                                                      const int *__restrict__ hpair_begin,
-                                                      const int *__restrict__ hpair_built, int level, int n_bins) {
+__global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int level) {
     __shared__ long long s_g[kMergeGroups][kMergeBins], s_h[kMergeGroups][kMergeBins];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const longlong2 *__restrict__ partial = tb.partial;
+    longlong2 *__restrict__ cur_q = tb.hist(level);
+    const longlong2 *__restrict__ prev_q = tb.hist(level + 1);
+    const int *__restrict__ hpair_begin = tb.hpair_begin;
+    const int *__restrict__ hpair_built = tb.hpair_built;
+    const int n_bins = tb.n_bins;
     const int p = blockIdx.y;
     const int built = hpair_built[p];
     if (built < 0) return;
@@ -489,10 +499,11 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(const longlong2 *__restri
 // feature), so every stored value adds its row's fixed-point gradient pair to the node's histogram
 // in HBM with two 64-bit integer atomics (exact and order-independent, unlike the float atomics of
 // hist_tree_builder_single.cu:203-216 / :485-505). One wavefront walks one row at a time.
-__global__ __launch_bounds__(kBlock) void k_hist_zero_built(longlong2 *__restrict__ cur_q,
-                                                           const int *__restrict__ hpair_built, int level,
-                                                           int n_bins) {
-    const int built = hpair_built[blockIdx.y];
+__global__ __launch_bounds__(kBlock) void k_hist_zero_built(TreeBuffers tb_all, int level) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    longlong2 *__restrict__ cur_q = tb.hist(level);
+    const int n_bins = tb.n_bins;
+    const int built = tb.hpair_built[blockIdx.y];
     if (built < 0) return;
     const int off = (1 << level) - 1;
     longlong2 *h = cur_q + (size_t)(built - off) * n_bins;
@@ -500,10 +511,13 @@ __global__ __launch_bounds__(kBlock) void k_hist_zero_built(longlong2 *__restric
 }
 
 template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb, CsrBins bins, const GHPair *__restrict__ gh,
-                                                    const int *__restrict__ ridx, longlong2 *__restrict__ cur_q,
+__global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict__ gh,
                                                     int n_pairs, int level) {
     __shared__ int s_info[3];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    gh += (size_t)blockIdx.z * tb.n;
+    const int *__restrict__ ridx = tb.list(level);
+    longlong2 *__restrict__ cur_q = tb.hist(level);
     const LevelCtl c = tb.ctl[level];
     const int item = blockIdx.x;
     if (item >= c.n_hitems) return;
@@ -542,10 +556,13 @@ __global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb, CsrBins bin
 // 1024 threads (16 wavefronts, one row each, the next row's header prefetched), two workgroups per CU.
 template <bool DIRECT>
 __global__ __launch_bounds__(TGBM_HIST_BLOCK) __attribute__((amdgpu_waves_per_eu(8)))
-void k_hist_csr_head(TreeBuffers tb, CsrBins bins, const GHPair *__restrict__ gh, const int *__restrict__ ridx,
-                     longlong2 *__restrict__ cur_q, int n_pairs, int level) {
+void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict__ gh, int n_pairs, int level) {
     extern __shared__ unsigned long long lds[];  // [2 * head_bins]: gradient, hessian of every slot
     __shared__ int s_info[3];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    gh += (size_t)blockIdx.z * tb.n;
+    const int *__restrict__ ridx = tb.list(level);
+    longlong2 *__restrict__ cur_q = tb.hist(level);
     const LevelCtl c = tb.ctl[level];
     const int item = blockIdx.x;
     if (item >= c.n_hitems) return;
@@ -613,11 +630,13 @@ void k_hist_csr_head(TreeBuffers tb, CsrBins bins, const GHPair *__restrict__ gh
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_hist_sub_csr(longlong2 *__restrict__ cur_q,
-                                                        const longlong2 *__restrict__ prev_q,
-                                                        const int *__restrict__ hpair_built, int level, int n_bins) {
+__global__ __launch_bounds__(kBlock) void k_hist_sub_csr(TreeBuffers tb_all, int level) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    longlong2 *__restrict__ cur_q = tb.hist(level);
+    const longlong2 *__restrict__ prev_q = tb.hist(level + 1);
+    const int n_bins = tb.n_bins;
     const int p = blockIdx.y;
-    const int built = hpair_built[p];
+    const int built = tb.hpair_built[p];
     if (built < 0) return;
     const int off = (1 << level) - 1;
     const int sib = (built & 1) ? built + 1 : built - 1;
@@ -653,10 +672,11 @@ __device__ __forceinline__ bool csr_goes_right(const CsrBins &bins, int row, int
 }
 
 template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb, CsrBins bins, const int *__restrict__ ridx,
-                                                          int level) {
+__global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, CsrBins bins, int level) {
     __shared__ int lds[kWaves];
     __shared__ int s_x;
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const int *__restrict__ ridx = tb.list(level);
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
@@ -709,9 +729,10 @@ __device__ __forceinline__ long long shfl_up_ll(long long v, int d) {
 // left = sum of the feature's bins below it, missing = node sum - feature total, gain with missing
 // values sent right and left (hist_tree_builder_single.cu:257-325 / :614-681 of the reference);
 // the wavefront keeps its best candidate: largest |gain|, ties to the smaller bin index (:330-335).
-__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const longlong2 *__restrict__ hist_q, int level,
-                                                      float mcw, float lambda) {
+__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int level, float mcw, float lambda) {
 #pragma clang fp contract(off)
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const longlong2 *__restrict__ hist_q = tb.hist(level);
     __shared__ GHPair s_miss[kWaves][kEvalPackBins];
     const int lane = lane_id(), w = wave_id();
     const int pack = blockIdx.x * kWaves + w;
@@ -853,7 +874,8 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb, const lon
 
 // Per node: reduce the wavefront candidates, fill the split record (hist_tree_builder_single.cu
 // :365-389) and apply it to the tree (update_tree, :860-899). One workgroup per node of the level.
-__global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb, int level, float rt_eps, float lambda) {
+__global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int level, float rt_eps, float lambda) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     __shared__ float s_abs[kWaves];
     __shared__ int s_idx[kWaves];
     __shared__ int s_pack[kWaves];
@@ -962,7 +984,8 @@ __device__ __forceinline__ bool node_splits(const TreeNode &nd) {
 }
 
 // Partition work items: every node of the level that was split gets ceil(rows / kPartChunk) items.
-__global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb, int level) {
+__global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb_all, int level) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     __shared__ int lds[kWaves];
     const int nl = 1 << level, off = nl - 1;
     int carry = 0;
@@ -989,10 +1012,11 @@ __global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb, int level)
 // (missing -> default direction, else right iff bin >= split bin; the reference's rule at
 // hist_tree_builder_single.cu:986-1011) and count the rows that go left.
 template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb, DenseBins bins,
-                                                            const int *__restrict__ ridx, int level) {
+__global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all, DenseBins bins, int level) {
     __shared__ int lds[kWaves];
     __shared__ int s_x;
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const int *__restrict__ ridx = tb.list(level);
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
@@ -1026,7 +1050,8 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb, Den
 // Scan the per-item left counts, publish the children's row segments and plan the histogram work
 // of the next level: per sibling pair the child with fewer rows is built (ties: the left one, as
 // hist_tree_builder_single.cu:466-467), the other one comes from subtraction. One workgroup.
-__global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb, int level) {
+__global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, int level) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     __shared__ int lds[kWaves];
     const int nl = 1 << level, off = nl - 1;
     const int n_p = tb.ctl[level].n_pitems;
@@ -1114,10 +1139,12 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb, int l
 // the histogram's gradient reads sequential but costs more in this kernel than it saves there.) The row -> node map is not touched here; it is rebuilt from the segments
 // when it is needed (k_nid_plan / k_nid_write).
 template <bool DIRECT>
-__global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const int *__restrict__ ridx_cur,
-                                                        int *__restrict__ ridx_next, int level) {
+__global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int level) {
     __shared__ int s_x;
     __shared__ int s_cnt[2][kWaves];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const int *__restrict__ ridx_cur = tb.list(level);
+    int *__restrict__ ridx_next = tb.list(level + 1);
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
@@ -1173,7 +1200,8 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb, const i
 // Bottom-up, level-parallel form of the reference's Tree::prune_self (src/thundergbm/tree.cu:96-128):
 // a node whose two children are valid leaves and whose gain is below gamma becomes a leaf and its
 // children are marked pruned; then final ids are renumbered over valid, unpruned nodes.
-__global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb, float gamma) {
+__global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb_all, float gamma) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     __shared__ int lds[kWaves];
     for (int level = tb.depth - 1; level >= 0; --level) {
         const int nl = 1 << level, off = nl - 1;
@@ -1293,7 +1321,8 @@ __device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBi
 // n_blocks), 0 everywhere for nodes that hold no rows: row block b then owns positions [bound[b][x],
 // bound[b + 1][x]) of every list. One thread per entry; neighbouring threads search neighbouring
 // boundaries of the same list.
-__global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb, int lookup_level, int n_blocks) {
+__global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb_all, int lookup_level, int n_blocks) {
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     const int n_holders = (1 << tb.depth) - 1;
     const size_t total = (size_t)n_holders * (n_blocks + 1);
     for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
@@ -1308,7 +1337,7 @@ __global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb, int looku
                 if (level == 0) {  // the root's list is the identity
                     pos = (int)min(max(r, (long long)sg.x), (long long)sg.y);
                 } else {
-                    const int *list = tb.ridx[level & 1];
+                    const int *list = tb.list(level);
                     const int first = list[sg.x], last = list[sg.y - 1];
                     pos = r <= first ? sg.x : (r > last ? sg.y : list_lower_bound(list, sg.x, sg.y, first, last, (int)r));
                 }
@@ -1319,8 +1348,10 @@ __global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb, int looku
 }
 
 template <int MODE, bool SPARSE>
-__global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb, DenseBins dbins, CsrBins cbins, TreeEndArgs a) {
+__global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBins dbins, CsrBins cbins, TreeEndArgs a) {
     __shared__ int s_leaf[kRowBlock];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    if (MODE == 1) a.yp += (size_t)blockIdx.z * tb.n;  // class-major predictions
     __shared__ int s_list[kEndListCap][3];  // node, first and one-past-last list position
     __shared__ int s_split[kEndListCap];    // -1: the rows stay in the node; else feature | bin << 16 | default_right << 24
     __shared__ int s_off[kEndListCap];
@@ -1347,7 +1378,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb, DenseBins d
                              ? -1
                              : (nd.split_feature_id | (int)nd.split_bid << 16 | (nd.default_right ? 1 : 0) << 24);
         } else {
-            const int *list = tb.ridx[(31 - __clz(x + 1)) & 1];
+            const int *list = tb.list(31 - __clz(x + 1));
             for (int p = pa; p < pb; ++p) {
                 const int row = x == 0 ? p : list[p];
                 s_leaf[row - r0] = nd.split_feature_id >= 0 ? end_child_of<SPARSE>(tb, dbins, cbins, nd, row) : x;
@@ -1384,7 +1415,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb, DenseBins d
                 node[u] = s_list[lo][0];
                 split[u] = s_split[lo];
                 const int p = s_list[lo][1] + (j - s_off[lo]);
-                row[u] = node[u] == 0 ? p : tb.ridx[(31 - __clz(node[u] + 1)) & 1][p];
+                row[u] = node[u] == 0 ? p : tb.list(31 - __clz(node[u] + 1))[p];
             }
         }
         if (SPARSE) {
@@ -1556,16 +1587,21 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
 }
 
-void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, bool stats_ready) {
-    if (!stats_ready) k_sum_gh<<<tb.n_grad_blocks, kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);  // n_grad_blocks == row_blocks(n)
-    k_tree_init<<<1, kBlock, 0, s>>>(tb, tb.root_partial, lambda);
+// Launchers: `tb` is the first buffer set to use, `n_class` consecutive sets (class trees of one round)
+// are served by the same launch through blockIdx.z; gradient and prediction pointers address the
+// first of those classes.
+void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, bool stats_ready,
+                      int n_class) {
+    if (!stats_ready)  // n_grad_blocks == row_blocks(n)
+        k_sum_gh<<<dim3(tb.n_grad_blocks, 1, n_class), kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
+    k_tree_init<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, lambda);
 }
 
 template <int LPR, int SLOTS>
 static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
-                              int level) {
+                              int level, int n_class) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
-    dim3 grid(tb.max_hitems, bins.n_blocks);
+    dim3 grid(tb.max_hitems, bins.n_blocks, n_class);
     size_t lds = (size_t)tb.max_block_bins * sizeof(unsigned long long);
     if (lds > 64 * 1024) {
         // more than the default dynamic LDS window: opt in once per kernel instance and size
@@ -1580,53 +1616,47 @@ static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseB
             opted = lds;
         }
     }
-    if (level == 0) {
-        k_hist_dense<LPR, true, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
-            bins, gh, nullptr, tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
-            tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
-    } else {
-        k_hist_dense<LPR, false, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(
-            bins, gh, tb.ridx[level & 1], tb.seg, tb.hpair_begin, tb.hpair_built, n_pairs, tb.ctl + level, tb.quant,
-            tb.blk_bin_begin, tb.feat_lds_off, tb.partial, tb.n_bins);
-    }
+    if (level == 0)
+        k_hist_dense<LPR, true, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
+    else
+        k_hist_dense<LPR, false, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
 }
 
 template <int LPR>
 static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
-                                int level) {
+                                int level, int n_class) {
     const int slots = (tb.max_block_bins + kHistBlock - 1) / kHistBlock;  // bins drained per thread
-    if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level);
-    else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level);
-    else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level);
-    else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level);
-    else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level);
+    if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level, n_class);
     else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
 }
 
-void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level) {
-    switch (bins.W / 4) {
-        case 1: hist_dense_dispatch<1>(s, tb, bins, gh, level); break;
-        case 2: hist_dense_dispatch<2>(s, tb, bins, gh, level); break;
-        case 4: hist_dense_dispatch<4>(s, tb, bins, gh, level); break;
-        case 8: hist_dense_dispatch<8>(s, tb, bins, gh, level); break;
-        case 16: hist_dense_dispatch<16>(s, tb, bins, gh, level); break;
+void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level,
+                       int n_class) {
+    switch (bins.W) {
+        case 4: hist_dense_dispatch<1>(s, tb, bins, gh, level, n_class); break;
+        case 8: hist_dense_dispatch<2>(s, tb, bins, gh, level, n_class); break;
+        case 16: hist_dense_dispatch<4>(s, tb, bins, gh, level, n_class); break;
+        case 32: hist_dense_dispatch<8>(s, tb, bins, gh, level, n_class); break;
+        case 64: hist_dense_dispatch<16>(s, tb, bins, gh, level, n_class); break;
         default: fatal("unsupported dense block width %d", bins.W);
     }
 }
 
-void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level) {
+void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
-
-    dim3 grid((tb.n_bins + kMergeBins - 1) / kMergeBins, n_pairs);
-    k_hist_merge<<<grid, kBlock, 0, s>>>(tb.partial, tb.hist_q[level & 1], tb.hist_q[(level + 1) & 1], tb.hpair_begin,
-                                        tb.hpair_built, level, tb.n_bins);
+    dim3 grid((tb.n_bins + kMergeBins - 1) / kMergeBins, n_pairs, n_class);
+    k_hist_merge<<<grid, kBlock, 0, s>>>(tb, level);
 }
 
-void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level) {
+void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
+                     int n_class) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
     const int zgrid = std::min(1024, (tb.n_bins + kBlock - 1) / kBlock);
-    longlong2 *cur = tb.hist_q[level & 1];
-    k_hist_zero_built<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hpair_built, level, tb.n_bins);
+    k_hist_zero_built<<<dim3(zgrid, n_pairs, n_class), kBlock, 0, s>>>(tb, level);
     const size_t lds = (size_t)bins.head_bins * 2 * sizeof(unsigned long long);
     if (bins.hist_word != nullptr && lds > 64 * 1024) {
         static size_t opted = 0;  // more than the default dynamic LDS window: opt in once
@@ -1638,76 +1668,72 @@ void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, 
             opted = lds;
         }
     }
-    const int *list = level == 0 ? nullptr : tb.ridx[level & 1];
+    const dim3 grid(tb.max_hitems, 1, n_class);
     if (bins.hist_word != nullptr) {
-        if (level == 0) k_hist_csr_head<true><<<tb.max_hitems, kHistBlock, lds, s>>>(tb, bins, gh, list, cur, n_pairs, level);
-        else k_hist_csr_head<false><<<tb.max_hitems, kHistBlock, lds, s>>>(tb, bins, gh, list, cur, n_pairs, level);
+        if (level == 0) k_hist_csr_head<true><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, n_pairs, level);
+        else k_hist_csr_head<false><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, n_pairs, level);
     } else {
-        if (level == 0) k_hist_csr<true><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, list, cur, n_pairs, level);
-        else k_hist_csr<false><<<tb.max_hitems, kBlock, 0, s>>>(tb, bins, gh, list, cur, n_pairs, level);
+        if (level == 0) k_hist_csr<true><<<grid, kBlock, 0, s>>>(tb, bins, gh, n_pairs, level);
+        else k_hist_csr<false><<<grid, kBlock, 0, s>>>(tb, bins, gh, n_pairs, level);
     }
-    if (level > 0)
-        k_hist_sub_csr<<<dim3(zgrid, n_pairs), kBlock, 0, s>>>(cur, tb.hist_q[(level + 1) & 1], tb.hpair_built, level,
-                                                              tb.n_bins);
+    if (level > 0) k_hist_sub_csr<<<dim3(zgrid, n_pairs, n_class), kBlock, 0, s>>>(tb, level);
 }
 
-void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda) {
-    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level);
-    k_eval_split<<<grid, kBlock, 0, s>>>(tb, tb.hist_q[level & 1], level, mcw, lambda);
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class) {
+    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level, n_class);
+    k_eval_split<<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda);
 }
 
-void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda) {
-    k_best_update<<<1 << level, kBlock, 0, s>>>(tb, level, rt_eps, lambda);
+void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class) {
+    k_best_update<<<dim3(1 << level, 1, n_class), kBlock, 0, s>>>(tb, level, rt_eps, lambda);
 }
 
-void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level) {
+void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class) {
     if (level == tb.depth - 1) return;  // the last level's children never get row lists (see k_tree_end)
-    k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
-    const int *cur = tb.ridx[level & 1];
-    int *next = tb.ridx[(level + 1) & 1];
+    const dim3 one(1, 1, n_class), items(tb.max_pitems, 1, n_class);
+    k_part_plan<<<one, kBlock, 0, s>>>(tb, level);
     if (level == 0) {
-        k_part_count_dense<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
-        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
-        k_part_scatter<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+        k_part_count_dense<true><<<items, kBlock, 0, s>>>(tb, bins, level);
+        k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<true><<<items, kBlock, 0, s>>>(tb, level);
     } else {
-        k_part_count_dense<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
-        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
-        k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+        k_part_count_dense<false><<<items, kBlock, 0, s>>>(tb, bins, level);
+        k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<false><<<items, kBlock, 0, s>>>(tb, level);
     }
 }
 
-void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level) {
+void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class) {
     if (level == tb.depth - 1) return;
-    k_part_plan<<<1, kBlock, 0, s>>>(tb, level);
-    const int *cur = tb.ridx[level & 1];
-    int *next = tb.ridx[(level + 1) & 1];
+    const dim3 one(1, 1, n_class), items(tb.max_pitems, 1, n_class);
+    k_part_plan<<<one, kBlock, 0, s>>>(tb, level);
     if (level == 0) {
-        k_part_count_csr<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
-        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
-        k_part_scatter<true><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+        k_part_count_csr<true><<<items, kBlock, 0, s>>>(tb, bins, level);
+        k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<true><<<items, kBlock, 0, s>>>(tb, level);
     } else {
-        k_part_count_csr<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, bins, cur, level);
-        k_part_scan_plan<<<1, kBlock, 0, s>>>(tb, level);
-        k_part_scatter<false><<<tb.max_pitems, kBlock, 0, s>>>(tb, cur, next, level);
+        k_part_count_csr<false><<<items, kBlock, 0, s>>>(tb, bins, level);
+        k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
+        k_part_scatter<false><<<items, kBlock, 0, s>>>(tb, level);
     }
 }
 
 template <bool SPARSE>
 static void tree_end_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &d, const CsrBins &c, int mode,
-                            const TreeEndArgs &a) {
-    const int grid = row_blocks(tb.n);
+                            const TreeEndArgs &a, int n_class) {
+    const dim3 grid(row_blocks(tb.n), 1, n_class);
     if (mode == 0) k_tree_end<0, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
     else if (mode == 1) k_tree_end<1, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
     else k_tree_end<2, SPARSE><<<grid, kBlock, 0, s>>>(tb, d, c, a);
 }
 
 static void tree_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins, int mode,
-                     const TreeEndArgs &a) {
+                     const TreeEndArgs &a, int n_class = 1) {
     const int n_blocks = row_blocks(tb.n);
     const size_t entries = (size_t)((1 << tb.depth) - 1) * (n_blocks + 1);
-    k_end_bounds<<<grid_for(entries, 8192), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
-    if (tb.sparse) tree_end_launch<true>(s, tb, DenseBins{}, *cbins, mode, a);
-    else tree_end_launch<false>(s, tb, *dbins, CsrBins{}, mode, a);
+    k_end_bounds<<<dim3(grid_for(entries, 8192), 1, n_class), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
+    if (tb.sparse) tree_end_launch<true>(s, tb, DenseBins{}, *cbins, mode, a, n_class);
+    else tree_end_launch<false>(s, tb, *dbins, CsrBins{}, mode, a, n_class);
 }
 
 void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
@@ -1718,12 +1744,12 @@ void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *d
 }
 
 void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
-                                int lookup_level, float *yp_class, float lr) {
+                                int lookup_level, float *yp_class, float lr, int n_class) {
     TreeEndArgs a{};
     a.lookup_level = lookup_level;
     a.yp = yp_class;
     a.lr = lr;
-    tree_end(s, tb, dbins, cbins, 1, a);
+    tree_end(s, tb, dbins, cbins, 1, a, n_class);
 }
 
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
@@ -1743,7 +1769,9 @@ void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbi
     k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, row_blocks(tb.n), metric_scratch, metric_out);
 }
 
-void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma) { k_prune<<<1, kBlock, 0, s>>>(tb, gamma); }
+void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma, int n_class) {
+    k_prune<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, gamma);
+}
 
 void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
                    float *out) {
