@@ -432,6 +432,13 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         }
     }
     __syncthreads();
+    if (c.hchunk <= kHistFlushEvery) {
+        // an item this short was never drained: its packed LDS words are the complete sums and go out as
+        // they are (8 bytes per bin instead of 16; k_hist_merge unpacks them)
+        unsigned long long *out = reinterpret_cast<unsigned long long *>(partial) + (size_t)item * n_bins + bin0;
+        for (int i = threadIdx.x; i < nb; i += BLK) out[i] = lds[i];
+        return;
+    }
     longlong2 *out = partial + (size_t)item * n_bins + bin0;
 #pragma unroll
     for (int k = 0; k < SLOTS; ++k) {
@@ -470,10 +477,20 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
     long long sg = 0, sh = 0;
     if (j < n_bins) {
-        for (int it = ib + ig; it < ie; it += kMergeGroups) {
-            longlong2 v = partial[(size_t)it * n_bins + j];
-            sg += v.x;
-            sh += v.y;
+        if (tb.ctl[level].hchunk <= kHistFlushEvery) {  // packed 8-byte partials (see k_hist_dense)
+            const unsigned long long *packed = reinterpret_cast<const unsigned long long *>(partial);
+            for (int it = ib + ig; it < ie; it += kMergeGroups) {
+                const unsigned long long t = packed[(size_t)it * n_bins + j];
+                const unsigned lo = (unsigned)t;
+                sg += (int)((long long)(t - lo) >> 32);
+                sh += lo;
+            }
+        } else {
+            for (int it = ib + ig; it < ie; it += kMergeGroups) {
+                longlong2 v = partial[(size_t)it * n_bins + j];
+                sg += v.x;
+                sh += v.y;
+            }
         }
     }
     s_g[ig][jl] = sg;
