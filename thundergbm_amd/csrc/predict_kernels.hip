@@ -62,6 +62,48 @@ __global__ __launch_bounds__(kBlock) void k_predict(int n, const int *__restrict
     }
 }
 
+// The reference's shared-memory path (predictor.cu:85-160): every thread first spreads its row into a dense
+// vector of F floats (+inf = not stored, which is why a stored +inf counts as missing there), then walks
+// all trees with one LDS read per node instead of a binary search of the CSR row. Feature-major LDS layout
+// (f * kStageBlock + thread) keeps the reads of a wavefront on distinct banks. Sums are double as in the
+// reference's path.
+constexpr int kStageBlock = 128;
+
+__global__ __launch_bounds__(kStageBlock) void k_predict_staged(int n, int F, const int *__restrict__ row_ptr,
+                                                               const int *__restrict__ col,
+                                                               const float *__restrict__ val,
+                                                               const TreeNode *__restrict__ model, int n_iter,
+                                                               int n_class_trees, int n_nodes, float lr,
+                                                               float base_score, float *__restrict__ out) {
+    extern __shared__ float dense[];  // [F][kStageBlock]
+    const int i = blockIdx.x * kStageBlock + threadIdx.x;
+    for (int f = 0; f < F; ++f) dense[f * kStageBlock + threadIdx.x] = INFINITY;
+    if (i >= n) return;  // no barrier below: a thread only reads what it wrote
+    const int rb = row_ptr[i], re = row_ptr[i + 1];
+    for (int e = rb; e < re; ++e) {
+        const int c = col[e];
+        if (c < F) dense[c * kStageBlock + threadIdx.x] = val[e];
+    }
+    for (int t = 0; t < n_class_trees; ++t) {
+        double sum = base_score;
+        for (int it = 0; it < n_iter; ++it) {
+            const TreeNode *nd = model + ((size_t)it * n_class_trees + t) * n_nodes;
+            int cur = 0;
+            while (!nd[cur].is_leaf) {
+                const TreeNode &c = nd[cur];
+                const int f = c.split_feature_id;
+                const float v = f < F ? dense[f * kStageBlock + threadIdx.x] : INFINITY;
+                if (v < INFINITY)
+                    cur = v < c.split_value ? c.lch_index : c.rch_index;
+                else
+                    cur = c.default_right ? c.rch_index : c.lch_index;
+            }
+            sum += lr * nd[cur].base_weight;
+        }
+        out[(size_t)t * n + i] += (float)sum;
+    }
+}
+
 // kind 1: binary label lookup, 2: arg-max label lookup, 3: softmax probabilities in place,
 // 4: sigmoid (reg:logistic). regression_obj.h:27-32,76-92 and multiclass_obj.cu:44-88 of the reference.
 __global__ void k_predict_transform(int kind, int n, int K, const float *__restrict__ label, float *__restrict__ y) {
@@ -106,8 +148,8 @@ void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *
     const bool dense_path = (size_t)F * 128 * sizeof(float) <= 48 * 1024;
     int grid = (n + kBlock - 1) / kBlock;
     if (dense_path)
-        k_predict<double, true><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr,
-                                                       base_score, out);
+        k_predict_staged<<<(n + kStageBlock - 1) / kStageBlock, kStageBlock, (size_t)F * kStageBlock * sizeof(float), s>>>(
+            n, F, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr, base_score, out);
     else
         k_predict<float, false><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr,
                                                        base_score, out);
