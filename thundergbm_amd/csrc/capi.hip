@@ -192,9 +192,9 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
     p.tree_method = "hist";
     t->dataset.load_from_sparse(row_size, val, row_ptr, col_ptr, label, nullptr, 0, p);
     t->impl.reset(new Trainer(t->dataset, p));
-    t->dataset.csr_val = std::vector<float>();
-    t->dataset.csr_col_idx = std::vector<int>();
-    t->dataset.csr_row_ptr = std::vector<int>();
+    t->dataset.val = nullptr;  // the caller's buffers are not referenced after this call
+    t->dataset.col_idx = nullptr;
+    t->dataset.row_ptr = nullptr;
     return t;
 }
 

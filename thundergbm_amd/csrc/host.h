@@ -10,9 +10,17 @@ namespace tgbm {
 
 // Host CSR dataset (the reference's DataSet, include/thundergbm/dataset.h).
 struct DataSet {
+    // Owned CSR arrays (filled by load_from_file only).
     std::vector<float> csr_val;
     std::vector<int> csr_row_ptr;
     std::vector<int> csr_col_idx;
+    // The CSR arrays the device code uploads: the caller's buffers after load_from_sparse (not copied; they
+    // must stay valid while the trainer / predictor is being constructed), the owned vectors after
+    // load_from_file.
+    const float *val = nullptr;
+    const int *row_ptr = nullptr;
+    const int *col_idx = nullptr;
+    long nnz = 0;
     std::vector<float> y;
     std::vector<float> label;  // distinct class labels, ascending
     std::vector<int> group;

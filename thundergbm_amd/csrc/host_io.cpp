@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstring>
 #include <fstream>
+#include <thread>
 #include <map>
 #include <sstream>
 
@@ -63,11 +64,25 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
     const int nnz = row_ptr[n_rows];
     y.assign(n_rows, 0.f);
     if (labels != nullptr) std::copy(labels, labels + n_rows, y.begin());
-    csr_val.assign(val, val + nnz);
-    csr_col_idx.assign(col_idx, col_idx + nnz);
-    csr_row_ptr.assign(row_ptr, row_ptr + n_rows + 1);
+    this->val = val;
+    this->row_ptr = row_ptr;
+    this->col_idx = col_idx;
+    this->nnz = nnz;
+    // largest column index, on a few threads when the matrix is large
+    const int n_thr = nnz > (1 << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
+    std::vector<int> part_max(n_thr, 0);
+    auto scan = [&](int t) {
+        const long b = (long)nnz * t / n_thr, e = (long)nnz * (t + 1) / n_thr;
+        int m = 0;
+        for (long i = b; i < e; ++i) m = std::max(m, col_idx[i]);
+        part_max[t] = m;
+    };
+    std::vector<std::thread> pool;
+    for (int t = 1; t < n_thr; ++t) pool.emplace_back(scan, t);
+    scan(0);
+    for (auto &th : pool) th.join();
     int max_col = 0;
-    for (int i = 0; i < nnz; ++i) max_col = std::max(max_col, col_idx[i]);
+    for (int m : part_max) max_col = std::max(max_col, m);
     n_features_ = (size_t)max_col + 1;
     log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
     if (labels != nullptr && objective_needs_group_label(param.objective)) {
@@ -129,6 +144,10 @@ void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {
         }
         csr_row_ptr.push_back((int)csr_val.size());
     }
+    val = csr_val.data();
+    row_ptr = csr_row_ptr.data();
+    col_idx = csr_col_idx.data();
+    nnz = (long)csr_val.size();
     label = y;  // the reference keeps a copy of all labels here (dataset.cpp:290-291) ...
     log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
     if (objective_needs_group_label(param.objective)) {

@@ -22,7 +22,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     TGBM_CHECK(e == hipSuccess && n_dev >= 1, "no HIP device available: this library has no CPU path");
     const int n = (int)ds.n_instances();
     const int F = (int)ds.n_features();
-    const long nnz = (long)ds.csr_val.size();
+    const long nnz = ds.nnz;
     TGBM_CHECK(!model.empty() && !model.front().empty(), "empty model");
     const int n_iter = (int)model.size();
     const int nct = (int)model.front().size();
@@ -49,10 +49,10 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipMalloc(&d_model, sizeof(TreeNode) * flat.size()));
     HIP_CHECK(hipMalloc(&d_out, sizeof(float) * std::max(n_out, (size_t)1)));
     if (nnz) {
-        HIP_CHECK(hipMemcpyAsync(d_val, ds.csr_val.data(), sizeof(float) * (size_t)nnz, hipMemcpyHostToDevice, s));
-        HIP_CHECK(hipMemcpyAsync(d_col, ds.csr_col_idx.data(), sizeof(int) * (size_t)nnz, hipMemcpyHostToDevice, s));
+        HIP_CHECK(hipMemcpyAsync(d_val, ds.val, sizeof(float) * (size_t)nnz, hipMemcpyHostToDevice, s));
+        HIP_CHECK(hipMemcpyAsync(d_col, ds.col_idx, sizeof(int) * (size_t)nnz, hipMemcpyHostToDevice, s));
     }
-    HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.csr_row_ptr.data(), sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
+    HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.row_ptr, sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
     HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));
     launch_fill_f32(s, d_out, 0.f, n_out);
     launch_predict(s, n, F, d_row_ptr, d_col, d_val, d_model, n_iter, nct, n_nodes, param.learning_rate,

@@ -34,7 +34,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     HIP_CHECK(hipStreamCreate(&stream_));
     n_ = (int)ds.n_instances();
     F_ = (int)ds.n_features();
-    nnz_ = (long)ds.csr_val.size();
+    nnz_ = ds.nnz;
     TGBM_CHECK(n_ > 0, "empty dataset");
     TGBM_CHECK(param.depth >= 1 && param.depth <= 14, "depth %d out of the supported range 1..14", param.depth);
     TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 255,
@@ -78,11 +78,17 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     HIP_CHECK(hipMalloc(&d_val, sizeof(float) * (size_t)std::max(nnz_, 1l)));
     HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz_, 1l)));
     HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n_ + 1)));
-    upload(stream_, d_val, ds.csr_val.data(), (size_t)nnz_);
-    upload(stream_, d_col, ds.csr_col_idx.data(), (size_t)nnz_);
-    upload(stream_, d_row_ptr, ds.csr_row_ptr.data(), (size_t)n_ + 1);
+    auto t_up = std::chrono::steady_clock::now();
+    upload(stream_, d_val, ds.val, (size_t)nnz_);
+    upload(stream_, d_col, ds.col_idx, (size_t)nnz_);
+    upload(stream_, d_row_ptr, ds.row_ptr, (size_t)n_ + 1);
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    log_debug("upload of %.2f GB: %.3f s", (double)nnz_ * 8e-9,
+              std::chrono::duration<double>(std::chrono::steady_clock::now() - t_up).count());
     log_info("Fast getting cut points...");
+    auto t_cut = std::chrono::steady_clock::now();
     cuts_ = build_cut_points(stream_, F_, nnz_, d_val, d_col, param_.max_num_bin);
+    log_debug("cut points: %.3f s", std::chrono::duration<double>(std::chrono::steady_clock::now() - t_cut).count());
     n_bins_ = cuts_.n_bins;
     allocs_.push_back(cuts_.cut_row_ptr);
     if (cuts_.cut_val) allocs_.push_back(cuts_.cut_val);
