@@ -94,19 +94,34 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
 }
 
 void DataSet::group_label() {
-    std::vector<int> distinct(y.begin(), y.end());  // labels are truncated to int for the label set
-    std::sort(distinct.begin(), distinct.end());
-    distinct.erase(std::unique(distinct.begin(), distinct.end()), distinct.end());
-    std::map<float, int> index_of;
-    label.clear();
-    for (int v : distinct) {
-        index_of[(float)v] = (int)label.size();
-        label.push_back((float)v);
+    // labels are truncated to int for the label set; the set is small, so it is kept sorted while scanning
+    // (no sort of all rows)
+    std::vector<int> distinct;
+    bool have_last = false;
+    int last = 0;
+    for (float v : y) {
+        const int iv = (int)v;
+        if (have_last && iv == last) continue;
+        have_last = true;
+        last = iv;
+        auto it = std::lower_bound(distinct.begin(), distinct.end(), iv);
+        if (it == distinct.end() || *it != iv) distinct.insert(it, iv);
     }
-    for (float &v : y) {
-        auto it = index_of.find(v);
-        v = it == index_of.end() ? 0.f : (float)it->second;  // unknown keys read as class 0
-    }
+    label.assign(distinct.begin(), distinct.end());
+    // a row's class is the position of its label in the set; labels that are not in it (non-integers)
+    // read as class 0, like a failed lookup in the reference's map
+    const int n_thr = y.size() > (1u << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
+    auto remap = [&](int t) {
+        const size_t b = y.size() * t / n_thr, e = y.size() * (t + 1) / n_thr;
+        for (size_t i = b; i < e; ++i) {
+            auto it = std::lower_bound(label.begin(), label.end(), y[i]);
+            y[i] = (it != label.end() && *it == y[i]) ? (float)(it - label.begin()) : 0.f;
+        }
+    };
+    std::vector<std::thread> pool;
+    for (int t = 1; t < n_thr; ++t) pool.emplace_back(remap, t);
+    remap(0);
+    for (auto &th : pool) th.join();
 }
 
 void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {

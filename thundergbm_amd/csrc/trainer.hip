@@ -5,6 +5,7 @@
 #include "trainer.h"
 
 #include <algorithm>
+#include <thread>
 #include <chrono>
 #include <cmath>
 #include <cstdlib>
@@ -25,6 +26,45 @@ template <typename T>
 static T *upload(hipStream_t s, T *dst, const T *src, size_t count) {
     if (count) HIP_CHECK(hipMemcpyAsync(dst, src, count * sizeof(T), hipMemcpyHostToDevice, s));
     return dst;
+}
+
+// Host -> device copy of a large pageable array: chunks are copied by a few host threads into two pinned
+// staging buffers and sent with asynchronous DMA, so the host copy of one chunk overlaps the transfer of
+// the previous one (a plain hipMemcpy of pageable memory stages through one thread).
+static void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes) {
+    constexpr size_t kChunk = (size_t)32 << 20;
+    if (bytes < 4 * kChunk) {
+        if (bytes) HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
+        return;
+    }
+    void *pin[2] = {nullptr, nullptr};
+    hipEvent_t done[2];
+    for (int b = 0; b < 2; ++b) {
+        HIP_CHECK(hipHostMalloc(&pin[b], kChunk, hipHostMallocDefault));
+        HIP_CHECK(hipEventCreateWithFlags(&done[b], hipEventDisableTiming));
+    }
+    const int n_thr = (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency()));
+    size_t off = 0;
+    for (int i = 0; off < bytes; ++i, off += kChunk) {
+        const int b = i & 1;
+        const size_t len = std::min(kChunk, bytes - off);
+        if (i >= 2) HIP_CHECK(hipEventSynchronize(done[b]));  // the DMA that last read this buffer
+        std::vector<std::thread> pool;
+        auto part = [&](int t) {
+            const size_t pb = len * t / n_thr, pe = len * (t + 1) / n_thr;
+            std::memcpy(static_cast<char *>(pin[b]) + pb, static_cast<const char *>(src) + off + pb, pe - pb);
+        };
+        for (int t = 1; t < n_thr; ++t) pool.emplace_back(part, t);
+        part(0);
+        for (auto &th : pool) th.join();
+        HIP_CHECK(hipMemcpyAsync(static_cast<char *>(dst) + off, pin[b], len, hipMemcpyHostToDevice, s));
+        HIP_CHECK(hipEventRecord(done[b], s));
+    }
+    HIP_CHECK(hipStreamSynchronize(s));
+    for (int b = 0; b < 2; ++b) {
+        HIP_CHECK(hipEventDestroy(done[b]));
+        HIP_CHECK(hipHostFree(pin[b]));
+    }
 }
 
 Trainer::Trainer(const DataSet &ds, GBMParam &param) {
@@ -79,8 +119,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz_, 1l)));
     HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n_ + 1)));
     auto t_up = std::chrono::steady_clock::now();
-    upload(stream_, d_val, ds.val, (size_t)nnz_);
-    upload(stream_, d_col, ds.col_idx, (size_t)nnz_);
+    upload_large(stream_, d_val, ds.val, sizeof(float) * (size_t)nnz_);
+    upload_large(stream_, d_col, ds.col_idx, sizeof(int) * (size_t)nnz_);
     upload(stream_, d_row_ptr, ds.row_ptr, (size_t)n_ + 1);
     HIP_CHECK(hipStreamSynchronize(stream_));
     log_debug("upload of %.2f GB: %.3f s", (double)nnz_ * 8e-9,
