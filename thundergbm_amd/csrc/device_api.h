@@ -215,6 +215,9 @@ struct DeviceCuts {
 };
 DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, const int *d_col, int max_num_bin);
 
+// Host -> device copy of a large pageable array through pinned staging buffers (returns when done).
+void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);
+
 // prediction
 void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
                     const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,

@@ -49,8 +49,8 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipMalloc(&d_model, sizeof(TreeNode) * flat.size()));
     HIP_CHECK(hipMalloc(&d_out, sizeof(float) * std::max(n_out, (size_t)1)));
     if (nnz) {
-        HIP_CHECK(hipMemcpyAsync(d_val, ds.val, sizeof(float) * (size_t)nnz, hipMemcpyHostToDevice, s));
-        HIP_CHECK(hipMemcpyAsync(d_col, ds.col_idx, sizeof(int) * (size_t)nnz, hipMemcpyHostToDevice, s));
+        upload_large(s, d_val, ds.val, sizeof(float) * (size_t)nnz);
+        upload_large(s, d_col, ds.col_idx, sizeof(int) * (size_t)nnz);
     }
     HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.row_ptr, sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
     HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));

@@ -31,7 +31,7 @@ static T *upload(hipStream_t s, T *dst, const T *src, size_t count) {
 // Host -> device copy of a large pageable array: chunks are copied by a few host threads into two pinned
 // staging buffers and sent with asynchronous DMA, so the host copy of one chunk overlaps the transfer of
 // the previous one (a plain hipMemcpy of pageable memory stages through one thread).
-static void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes) {
+void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes) {
     constexpr size_t kChunk = (size_t)32 << 20;
     if (bytes < 4 * kChunk) {
         if (bytes) HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
