@@ -176,7 +176,10 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_cl
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
                      int n_class = 1);
 void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
-void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class = 1);
+// store_sibling (sparse layout only): keep the derived sibling histograms; nobody reads those of a tree's
+// last level
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class = 1,
+                       bool store_sibling = true);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class = 1);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class = 1);
 // Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level

@@ -86,6 +86,7 @@ class Trainer {
     float *d_metric_ = nullptr;
     double *d_metric_scratch_ = nullptr;
     int cur_class_ = 0;
+    bool in_boost_ = false;
     int lookup_level_ = -1;          // level whose split nodes have not been partitioned into row lists yet
     bool next_round_ready_ = false;  // d_gh_ and the root statistics already belong to the next round
     // profiling

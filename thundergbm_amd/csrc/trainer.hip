@@ -415,7 +415,9 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
         build_level_hist(tb, level, gh, n_class);
     }
     if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
-    launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class);
+    // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them)
+    launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
+                      !(in_boost_ && level == param_.depth - 1));
     launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
 }
@@ -500,6 +502,7 @@ float Trainer::metric() {
 
 void Trainer::boost(int rounds) {
     static const char *names[] = {"RMSE", "test error", "multi-class accuracy"};
+    in_boost_ = true;
     for (int r = 0; r < rounds; ++r) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
         const bool fuse = objective_ != OBJ_SOFTMAX && param_.tree_per_rounds == 1;
@@ -529,6 +532,7 @@ void Trainer::boost(int rounds) {
         }
         ++rounds_done_;
     }
+    in_boost_ = false;
 }
 
 std::vector<std::vector<Tree>> Trainer::model_to_host() {

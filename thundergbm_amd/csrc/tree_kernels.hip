@@ -647,25 +647,6 @@ void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict_
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_hist_sub_csr(TreeBuffers tb_all, int level) {
-    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
-    longlong2 *__restrict__ cur_q = tb.hist(level);
-    const longlong2 *__restrict__ prev_q = tb.hist(level + 1);
-    const int n_bins = tb.n_bins;
-    const int p = blockIdx.y;
-    const int built = tb.hpair_built[p];
-    if (built < 0) return;
-    const int off = (1 << level) - 1;
-    const int sib = (built & 1) ? built + 1 : built - 1;
-    const longlong2 *b = cur_q + (size_t)(built - off) * n_bins;
-    longlong2 *sq = cur_q + (size_t)(sib - off) * n_bins;
-    const longlong2 *par = prev_q + (size_t)p * n_bins;
-    for (int j = blockIdx.x * kBlock + threadIdx.x; j < n_bins; j += gridDim.x * kBlock) {
-        longlong2 pv = par[j], bv = b[j];
-        sq[j] = make_longlong2(pv.x - bv.x, pv.y - bv.y);
-    }
-}
-
 // Left/right decision of the sparse layout: binary search of the row's bin ids for the one inside
 // the split feature's bin range (absent = missing), hist_tree_builder_single.cu:941-1011.
 // Does the row go right at a split of the feature whose global bins are [cb, ce)? Binary search of the
@@ -746,10 +727,15 @@ __device__ __forceinline__ long long shfl_up_ll(long long v, int d) {
 // left = sum of the feature's bins below it, missing = node sum - feature total, gain with missing
 // values sent right and left (hist_tree_builder_single.cu:257-325 / :614-681 of the reference);
 // the wavefront keeps its best candidate: largest |gain|, ties to the smaller bin index (:330-335).
-__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int level, float mcw, float lambda) {
+// SUB (sparse layout, whose histograms are not merged from work-item partials): the node of a pair that
+// was not built from rows is derived here as parent - built while it is scanned, and stored for the next
+// level, instead of by a separate pass over the (very long) histograms.
+template <bool SUB>
+__global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int level, float mcw, float lambda,
+                                                      bool store_sibling) {
 #pragma clang fp contract(off)
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
-    const longlong2 *__restrict__ hist_q = tb.hist(level);
+    longlong2 *__restrict__ hist_q = tb.hist(level);
     __shared__ GHPair s_miss[kWaves][kEvalPackBins];
     const int lane = lane_id(), w = wave_id();
     const int pack = blockIdx.x * kWaves + w;
@@ -763,9 +749,37 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
         b_end = tb.pack_begin[pack + 1];
     }
     const GHPair S = nd.sum_gh_pair;
-    const longlong2 *h = hist_q + (size_t)x_in * tb.n_bins;
+    longlong2 *h = hist_q + (size_t)x_in * tb.n_bins;
     const double inv_g = tb.quant->inv_g, inv_h = tb.quant->inv_h;
+    // SUB: is this node the sibling of the pair's built node?
+    const longlong2 *h_par = nullptr, *h_built = nullptr;
+    if (SUB && level > 0 && active) {
+        const int built = tb.hpair_built[x_in >> 1];
+        if (built >= 0 && built != x) {
+            h_par = tb.hist(level + 1) + (size_t)(x_in >> 1) * tb.n_bins;
+            h_built = hist_q + (size_t)(built - ((1 << level) - 1)) * tb.n_bins;
+        }
+    }
 
+    // The pack's bins are read with consecutive lanes on consecutive bins (whole lines per load) and handed
+    // over through LDS to the scan's layout of four consecutive bins per lane.
+    __shared__ longlong2 s_v[kWaves][kEvalPackBins];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int b = b_begin + j * 64 + lane;
+        if (b < b_end) {
+            longlong2 v;
+            if (SUB && h_par != nullptr) {
+                const longlong2 pv = h_par[b], bv = h_built[b];
+                v = make_longlong2(pv.x - bv.x, pv.y - bv.y);
+                if (store_sibling) h[b] = v;
+            } else {
+                v = h[b];
+            }
+            s_v[w][j * 64 + lane] = v;
+        }
+    }
+    __syncthreads();
     long long incg[4], inch[4];
     int lastb[4];  // pack-relative index of the last bin of the element's feature
     bool valid[4], head[4], last[4];
@@ -780,7 +794,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
         last[j] = false;
         incg[j] = inch[j] = 0;
         if (valid[j]) {
-            longlong2 v = h[b];
+            const longlong2 v = s_v[w][lane * 4 + j];
             const int f = tb.cut_fid[b];
             const int fend = tb.cut_row_ptr[f + 1];
             head[j] = tb.cut_row_ptr[f] == b;
@@ -1693,12 +1707,14 @@ void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, 
         if (level == 0) k_hist_csr<true><<<grid, kBlock, 0, s>>>(tb, bins, gh, n_pairs, level);
         else k_hist_csr<false><<<grid, kBlock, 0, s>>>(tb, bins, gh, n_pairs, level);
     }
-    if (level > 0) k_hist_sub_csr<<<dim3(zgrid, n_pairs, n_class), kBlock, 0, s>>>(tb, level);
+    // the sibling histograms (parent - built) are produced by k_eval_split<true>
 }
 
-void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class) {
+void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class,
+                       bool store_sibling) {
     dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level, n_class);
-    k_eval_split<<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda);
+    if (tb.sparse) k_eval_split<true><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, store_sibling);
+    else k_eval_split<false><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, true);
 }
 
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class) {
