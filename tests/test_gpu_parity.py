@@ -484,6 +484,63 @@ def test_full_size_properties_config2(T):
     s.close()
 
 
+def _check_boosted_round(T, val, rp, col, y, n_sample, **kw):
+    """One production boost() round at full size, checked through properties that need no oracle run:
+    every tree's root sum is the fp64 sum of its class's gradients; the rows that ended in a node (last
+    class tree) reproduce that node's sums in an fp64 recount; children add up to their parent; the
+    predictor on a sample of training rows reproduces the training-time predictions."""
+    n = len(rp) - 1
+    s = T.Session(val, rp, col, y, n_trees=2, learning_rate=0.3, **kw)
+    K = s.tree_per_rounds
+    s.gradient()
+    gh = s.gh().astype(np.float64)
+    s.boost(1)
+    model = s.model()
+    for k in range(K):
+        ghk = gh[k * n:(k + 1) * n]
+        Ag, Ah = np.abs(ghk[:, 0]).sum(), np.abs(ghk[:, 1]).sum()
+        nodes = model[0, k]
+        assert nodes[0]["is_valid"]
+        assert abs(nodes[0]["sum_g"] - ghk[:, 0].sum()) <= 1e-5 * Ag and abs(nodes[0]["sum_h"] - ghk[:, 1].sum()) <= 1e-5 * Ah
+        inner = np.flatnonzero((nodes["is_valid"] == 1) & (nodes["split_fid"] >= 0))
+        l, r = nodes["lch"][inner], nodes["rch"][inner]
+        assert np.all(np.abs(nodes["sum_g"][l].astype(np.float64) + nodes["sum_g"][r] - nodes["sum_g"][inner]) <= 1e-5 * Ag)
+        assert np.all(np.abs(nodes["sum_h"][l].astype(np.float64) + nodes["sum_h"][r] - nodes["sum_h"][inner]) <= 1e-5 * Ah)
+    nid = s.nid()  # of the last class tree
+    cnt = np.bincount(nid, minlength=len(nodes))
+    occupied = np.flatnonzero(cnt > 0)
+    assert np.all(nodes["is_valid"][occupied] == 1) and np.all(nodes["split_fid"][occupied] < 0)
+    np.testing.assert_allclose(nodes["sum_h"][occupied], np.bincount(nid, weights=ghk[:, 1], minlength=len(nodes))[occupied],
+                               rtol=0, atol=1e-5 * Ah)
+    np.testing.assert_allclose(nodes["sum_g"][occupied], np.bincount(nid, weights=ghk[:, 0], minlength=len(nodes))[occupied],
+                               rtol=0, atol=1e-5 * Ag)
+    yp = s.y_pred().reshape(-1, n)
+    L = T.load()
+    handle = C.c_void_p(s.export_model())
+    m = n_sample
+    out = np.zeros(K * m, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    srp = rp[: m + 1].copy()
+    L.tgbm_predict_raw(m, p(val), p(srp), p(col), handle, 1, K, 0.3, s.base_score if K == 1 else 0.0, p(out))
+    np.testing.assert_allclose(out.reshape(K, m), yp[:, :m], rtol=1e-5, atol=1e-6)
+    L.model_free(C.byref(handle))
+    s.close()
+
+
+def test_full_size_properties_config5_softmax(T):
+    """1 M x 54, 8 classes: the class trees of the round are built by common launches."""
+    X, y = D.config5()
+    val, rp, col = D.dense_to_csr(X)
+    del X
+    _check_boosted_round(T, val, rp, col, y, 100000, objective="multi:softmax", depth=8, max_num_bin=255)
+
+
+def test_full_size_properties_config4_sparse(T):
+    """2 M x 100k CSR with Zipf-distributed feature ids: sparse layout with the LDS head."""
+    val, rp, col, y = D.config4()
+    _check_boosted_round(T, val, rp, col, y, 100000, objective="binary:logistic", depth=8, max_num_bin=63)
+
+
 def test_cli_train_and_predict_on_a1a(T, tmp_path):
     """thundergbm-train <conf> + thundergbm-predict <conf> (reference: docs/how-to.md:20-31): LIBSVM
     loader, key=value parser, model file with base score, predictor and metric."""
