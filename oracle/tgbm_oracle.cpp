@@ -12,7 +12,9 @@
 //   cut points      closed-form rule on hand inputs, invariants, the a1a fixture (one cut = 1.0 per feature)
 //   bin ids         brute force min(#cuts<=v, k-1) against numpy searchsorted
 //   gradients       float64 closed forms
-//   histogram       brute-force float64 accumulation; bin counts for squared loss
+//   histogram       brute-force float64 accumulation; bin counts for squared loss (the oracle itself
+//                   accumulates in float64 and rounds once: the reference's float atomics have no defined
+//                   order, so their result is only defined up to float round-off)
 //   split finding   brute-force enumeration of (feature, bin, direction) in numpy float64
 //   update/partition row counts equal hessian sums for squared loss; raw-value threshold consistency
 //   prune           hand-built 7-node trees
@@ -301,46 +303,40 @@ void build_hist(Oracle &o, const int *rows, long cnt, GH *out, double *out64) {
     nt = omp_get_max_threads();
 #endif
     if (cnt < 4096) nt = 1;
-    std::vector<GH> priv((size_t)nt * B, GH{0, 0});
-    std::vector<double> priv64;
-    if (out64) priv64.assign((size_t)nt * B * 2, 0.0);
+    // The reference adds with float atomics in no defined order, so its own result varies from run to run
+    // by float round-off that grows with the number of rows per bin. The oracle accumulates in fp64 and
+    // rounds once: the centre of those possible results, and what the 1e-5 parity tolerance refers to.
+    std::vector<double> priv64((size_t)nt * B * 2, 0.0);
 #pragma omp parallel num_threads(nt)
     {
         int t = 0;
 #ifdef _OPENMP
         t = omp_get_thread_num();
 #endif
-        GH *h = priv.data() + (size_t)t * B;
-        double *h64 = out64 ? priv64.data() + (size_t)t * B * 2 : nullptr;
+        double *h64 = priv64.data() + (size_t)t * B * 2;
         long b = cnt * t / nt, e = cnt * (t + 1) / nt;
         for (long r = b; r < e; ++r) {
             int i = rows ? rows[r] : (int)r;
             GH s = gh[i];
             for (int j = o.row_ptr[i]; j < o.row_ptr[i + 1]; ++j) {
                 int bid = o.bin_id[j];
-                h[bid].g += s.g;
-                h[bid].h += s.h;
-                if (h64) {
-                    h64[2 * bid] += (double)s.g;
-                    h64[2 * bid + 1] += (double)s.h;
-                }
+                h64[2 * bid] += (double)s.g;
+                h64[2 * bid + 1] += (double)s.h;
             }
         }
     }
     for (int b = 0; b < B; ++b) {
-        float g = 0, h = 0;
+        double g = 0, h = 0;
         for (int t = 0; t < nt; ++t) {
-            g += priv[(size_t)t * B + b].g;
-            h += priv[(size_t)t * B + b].h;
+            g += priv64[(size_t)t * B * 2 + 2 * b];
+            h += priv64[(size_t)t * B * 2 + 2 * b + 1];
         }
-        out[b] = GH{g, h};
+        out[b] = GH{(float)g, (float)h};
+        if (out64) {
+            out64[2 * b] = g;
+            out64[2 * b + 1] = h;
+        }
     }
-    if (out64)
-        for (int b = 0; b < 2 * B; ++b) {
-            double s = 0;
-            for (int t = 0; t < nt; ++t) s += priv64[(size_t)t * B * 2 + b];
-            out64[b] = s;
-        }
     o.rows_built_total += cnt;
 }
 
