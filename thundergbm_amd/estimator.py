@@ -16,9 +16,17 @@ _PARAMS = ("depth", "n_trees", "n_gpus", "min_child_weight", "lambda_tgbm", "gam
 
 
 def _csr(X):
-    X = X.tocsr(copy=True) if sp.issparse(X) else sp.csr_matrix(np.asarray(X))
-    X.data = np.ascontiguousarray(X.data, dtype=np.float32)
-    X.sort_indices()
+    """CSR view of X with float32 values and ascending column indices; the caller's matrix is only copied
+    when it has to be changed."""
+    if not sp.issparse(X):
+        X = sp.csr_matrix(np.asarray(X))
+    elif X.format != "csr":
+        X = X.tocsr()
+    if X.data.dtype != np.float32 or not X.data.flags.c_contiguous:
+        X = sp.csr_matrix((np.ascontiguousarray(X.data, dtype=np.float32), X.indices, X.indptr), shape=X.shape)
+    if not X.has_sorted_indices:
+        X = X.copy()
+        X.sort_indices()
     return X
 
 
@@ -53,7 +61,7 @@ class TGBMModel(BaseEstimator):
             raise ValueError("X and y have different numbers of rows")
         indptr = np.ascontiguousarray(X.indptr, dtype=np.int32)
         indices = np.ascontiguousarray(X.indices, dtype=np.int32)
-        n_labels = len(set(y.tolist()))
+        n_labels = len(np.unique(y))
         group_label = (C.c_float * max(n_labels, 1))()
         n_class = (C.c_int * 1)(self.num_class)
         per_iter = (C.c_int * 1)(0)
