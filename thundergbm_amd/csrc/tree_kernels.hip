@@ -1167,8 +1167,9 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
 
 // Stable two-way compaction of a work item's rows into the children's segments with wavefront
 // ballots and popcounts. (Moving the gradient pairs along with the row ids was measured: it makes
-// the histogram's gradient reads sequential but costs more in this kernel than it saves there.) The row -> node map is not touched here; it is rebuilt from the segments
-// when it is needed (k_nid_plan / k_nid_write).
+// the histogram's gradient reads sequential but costs more in this kernel than it saves there.)
+// The row -> node map is not touched here; k_end_bounds / k_tree_end derive it from the row lists
+// when it is needed.
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int level) {
     __shared__ int s_x;
