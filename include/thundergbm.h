@@ -31,8 +31,10 @@ void set_logger(int verbose);
 
 /* scikit_tgbm.cpp:26-80. CSR input (float32 values, int32 indices, ascending columns per row).
  * num_class is in/out, group_label receives the distinct labels (caller allocates one float per
- * distinct label), tree_per_iter and *model are outputs. n_device, bagging, column_sampling_rate,
- * n_parallel_trees, group and num_group are accepted for signature compatibility and ignored. */
+ * distinct label), tree_per_iter and *model are outputs. column_sampling_rate < 1 samples columns per
+ * round as the reference does (see tgbm_trainer_set_option). n_device, bagging (never applied by the
+ * reference either), n_parallel_trees, group and num_group are accepted for signature compatibility and
+ * ignored. */
 void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *label, int depth, int n_trees,
                          int n_device, float min_child_weight, float lambda, float gamma, int max_num_bin,
                          int verbose, float column_sampling_rate, int bagging, int n_parallel_trees,
@@ -79,6 +81,13 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
                                   float gamma, int max_num_bin, float learning_rate, const char *objective,
                                   int num_class, int verbose);
 void tgbm_trainer_destroy(tgbm_trainer *t);
+
+/* Options that tgbm_trainer_create has no argument for. "column_sampling_rate" (GBMParam, common.h:92):
+ * below 1 every boosting round ignores max(1, int(n_features * rate)) randomly chosen columns in its split
+ * search (Shard::column_sampling, builder/shard.cu:8-22; the shuffle draws from the process-wide rand()). */
+void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value);
+/* The column sampling of one round for stage-wise driving (tgbm_trainer_boost does it itself). */
+void tgbm_trainer_sample_columns(tgbm_trainer *t);
 
 /* `rounds` iterations of Booster::boost (booster.h:76-93); returns after the GPU finished. */
 void tgbm_trainer_boost(tgbm_trainer *t, int rounds);

@@ -80,6 +80,8 @@ inline float compute_gain(GH f, GH l, GH r, float mcw, float lambda) {
 }
 
 struct Oracle {
+    float column_sampling_rate = 1.f;
+    std::vector<char> ignored;  // per feature, this round (empty: none)
     // data (DataSet, src/thundergbm/dataset.cpp:20-63)
     int n = 0, F = 0;
     long nnz = 0;
@@ -342,6 +344,21 @@ void build_hist(Oracle &o, const int *rows, long cnt, GH *out, double *out64) {
 
 // Scan + missing + gain + argmax + record for one node given its raw histogram.
 // hist_tree_builder_single.cu:257-390 (root) / :614-752 (pair member).
+// Shard::column_sampling, src/thundergbm/builder/shard.cu:8-22, called once per boosting round
+// (builder/tree_builder.cu:150-152): shuffle 0..F-1 with std::random_shuffle (process-wide rand()) and mark
+// the first max(1, int(F * rate)) columns as *ignored* for the round (the array is re-created, i.e. zeroed,
+// by every call: syncarray.h:103-113, syncmem.cpp:76-120). The oracle calls the very library routine the
+// reference calls.
+void sample_columns(Oracle &o) {
+    if (!(o.column_sampling_rate < 1)) return;
+    std::vector<int> idx(o.F);
+    for (int i = 0; i < o.F; ++i) idx[i] = i;
+    std::random_shuffle(idx.begin(), idx.end());
+    int sample_count = std::max(1, int(o.F * o.column_sampling_rate));
+    o.ignored.assign(o.F, 0);
+    for (int i = 0; i < sample_count; ++i) o.ignored[idx[i]] = 1;
+}
+
 void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
     const int B = o.n_bins, F = o.F;
     const Node &nd = o.nodes[node];
@@ -382,6 +399,7 @@ void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
         GH r2 = GH{S.g - l2.g, S.h - l2.h};
         float gl = fmaxf(0.f, compute_gain(S, l2, r2, o.mcw, o.lambda));
         float score = (gl > gr) ? gl : -gr;
+        if (!o.ignored.empty() && o.ignored[f]) score = 0;  // :304 / :663: an ignored column's gain is 0
         if (dbg) dbg[b] = score;
         // arg_abs_max (:330-335): larger |gain| wins, ties keep the smaller index
         if (first || fabsf(score) > fabsf(best_score)) {
@@ -667,6 +685,7 @@ void build_tree(Oracle &o, int k) {
 
 // Booster::boost, include/thundergbm/booster.h:76-93
 void boost_round(Oracle &o) {
+    sample_columns(o);
     gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
     std::vector<Node> round_trees;
     for (int k = 0; k < o.tree_per_rounds; ++k) {
@@ -818,6 +837,8 @@ void orc_prepare(void *h) {
     init_base_score(o);
 }
 
+void orc_set_column_sampling_rate(void *h, float rate) { ((Oracle *)h)->column_sampling_rate = rate; }
+void orc_sample_columns(void *h) { sample_columns(*(Oracle *)h); }
 void orc_boost(void *h, int rounds) {
     Oracle &o = *(Oracle *)h;
     for (int r = 0; r < rounds; ++r) boost_round(o);

@@ -44,6 +44,8 @@ def lib():
             getattr(L, name).restype = None
         L.orc_set_debug.argtypes = [C.c_void_p, C.c_int, C.c_int]
         L.orc_boost.argtypes = [C.c_void_p, C.c_int]
+        L.orc_set_column_sampling_rate.argtypes = [C.c_void_p, C.c_float]
+        L.orc_sample_columns.argtypes = [C.c_void_p]
         for name in ("orc_tree_init", "orc_find_split", "orc_predict_in_training", "orc_build_tree"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_int]
             getattr(L, name).restype = None
@@ -139,6 +141,12 @@ class Oracle:
         self.tree_per_rounds = self.L.orc_tree_per_rounds(self.h)
         self.n_nodes = self.L.orc_n_nodes(self.h)
         return self
+
+    def set_column_sampling_rate(self, rate):
+        self.L.orc_set_column_sampling_rate(self.h, rate)
+
+    def sample_columns(self):
+        self.L.orc_sample_columns(self.h)
 
     def boost(self, rounds=1):
         self.L.orc_boost(self.h, rounds)

@@ -245,6 +245,48 @@ def test_class_trees_built_together_equal_one_by_one(T, layout):
         s.close()
 
 
+@pytest.mark.parametrize("objective,kind,rate", [("reg:linear", "reg", 0.5), ("binary:logistic", "bin", 0.3),
+                                                 ("multi:softmax", "multi", 0.7), ("reg:linear", "reg", 0.05)])
+def test_column_sampling_matches_oracle(T, objective, kind, rate):
+    """column_sampling_rate < 1: every round ignores max(1, int(F * rate)) shuffled columns. The library
+    restates libstdc++'s std::random_shuffle over the process-wide rand(); the oracle calls
+    std::random_shuffle itself. Both are started from the same srand() seed; whole boosting runs (no
+    teacher forcing) must then pick the same columns and build the same trees."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    n, F = 3000, 11
+    val, rp, col = _ragged(n, F, 21, F)
+    y = _target(val, rp, col, n, F, 21, kind)
+    kw = dict(objective=objective, n_trees=5, depth=4, max_num_bin=32, learning_rate=0.5)
+    s = T.Session(val, rp, col, y, **kw)
+    s.set_option("column_sampling_rate", rate)
+    o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    o.set_column_sampling_rate(rate)
+    n_ignored = max(1, int(F * rate))
+    for r in range(5):
+        o.set_y_pred(s.y_pred())
+        s.gradient()
+        gh = s.gh()
+        libc.srand(1234 + r)
+        s.boost(1)
+        libc.srand(1234 + r)
+        o.sample_columns()
+        o.compute_gradient()
+        o.set_gh(gh)
+        model = s.model()
+        used = set()
+        for k in range(s.tree_per_rounds):
+            o.build_tree(k)
+            ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
+            d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=s.cuts()[1], orc_scores=o.tree_scores(),
+                                abs_scale=(ghk[0], ghk[1]))
+            assert not d.near_ties
+            nodes = model[r, k]
+            used |= set(int(f) for f in nodes["split_fid"][(nodes["is_valid"] == 1) & (nodes["split_fid"] >= 0)])
+        assert len(used) <= F - n_ignored  # the round's trees only split on columns that were not ignored
+    s.close()
+
+
 def test_predict_transforms_through_the_c_abi(T):
     """sparse_predict_scikit for every objective against the oracle's predictor + transform on unseen rows."""
     n, F = 1500, 7

@@ -583,3 +583,38 @@ def test_a1a_quickstart_known_answer():
     o2 = O.Oracle(val, rp, col, y, depth=6, n_trees=40, learning_rate=1.0).prepare()
     o2.boost(40)
     assert abs(float(o2.metric_log()[-1]) - 0.52842) < 1e-3
+
+
+def test_column_sampling_ignores_the_shuffled_head():
+    """Shard::column_sampling (shard.cu:8-22): with F columns and rate r, max(1, int(F * r)) columns are
+    ignored per round and no tree of the round splits on them; rate 1 ignores nothing. The shuffle is
+    std::random_shuffle over rand(): two runs from the same srand() seed agree, another seed differs."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    rng = np.random.default_rng(5)
+    n, F = 2000, 10
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    y = (X @ rng.standard_normal(F) + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    kw = dict(objective="reg:linear", n_trees=6, depth=4, max_num_bin=32, learning_rate=0.5)
+
+    def run(rate, seed):
+        o = O.Oracle(val, rp, col, y, **kw).prepare()
+        o.set_column_sampling_rate(rate)
+        libc.srand(seed)
+        o.boost(6)
+        m = o.model()
+        used = [set(int(f) for f in t[0]["split_fid"][(t[0]["is_valid"] == 1) & (t[0]["split_fid"] >= 0)]) for t in m]
+        return m, used
+
+    m_a, used_a = run(0.6, 7)
+    m_b, _ = run(0.6, 7)
+    m_c, used_c = run(0.6, 8)
+    assert m_a.tobytes() == m_b.tobytes()
+    assert m_a.tobytes() != m_c.tobytes()
+    assert all(len(u) <= F - 6 for u in used_a + used_c)  # int(10 * 0.6) = 6 ignored columns per round
+    assert len(set().union(*used_a)) > F - 6  # a fresh sample every round: over 6 rounds more columns appear
+    m_full, used_full = run(1.0, 7)
+    assert max(len(u) for u in used_full) > 4
+    _, used_tiny = run(0.01, 7)  # max(1, int(0.1)) = 1 ignored column
+    assert all(len(u) <= F - 1 for u in used_tiny)

@@ -200,6 +200,9 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
 
 void tgbm_trainer_destroy(tgbm_trainer *t) { delete t; }
 
+void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value) { t->impl->set_option(key, value); }
+void tgbm_trainer_sample_columns(tgbm_trainer *t) { t->impl->sample_columns(); }
+
 void tgbm_trainer_boost(tgbm_trainer *t, int rounds) {
     t->impl->boost(rounds);
     t->impl->sync();

@@ -111,6 +111,7 @@ struct TreeBuffers {
     // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1]) (whole features)
     const int *pack_begin = nullptr;
     int n_packs = 0;
+    const uint8_t *ignored = nullptr;  // [F] columns whose candidates score 0 this round (nullptr: none)
     const int *cut_row_ptr = nullptr;
     const int *cut_fid = nullptr;
     const float *cut_val = nullptr;

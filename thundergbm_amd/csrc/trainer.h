@@ -30,6 +30,8 @@ class Trainer {
     // One call = `rounds` iterations of Booster::boost: gradients, tree_per_rounds trees, metric.
     void boost(int rounds);
     // step-wise driving (used by parity tests)
+    void sample_columns();  // column sampling of one boosting round (no-op for rate >= 1); boost() calls it
+    void set_option(const std::string &key, double value);  // "column_sampling_rate"
     void compute_gradient();
     void tree_init(int k);
     void find_split(int level);  // histogram, merge/subtract, split search, update_tree
@@ -85,6 +87,8 @@ class Trainer {
     int trees_built_ = 0, rounds_done_ = 0, model_cap_trees_ = 0;
     float *d_metric_ = nullptr;
     double *d_metric_scratch_ = nullptr;
+    std::vector<uint8_t> h_ignored_;
+    uint8_t *d_ignored_ = nullptr;
     int cur_class_ = 0;
     bool in_boost_ = false;
     int lookup_level_ = -1;          // level whose split nodes have not been partitioned into row lists yet

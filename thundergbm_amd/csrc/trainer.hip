@@ -80,8 +80,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 255,
                "max_num_bin %d out of the supported range 2..255", param.max_num_bin);
     TGBM_CHECK(objective_supported(param.objective), "undefined objective %s", param.objective.c_str());
-    if (param.bagging || param.column_sampling_rate < 1.f)
-        log_info("bagging / column sampling are not part of this build and are ignored");
+    if (param.bagging) log_info("bagging is ignored (the reference never calls its row sampler either)");
+    TGBM_CHECK(param.column_sampling_rate > 0.f, "column_sampling_rate must be positive");
     // class bookkeeping of TreeTrainer::train (src/thundergbm/trainer.cu:24-37)
     if (param.objective.find("multi:") != std::string::npos || param.objective.find("binary:") != std::string::npos) {
         int nc = (int)ds.label.size();
@@ -388,6 +388,37 @@ void Trainer::compute_gradient() {
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
 }
 
+// Shard::column_sampling (src/thundergbm/builder/shard.cu:8-22), once per boosting round
+// (builder/tree_builder.cu:150-152): the columns 0..F-1 are shuffled the way libstdc++'s
+// std::random_shuffle does it (i = 1..F-1: swap with position rand() % (i + 1), process-wide rand() as
+// in the reference) and the first max(1, int(F * rate)) of them are ignored by this round's split search.
+void Trainer::sample_columns() {
+    if (!(param_.column_sampling_rate < 1.f)) return;
+    std::vector<int> idx(F_);
+    for (int i = 0; i < F_; ++i) idx[i] = i;
+    for (int i = 1; i < F_; ++i) {
+        const int j = std::rand() % (i + 1);
+        if (i != j) std::swap(idx[i], idx[j]);
+    }
+    const int sample_count = std::max(1, (int)(F_ * param_.column_sampling_rate));
+    h_ignored_.assign(F_, 0);
+    for (int i = 0; i < sample_count; ++i) h_ignored_[idx[i]] = 1;
+    if (d_ignored_ == nullptr) d_ignored_ = dalloc<uint8_t>((size_t)F_);
+    HIP_CHECK(hipMemcpyAsync(d_ignored_, h_ignored_.data(), (size_t)F_, hipMemcpyHostToDevice, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));  // h_ignored_ is reused by the next round
+    tb_.ignored = d_ignored_;
+}
+
+void Trainer::set_option(const std::string &key, double value) {
+    if (key == "column_sampling_rate") {
+        TGBM_CHECK(value > 0, "column_sampling_rate must be positive");
+        param_.column_sampling_rate = (float)value;
+        if (!(value < 1)) tb_.ignored = nullptr;
+    } else {
+        fatal("unknown trainer option %s", key.c_str());
+    }
+}
+
 // Buffer set of class tree k, and the first set with the item target of a whole round built at once.
 TreeBuffers Trainer::set_of(int k) const { return tb_.for_class(n_sets_ > 1 ? k : 0); }
 
@@ -506,6 +537,7 @@ void Trainer::boost(int rounds) {
     for (int r = 0; r < rounds; ++r) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
         const bool fuse = objective_ != OBJ_SOFTMAX && param_.tree_per_rounds == 1;
+        sample_columns();
         if (!next_round_ready_) compute_gradient();
         if (n_sets_ > 1) {
             build_round_together();

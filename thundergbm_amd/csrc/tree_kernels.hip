@@ -782,7 +782,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
     __syncthreads();
     long long incg[4], inch[4];
     int lastb[4];  // pack-relative index of the last bin of the element's feature
-    bool valid[4], head[4], last[4];
+    bool valid[4], head[4], last[4], ign[4];
     long long rung = 0, runh = 0;
     bool any_head = false;
 #pragma unroll
@@ -792,10 +792,12 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
         lastb[j] = 0;
         head[j] = false;
         last[j] = false;
+        ign[j] = false;
         incg[j] = inch[j] = 0;
         if (valid[j]) {
             const longlong2 v = s_v[w][lane * 4 + j];
             const int f = tb.cut_fid[b];
+            ign[j] = tb.ignored != nullptr && tb.ignored[f] != 0;
             const int fend = tb.cut_row_ptr[f + 1];
             head[j] = tb.cut_row_ptr[f] == b;
             last[j] = fend == b + 1;
@@ -866,6 +868,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
             GHPair l2{l.g + m.g, l.h + m.h};
             float gl = split_gain(S, l2, mcw, lambda);
             float score = (gl > gr) ? gl : -gr;
+            if (ign[j]) score = 0.f;  // column sampling: hist_tree_builder_single.cu:304 / :663
             float a = fabsf(score);
             if (a > best) {
                 best = a;

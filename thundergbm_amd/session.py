@@ -64,6 +64,12 @@ class Session:
     def base_score(self):
         return self.L.tgbm_trainer_base_score(self.h)
 
+    def set_option(self, key, value):
+        self.L.tgbm_trainer_set_option(self.h, key.encode(), float(value))
+
+    def sample_columns(self):
+        self.L.tgbm_trainer_sample_columns(self.h)
+
     def boost(self, rounds=1):
         self.L.tgbm_trainer_boost(self.h, rounds)
 
