@@ -541,6 +541,22 @@ def test_full_size_properties_config4_sparse(T):
     _check_boosted_round(T, val, rp, col, y, 100000, objective="binary:logistic", depth=8, max_num_bin=63)
 
 
+def test_estimator_cross_validation(T):
+    """TGBMModel.cv (python/thundergbm/thundergbm.py:223-282): five folds from a seeded permutation; the
+    test accuracy of a separable problem is high and below the train accuracy's ceiling of 1."""
+    rng = np.random.default_rng(3)
+    X = rng.standard_normal((3000, 6)).astype(np.float32)
+    y = (X[:, 0] + 0.5 * X[:, 1] > 0).astype(np.float32)
+    clf = T.TGBMClassifier(depth=4, n_trees=10, objective="binary:logistic", learning_rate=0.5, verbose=0)
+    res = clf.cv(X, y, nfold=5, seed=1)
+    assert set(res) == {"train-accuracy-mean", "train-accuracy-std", "test-accuracy-mean", "test-accuracy-std"}
+    assert 0.9 < res["test-accuracy-mean"] <= res["train-accuracy-mean"] <= 1.0
+    reg = T.TGBMRegressor(depth=4, n_trees=10, objective="reg:linear", learning_rate=0.5, verbose=0)
+    yr = (X @ rng.standard_normal(6)).astype(np.float32)
+    res = reg.cv(X, yr, nfold=4, shuffle=False)
+    assert res["train-RMSE-mean"] < res["test-RMSE-mean"] < float(np.var(yr))
+
+
 def test_cli_train_and_predict_on_a1a(T, tmp_path):
     """thundergbm-train <conf> + thundergbm-predict <conf> (reference: docs/how-to.md:20-31): LIBSVM
     loader, key=value parser, model file with base score, predictor and metric."""

@@ -162,6 +162,49 @@ class TGBMModel(BaseEstimator):
             trees.append(d)
         return trees
 
+    def get_shap_trees(self):
+        """The trees as shap.explainers.tree.Tree objects (python/thundergbm/thundergbm.py:284-348); like
+        the reference only for models with one tree per iteration, and only when shap is installed."""
+        if self.objective != "binary:logistic" and self.tree_per_iter != 1:
+            raise RuntimeError("not supported yet!")
+        import shap.explainers.tree as shap_tree
+        return [shap_tree.Tree(t) for t in self.get_trees()[:: max(self.tree_per_iter, 1)]]
+
+    def cv(self, X, y, folds=None, nfold=5, shuffle=True, seed=0):
+        """k-fold cross-validation with the reference's fold construction and result keys
+        (python/thundergbm/thundergbm.py:223-282): fold size int(n / nfold), folds cut from a seeded
+        permutation, accuracy for classifiers and mean squared error (reported under the RMSE keys, as
+        there) for regressors."""
+        import statistics
+
+        X = _csr(X)
+        y = np.ascontiguousarray(y, dtype=np.float32)
+        n = X.shape[0]
+        if folds is not None:
+            train_ids = [f[0] for f in folds]
+            test_ids = [f[1] for f in folds]
+            nfold = len(folds)
+        else:
+            order = np.random.RandomState(seed).permutation(n) if shuffle else np.arange(n)
+            step = int(n / nfold)
+            test_ids = [order[i:i + step] for i in range(0, n, step)]
+            train_ids = [np.concatenate([test_ids[i] for i in range(nfold) if i != k]) for k in range(nfold)]
+        classifier = getattr(self, "_impl", "") == "classifier"
+        train_scores, test_scores = [], []
+        for k in range(nfold):
+            self.fit(X[train_ids[k], :], y[train_ids[k]])
+            for ids, scores in ((train_ids[k], train_scores), (test_ids[k], test_scores)):
+                pred = self.predict(X[ids, :])
+                if classifier:
+                    scores.append(float(np.mean(pred == y[ids])))
+                else:
+                    scores.append(float(np.mean((pred - y[ids]) ** 2)))
+        name = "accuracy" if classifier else "RMSE"
+        self.eval_res = {
+            "train-%s-mean" % name: statistics.mean(train_scores), "train-%s-std" % name: statistics.stdev(train_scores),
+            "test-%s-mean" % name: statistics.mean(test_scores), "test-%s-std" % name: statistics.stdev(test_scores)}
+        return self.eval_res
+
 
 class TGBMClassifier(TGBMModel, ClassifierMixin):
     _impl = "classifier"
