@@ -287,6 +287,24 @@ def test_column_sampling_matches_oracle(T, objective, kind, rate):
     s.close()
 
 
+@pytest.mark.parametrize("layout", ["dense", "sparse"])
+def test_training_is_bit_reproducible(T, layout):
+    """Histograms are exact integer sums (LDS and HBM atomics alike) and every float reduction has a fixed
+    order, so two runs on the same input give the same bytes - which the reference's float atomics do not."""
+    os.environ["TGBM_LAYOUT"] = layout
+    n, F = 40000, 20
+    val, rp, col = _ragged(n, F, 5, F)
+    y = _target(val, rp, col, n, F, 5, "bin")
+    kw = dict(objective="binary:logistic", n_trees=8, depth=6, max_num_bin=64, learning_rate=0.3)
+    runs = []
+    for _ in range(3):
+        s = T.Session(val, rp, col, y, **kw)
+        s.boost(8)
+        runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.metric_log().tobytes()))
+        s.close()
+    assert runs[0] == runs[1] == runs[2]
+
+
 def test_predict_transforms_through_the_c_abi(T):
     """sparse_predict_scikit for every objective against the oracle's predictor + transform on unseen rows."""
     n, F = 1500, 7
