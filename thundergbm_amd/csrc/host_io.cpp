@@ -124,40 +124,98 @@ void DataSet::group_label() {
     for (auto &th : pool) th.join();
 }
 
+// One chunk of LIBSVM text: whole lines in [b, e). strtof / strtol never run past a line end because a
+// newline is not part of a number and is never skipped as leading white space here.
+namespace {
+struct LibsvmChunk {
+    std::vector<float> y, val;
+    std::vector<int> col, row_len;
+    size_t max_fid = 0;
+};
+
+void parse_libsvm_chunk(const char *b, const char *e, LibsvmChunk &out) {
+    const char *line = b;
+    while (line < e) {
+        const char *eol = static_cast<const char *>(std::memchr(line, '\n', (size_t)(e - line)));
+        if (eol == nullptr) eol = e;
+        const char *p = line;
+        line = eol + 1;
+        while (p < eol && (*p == ' ' || *p == '\t')) ++p;
+        if (p >= eol || *p == '#' || *p == '\r') continue;
+        char *end = nullptr;
+        float lab = std::strtof(p, &end);
+        if (end == p) continue;
+        out.y.push_back(lab);
+        p = end;
+        int len = 0;
+        for (;;) {
+            while (p < eol && (*p == ' ' || *p == '\t' || *p == '\r')) ++p;
+            if (p >= eol || *p == '#') break;
+            long fid = std::strtol(p, &end, 10);
+            if (end == p || *end != ':') break;
+            p = end + 1;
+            if (p >= eol) break;
+            float v = std::strtof(p, &end);
+            if (end == p) break;
+            p = end;
+            out.col.push_back((int)fid - 1);
+            out.val.push_back(v);
+            ++len;
+            if ((size_t)fid > out.max_fid) out.max_fid = (size_t)fid;
+        }
+        out.row_len.push_back(len);
+    }
+}
+}  // namespace
+
 void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {
     log_info("loading LIBSVM dataset from file ## %s ##", file_name.c_str());
-    std::ifstream ifs(file_name, std::ifstream::binary);
+    std::ifstream ifs(file_name, std::ifstream::binary | std::ifstream::ate);
     TGBM_CHECK(ifs.is_open(), "file ## %s ## not found. ", file_name.c_str());
+    const size_t bytes = (size_t)ifs.tellg();
+    ifs.seekg(0);
+    std::string text(bytes + 1, '\0');  // one terminating NUL: the number parsers stop there
+    ifs.read(&text[0], (std::streamsize)bytes);
+    // chunks of whole lines, parsed by a few threads (the reference's loader splits the file the same way,
+    // src/thundergbm/dataset.cpp:170-320), then concatenated in file order
+    const int n_thr = bytes > (1u << 22) ? (int)std::min(16u, std::max(1u, std::thread::hardware_concurrency())) : 1;
+    std::vector<size_t> cut(n_thr + 1, bytes);
+    cut[0] = 0;
+    for (int t = 1; t < n_thr; ++t) {
+        size_t pos = std::max(cut[t - 1], bytes * t / n_thr);
+        const char *nl = pos < bytes ? static_cast<const char *>(std::memchr(text.data() + pos, '\n', bytes - pos)) : nullptr;
+        cut[t] = nl ? (size_t)(nl - text.data()) + 1 : bytes;
+    }
+    std::vector<LibsvmChunk> chunks(n_thr);
+    {
+        std::vector<std::thread> pool;
+        for (int t = 1; t < n_thr; ++t)
+            pool.emplace_back([&, t] { parse_libsvm_chunk(text.data() + cut[t], text.data() + cut[t + 1], chunks[t]); });
+        parse_libsvm_chunk(text.data() + cut[0], text.data() + cut[1], chunks[0]);
+        for (auto &th : pool) th.join();
+    }
     y.clear();
     label.clear();
     csr_val.clear();
     csr_col_idx.clear();
     csr_row_ptr.assign(1, 0);
     n_features_ = 0;
-    std::string line;
-    while (std::getline(ifs, line)) {
-        const char *p = line.c_str();
-        while (*p == ' ' || *p == '\t') ++p;
-        if (*p == '\0' || *p == '#' || *p == '\r') continue;
-        char *end = nullptr;
-        float lab = std::strtof(p, &end);
-        if (end == p) continue;
-        y.push_back(lab);
-        p = end;
-        for (;;) {
-            while (*p == ' ' || *p == '\t' || *p == '\r') ++p;
-            if (*p == '\0' || *p == '#') break;
-            long fid = std::strtol(p, &end, 10);
-            if (end == p || *end != ':') break;
-            p = end + 1;
-            float v = std::strtof(p, &end);
-            if (end == p) break;
-            p = end;
-            csr_col_idx.push_back((int)fid - 1);
-            csr_val.push_back(v);
-            if ((size_t)fid > n_features_) n_features_ = (size_t)fid;
-        }
-        csr_row_ptr.push_back((int)csr_val.size());
+    size_t rows = 0, entries = 0;
+    for (const LibsvmChunk &c : chunks) {
+        rows += c.y.size();
+        entries += c.val.size();
+    }
+    TGBM_CHECK(entries < ((size_t)1 << 31), "more than 2^31 stored values");
+    y.reserve(rows);
+    csr_val.reserve(entries);
+    csr_col_idx.reserve(entries);
+    csr_row_ptr.reserve(rows + 1);
+    for (const LibsvmChunk &c : chunks) {
+        y.insert(y.end(), c.y.begin(), c.y.end());
+        csr_val.insert(csr_val.end(), c.val.begin(), c.val.end());
+        csr_col_idx.insert(csr_col_idx.end(), c.col.begin(), c.col.end());
+        for (int len : c.row_len) csr_row_ptr.push_back(csr_row_ptr.back() + len);
+        n_features_ = std::max(n_features_, c.max_fid);
     }
     val = csr_val.data();
     row_ptr = csr_row_ptr.data();
