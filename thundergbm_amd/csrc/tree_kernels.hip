@@ -1663,7 +1663,10 @@ static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const Dens
     const int slots = (tb.max_block_bins + kHistBlock - 1) / kHistBlock;  // bins drained per thread
     if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level, n_class);
     else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 3) hist_dense_launch<LPR, 3>(s, tb, bins, gh, level, n_class);
     else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 6) hist_dense_launch<LPR, 6>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 7) hist_dense_launch<LPR, 7>(s, tb, bins, gh, level, n_class);  // fewer accumulator registers
     else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level, n_class);
     else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level, n_class);
     else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
