@@ -396,7 +396,8 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         // the next step's rows are requested before this step's atomics (and before a drain's
         // barriers), so the memory pipeline stays busy
         if (base + RPS * U < end) load_rows(base + RPS * U, pk_next, s_next);
-        if (pending + RPS * U > kHistFlushEvery) {
+        const int step_rows = min(RPS * U, end - base);
+        if (pending + step_rows > kHistFlushEvery) {
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < SLOTS; ++k) {
@@ -412,7 +413,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
             __syncthreads();
             pending = 0;
         }
-        pending += RPS * U;
+        pending += step_rows;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const unsigned v = pk[u];
