@@ -366,7 +366,8 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     const int begin = s_range[0], end = s_range[1];
     const float scale_g = quant->scale_g, scale_h = quant->scale_h;
     constexpr int RPS = BLK / LPR;  // rows per step of the whole block
-    constexpr int U = 4;
+    // steps in flight per thread: three keep the 64-register variants (8 waves per SIMD) free of spills
+    constexpr int U = SLOTS <= 8 ? 3 : 4;
     static_assert(RPS * U <= kHistFlushRows, "one iteration must not exceed the flush interval");
     const int q = threadIdx.x % LPR;
     const int rsub = threadIdx.x / LPR;
@@ -1067,14 +1068,22 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     const bool dr = nd.default_right;
     const uint8_t *column = bins.col + (size_t)f * bins.col_stride;
     int nleft = 0;
+    // all row ids first, then all bin bytes, then the stores: the three phases keep a thread's eight
+    // gathers in flight together (the byte store may alias the byte loads for the compiler)
+    constexpr int R = kPartChunk / kBlock;
+    int row[R], b[R];
 #pragma unroll
-    for (int k = 0; k < kPartChunk / kBlock; ++k) {
-        int pos = pb + k * kBlock + threadIdx.x;
-        if (pos < pe) {
-            int row = DIRECT ? pos : ridx[pos];
-            int b = column[row];
-            bool right = (b == kMissingBin) ? dr : (b >= sbid);
-            tb.goes_right[pos] = right ? 1 : 0;
+    for (int k = 0; k < R; ++k) {
+        const int pos = pb + k * kBlock + threadIdx.x;
+        row[k] = pos < pe ? (DIRECT ? pos : ridx[pos]) : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < R; ++k) b[k] = row[k] >= 0 ? column[row[k]] : 0;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        if (row[k] >= 0) {
+            const bool right = (b[k] == kMissingBin) ? dr : (b[k] >= sbid);
+            tb.goes_right[pb + k * kBlock + threadIdx.x] = right ? 1 : 0;
             nleft += right ? 0 : 1;
         }
     }
