@@ -32,9 +32,10 @@ void set_logger(int verbose);
 /* scikit_tgbm.cpp:26-80. CSR input (float32 values, int32 indices, ascending columns per row).
  * num_class is in/out, group_label receives the distinct labels (caller allocates one float per
  * distinct label), tree_per_iter and *model are outputs. column_sampling_rate < 1 samples columns per
- * round as the reference does (see tgbm_trainer_set_option). n_device, bagging (never applied by the
- * reference either), n_parallel_trees, group and num_group are accepted for signature compatibility and
- * ignored. */
+ * round as the reference does (see tgbm_trainer_set_option). group / num_group are the query group sizes
+ * of the ranking objectives (rank:pairwise, rank:ndcg; dataset.cpp:64-68) and ignored otherwise. n_device,
+ * bagging (never applied by the reference either) and n_parallel_trees are accepted for signature
+ * compatibility and ignored. */
 void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *label, int depth, int n_trees,
                          int n_device, float min_child_weight, float lambda, float gamma, int max_num_bin,
                          int verbose, float column_sampling_rate, int bagging, int n_parallel_trees,
@@ -42,7 +43,8 @@ void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, f
                          int *tree_per_iter, float *group_label, int *group, int num_group);
 
 /* scikit_tgbm.cpp:83-121. y_pred: row_size floats, or row_size * num_class (class-major) for
- * multi:softprob. As in the reference the base score is not part of this path. */
+ * multi:softprob. As in the reference the base score is not part of this path. group / num_group: query
+ * groups of the rows for a ranking objective; they only feed the metric line of the log and may be absent. */
 void sparse_predict_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *y_pred, tgbm_model **model,
                            int n_trees, int trees_per_iter, char *objective, int num_class, float learning_rate,
                            float *group_label, int *group, int num_group, int verbose);
@@ -80,6 +82,15 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
                                   const float *label, int depth, int n_trees, float min_child_weight, float lambda,
                                   float gamma, int max_num_bin, float learning_rate, const char *objective,
                                   int num_class, int verbose);
+/* The same with query groups for the ranking objectives rank:pairwise / rank:ndcg (LambdaRank,
+ * LambdaRankNDCG: objective/ranking_obj.cpp:11-18, :100-103): `group` holds num_group sizes of consecutive
+ * runs of rows that sum to row_size, as in the group / num_group arguments of sparse_train_scikit
+ * (scikit_tgbm.cpp:31, dataset.cpp:64-68). Other objectives ignore them. */
+tgbm_trainer *tgbm_trainer_create_grouped(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
+                                          const float *label, int depth, int n_trees, float min_child_weight,
+                                          float lambda, float gamma, int max_num_bin, float learning_rate,
+                                          const char *objective, int num_class, int verbose, const int *group,
+                                          int num_group);
 void tgbm_trainer_destroy(tgbm_trainer *t);
 
 /* Options that tgbm_trainer_create has no argument for. "column_sampling_rate" (GBMParam, common.h:92):
@@ -111,7 +122,8 @@ float tgbm_trainer_base_score(tgbm_trainer *t);
 
 /* Copies a device buffer to `out` when `cap` is large enough; always returns its size in bytes.
  * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist_q0, hist_q1,
- * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels. After tgbm_trainer_boost `gh` may already
+ * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels, rank_order (ranking objectives: the rows in
+ * the order of the last gradient or metric pass). After tgbm_trainer_boost `gh` may already
  * hold the gradients of the next round (single-tree objectives compute them in the round's last pass). */
 size_t tgbm_trainer_get(tgbm_trainer *t, const char *name, void *out, size_t cap);
 /* Overwrites gh or y_pred (lock-step tests feed both implementations the same state). */

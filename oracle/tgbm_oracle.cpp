@@ -20,9 +20,15 @@
 //   prune           hand-built 7-node trees
 //   predictor       equality with the training-time prediction on the training rows
 //   metrics         reference KATs src/test/test_metrics.cpp:70,84,96; tree size src/test/test_tree.cpp:68
+//   ranking         LambdaRank gradients: two-row groups (closed form), pair bookkeeping by brute force over the
+//                   group (every drawing position pairs with a position outside its run of equal labels, the
+//                   lambdas of a pair cancel), |delta NDCG| = the change of DCG when the two positions swap;
+//                   MAP / NDCG: hand-computed lists, a perfect ranking scores 1
 // Parity unpinned (no run of the reference is possible): the association order of the reference's
 // fp32 sums (atomics, thrust scan/reduce), device expf ulps, ordering of +0.0/-0.0 duplicates in
-// the cut-point sort.
+// the cut-point sort; for the ranking objectives the tie order of std::sort and the std::mt19937 partner
+// draws seeded from rand() inside an OpenMP loop (both unspecified in the reference: ties keep row order here
+// and draws are a function of (round seed, position)).
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -89,6 +95,7 @@ struct Oracle {
     std::vector<int> col, row_ptr;
     std::vector<float> y;      // mapped to class index for classification
     std::vector<float> label;  // distinct labels
+    std::vector<int> group;    // query group sizes (ranking objectives, dataset.cpp:64-68)
     // params (GBMParam, include/thundergbm/common.h:86-111)
     int depth = 6, n_trees = 40, max_num_bin = 255, num_class = 1, tree_per_rounds = 1;
     float mcw = 1, lambda = 1, gamma = 1, rt_eps = 1e-6f, lr = 1, base_score = 0;
@@ -618,6 +625,160 @@ void predict_in_training(Oracle &o, int k) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Ranking objectives. NDCG::discounted_gain, include/thundergbm/metric/ranking_metric.h:43-45.
+inline float discounted_gain(int label, int rank) { return ((1 << label) - 1) / log2f(rank + 1 + 1); }
+
+// NDCG::get_IDCG, src/thundergbm/metric/rank_metric.cpp:106-123
+std::vector<float> get_idcg(const std::vector<int> &gptr, const float *y) {
+    const int n_group = (int)gptr.size() - 1;
+    std::vector<float> idcg(n_group, 0.f);
+    for (int k = 0; k < n_group; ++k) {
+        std::vector<float> sorted_label(y + gptr[k], y + gptr[k + 1]);
+        std::sort(sorted_label.begin(), sorted_label.end(), std::greater<float>());
+        for (size_t i = 0; i < sorted_label.size(); ++i) idcg[k] += discounted_gain((int)sorted_label[i], (int)i);
+    }
+    return idcg;
+}
+
+// RankListMetric::configure_gptr, rank_metric.cpp:39-44
+std::vector<int> make_gptr(const std::vector<int> &group) {
+    std::vector<int> gptr(group.size() + 1, 0);
+    for (size_t i = 1; i < gptr.size(); ++i) gptr[i] = gptr[i - 1] + group[i - 1];
+    return gptr;
+}
+
+// The partner draw that stands in for std::uniform_int_distribution over std::mt19937(std::rand()): a pure
+// function of the round's seed and the drawing row's position in the dataset-wide (group, label order) list.
+inline unsigned rank_draw(unsigned seed, unsigned pos, unsigned range) {
+    unsigned long long x = ((unsigned long long)seed << 32) | pos;
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    return (unsigned)(((x >> 32) * (unsigned long long)range) >> 32);
+}
+
+// LambdaRank::get_gradient, src/thundergbm/objective/ranking_obj.cpp:20-96, with get_delta_z of LambdaRank
+// (ranking_obj.h:32) or LambdaRankNDCG (ranking_obj.cpp:105-113). The sums per row are kept in double and
+// rounded once. order_out (optional): row at every position of the (label, score) order; pair_out (optional):
+// per position the partner's position or -1.
+void rank_gradient(bool ndcg, int n, const float *y, const float *score0, const std::vector<int> &group, unsigned seed,
+                   GH *gh, int *order_out, int *pair_out) {
+    const std::vector<int> gptr = make_gptr(group);
+    std::vector<float> idcg;
+    if (ndcg) idcg = get_idcg(gptr, y);
+    std::vector<double> acc(2 * (size_t)n, 0.0);
+    if (pair_out)
+        for (int i = 0; i < n; ++i) pair_out[i] = -1;
+    const int n_group = (int)group.size();
+    for (int k = 0; k < n_group; ++k) {
+        const int group_start = gptr[k];
+        const int len = gptr[k + 1] - group_start;
+        const float *score = score0 + group_start;
+        const float *label_data = y + group_start;
+        std::vector<int> idx(len);
+        for (int i = 0; i < len; ++i) idx[i] = i;
+        std::stable_sort(idx.begin(), idx.end(), [=](int a, int b) { return score[a] > score[b]; });
+        std::vector<std::pair<float, int>> label_idx(len);
+        for (int i = 0; i < len; ++i) {
+            label_idx[i].first = label_data[idx[i]];
+            label_idx[i].second = idx[i];
+        }
+        std::stable_sort(label_idx.begin(), label_idx.end(),
+                         [](const std::pair<float, int> &a, const std::pair<float, int> &b) { return a.first > b.first; });
+        if (order_out)
+            for (int i = 0; i < len; ++i) order_out[group_start + i] = group_start + label_idx[i].second;
+        for (int i = 0; i < len; ++i) {
+            int j = i + 1;
+            while (j < len && label_idx[i].first == label_idx[j].first) j++;
+            const int nleft = i;
+            const int nright = len - j;
+            if (nleft + nright != 0) {
+                for (int l = i; l < j; ++l) {
+                    const int m = (int)rank_draw(seed, (unsigned)(group_start + l), (unsigned)(nleft + nright));
+                    int high = 0, low = 0;
+                    if (m < nleft) {
+                        high = m;
+                        low = l;
+                    } else {
+                        high = l;
+                        low = m + j - i;
+                    }
+                    if (pair_out) pair_out[group_start + l] = group_start + (m < nleft ? high : low);
+                    const float high_label = label_idx[high].first;
+                    const float low_label = label_idx[low].first;
+                    const int high_idx = label_idx[high].second;
+                    const int low_idx = label_idx[low].second;
+                    float delta_z = 1;
+                    if (ndcg) {
+                        if (idcg[k] == 0) {
+                            delta_z = 0;
+                        } else {
+                            const float dgI1 = discounted_gain((int)high_label, high);
+                            const float dgJ1 = discounted_gain((int)low_label, low);
+                            const float dgI2 = discounted_gain((int)high_label, low);
+                            const float dgJ2 = discounted_gain((int)low_label, high);
+                            delta_z = (dgI1 + dgJ1 - dgI2 - dgJ2) / idcg[k];
+                        }
+                    }
+                    const float abs_delta_z = fabsf(delta_z);
+                    const float rhoIJ = 1 / (1 + expf((score[high_idx] - score[low_idx])));
+                    const float lambda = -abs_delta_z * rhoIJ;
+                    const float hessian = 2 * fmaxf(abs_delta_z * rhoIJ * (1 - rhoIJ), 1e-16f);
+                    acc[2 * (size_t)(group_start + high_idx)] += lambda;
+                    acc[2 * (size_t)(group_start + high_idx) + 1] += hessian;
+                    acc[2 * (size_t)(group_start + low_idx)] -= lambda;
+                    acc[2 * (size_t)(group_start + low_idx) + 1] += hessian;
+                }
+            }
+            i = j;  // and the loop header adds one more: the first position of the next run is stepped over
+        }
+    }
+    for (int i = 0; i < n; ++i) gh[i] = GH{(float)acc[2 * (size_t)i], (float)acc[2 * (size_t)i + 1]};
+}
+
+// RankListMetric::get_score with MAP::eval_query_group / NDCG::eval_query_group, rank_metric.cpp:9-104
+// (topn = INT_MAX). Ties between equal scores keep row order.
+float rank_metric(bool ndcg, int n, const float *y, const float *yp, const std::vector<int> &group) {
+    const std::vector<int> gptr = make_gptr(group);
+    std::vector<float> idcg;
+    if (ndcg) idcg = get_idcg(gptr, y);
+    const int n_group = (int)group.size();
+    float sum_score = 0;
+    for (int k = 0; k < n_group; ++k) {
+        const int len = gptr[k + 1] - gptr[k];
+        const float *label = y + gptr[k];
+        const float *score = yp + gptr[k];
+        std::vector<int> idx(len);
+        for (int i = 0; i < len; ++i) idx[i] = i;
+        std::stable_sort(idx.begin(), idx.end(), [=](int a, int b) { return score[a] > score[b]; });
+        if (ndcg) {
+            if (idcg[k] == 0) {
+                sum_score += 1;
+                continue;
+            }
+            float dcg = 0;
+            for (int i = 0; i < len; ++i) dcg += discounted_gain((int)label[idx[i]], i);
+            sum_score += dcg / idcg[k];
+        } else {
+            int nhits = 0;
+            double sum_ap = 0;
+            for (int i = 0; i < len; ++i) {
+                if (label[idx[i]] != 0) {
+                    nhits++;
+                    sum_ap += (double)nhits / (i + 1);
+                }
+            }
+            sum_score += nhits != 0 ? (float)(sum_ap / nhits) : 1.f;
+        }
+    }
+    (void)n;
+    return sum_score / n_group;
+}
+
+bool is_rank(const std::string &obj) { return obj == "rank:pairwise" || obj == "rank:ndcg"; }
+
 // a12  metrics: RMSE src/thundergbm/metric/pointwise_metric.cu:8-22, accuracy / error
 // src/thundergbm/metric/multiclass_metric.cu:9-46
 float metric(const std::string &obj, int n, int num_class, const float *y, const float *yp) {
@@ -686,14 +847,21 @@ void build_tree(Oracle &o, int k) {
 // Booster::boost, include/thundergbm/booster.h:76-93
 void boost_round(Oracle &o) {
     sample_columns(o);
-    gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+    if (is_rank(o.objective))
+        rank_gradient(o.objective == "rank:ndcg", o.n, o.y.data(), o.y_pred.data(), o.group, (unsigned)std::rand(),
+                      o.gh.data(), nullptr, nullptr);
+    else
+        gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
     std::vector<Node> round_trees;
     for (int k = 0; k < o.tree_per_rounds; ++k) {
         build_tree(o, k);
         round_trees.insert(round_trees.end(), o.nodes.begin(), o.nodes.end());
     }
     o.model.push_back(round_trees);
-    o.metric_log.push_back(metric(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data()));
+    if (is_rank(o.objective))
+        o.metric_log.push_back(rank_metric(o.objective == "rank:ndcg", o.n, o.y.data(), o.y_pred.data(), o.group));
+    else
+        o.metric_log.push_back(metric(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data()));
 }
 
 // a13  Predictor::predict_raw, src/thundergbm/predictor.cu:32-189. double accumulation when the
@@ -837,6 +1005,18 @@ void orc_prepare(void *h) {
     init_base_score(o);
 }
 
+void orc_set_groups(void *h, const int *group, int num_group) {
+    ((Oracle *)h)->group.assign(group, group + num_group);
+}
+// one LambdaRank gradient pass; order_out / pair_out may be null
+void orc_rank_gradient(int ndcg, int n, const float *y, const float *score, const int *group, int num_group,
+                       unsigned seed, float *gh, int *order_out, int *pair_out) {
+    rank_gradient(ndcg != 0, n, y, score, std::vector<int>(group, group + num_group), seed, (GH *)gh, order_out,
+                  pair_out);
+}
+float orc_rank_metric(int ndcg, int n, const float *y, const float *score, const int *group, int num_group) {
+    return rank_metric(ndcg != 0, n, y, score, std::vector<int>(group, group + num_group));
+}
 void orc_set_column_sampling_rate(void *h, float rate) { ((Oracle *)h)->column_sampling_rate = rate; }
 void orc_sample_columns(void *h) { sample_columns(*(Oracle *)h); }
 void orc_boost(void *h, int rounds) {
@@ -847,7 +1027,11 @@ void orc_boost(void *h, int rounds) {
 // step-wise driving for lock-step tests
 void orc_compute_gradient(void *h) {
     Oracle &o = *(Oracle *)h;
-    gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+    if (is_rank(o.objective))
+        rank_gradient(o.objective == "rank:ndcg", o.n, o.y.data(), o.y_pred.data(), o.group, (unsigned)std::rand(),
+                      o.gh.data(), nullptr, nullptr);
+    else
+        gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
 }
 void orc_tree_init(void *h, int k) { tree_init(*(Oracle *)h, k); }
 void orc_find_split(void *h, int level) { find_split(*(Oracle *)h, level); }
@@ -861,6 +1045,7 @@ void orc_predict_in_training(void *h, int k) { predict_in_training(*(Oracle *)h,
 void orc_build_tree(void *h, int k) { build_tree(*(Oracle *)h, k); }
 float orc_metric(void *h) {
     Oracle &o = *(Oracle *)h;
+    if (is_rank(o.objective)) return rank_metric(o.objective == "rank:ndcg", o.n, o.y.data(), o.y_pred.data(), o.group);
     return metric(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data());
 }
 

@@ -46,6 +46,13 @@ def lib():
         L.orc_boost.argtypes = [C.c_void_p, C.c_int]
         L.orc_set_column_sampling_rate.argtypes = [C.c_void_p, C.c_float]
         L.orc_sample_columns.argtypes = [C.c_void_p]
+        L.orc_set_groups.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_set_groups.restype = None
+        L.orc_rank_gradient.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_uint,
+                                        C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_rank_gradient.restype = None
+        L.orc_rank_metric.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_rank_metric.restype = C.c_float
         for name in ("orc_tree_init", "orc_find_split", "orc_predict_in_training", "orc_build_tree"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_int]
             getattr(L, name).restype = None
@@ -111,7 +118,7 @@ def dense_to_csr(X):
 class Oracle:
     def __init__(self, val, row_ptr, col, y, depth=6, n_trees=40, min_child_weight=1.0, lambda_=1.0, gamma=1.0,
                  max_num_bin=255, learning_rate=1.0, objective="reg:linear", num_class=1, debug=False,
-                 shadow64=False):
+                 shadow64=False, groups=None):
         self.L = lib()
         self.val = np.ascontiguousarray(val, dtype=np.float32)
         self.row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
@@ -125,6 +132,9 @@ class Oracle:
                                    min_child_weight, lambda_, gamma, max_num_bin, learning_rate,
                                    objective.encode(), num_class)
         self.L.orc_set_debug(self.h, int(debug), int(shadow64))
+        if groups is not None:
+            grp = np.ascontiguousarray(groups, dtype=np.int32)
+            self.L.orc_set_groups(self.h, _p(grp), len(grp))
         self.shadow64 = shadow64
 
     def __del__(self):
@@ -315,6 +325,30 @@ def gradient(objective, y, yp, num_class=1):
     out = np.zeros((yp.size, 2), dtype=np.float32)
     L.orc_gradient(objective.encode(), n, num_class, _p(y), _p(yp), _p(out))
     return out
+
+
+def rank_gradient(objective, y, score, groups, seed):
+    """One LambdaRank pass: (gh [n, 2], order [n] = row at every position of the (label, score) order of its
+    group, pair [n] = partner position of every drawing position or -1)."""
+    L = lib()
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    score = np.ascontiguousarray(score, dtype=np.float32)
+    grp = np.ascontiguousarray(groups, dtype=np.int32)
+    n = len(y)
+    gh = np.zeros((n, 2), dtype=np.float32)
+    order = np.zeros(n, dtype=np.int32)
+    pair = np.zeros(n, dtype=np.int32)
+    L.orc_rank_gradient(int(objective == "rank:ndcg"), n, _p(y), _p(score), _p(grp), len(grp), int(seed), _p(gh),
+                        _p(order), _p(pair))
+    return gh, order, pair
+
+
+def rank_metric(objective, y, score, groups):
+    L = lib()
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    score = np.ascontiguousarray(score, dtype=np.float32)
+    grp = np.ascontiguousarray(groups, dtype=np.int32)
+    return L.orc_rank_metric(int(objective == "rank:ndcg"), len(y), _p(y), _p(score), _p(grp), len(grp))
 
 
 def metric_score(objective, y, yp, num_class=1):

@@ -24,6 +24,8 @@ SIGNATURES = {
     "model_free": (None, [_P]),
     "tgbm_trainer_create": (_P, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
                                  C.c_float, C.c_char_p, C.c_int, C.c_int]),
+    "tgbm_trainer_create_grouped": (_P, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float,
+                                         C.c_int, C.c_float, C.c_char_p, C.c_int, C.c_int, _P, C.c_int]),
     "tgbm_trainer_destroy": (None, [_P]),
     "tgbm_trainer_set_option": (None, [_P, C.c_char_p, C.c_double]),
     "tgbm_trainer_sample_columns": (None, [_P]),

@@ -176,6 +176,16 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
                                   const float *label, int depth, int n_trees, float min_child_weight, float lambda,
                                   float gamma, int max_num_bin, float learning_rate, const char *objective,
                                   int num_class, int verbose) {
+    return tgbm_trainer_create_grouped(row_size, val, row_ptr, col_ptr, label, depth, n_trees, min_child_weight,
+                                       lambda, gamma, max_num_bin, learning_rate, objective, num_class, verbose,
+                                       nullptr, 0);
+}
+
+tgbm_trainer *tgbm_trainer_create_grouped(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
+                                          const float *label, int depth, int n_trees, float min_child_weight,
+                                          float lambda, float gamma, int max_num_bin, float learning_rate,
+                                          const char *objective, int num_class, int verbose, const int *group,
+                                          int num_group) {
     set_logger(verbose);
     tgbm_trainer *t = new tgbm_trainer;
     GBMParam &p = t->param;
@@ -190,7 +200,7 @@ tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row
     p.num_class = num_class;
     p.verbose = verbose;
     p.tree_method = "hist";
-    t->dataset.load_from_sparse(row_size, val, row_ptr, col_ptr, label, nullptr, 0, p);
+    t->dataset.load_from_sparse(row_size, val, row_ptr, col_ptr, label, group, num_group, p);
     t->impl.reset(new Trainer(t->dataset, p));
     t->dataset.val = nullptr;  // the caller's buffers are not referenced after this call
     t->dataset.col_idx = nullptr;

@@ -162,7 +162,7 @@ struct TreeBuffers {
 };
 
 // objective codes
-enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2 };
+enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2, OBJ_RANK = 3 };
 
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
@@ -218,6 +218,35 @@ struct DeviceCuts {
     std::vector<long> feature_nnz;  // host: stored values per feature
 };
 DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, const int *d_col, int max_num_bin);
+
+// Tile sums of the device-wide exclusive scan, one pair of arrays per recursion level (grown on demand).
+struct ScanScratch {
+    struct Level {
+        unsigned *sums = nullptr, *scanned = nullptr;
+        size_t cap = 0;
+    };
+    std::vector<Level> levels;
+    void release();
+};
+
+// out[i] = in[0] + ... + in[i-1] over n 32-bit counters, *d_total (device) = the sum of all of them.
+void device_exclusive_scan(hipStream_t s, const unsigned *in, unsigned *out, long n, unsigned *d_total,
+                           ScanScratch &sc);
+
+// Buffers of sort_pairs for up to `cap` (64-bit key, 32-bit payload) pairs; allocated once, reused per call.
+struct PairSorter {
+    long cap = 0, n_tiles = 0;
+    unsigned long long *keys[2] = {nullptr, nullptr};
+    int *vals[2] = {nullptr, nullptr};
+    unsigned *counts = nullptr, *offsets = nullptr, *d_total = nullptr;
+    ScanScratch scan;
+    void alloc(long n);
+    void release();
+};
+// Stable LSD radix sort (8 bits per pass) of the n pairs in keys[0] / vals[0] by the key bits [0, key_bits),
+// ascending. Returns which of the two buffer pairs (0 or 1) holds the result. Stream-ordered; allocates only
+// when the scan scratch has to grow (first call).
+int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
 
 // Host -> device copy of a large pageable array through pinned staging buffers (returns when done).
 void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);

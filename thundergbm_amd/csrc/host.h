@@ -36,9 +36,12 @@ struct DataSet {
     void load_from_file(const std::string &file_name, GBMParam &param);
     // src/thundergbm/dataset.cpp:83-101
     void group_label();
+    // src/thundergbm/dataset.cpp:71-81 (sizes of the query groups, one number per token)
+    void load_group_file(const std::string &file_name);
 };
 
 bool objective_needs_group_label(const std::string &objective);
+bool objective_needs_groups(const std::string &objective);  // rank:pairwise, rank:ndcg
 bool objective_supported(const std::string &objective);
 
 // Parameter parsing and the raw binary model format (src/thundergbm/parser.cpp).

@@ -50,9 +50,12 @@ bool objective_needs_group_label(const std::string &o) {
     return o == "multi:softprob" || o == "multi:softmax" || o == "binary:logistic";
 }
 
+// ObjectiveFunction::need_load_group_file (src/thundergbm/objective/objective_function.cu:23-25)
+bool objective_needs_groups(const std::string &o) { return o == "rank:pairwise" || o == "rank:ndcg"; }
+
 bool objective_supported(const std::string &o) {
     return o == "reg:linear" || o == "reg:logistic" || o == "binary:logistic" || o == "multi:softprob" ||
-           o == "multi:softmax";
+           o == "multi:softmax" || objective_needs_groups(o);
 }
 
 void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr, const int *col_idx,
@@ -89,8 +92,22 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
         group_label();
         param.num_class = (int)label.size();
     }
-    (void)grp;
-    (void)num_group;  // query groups belong to the ranking objectives, which this library does not train
+    // query group sizes of the ranking objectives (dataset.cpp:64-68)
+    if (objective_needs_groups(param.objective)) {
+        for (int i = 0; i < num_group; ++i) group.push_back(grp[i]);
+        log_info("#groups = %zu", group.size());
+    }
+}
+
+// dataset.cpp:71-81: one group size per whitespace-separated token
+void DataSet::load_group_file(const std::string &file_name) {
+    log_info("loading group info from file \"%s\"", file_name.c_str());
+    group.clear();
+    std::ifstream ifs(file_name);
+    TGBM_CHECK(ifs.is_open(), "ranking objective needs a group file, but file %s not found", file_name.c_str());
+    int group_size;
+    while (ifs >> group_size) group.push_back(group_size);
+    log_info("#groups = %zu", group.size());
 }
 
 void DataSet::group_label() {
@@ -223,6 +240,7 @@ void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {
     nnz = (long)csr_val.size();
     label = y;  // the reference keeps a copy of all labels here (dataset.cpp:290-291) ...
     log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
+    if (objective_needs_groups(param.objective)) load_group_file(file_name + ".group");  // dataset.cpp:302
     if (objective_needs_group_label(param.objective)) {
         group_label();  // ... which grouping replaces by the distinct ones
         param.num_class = (int)label.size();

@@ -3,6 +3,7 @@
 
 #include "device_api.h"
 #include "host.h"
+#include "rank.h"
 
 namespace tgbm {
 
@@ -58,7 +59,24 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     launch_predict(s, n, F, d_row_ptr, d_col, d_val, d_model, n_iter, nct, n_nodes, param.learning_rate,
                    param.base_score, d_out);
     size_t n_ret = n_out;
-    if (log_metric && (int)ds.y.size() == n && n > 0) {
+    if (log_metric && objective_needs_groups(param.objective)) {
+        // MAP / NDCG need the query groups of the rows that are scored (Predictor::predict configures the
+        // objective with the dataset's groups, predictor.cu:16-24); without them the metric line is left out
+        long covered = 0;
+        for (int g : ds.group) covered += g;
+        if (!ds.group.empty() && covered == (long)n && (int)ds.y.size() == n) {
+            const bool ndcg = param.objective == "rank:ndcg";
+            RankContext rc(s, ds.y, ds.group, ndcg);
+            float *d_m = nullptr;
+            HIP_CHECK(hipMalloc(&d_m, sizeof(float)));
+            rc.metric(ndcg ? RANK_METRIC_NDCG : RANK_METRIC_MAP, d_out, d_m);
+            float v = 0;
+            HIP_CHECK(hipMemcpyAsync(&v, d_m, sizeof(float), hipMemcpyDeviceToHost, s));
+            HIP_CHECK(hipStreamSynchronize(s));
+            log_info("%s = %g", ndcg ? "NDCG" : "MAP", v);
+            HIP_CHECK(hipFree(d_m));
+        }
+    } else if (log_metric && (int)ds.y.size() == n && n > 0) {
         int kind = 0;
         if (param.objective == "binary:logistic") kind = 1;
         if (param.objective.find("multi:") == 0) kind = 2;

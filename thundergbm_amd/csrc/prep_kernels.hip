@@ -59,9 +59,11 @@ __global__ __launch_bounds__(kBlock) void k_radix_count(const unsigned long long
         for (int d = lane; d < 256; d += 64) counts[(size_t)d * n_tiles + tile] = cnt[w][d];
 }
 
+template <bool PAYLOAD>
 __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long long *__restrict__ in,
                                                          unsigned long long *__restrict__ out, long n, int shift,
-                                                         long n_tiles, const unsigned *__restrict__ offsets) {
+                                                         long n_tiles, const unsigned *__restrict__ offsets,
+                                                         const int *__restrict__ in_val, int *__restrict__ out_val) {
     __shared__ unsigned run[kWaves][256];
     const int w = wave_id(), lane = lane_id();
     const long tile = (long)blockIdx.x * kWaves + w;
@@ -74,6 +76,8 @@ __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long lo
         long i = base + (long)r * 64 + lane;
         bool valid = live && i < n;
         unsigned long long key = valid ? in[i] : 0ull;
+        int payload = 0;
+        if (PAYLOAD && valid) payload = in_val[i];
         unsigned d = (unsigned)(key >> shift) & 255u;
         // lanes holding the same digit (match-any built from eight ballots)
         unsigned long long mask = __ballot(valid);
@@ -88,6 +92,7 @@ __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long lo
         __syncthreads();
         if (valid) {
             out[(size_t)first + rank] = key;
+            if (PAYLOAD) out_val[(size_t)first + rank] = payload;
             if (rank == 0) run[w][d] = first + (unsigned)__popcll(mask);
         }
         __syncthreads();
@@ -153,20 +158,25 @@ __global__ __launch_bounds__(kBlock) void k_scan_add(unsigned *__restrict__ out,
     }
 }
 
-// out[i] = sum of in[0..i); returns nothing, the total is written to *d_total (device).
+// out[i] = sum of in[0..i); returns nothing, the total is written to *d_total (device). The tile sums of
+// every recursion level live in `sc`, which grows on demand and is reused by later calls.
 template <bool FROM_KEYS>
-void exclusive_scan(hipStream_t s, const void *in, unsigned *out, long n, unsigned *d_total,
-                    std::vector<void *> &scratch) {
+void exclusive_scan(hipStream_t s, const void *in, unsigned *out, long n, unsigned *d_total, ScanScratch &sc,
+                    size_t level = 0) {
     long tiles = (n + kScanTile - 1) / kScanTile;
-    unsigned *sums = nullptr;
-    HIP_CHECK(hipMalloc(&sums, sizeof(unsigned) * (size_t)(tiles + 1)));
-    scratch.push_back(sums);
+    if (sc.levels.size() <= level) sc.levels.resize(level + 1);
+    ScanScratch::Level &lv = sc.levels[level];
+    if (lv.cap < (size_t)tiles + 1) {
+        if (lv.sums) HIP_CHECK(hipFree(lv.sums));
+        if (lv.scanned) HIP_CHECK(hipFree(lv.scanned));
+        lv.cap = (size_t)tiles + 1;
+        HIP_CHECK(hipMalloc(&lv.sums, sizeof(unsigned) * lv.cap));
+        HIP_CHECK(hipMalloc(&lv.scanned, sizeof(unsigned) * lv.cap));
+    }
+    unsigned *sums = lv.sums, *sums_scanned = lv.scanned;  // the recursion may move sc.levels
     k_scan_tiles<FROM_KEYS><<<(unsigned)tiles, kBlock, 0, s>>>(in, out, n, sums);
     if (tiles > 1) {
-        unsigned *sums_scanned = nullptr;
-        HIP_CHECK(hipMalloc(&sums_scanned, sizeof(unsigned) * (size_t)(tiles + 1)));
-        scratch.push_back(sums_scanned);
-        exclusive_scan<false>(s, sums, sums_scanned, tiles, d_total, scratch);
+        exclusive_scan<false>(s, sums, sums_scanned, tiles, d_total, sc, level + 1);
         k_scan_add<<<(unsigned)tiles, kBlock, 0, s>>>(out, n, sums_scanned);
     } else {
         HIP_CHECK(hipMemcpyAsync(d_total, sums, sizeof(unsigned), hipMemcpyDeviceToDevice, s));
@@ -288,7 +298,7 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
         out.feature_nnz.assign(F, 0);
         return out;
     }
-    std::vector<void *> scratch;
+    ScanScratch scratch;
     unsigned long long *keys[2];
     HIP_CHECK(hipMalloc(&keys[0], sizeof(unsigned long long) * (size_t)nnz));
     HIP_CHECK(hipMalloc(&keys[1], sizeof(unsigned long long) * (size_t)nnz));
@@ -309,7 +319,8 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
         const int shift = 8 * p;
         k_radix_count<<<sort_grid, kBlock, 0, s>>>(keys[cur], nnz, shift, n_tiles, counts);
         exclusive_scan<false>(s, counts, offsets, (long)n_counts, d_total, scratch);
-        k_radix_scatter<<<sort_grid, kBlock, 0, s>>>(keys[cur], keys[cur ^ 1], nnz, shift, n_tiles, offsets);
+        k_radix_scatter<false><<<sort_grid, kBlock, 0, s>>>(keys[cur], keys[cur ^ 1], nnz, shift, n_tiles, offsets,
+                                                            nullptr, nullptr);
         cur ^= 1;
     }
     const unsigned long long *sorted = keys[cur];
@@ -342,7 +353,7 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     k_emit_cuts<<<grid_for(nnz), kBlock, 0, s>>>(sorted, uidx, nnz, ustart, out.cut_row_ptr, max_num_bin, out.cut_val,
                                                out.cut_fid);
     HIP_CHECK(hipStreamSynchronize(s));
-    for (void *p : scratch) HIP_CHECK(hipFree(p));
+    scratch.release();
     HIP_CHECK(hipFree(keys[0]));
     HIP_CHECK(hipFree(keys[1]));
     HIP_CHECK(hipFree(counts));
@@ -352,6 +363,67 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     HIP_CHECK(hipFree(estart));
     HIP_CHECK(hipFree(ustart));
     return out;
+}
+
+void ScanScratch::release() {
+    for (Level &lv : levels) {
+        if (lv.sums) (void)hipFree(lv.sums);
+        if (lv.scanned) (void)hipFree(lv.scanned);
+    }
+    levels.clear();
+}
+
+void device_exclusive_scan(hipStream_t s, const unsigned *in, unsigned *out, long n, unsigned *d_total,
+                           ScanScratch &sc) {
+    exclusive_scan<false>(s, in, out, n, d_total, sc);
+}
+
+void PairSorter::alloc(long n) {
+    cap = n;
+    const size_t m = (size_t)std::max(n, 1l);
+    n_tiles = (n + kSortTile - 1) / kSortTile;
+    const size_t n_counts = (size_t)256 * (size_t)std::max(n_tiles, 1l);
+    for (int b = 0; b < 2; ++b) {
+        HIP_CHECK(hipMalloc(&keys[b], sizeof(unsigned long long) * m));
+        HIP_CHECK(hipMalloc(&vals[b], sizeof(int) * m));
+    }
+    HIP_CHECK(hipMalloc(&counts, sizeof(unsigned) * n_counts));
+    HIP_CHECK(hipMalloc(&offsets, sizeof(unsigned) * (n_counts + 1)));
+    HIP_CHECK(hipMalloc(&d_total, sizeof(unsigned)));
+}
+
+void PairSorter::release() {
+    for (int b = 0; b < 2; ++b) {
+        if (keys[b]) (void)hipFree(keys[b]);
+        if (vals[b]) (void)hipFree(vals[b]);
+        keys[b] = nullptr;
+        vals[b] = nullptr;
+    }
+    if (counts) (void)hipFree(counts);
+    if (offsets) (void)hipFree(offsets);
+    if (d_total) (void)hipFree(d_total);
+    counts = offsets = d_total = nullptr;
+    scan.release();
+    cap = 0;
+}
+
+int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits) {
+    TGBM_CHECK(n <= ps.cap, "sort_pairs: %ld pairs exceed the sorter's capacity %ld", n, ps.cap);
+    if (n <= 1) return 0;
+    const long n_tiles = (n + kSortTile - 1) / kSortTile;
+    const size_t n_counts = (size_t)256 * n_tiles;
+    const unsigned sort_grid = (unsigned)((n_tiles + kWaves - 1) / kWaves);
+    const int passes = (key_bits + 7) / 8;
+    int cur = 0;
+    for (int p = 0; p < passes; ++p) {
+        const int shift = 8 * p;
+        k_radix_count<<<sort_grid, kBlock, 0, s>>>(ps.keys[cur], n, shift, n_tiles, ps.counts);
+        exclusive_scan<false>(s, ps.counts, ps.offsets, (long)n_counts, ps.d_total, ps.scan);
+        k_radix_scatter<true><<<sort_grid, kBlock, 0, s>>>(ps.keys[cur], ps.keys[cur ^ 1], n, shift, n_tiles, ps.offsets,
+                                                           ps.vals[cur], ps.vals[cur ^ 1]);
+        cur ^= 1;
+    }
+    return cur;
 }
 
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,

@@ -3,11 +3,13 @@
 #include <hip/hip_runtime.h>
 
 #include <map>
+#include <memory>
 #include <string>
 #include <vector>
 
 #include "device_api.h"
 #include "host.h"
+#include "rank.h"
 
 namespace tgbm {
 
@@ -59,6 +61,7 @@ class Trainer {
     void build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class);
     void build_round_together();
     void log_plan(const TreeBuffers &tb);
+    void run_metric(float *slot);
     void alloc_tree_buffers();
     template <typename T>
     T *dalloc(size_t count);
@@ -90,6 +93,7 @@ class Trainer {
     std::vector<uint8_t> h_ignored_;
     uint8_t *d_ignored_ = nullptr;
     int cur_class_ = 0;
+    std::unique_ptr<RankContext> rank_;  // ranking objectives only
     bool in_boost_ = false;
     int lookup_level_ = -1;          // level whose split nodes have not been partitioned into row lists yet
     bool next_round_ready_ = false;  // d_gh_ and the root statistics already belong to the next round

@@ -93,7 +93,13 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     } else if (param.objective.find("reg:") != std::string::npos) {
         param.num_class = 1;
     }
-    if (param.objective == "reg:linear") {
+    if (objective_needs_groups(param.objective)) {
+        // LambdaRank / LambdaRankNDCG with their default metrics (ranking_obj.cpp:98,115); one score per row
+        objective_ = OBJ_RANK;
+        metric_kind_ = param.objective == "rank:ndcg" ? RANK_METRIC_NDCG : RANK_METRIC_MAP;
+        TGBM_CHECK(param.num_class == 1, "ranking objectives train one score per instance (num_class %d)",
+                   param.num_class);
+    } else if (param.objective == "reg:linear") {
         objective_ = OBJ_SQUARE;
         metric_kind_ = 0;
     } else if (param.objective == "reg:logistic") {
@@ -245,8 +251,10 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     launch_fill_f32(stream_, reinterpret_cast<float *>(d_gh_), 0.f, (size_t)param_.num_class * n_ * 2);
     alloc_tree_buffers();
 
+    if (objective_ == OBJ_RANK) rank_.reset(new RankContext(stream_, ds.y, ds.group, param_.objective == "rank:ndcg"));
+
     // base score (regression_obj.h:35-53, :95-114; only for squared / logistic objectives)
-    if (objective_ != OBJ_SOFTMAX) {
+    if (objective_ != OBJ_SOFTMAX && objective_ != OBJ_RANK) {
         launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
         launch_tree_init(stream_, tb_, d_gh_, param_.lambda);  // reuses the root-sum reduction
         TreeNode root;
@@ -385,6 +393,12 @@ void Trainer::sync() { HIP_CHECK(hipStreamSynchronize(stream_)); }
 
 void Trainer::compute_gradient() {
     next_round_ready_ = false;
+    if (objective_ == OBJ_RANK) {
+        // the round's partner draws hang off the process-wide rand(), which is what the reference seeds its
+        // per-group generators from (ranking_obj.cpp:53): srand() makes a run repeatable
+        rank_->gradient(d_yp_, d_gh_, (unsigned)std::rand());
+        return;
+    }
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
 }
 
@@ -522,9 +536,16 @@ void Trainer::build_round_together() {
     cur_class_ = K - 1;
 }
 
+void Trainer::run_metric(float *slot) {
+    if (objective_ == OBJ_RANK)
+        rank_->metric(metric_kind_, d_yp_, slot);
+    else
+        launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+}
+
 float Trainer::metric() {
     float *slot = d_metric_ + std::min(rounds_done_, std::max(1, param_.n_trees) - 1);
-    launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+    run_metric(slot);
     float v = 0;
     HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
@@ -532,11 +553,11 @@ float Trainer::metric() {
 }
 
 void Trainer::boost(int rounds) {
-    static const char *names[] = {"RMSE", "test error", "multi-class accuracy"};
+    static const char *names[] = {"RMSE", "test error", "multi-class accuracy", "MAP", "NDCG"};
     in_boost_ = true;
     for (int r = 0; r < rounds; ++r) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
-        const bool fuse = objective_ != OBJ_SOFTMAX && param_.tree_per_rounds == 1;
+        const bool fuse = (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && param_.tree_per_rounds == 1;
         sample_columns();
         if (!next_round_ready_) compute_gradient();
         if (n_sets_ > 1) {
@@ -555,7 +576,7 @@ void Trainer::boost(int rounds) {
             }
         }
         float *slot = d_metric_ + rounds_done_;
-        if (!fuse) launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
+        if (!fuse) run_metric(slot);
         if (g_verbose >= 1) {
             float v = 0;
             HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
@@ -673,6 +694,11 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "ridx1") src = cur.ridx[1], bytes = sizeof(int) * (size_t)n_;
     else if (name == "model") src = d_model_, bytes = sizeof(TreeNode) * (size_t)trees_built_ * tb_.n_nodes;
     else if (name == "metric_log") src = d_metric_, bytes = sizeof(float) * (size_t)rounds_done_;
+    else if (name == "rank_order") {
+        // rows in the order the last ranking gradient / metric pass sorted them
+        TGBM_CHECK(rank_ != nullptr, "rank_order belongs to the ranking objectives");
+        src = rank_->last_sorted_rows(), bytes = sizeof(int) * (size_t)n_;
+    }
     else fatal("unknown buffer %s", name.c_str());
     if (out != nullptr && cap >= bytes && bytes > 0) HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
     return bytes;

@@ -93,10 +93,11 @@ class TGBMModel(BaseEstimator):
         n_out = n * self.num_class if self.objective == "multi:softprob" else n
         out = np.zeros(max(n_out, n * max(self.tree_per_iter, 1)), dtype=np.float32)
         labels = np.asarray(self.group_label if self.group_label else [0.0], dtype=np.float32)
+        grp = None if groups is None else np.ascontiguousarray(groups, dtype=np.int32)
         lib.sparse_predict_scikit(n, _ptr(X.data), _ptr(indptr), _ptr(indices), _ptr(out),
                                   C.cast(C.byref(self.model), C.c_void_p), self.n_trees, self.tree_per_iter,
                                   self.objective.encode("utf-8"), self.num_class, self.learning_rate, _ptr(labels),
-                                  None, 0, self.verbose)
+                                  None if grp is None else _ptr(grp), 0 if grp is None else len(grp), self.verbose)
         if self.objective == "multi:softprob":
             # the library returns class-major probabilities; the reference wrapper reshapes them as
             # [-1, num_class] without transposing (thundergbm.py:169-171) and so does this one

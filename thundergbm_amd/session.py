@@ -31,7 +31,7 @@ class Session:
     """One training session on the GPU: CSR input is copied to HBM once, then boosted in place."""
 
     def __init__(self, val, row_ptr, col, y, depth=6, n_trees=40, min_child_weight=1.0, lambda_=1.0, gamma=1.0,
-                 max_num_bin=255, learning_rate=1.0, objective="reg:linear", num_class=1, verbose=0):
+                 max_num_bin=255, learning_rate=1.0, objective="reg:linear", num_class=1, verbose=0, groups=None):
         self.L = _lib.load()
         val = np.ascontiguousarray(val, dtype=np.float32)
         row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
@@ -40,9 +40,12 @@ class Session:
         self.n = len(row_ptr) - 1
         self.nnz = int(row_ptr[-1])
         self.depth = depth
-        self.h = self.L.tgbm_trainer_create(self.n, _p(val), _p(row_ptr), _p(col), _p(y), depth, n_trees,
-                                            min_child_weight, lambda_, gamma, max_num_bin, learning_rate,
-                                            objective.encode(), num_class, verbose)
+        # groups: sizes of the query groups (consecutive rows) of the ranking objectives
+        grp = np.ascontiguousarray(groups if groups is not None else [], dtype=np.int32)
+        self.h = self.L.tgbm_trainer_create_grouped(self.n, _p(val), _p(row_ptr), _p(col), _p(y), depth, n_trees,
+                                                    min_child_weight, lambda_, gamma, max_num_bin, learning_rate,
+                                                    objective.encode(), num_class, verbose,
+                                                    _p(grp) if len(grp) else None, len(grp))
         self.F = self.info("n_features")
         self.n_bins = self.info("n_bins")
         self.num_class = self.info("num_class")
