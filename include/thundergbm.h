@@ -3,7 +3,8 @@
  *
  * Part 1 is the drop-in boundary: the nine entry points that the reference's Python wrapper
  * (python/thundergbm/thundergbm.py) binds with ctypes, with the argument order, types and
- * ownership rules of src/thundergbm/scikit_tgbm.cpp. Where the reference declares `Tree *&model`
+ * ownership rules of src/thundergbm/scikit_tgbm.cpp, plus the two file-based entry points of the R
+ * interface (src/thundergbm/gbm_R_interface.cpp). Where the reference declares `Tree *&model`
  * the ABI passes the address of an 8-byte slot; it is spelled `tgbm_model **` here. The model is
  * opaque, owned by the library and released only by model_free().
  *
@@ -70,6 +71,16 @@ void get_a_tree(tgbm_model **model, int tree_id, int n_nodes, int *children_left
 
 /* scikit_tgbm.cpp:250-254. */
 void model_free(tgbm_model **model);
+
+/* gbm_R_interface.cpp:10-61 and :63-86, the two symbols R/gbm.R reaches with .C(): every argument is a
+ * pointer, strings are char**. train_R loads the LIBSVM file data[0] (plus data[0].group for a ranking
+ * objective), trains and writes the model file model_out[0]; predict_R loads model_in[0] and the file
+ * data[0], predicts and logs the metric. min_child_weight is an int here, as in the reference. */
+void train_R(int *depth, int *n_trees, int *n_gpus, int *verbose, int *profiling, char **data, int *max_num_bin,
+             double *column_sampling_rate, int *bagging, int *n_parallel_trees, double *learning_rate,
+             char **objective, int *num_class, int *min_child_weight, double *lambda_tgbm, double *gamma,
+             char **tree_method, char **model_out);
+void predict_R(char **data, char **model_in, int *verbose);
 
 /* ------------------------------------------------------------------- Part 2: session API */
 

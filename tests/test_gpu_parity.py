@@ -586,3 +586,41 @@ def test_cli_train_and_predict_on_a1a(T, tmp_path):
                           "verbosity=1"], capture_output=True, text=True, cwd=tmp_path, timeout=300)
     assert out.returncode == 0, out.stderr
     assert "[4/4] test error = " in out.stdout
+
+
+def test_r_entry_points(T, tmp_path):
+    """train_R / predict_R (gbm_R_interface.cpp:10-86) the way R's .C() calls them: every argument a pointer,
+    strings as char**. The model file they write equals what the estimator saves for the same parameters."""
+    L = T.load()
+    ci = lambda v: C.byref(C.c_int(v))
+    cd = lambda v: C.byref(C.c_double(v))
+
+    def cs(v):
+        arr = (C.c_char_p * 1)(str(v).encode())
+        return arr
+
+    model_path = tmp_path / "r.model"
+    data, obj, method, out = cs(D.A1A), cs("binary:logistic"), cs("hist"), cs(model_path)
+    L.train_R(ci(4), ci(6), ci(1), ci(0), ci(0), data, ci(63), cd(1.0), ci(0), ci(1), cd(0.5), obj, ci(2), ci(1),
+              cd(1.0), cd(0.5), method, out)
+    assert os.path.getsize(model_path) > 0
+    m = T.TGBMClassifier(verbose=0)
+    m.load_model(str(model_path))
+    assert (m.n_trees, m.num_class, m.tree_per_iter) == (6, 2, 1) and abs(m.learning_rate - 0.5) < 1e-7
+    val, rp, col, y = D.read_libsvm(D.A1A)
+    import scipy.sparse as sp
+    X = sp.csr_matrix((val, col, rp), shape=(len(y), 119))
+    ref = T.TGBMClassifier(depth=4, n_trees=6, max_num_bin=63, learning_rate=0.5, objective="binary:logistic",
+                           gamma=0.5, verbose=0, tree_method="hist").fit(X, y)
+    for t in range(6):
+        a, b = m.get_trees()[t], ref.get_trees()[t]
+        assert np.array_equal(a["feature"], b["feature"]) and np.array_equal(a["threshold"], b["threshold"])
+        assert np.array_equal(a["value"], b["value"])
+    import subprocess, sys
+    code = ("import ctypes as C, thundergbm_amd as T; L = T.load();"
+            "L.predict_R((C.c_char_p * 1)(%r.encode()), (C.c_char_p * 1)(%r.encode()), C.byref(C.c_int(1)))")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", code % (D.A1A, str(model_path))], capture_output=True, text=True,
+                         cwd=root, timeout=300)
+    assert res.returncode == 0, res.stderr
+    assert "test error = " in res.stdout

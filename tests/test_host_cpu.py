@@ -33,7 +33,7 @@ def lib():
 def _declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b([a-z_][a-z0-9_]*)\s*\(", text)) - {"defined"})
+    return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text)) - {"defined"})
 
 
 def test_header_symbols_are_exported(lib):
@@ -41,6 +41,8 @@ def test_header_symbols_are_exported(lib):
     # the nine entry points of the reference's scikit_tgbm.cpp must all be there
     for ref in ("set_logger", "sparse_train_scikit", "sparse_predict_scikit", "save", "load_model", "load_config",
                 "get_n_nodes", "get_a_tree", "model_free"):
+        assert ref in names
+    for ref in ("train_R", "predict_R"):  # gbm_R_interface.cpp
         assert ref in names
     for n in names:
         assert hasattr(lib, n), "declared in the header but not exported: %s" % n

@@ -22,6 +22,8 @@ SIGNATURES = {
     "get_n_nodes": (None, [_P, _P, C.c_int, C.c_int]),
     "get_a_tree": (None, [_P, C.c_int, C.c_int, _P, _P, _P, _P, _P, _P, _P]),
     "model_free": (None, [_P]),
+    "train_R": (None, [_P] * 18),
+    "predict_R": (None, [_P] * 3),
     "tgbm_trainer_create": (_P, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.c_int,
                                  C.c_float, C.c_char_p, C.c_int, C.c_int]),
     "tgbm_trainer_create_grouped": (_P, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, C.c_float,

@@ -171,6 +171,51 @@ void model_free(tgbm_model **model) {
     }
 }
 
+// ----------------------------------------------------------------------------- R entry points
+// R's .C() convention: every argument is a pointer, strings arrive as char**. File in, file out.
+void train_R(int *depth, int *n_trees, int *n_gpus, int *verbose, int *profiling, char **data, int *max_num_bin,
+             double *column_sampling_rate, int *bagging, int *n_parallel_trees, double *learning_rate,
+             char **objective, int *num_class, int *min_child_weight, double *lambda_tgbm, double *gamma,
+             char **tree_method, char **model_out) {
+    set_logger(*verbose);
+    GBMParam p;
+    p.depth = *depth;
+    p.n_trees = *n_trees;
+    p.n_device = *n_gpus;
+    p.verbose = *verbose;
+    p.profiling = *profiling != 0;
+    p.path = data[0];
+    p.max_num_bin = *max_num_bin;
+    p.column_sampling_rate = (float)*column_sampling_rate;
+    p.bagging = *bagging != 0;
+    p.n_parallel_trees = *n_parallel_trees;
+    p.learning_rate = (float)*learning_rate;
+    p.objective = objective[0];
+    p.num_class = *num_class;
+    p.min_child_weight = (float)*min_child_weight;
+    p.lambda = (float)*lambda_tgbm;
+    p.gamma = (float)*gamma;
+    p.tree_method = tree_method[0];
+    p.rt_eps = 1e-6f;
+    p.tree_per_rounds = 1;
+    DataSet dataset;
+    dataset.load_from_file(p.path, p);
+    std::vector<std::vector<Tree>> model = train(p, dataset);
+    Parser::save_model(model_out[0], p, model, dataset);
+}
+
+void predict_R(char **data, char **model_in, int *verbose) {
+    set_logger(*verbose);
+    GBMParam p;
+    DataSet dataset;
+    std::vector<std::vector<Tree>> model;
+    Parser::load_model(model_in[0], p, model, dataset);
+    std::vector<float> model_labels = dataset.label;
+    dataset.load_from_file(data[0], p);
+    if (!objective_needs_group_label(p.objective)) dataset.label = model_labels;
+    (void)predict(p, model, dataset, true);
+}
+
 // ------------------------------------------------------------------------------- session API
 tgbm_trainer *tgbm_trainer_create(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
                                   const float *label, int depth, int n_trees, float min_child_weight, float lambda,
