@@ -45,20 +45,30 @@ __global__ __launch_bounds__(kBlock) void k_radix_count(const unsigned long long
     __shared__ unsigned cnt[kWaves][256];
     const int w = wave_id(), lane = lane_id();
     const long tile = (long)blockIdx.x * kWaves + w;
+    if (tile >= n_tiles) return;  // a wavefront only touches its own row of counters: no workgroup barrier
     for (int d = lane; d < 256; d += 64) cnt[w][d] = 0;
-    __syncthreads();
-    if (tile < n_tiles) {
-        const long base = tile * kSortTile;
-        for (int r = 0; r < kSortRounds; ++r) {
-            long i = base + (long)r * 64 + lane;
-            if (i < n) atomicAdd(&cnt[w][(unsigned)(keys[i] >> shift) & 255u], 1u);
+    __builtin_amdgcn_wave_barrier();
+    const long base = tile * kSortTile;
+    constexpr int kBatch = 16;
+    for (int r0 = 0; r0 < kSortRounds; r0 += kBatch) {
+        unsigned long long k[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const long i = base + (long)(r0 + b) * 64 + lane;
+            k[b] = i < n ? keys[i] : 0ull;
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const long i = base + (long)(r0 + b) * 64 + lane;
+            if (i < n) atomicAdd(&cnt[w][(unsigned)(k[b] >> shift) & 255u], 1u);
         }
     }
-    __syncthreads();
-    if (tile < n_tiles)
-        for (int d = lane; d < 256; d += 64) counts[(size_t)d * n_tiles + tile] = cnt[w][d];
+    __builtin_amdgcn_wave_barrier();
+    for (int d = lane; d < 256; d += 64) counts[(size_t)d * n_tiles + tile] = cnt[w][d];
 }
 
+// A wavefront owns its tile and its row of running offsets, so the rounds need no workgroup barrier: the LDS
+// serves one wavefront's reads and writes in program order. Keys are fetched a batch of rounds ahead.
 template <bool PAYLOAD>
 __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long long *__restrict__ in,
                                                          unsigned long long *__restrict__ out, long n, int shift,
@@ -67,35 +77,45 @@ __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long lo
     __shared__ unsigned run[kWaves][256];
     const int w = wave_id(), lane = lane_id();
     const long tile = (long)blockIdx.x * kWaves + w;
-    const bool live = tile < n_tiles;
-    if (live)
-        for (int d = lane; d < 256; d += 64) run[w][d] = offsets[(size_t)d * n_tiles + tile];
-    __syncthreads();
+    if (tile >= n_tiles) return;
+    for (int d = lane; d < 256; d += 64) run[w][d] = offsets[(size_t)d * n_tiles + tile];
+    __builtin_amdgcn_wave_barrier();
     const long base = tile * kSortTile;
-    for (int r = 0; r < kSortRounds; ++r) {
-        long i = base + (long)r * 64 + lane;
-        bool valid = live && i < n;
-        unsigned long long key = valid ? in[i] : 0ull;
-        int payload = 0;
-        if (PAYLOAD && valid) payload = in_val[i];
-        unsigned d = (unsigned)(key >> shift) & 255u;
-        // lanes holding the same digit (match-any built from eight ballots)
-        unsigned long long mask = __ballot(valid);
+    constexpr int kBatch = 8;
+    static_assert(kSortRounds % kBatch == 0, "rounds come in whole batches");
+    for (int r0 = 0; r0 < kSortRounds; r0 += kBatch) {
+        unsigned long long keys[kBatch];
+        int payload[kBatch];
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            bool bit = (d >> b) & 1u;
-            unsigned long long m = __ballot(bit);
-            mask &= bit ? m : ~m;
+        for (int b = 0; b < kBatch; ++b) {
+            const long i = base + (long)(r0 + b) * 64 + lane;
+            keys[b] = i < n ? in[i] : 0ull;
+            payload[b] = (PAYLOAD && i < n) ? in_val[i] : 0;
         }
-        unsigned first = valid ? run[w][d] : 0u;
-        int rank = lanes_below(mask);
-        __syncthreads();
-        if (valid) {
-            out[(size_t)first + rank] = key;
-            if (PAYLOAD) out_val[(size_t)first + rank] = payload;
-            if (rank == 0) run[w][d] = first + (unsigned)__popcll(mask);
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+            const long i = base + (long)(r0 + b) * 64 + lane;
+            const bool valid = i < n;
+            const unsigned long long key = keys[b];
+            const unsigned d = (unsigned)(key >> shift) & 255u;
+            // lanes holding the same digit (match-any built from eight ballots)
+            unsigned long long mask = __ballot(valid);
+#pragma unroll
+            for (int bit_i = 0; bit_i < 8; ++bit_i) {
+                const bool bit = (d >> bit_i) & 1u;
+                const unsigned long long m = __ballot(bit);
+                mask &= bit ? m : ~m;
+            }
+            const unsigned first = valid ? run[w][d] : 0u;
+            const int rank = lanes_below(mask);
+            __builtin_amdgcn_wave_barrier();
+            if (valid) {
+                out[(size_t)first + rank] = key;
+                if (PAYLOAD) out_val[(size_t)first + rank] = payload[b];
+                if (rank == 0) run[w][d] = first + (unsigned)__popcll(mask);
+            }
+            __builtin_amdgcn_wave_barrier();
         }
-        __syncthreads();
     }
 }
 
