@@ -98,6 +98,11 @@ def test_rank_gradient_and_metric_parity(T, objective, name, ties):
         m = s.metric()
         om = O.rank_metric(objective, y, score, groups)
         assert abs(m - om) <= 1e-5 * max(1.0, abs(om))
+        # right after a metric pass the gradient re-sorts the metric's order by run id only: same bits
+        _round_seed(seed)
+        s.gradient()
+        assert np.array_equal(s.get("rank_order", np.int32), order)
+        assert np.array_equal(s.gh(), gh)
     s.close()
 
 

@@ -32,7 +32,9 @@ class RankContext {
 
     // LambdaRank::get_gradient (ranking_obj.cpp:20-96): gh[row] = sum of the lambdas of the sampled pairs the
     // row takes part in. `seed` selects the round's partner draws.
-    void gradient(const float *d_score, GHPair *d_gh, unsigned seed);
+    // order_is_fresh: d_score has not changed since the last metric() call, whose (group, score) order then
+    // only needs a stable re-sort by run id
+    void gradient(const float *d_score, GHPair *d_gh, unsigned seed, bool order_is_fresh = false);
     // RankListMetric::get_score with MAP or NDCG (metric/rank_metric.cpp:9-104); writes one float to d_out
     void metric(int kind, const float *d_score, float *d_out);
     // the row order and partner draws of the last gradient() call (tests): sorted rows [n]
@@ -53,6 +55,7 @@ class RankContext {
     float *d_y_ = nullptr;
     int *d_static_row_ = nullptr;  // rows of every group by label descending (ties: row ascending)
     int *d_run_of_ = nullptr;      // run of a position of that order
+    int *d_run_of_row_ = nullptr;  // run of a row
     RankRun *d_runs_ = nullptr;
     int *d_group_of_ = nullptr;    // group of a row
     int *d_gptr_ = nullptr;
@@ -64,6 +67,7 @@ class RankContext {
     int n_partial_ = 0;
     PairSorter sorter_;
     int last_cur_ = 0;
+    bool have_metric_order_ = false;  // sorter_.vals[last_cur_] is the (group, score) order of a metric() call
 };
 
 }  // namespace tgbm

@@ -65,6 +65,17 @@ __global__ __launch_bounds__(kBlock) void k_rank_train_keys(int n, const int *__
     vals[p] = row;
 }
 
+// Keys for the short re-sort of rows that are already in (group, score) order: the run id alone.
+__global__ __launch_bounds__(kBlock) void k_rank_run_keys(int n, const int *__restrict__ run_of_row,
+                                                         const int *sorted_row, unsigned long long *__restrict__ keys,
+                                                         int *vals) {
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= n) return;
+    const int row = sorted_row[p];  // may alias vals: every thread reads and writes its own element
+    keys[p] = (unsigned long long)(unsigned)run_of_row[row];
+    vals[p] = row;
+}
+
 __global__ __launch_bounds__(kBlock) void k_rank_metric_keys(int n, const int *__restrict__ group_of,
                                                             const float *__restrict__ score,
                                                             unsigned long long *__restrict__ keys, int *__restrict__ vals) {
@@ -232,7 +243,7 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
     for (float v : y) labels_ok = labels_ok && v >= 0.f && v < 31.f;
     TGBM_CHECK(!ndcg || labels_ok, "rank:ndcg needs labels in 0..30");
 
-    std::vector<int> static_row(n_), run_of(n_), group_of(n_), hits(n_groups_, 0);
+    std::vector<int> static_row(n_), run_of(n_), run_of_row(n_), group_of(n_), hits(n_groups_, 0);
     std::vector<RankRun> runs;
     std::vector<float> idcg(n_groups_, 0.f);
     int ndcg_one = 0;  // groups whose NDCG is 1 by definition (IDCG == 0)
@@ -265,7 +276,10 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
             r.group = g;
             r.pad = 0;
             skip_first = r.first_l < j;  // a processed run makes the loop step over the next run's first position
-            for (int k = i; k < j; ++k) run_of[k] = (int)runs.size();
+            for (int k = i; k < j; ++k) {
+                run_of[k] = (int)runs.size();
+                run_of_row[static_row[k]] = (int)runs.size();
+            }
             runs.push_back(r);
             i = j;
         }
@@ -279,6 +293,7 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
     d_y_ = dalloc<float>(n_);
     d_static_row_ = dalloc<int>(n_);
     d_run_of_ = dalloc<int>(n_);
+    d_run_of_row_ = dalloc<int>(n_);
     d_group_of_ = dalloc<int>(n_);
     d_runs_ = dalloc<RankRun>(runs.size());
     d_gptr_ = dalloc<int>(gptr.size());
@@ -295,6 +310,7 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
     up(d_y_, y.data(), sizeof(float) * (size_t)n_);
     up(d_static_row_, static_row.data(), sizeof(int) * (size_t)n_);
     up(d_run_of_, run_of.data(), sizeof(int) * (size_t)n_);
+    up(d_run_of_row_, run_of_row.data(), sizeof(int) * (size_t)n_);
     up(d_group_of_, group_of.data(), sizeof(int) * (size_t)n_);
     up(d_runs_, runs.data(), sizeof(RankRun) * runs.size());
     up(d_gptr_, gptr.data(), sizeof(int) * gptr.size());
@@ -310,12 +326,21 @@ RankContext::~RankContext() {
     for (void *p : allocs_) (void)hipFree(p);
 }
 
-void RankContext::gradient(const float *d_score, GHPair *d_gh, unsigned seed) {
+void RankContext::gradient(const float *d_score, GHPair *d_gh, unsigned seed, bool order_is_fresh) {
     if (n_ == 0) return;
     const int grid = grid_for(n_);
-    k_rank_train_keys<<<grid, kBlock, 0, stream_>>>(n_, d_static_row_, d_run_of_, d_score, sorter_.keys[0],
-                                                   sorter_.vals[0]);
-    last_cur_ = sort_pairs(stream_, sorter_, n_, 32 + run_bits_);
+    if (order_is_fresh && have_metric_order_) {
+        // rows already ordered by (group, score descending, row): a stable sort by run id yields
+        // (run, score descending, row), the same order as the full sort below
+        k_rank_run_keys<<<grid, kBlock, 0, stream_>>>(n_, d_run_of_row_, sorter_.vals[last_cur_], sorter_.keys[0],
+                                                     sorter_.vals[0]);
+        last_cur_ = sort_pairs(stream_, sorter_, n_, run_bits_);
+    } else {
+        k_rank_train_keys<<<grid, kBlock, 0, stream_>>>(n_, d_static_row_, d_run_of_, d_score, sorter_.keys[0],
+                                                       sorter_.vals[0]);
+        last_cur_ = sort_pairs(stream_, sorter_, n_, 32 + run_bits_);
+    }
+    have_metric_order_ = false;
     k_rank_pairs<<<grid, kBlock, 0, stream_>>>(n_, d_runs_, d_run_of_, sorter_.vals[last_cur_], d_score, d_y_,
                                               ndcg_ ? d_idcg_ : nullptr, seed,
                                               reinterpret_cast<unsigned long long *>(d_acc_));
@@ -342,6 +367,7 @@ void RankContext::metric(int kind, const float *d_score, float *d_out) {
     }
     k_rank_metric_final<<<1, 64, 0, stream_>>>(d_partial_, n_partial_, constant, n_groups_, d_out);
     last_cur_ = cur;
+    have_metric_order_ = true;
 }
 
 }  // namespace tgbm

@@ -94,6 +94,7 @@ class Trainer {
     uint8_t *d_ignored_ = nullptr;
     int cur_class_ = 0;
     std::unique_ptr<RankContext> rank_;  // ranking objectives only
+    bool rank_order_fresh_ = false;      // d_yp_ unchanged since the last ranking metric pass
     bool in_boost_ = false;
     int lookup_level_ = -1;          // level whose split nodes have not been partitioned into row lists yet
     bool next_round_ready_ = false;  // d_gh_ and the root statistics already belong to the next round

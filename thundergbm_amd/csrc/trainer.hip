@@ -396,7 +396,8 @@ void Trainer::compute_gradient() {
     if (objective_ == OBJ_RANK) {
         // the round's partner draws hang off the process-wide rand(), which is what the reference seeds its
         // per-group generators from (ranking_obj.cpp:53): srand() makes a run repeatable
-        rank_->gradient(d_yp_, d_gh_, (unsigned)std::rand());
+        rank_->gradient(d_yp_, d_gh_, (unsigned)std::rand(), rank_order_fresh_);
+        rank_order_fresh_ = false;
         return;
     }
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
@@ -495,6 +496,7 @@ void Trainer::log_plan(const TreeBuffers &tb) {
 
 void Trainer::finish_tree(int k, bool fuse_round_end) {
     const TreeBuffers tb = set_of(k);
+    rank_order_fresh_ = false;  // the scores change below
     launch_prune(stream_, tb, param_.gamma);
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
@@ -537,9 +539,10 @@ void Trainer::build_round_together() {
 }
 
 void Trainer::run_metric(float *slot) {
-    if (objective_ == OBJ_RANK)
+    if (objective_ == OBJ_RANK) {
         rank_->metric(metric_kind_, d_yp_, slot);
-    else
+        rank_order_fresh_ = true;
+    } else
         launch_metric(stream_, metric_kind_, n_, param_.num_class, d_y_, d_yp_, d_metric_scratch_, slot);
 }
 
@@ -707,6 +710,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
 void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     sync();
     next_round_ready_ = false;
+    rank_order_fresh_ = false;
     void *dst = nullptr;
     size_t want = 0;
     if (name == "gh") dst = d_gh_, want = sizeof(GHPair) * (size_t)param_.num_class * n_;
