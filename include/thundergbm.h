@@ -34,9 +34,10 @@ void set_logger(int verbose);
  * num_class is in/out, group_label receives the distinct labels (caller allocates one float per
  * distinct label), tree_per_iter and *model are outputs. column_sampling_rate < 1 samples columns per
  * round as the reference does (see tgbm_trainer_set_option). group / num_group are the query group sizes
- * of the ranking objectives (rank:pairwise, rank:ndcg; dataset.cpp:64-68) and ignored otherwise. n_device,
- * bagging (never applied by the reference either) and n_parallel_trees are accepted for signature
- * compatibility and ignored. */
+ * of the ranking objectives (rank:pairwise, rank:ndcg; dataset.cpp:64-68) and ignored otherwise. bagging != 0
+ * resamples the gradients every round (RowSampler::do_bagging, row_sampler.cu:9-38, booster.h:84). n_device
+ * and n_parallel_trees (never read by the reference either) are accepted for signature compatibility and
+ * ignored. */
 void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *label, int depth, int n_trees,
                          int n_device, float min_child_weight, float lambda, float gamma, int max_num_bin,
                          int verbose, float column_sampling_rate, int bagging, int n_parallel_trees,
@@ -106,7 +107,9 @@ void tgbm_trainer_destroy(tgbm_trainer *t);
 
 /* Options that tgbm_trainer_create has no argument for. "column_sampling_rate" (GBMParam, common.h:92):
  * below 1 every boosting round ignores max(1, int(n_features * rate)) randomly chosen columns in its split
- * search (Shard::column_sampling, builder/shard.cu:8-22; the shuffle draws from the process-wide rand()). */
+ * search (Shard::column_sampling, builder/shard.cu:8-22; the shuffle draws from the process-wide rand()).
+ * "bagging" (common.h:97): non-zero makes every gradient pass multiply the gradient pairs by bootstrap draw
+ * counts (RowSampler::do_bagging, row_sampler.cu:9-38; seeded with one rand() per pass). */
 void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value);
 /* The column sampling of one round for stage-wise driving (tgbm_trainer_boost does it itself). */
 void tgbm_trainer_sample_columns(tgbm_trainer *t);
@@ -115,7 +118,7 @@ void tgbm_trainer_sample_columns(tgbm_trainer *t);
 void tgbm_trainer_boost(tgbm_trainer *t, int rounds);
 
 /* Stage-wise driving; each call returns after enqueueing (tgbm_trainer_get synchronises).
- * gradient = ObjectiveFunction::get_gradient; tree_init = Tree::init2; find_split = find_split +
+ * gradient = ObjectiveFunction::get_gradient (then do_bagging when the option is on); tree_init = Tree::init2; find_split = find_split +
  * update_tree of the level; partition = update_ins2node_id; finish_tree = prune_self +
  * predict_in_training. */
 void tgbm_trainer_gradient(tgbm_trainer *t);

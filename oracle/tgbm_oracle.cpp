@@ -20,6 +20,8 @@
 //   prune           hand-built 7-node trees
 //   predictor       equality with the training-time prediction on the training rows
 //   metrics         reference KATs src/test/test_metrics.cpp:70,84,96; tree size src/test/test_tree.cpp:68
+//   bagging         the draws against vectors produced by the thrust headers this image ships (rocThrust;
+//                   tests/golden/bagging_thrust_vectors.hip), the engine is libstdc++'s std::minstd_rand
 //   ranking         LambdaRank gradients: two-row groups (closed form), pair bookkeeping by brute force over the
 //                   group (every drawing position pairs with a position outside its run of equal labels, the
 //                   lambdas of a pair cancel), |delta NDCG| = the change of DCG when the two positions swap;
@@ -36,6 +38,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <random>
 #include <string>
 #include <vector>
 #ifdef _OPENMP
@@ -87,6 +90,7 @@ inline float compute_gain(GH f, GH l, GH r, float mcw, float lambda) {
 
 struct Oracle {
     float column_sampling_rate = 1.f;
+    bool bagging = false;
     std::vector<char> ignored;  // per feature, this round (empty: none)
     // data (DataSet, src/thundergbm/dataset.cpp:20-63)
     int n = 0, F = 0;
@@ -777,6 +781,35 @@ float rank_metric(bool ndcg, int n, const float *y, const float *yp, const std::
     return sum_score / n_group;
 }
 
+// RowSampler::do_bagging, src/thundergbm/row_sampler.cu:9-38. The reference draws with thrust (a dependency
+// from the CUDA toolkit, not part of its checkout): thrust::default_random_engine is minstd_rand, the same
+// generator as std::minstd_rand (x <- 48271 x mod 2^31 - 1); thrust::uniform_int_distribution<int>(a, b) maps
+// one engine output u through uniform_real_distribution<double>(a, b + 1):
+// (u - min) / (1 + (max - min)) * ((b + 1) - a) + a, truncated
+// (thrust/random/detail/uniform_int_distribution.inl, uniform_real_distribution.inl).
+// Entry i takes the output that follows discard(i), i.e. output i + 1 of one engine seeded once: the draws
+// of all entries are the engine's outputs in order.
+void bagging_draws(int seed, int N, int count, int *out) {
+    std::minstd_rand rng((unsigned)seed);
+    const double a = 0.0, b = (double)(N - 1) + 1.0;
+    for (int i = 0; i < count; ++i) {
+        double result = (double)(rng() - std::minstd_rand::min());
+        result /= 1.0 + (double)(std::minstd_rand::max() - std::minstd_rand::min());
+        out[i] = (int)(result * (b - a) + a);
+    }
+}
+
+void do_bagging(std::vector<GH> &gh, int seed) {
+    const int N = (int)gh.size();
+    std::vector<int> idx(N), ins_count(N, 0);
+    bagging_draws(seed, N, N, idx.data());
+    for (int i = 0; i < N; ++i) ins_count[idx[i]] += 1;
+    for (int i = 0; i < N; ++i) {
+        gh[i].g = gh[i].g * ins_count[i];
+        gh[i].h = gh[i].h * ins_count[i];
+    }
+}
+
 bool is_rank(const std::string &obj) { return obj == "rank:pairwise" || obj == "rank:ndcg"; }
 
 // a12  metrics: RMSE src/thundergbm/metric/pointwise_metric.cu:8-22, accuracy / error
@@ -852,6 +885,7 @@ void boost_round(Oracle &o) {
                       o.gh.data(), nullptr, nullptr);
     else
         gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+    if (o.bagging) do_bagging(o.gh, std::rand());  // booster.h:84
     std::vector<Node> round_trees;
     for (int k = 0; k < o.tree_per_rounds; ++k) {
         build_tree(o, k);
@@ -1005,6 +1039,9 @@ void orc_prepare(void *h) {
     init_base_score(o);
 }
 
+void orc_set_bagging(void *h, int on) { ((Oracle *)h)->bagging = on != 0; }
+// idx_i of RowSampler::do_bagging for i = 0..count-1
+void orc_bagging_draws(int seed, int N, int count, int *out) { bagging_draws(seed, N, count, out); }
 void orc_set_groups(void *h, const int *group, int num_group) {
     ((Oracle *)h)->group.assign(group, group + num_group);
 }
@@ -1032,6 +1069,7 @@ void orc_compute_gradient(void *h) {
                       o.gh.data(), nullptr, nullptr);
     else
         gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
+    if (o.bagging) do_bagging(o.gh, std::rand());
 }
 void orc_tree_init(void *h, int k) { tree_init(*(Oracle *)h, k); }
 void orc_find_split(void *h, int level) { find_split(*(Oracle *)h, level); }

@@ -46,6 +46,10 @@ def lib():
         L.orc_boost.argtypes = [C.c_void_p, C.c_int]
         L.orc_set_column_sampling_rate.argtypes = [C.c_void_p, C.c_float]
         L.orc_sample_columns.argtypes = [C.c_void_p]
+        L.orc_set_bagging.argtypes = [C.c_void_p, C.c_int]
+        L.orc_set_bagging.restype = None
+        L.orc_bagging_draws.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p]
+        L.orc_bagging_draws.restype = None
         L.orc_set_groups.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         L.orc_set_groups.restype = None
         L.orc_rank_gradient.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_uint,
@@ -157,6 +161,9 @@ class Oracle:
 
     def sample_columns(self):
         self.L.orc_sample_columns(self.h)
+
+    def set_bagging(self, on):
+        self.L.orc_set_bagging(self.h, int(on))
 
     def boost(self, rounds=1):
         self.L.orc_boost(self.h, rounds)
@@ -324,6 +331,15 @@ def gradient(objective, y, yp, num_class=1):
     n = len(y)
     out = np.zeros((yp.size, 2), dtype=np.float32)
     L.orc_gradient(objective.encode(), n, num_class, _p(y), _p(yp), _p(out))
+    return out
+
+
+def bagging_draws(seed, N, count=None):
+    """The indices RowSampler::do_bagging draws for entries 0..count-1 of an N-entry gradient array."""
+    L = lib()
+    count = N if count is None else count
+    out = np.zeros(count, dtype=np.int32)
+    L.orc_bagging_draws(int(seed), int(N), int(count), _p(out))
     return out
 
 

@@ -287,6 +287,80 @@ def test_column_sampling_matches_oracle(T, objective, kind, rate):
     s.close()
 
 
+@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin"),
+                                            ("multi:softmax", "multi")])
+def test_bagging_matches_oracle(T, objective, kind):
+    """bagging = 1 (RowSampler::do_bagging, row_sampler.cu:9-38; booster.h:84): every round multiplies the
+    gradient pairs by bootstrap draw counts from thrust's minstd engine seeded with one rand(). The draw
+    counts must be the oracle's exactly (integer work), and boosting on the bagged gradients must build the
+    oracle's trees."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    libc.rand.restype = ctypes.c_int
+    n, F = 3000, 9
+    val, rp, col = _ragged(n, F, 33, F)
+    y = _target(val, rp, col, n, F, 33, kind)
+    # min_child_weight 0.5: the bagged hessians of squared loss are whole numbers, so child sums would sit
+    # exactly on a gate of 1 and candidates that isolate the same rows through different features would tie
+    kw = dict(objective=objective, n_trees=4, depth=4, max_num_bin=32, learning_rate=0.5, min_child_weight=0.5)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    s.gradient()
+    plain = s.gh().copy()
+    s.set_option("bagging", 1)
+    o.set_bagging(True)
+    N = plain.shape[0]
+    assert N == s.num_class * n  # the whole gradient array is resampled, as in the reference
+    for seed in (7, 8):
+        libc.srand(seed)
+        draw_seed = libc.rand()
+        libc.srand(seed)
+        s.gradient()
+        counts = np.bincount(O.bagging_draws(draw_seed, N), minlength=N).astype(np.float32)
+        assert np.array_equal(s.gh(), plain * counts[:, None])
+    ties = 0
+    for r in range(4):
+        o.set_y_pred(s.y_pred())
+        libc.srand(100 + r)
+        s.gradient()
+        gh = s.gh()
+        libc.srand(100 + r)
+        o.compute_gradient()
+        np.testing.assert_allclose(gh, o.gh(), rtol=1e-5, atol=2e-6)
+        o.set_gh(gh)
+        libc.srand(100 + r)
+        s.boost(1)
+        model = s.model()
+        for k in range(s.tree_per_rounds):
+            o.build_tree(k)
+            ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
+            d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=s.cuts()[1], orc_scores=o.tree_scores(),
+                                abs_scale=(ghk[0], ghk[1]), mcw=0.5)
+            ties += len(d.near_ties)
+    # rows drawn zero times carry no weight, so neighbouring candidates can describe the same partition;
+    # compare_trees has checked that every differing choice is such a tie in the oracle's own gains
+    assert ties <= 3
+    s.close()
+
+
+def test_bagging_through_the_c_abi(T):
+    """The bagging argument of sparse_train_scikit: same srand() seed, same model; without bagging another."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    rng = np.random.default_rng(4)
+    X = rng.standard_normal((2000, 6)).astype(np.float32)
+    y = (X[:, 0] - X[:, 1] + 0.3 * rng.standard_normal(2000)).astype(np.float32)
+    preds = []
+    for bagging, seed in ((1, 5), (1, 5), (1, 6), (0, 5)):
+        libc.srand(seed)
+        m = T.TGBMRegressor(depth=4, n_trees=6, learning_rate=0.5, bagging=bagging, verbose=0).fit(X, y)
+        preds.append(np.asarray(m.predict(X), np.float32).copy())
+    assert np.array_equal(preds[0], preds[1])
+    assert not np.array_equal(preds[0], preds[2])
+    assert not np.array_equal(preds[0], preds[3])
+    assert np.sqrt(np.mean((preds[0] - y) ** 2)) < 0.8 * np.std(y)  # still learns
+
+
 @pytest.mark.parametrize("layout", ["dense", "sparse"])
 def test_training_is_bit_reproducible(T, layout):
     """Histograms are exact integer sums (LDS and HBM atomics alike) and every float reduction has a fixed

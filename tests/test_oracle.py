@@ -1,5 +1,7 @@
 """Pins the CPU oracle (oracle/tgbm_oracle.cpp) without running the reference: closed forms,
 brute force on small inputs, invariants, and the reference's own fixture / known answers."""
+import os
+
 import numpy as np
 import pytest
 
@@ -618,3 +620,44 @@ def test_column_sampling_ignores_the_shuffled_head():
     assert max(len(u) for u in used_full) > 4
     _, used_tiny = run(0.01, 7)  # max(1, int(0.1)) = 1 ignored column
     assert all(len(u) <= F - 1 for u in used_tiny)
+
+
+# ------------------------------------------------------------------------------------------ bagging
+def test_bagging_draws_match_thrust_vectors():
+    """RowSampler::do_bagging draws with thrust::default_random_engine and thrust::uniform_int_distribution.
+    The vectors were produced with the thrust headers of this image (tests/golden/bagging_thrust_vectors.hip);
+    the oracle's restatement (std::minstd_rand + thrust's mapping) must give the same indices."""
+    import json
+    cases = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                        "bagging_thrust_vectors.json")))
+    assert len(cases) == 30
+    for c in cases:
+        draws = O.bagging_draws(c["seed"], c["N"], max(int(p) for p in c["draws"]) + 1)
+        for pos, idx in c["draws"].items():
+            assert draws[int(pos)] == idx, (c["seed"], c["N"], pos)
+
+
+def test_bagging_engine_is_minstd_rand():
+    # the C++ standard fixes the 10000th output of minstd_rand (default seed 1) at 399268537; with N = m - 1
+    # the distribution's mapping is the identity on (output - 1)
+    m = 2147483647
+    assert O.bagging_draws(1, m - 1, 10000)[9999] == 399268537 - 1
+
+
+def test_bagging_scales_gradients_by_draw_counts():
+    import ctypes as C
+    libc = C.CDLL("libc.so.6")
+    libc.rand.restype = C.c_int
+    X, y = D.config1(500, 4, seed=3)
+    val, rp, col = O.dense_to_csr(X)
+    o = O.Oracle(val, rp, col, y, depth=3, n_trees=2).prepare()
+    o.compute_gradient()
+    plain = o.gh().copy()
+    o.set_bagging(True)
+    libc.srand(42)
+    seed = libc.rand()
+    libc.srand(42)
+    o.compute_gradient()
+    counts = np.bincount(O.bagging_draws(seed, 500), minlength=500)
+    assert counts.sum() == 500 and counts.max() > 1 and (counts == 0).sum() > 100  # a bootstrap sample
+    assert np.array_equal(o.gh(), plain * counts[:, None].astype(np.float32))

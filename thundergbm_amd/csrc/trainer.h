@@ -33,7 +33,7 @@ class Trainer {
     void boost(int rounds);
     // step-wise driving (used by parity tests)
     void sample_columns();  // column sampling of one boosting round (no-op for rate >= 1); boost() calls it
-    void set_option(const std::string &key, double value);  // "column_sampling_rate"
+    void set_option(const std::string &key, double value);  // "column_sampling_rate", "bagging"
     void compute_gradient();
     void tree_init(int k);
     void find_split(int level);  // histogram, merge/subtract, split search, update_tree
@@ -94,6 +94,7 @@ class Trainer {
     uint8_t *d_ignored_ = nullptr;
     int cur_class_ = 0;
     std::unique_ptr<RankContext> rank_;  // ranking objectives only
+    int *d_bag_count_ = nullptr;         // bagging: draws per gradient entry (zero between rounds)
     bool rank_order_fresh_ = false;      // d_yp_ unchanged since the last ranking metric pass
     bool in_boost_ = false;
     int lookup_level_ = -1;          // level whose split nodes have not been partitioned into row lists yet

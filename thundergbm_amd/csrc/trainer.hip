@@ -80,7 +80,6 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 255,
                "max_num_bin %d out of the supported range 2..255", param.max_num_bin);
     TGBM_CHECK(objective_supported(param.objective), "undefined objective %s", param.objective.c_str());
-    if (param.bagging) log_info("bagging is ignored (the reference never calls its row sampler either)");
     TGBM_CHECK(param.column_sampling_rate > 0.f, "column_sampling_rate must be positive");
     // class bookkeeping of TreeTrainer::train (src/thundergbm/trainer.cu:24-37)
     if (param.objective.find("multi:") != std::string::npos || param.objective.find("binary:") != std::string::npos) {
@@ -391,6 +390,8 @@ Trainer::~Trainer() {
 
 void Trainer::sync() { HIP_CHECK(hipStreamSynchronize(stream_)); }
 
+// The first two steps of Booster::boost (include/thundergbm/booster.h:80-84): the objective's gradients, then
+// bagging when it is switched on.
 void Trainer::compute_gradient() {
     next_round_ready_ = false;
     if (objective_ == OBJ_RANK) {
@@ -398,9 +399,17 @@ void Trainer::compute_gradient() {
         // per-group generators from (ranking_obj.cpp:53): srand() makes a run repeatable
         rank_->gradient(d_yp_, d_gh_, (unsigned)std::rand(), rank_order_fresh_);
         rank_order_fresh_ = false;
-        return;
+    } else {
+        launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
     }
-    launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
+    if (param_.bagging) {
+        const size_t N = (size_t)param_.num_class * n_;  // the whole gradient array, as in the reference
+        if (d_bag_count_ == nullptr) {
+            d_bag_count_ = dalloc<int>(N);
+            HIP_CHECK(hipMemsetAsync(d_bag_count_, 0, sizeof(int) * N, stream_));
+        }
+        launch_bagging(stream_, (int)N, (unsigned)std::rand(), d_bag_count_, d_gh_);  // row_sampler.cu:15
+    }
 }
 
 // Shard::column_sampling (src/thundergbm/builder/shard.cu:8-22), once per boosting round
@@ -429,6 +438,9 @@ void Trainer::set_option(const std::string &key, double value) {
         TGBM_CHECK(value > 0, "column_sampling_rate must be positive");
         param_.column_sampling_rate = (float)value;
         if (!(value < 1)) tb_.ignored = nullptr;
+    } else if (key == "bagging") {
+        param_.bagging = value != 0;
+        next_round_ready_ = false;
     } else {
         fatal("unknown trainer option %s", key.c_str());
     }
@@ -560,7 +572,9 @@ void Trainer::boost(int rounds) {
     in_boost_ = true;
     for (int r = 0; r < rounds; ++r) {
         TGBM_CHECK(rounds_done_ < std::max(1, param_.n_trees), "boost called more often than n_trees");
-        const bool fuse = (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && param_.tree_per_rounds == 1;
+        // (with bagging the next round's gradients are not the plain ones the fused pass would compute)
+        const bool fuse = (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && param_.tree_per_rounds == 1 &&
+                          !param_.bagging;
         sample_columns();
         if (!next_round_ready_) compute_gradient();
         if (n_sets_ > 1) {

@@ -137,6 +137,42 @@ __global__ void k_gradient_softmax(int n, int K, const float *__restrict__ y, co
     }
 }
 
+// Bagging, RowSampler::do_bagging (src/thundergbm/row_sampler.cu:9-38): entry i of the gradient array draws
+// idx_i from thrust::default_random_engine(seed) after discard(i) through
+// thrust::uniform_int_distribution<int>(0, N - 1); every gradient pair is multiplied by the number of draws
+// that hit its index. thrust's default engine is minstd_rand (x <- 48271 x mod 2^31 - 1, a seed of 0 mod m
+// becomes 1), its integer distribution maps the engine's output u in [1, m - 1] to
+// int((u - 1) / (m - 1) * N) in double precision. The i + 1 steps of the engine are one modular power.
+__global__ void k_bagging_draw(int N, unsigned seed, int *__restrict__ count) {
+    constexpr unsigned long long M = 2147483647ull, A = 48271ull;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
+        unsigned long long x = seed % M;
+        if (x == 0) x = 1;
+        unsigned long long base = A, e = (unsigned long long)i + 1ull;  // discard(i), then one draw
+        while (e) {
+            if (e & 1ull) x = x * base % M;
+            base = base * base % M;
+            e >>= 1;
+        }
+        double r = (double)(unsigned)(x - 1ull);
+        r /= 1.0 + (double)(unsigned)(M - 2ull);  // 1 + (max - min) with min = 1, max = m - 1
+        const double lo = 0.0, hi = (double)(N - 1) + 1.0;
+        const int idx = (int)(r * (hi - lo) + lo);
+        atomicAdd(count + idx, 1);
+    }
+}
+
+__global__ void k_bagging_apply(int N, int *__restrict__ count, GHPair *__restrict__ gh) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
+        const int c = count[i];
+        count[i] = 0;  // ready for the next round
+        GHPair v = gh[i];
+        v.g = v.g * c;
+        v.h = v.h * c;
+        gh[i] = v;
+    }
+}
+
 // Row-blocked reductions: workgroup b owns rows [b * kRowBlock, (b + 1) * kRowBlock), thread t adds its
 // rows t, t + kBlock, ... in that order, then lanes, then wavefronts. Every kernel that produces
 // gradient statistics or metric partials follows this order, so fused and separate passes give the
@@ -1630,6 +1666,11 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_softmax<<<grid_for(n), kBlock, 0, s>>>(n, num_class, y, yp, gh);
     else
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
+}
+
+void launch_bagging(hipStream_t s, int N, unsigned seed, int *count, GHPair *gh) {
+    k_bagging_draw<<<grid_for(N), kBlock, 0, s>>>(N, seed, count);
+    k_bagging_apply<<<grid_for(N), kBlock, 0, s>>>(N, count, gh);
 }
 
 // Launchers: `tb` is the first buffer set to use, `n_class` consecutive sets (class trees of one round)
