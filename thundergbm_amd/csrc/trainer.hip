@@ -96,8 +96,10 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         // LambdaRank / LambdaRankNDCG with their default metrics (ranking_obj.cpp:98,115); one score per row
         objective_ = OBJ_RANK;
         metric_kind_ = param.objective == "rank:ndcg" ? RANK_METRIC_NDCG : RANK_METRIC_MAP;
-        TGBM_CHECK(param.num_class == 1, "ranking objectives train one score per instance (num_class %d)",
-                   param.num_class);
+        if (param.num_class != 1) {
+            log_info("ranking objectives train one score per instance: num_class %d -> 1", param.num_class);
+            param.num_class = 1;
+        }
     } else if (param.objective == "reg:linear") {
         objective_ = OBJ_SQUARE;
         metric_kind_ = 0;
@@ -404,6 +406,7 @@ void Trainer::compute_gradient() {
     }
     if (param_.bagging) {
         const size_t N = (size_t)param_.num_class * n_;  // the whole gradient array, as in the reference
+        TGBM_CHECK(N < ((size_t)1 << 31), "bagging: %zu gradient pairs exceed the int index range", N);
         if (d_bag_count_ == nullptr) {
             d_bag_count_ = dalloc<int>(N);
             HIP_CHECK(hipMemsetAsync(d_bag_count_, 0, sizeof(int) * N, stream_));
