@@ -493,12 +493,13 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
 // instead of storing and merging them was measured: 0.5 ms per tree slower on the 10M x 28 benchmark.)
 // Sum the private histograms of the node that was built from rows (64-bit integers, exact, any
 // order gives the same bits) and derive its sibling as parent - built (the reference's subtraction
-// trick, hist_tree_builder_single.cu:526-540). A block covers 32 bins of one sibling pair; its eight
-// thread groups stride over the pair's work items and are combined through LDS.
-constexpr int kMergeBins = 32;
-constexpr int kMergeGroups = kBlock / kMergeBins;
-
+// trick, hist_tree_builder_single.cu:526-540). A block covers kMergeBins bins of one sibling pair; its
+// thread groups stride over the pair's work items and are combined through LDS. Near the root a pair has
+// hundreds of items and the level only a few pairs, so narrow blocks (8 bins, 32 groups) are used there:
+// four times the workgroups and a quarter of the loads per thread.
+template <int kMergeBins>
 __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int level) {
+    constexpr int kMergeGroups = kBlock / kMergeBins;
     __shared__ long long s_g[kMergeGroups][kMergeBins], s_h[kMergeGroups][kMergeBins];
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     const longlong2 *__restrict__ partial = tb.partial;
@@ -1136,7 +1137,7 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
     const int nl = 1 << level, off = nl - 1;
     const int n_p = tb.ctl[level].n_pitems;
     int carry = 0;
-    constexpr int IPT = 8;  // items per thread and step
+    constexpr int IPT = 20;  // items per thread and step (10 M rows are 4 883 items: one step)
     for (int base = 0; base < n_p; base += kBlock * IPT) {
         const int i0 = base + threadIdx.x * IPT;
         int v[IPT];
@@ -1157,6 +1158,48 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
     }
     if (threadIdx.x == 0) tb.pitem_loff[n_p] = carry;
     __syncthreads();
+    if (nl <= kBlock) {
+        // the usual case (levels up to 8): one node per thread, everything after the scan stays in registers
+        const int x_in = threadIdx.x;
+        int built = -1, rows = 0;
+        if (x_in < nl) {
+            const TreeNode &nd = tb.nodes[off + x_in];
+            const int2 sg = tb.seg[off + x_in];
+            if (node_splits(nd)) {
+                const int nleft = tb.pitem_loff[tb.pitem_begin[x_in + 1]] - tb.pitem_loff[tb.pitem_begin[x_in]];
+                const int nright = (sg.y - sg.x) - nleft;
+                tb.node_nleft[x_in] = nleft;
+                tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
+                tb.seg[nd.rch_index] = make_int2(sg.x + nleft, sg.y);
+                built = (nleft <= nright) ? nd.lch_index : nd.rch_index;
+                rows = min(nleft, nright);
+            } else {
+                tb.node_nleft[x_in] = 0;
+                tb.seg[nd.lch_index] = make_int2(0, 0);
+                tb.seg[nd.rch_index] = make_int2(0, 0);
+            }
+            tb.hpair_built[x_in] = built;
+        }
+        const int total_rows = block_sum(rows, lds);
+        const int n_built = block_sum(built >= 0 ? 1 : 0, lds);
+        const int room = max(tb.target_hitems / 4, tb.target_hitems - n_built);
+        int chunk = (total_rows + room - 1) / room;
+        chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
+        const int cnt = built >= 0 ? (rows + chunk - 1) / chunk : 0;
+        int tot;
+        const int ex = block_excl_scan(cnt, lds, &tot);
+        if (x_in < nl) tb.hpair_begin[x_in] = ex;
+        if (threadIdx.x == 0) {
+            tb.hpair_begin[nl] = tot;
+            LevelCtl c;
+            c.hchunk = chunk;
+            c.n_hitems = tot;
+            c.n_pitems = 0;
+            c.rows_built = total_rows;
+            tb.ctl[level + 1] = c;
+        }
+        return;
+    }
     // children segments + rows of the built child of every pair
     int rows_sum = 0;
     for (int x_in = threadIdx.x; x_in < nl; x_in += kBlock) {
@@ -1737,8 +1780,13 @@ void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bi
 
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
-    dim3 grid((tb.n_bins + kMergeBins - 1) / kMergeBins, n_pairs, n_class);
-    k_hist_merge<<<grid, kBlock, 0, s>>>(tb, level);
+    if (n_pairs * n_class <= 4) {
+        dim3 grid((tb.n_bins + 7) / 8, n_pairs, n_class);
+        k_hist_merge<8><<<grid, kBlock, 0, s>>>(tb, level);
+    } else {
+        dim3 grid((tb.n_bins + 31) / 32, n_pairs, n_class);
+        k_hist_merge<32><<<grid, kBlock, 0, s>>>(tb, level);
+    }
 }
 
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
