@@ -1473,7 +1473,7 @@ __global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb_all, int l
 
 template <int MODE, bool SPARSE>
 __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBins dbins, CsrBins cbins, TreeEndArgs a) {
-    __shared__ int s_leaf[kRowBlock];
+    __shared__ short s_leaf[kRowBlock];  // node of every row of the block (depth <= 14: ids below 2^15), -1: none
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     if (MODE == 1) a.yp += (size_t)blockIdx.z * tb.n;  // class-major predictions
     __shared__ int s_list[kEndListCap][3];  // node, first and one-past-last list position
@@ -1493,7 +1493,9 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
         const int pa = b_lo[x], pb = b_hi[x];
         if (pb <= pa) continue;
         const TreeNode &nd = tb.nodes[x];
-        if (pb - pa > kEndInline) {
+        // (trees of up to kEndListCap row-holding nodes list every sub-range: the inline walk is a chain of
+        // dependent loads)
+        if (pb - pa > kEndInline || n_holders <= kEndListCap) {
             int e = atomicAdd(&s_n, 1);
             s_list[e][0] = x;
             s_list[e][1] = pa;
