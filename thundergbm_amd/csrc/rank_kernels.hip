@@ -201,13 +201,19 @@ __global__ __launch_bounds__(kBlock) void k_rank_map_partial(int n, const unsign
     store_block_sum(c, partial);
 }
 
-// (sum of the partials + groups that score 1 by definition) / number of groups
-__global__ void k_rank_metric_final(const double *__restrict__ partial, int n_partial, double constant, int n_groups,
-                                    float *__restrict__ out) {
-    if (blockIdx.x != 0 || threadIdx.x != 0) return;
-    double s = 0;
-    for (int i = 0; i < n_partial; ++i) s += partial[i];
-    *out = (float)((s + constant) / (double)n_groups);
+// (sum of the partials + groups that score 1 by definition) / number of groups; one workgroup, fixed order
+__global__ __launch_bounds__(kBlock) void k_rank_metric_final(const double *__restrict__ partial, int n_partial,
+                                                             double constant, int n_groups, float *__restrict__ out) {
+    __shared__ double s[kBlock];
+    double v = 0;
+    for (int i = threadIdx.x; i < n_partial; i += kBlock) v += partial[i];
+    s[threadIdx.x] = v;
+    __syncthreads();
+    for (int w = kBlock / 2; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) s[threadIdx.x] += s[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = (float)((s[0] + constant) / (double)n_groups);
 }
 
 int bits_for(long count) {
@@ -365,7 +371,7 @@ void RankContext::metric(int kind, const float *d_score, float *d_out) {
                                                         d_group_hits_, d_partial_);
         constant = zero_hit_groups_;
     }
-    k_rank_metric_final<<<1, 64, 0, stream_>>>(d_partial_, n_partial_, constant, n_groups_, d_out);
+    k_rank_metric_final<<<1, kBlock, 0, stream_>>>(d_partial_, n_partial_, constant, n_groups_, d_out);
     last_cur_ = cur;
     have_metric_order_ = true;
 }

@@ -12,15 +12,8 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / 64;
 constexpr int kHistMinChunk = 1024;
-#ifndef TGBM_HIST_BLOCK
-#define TGBM_HIST_BLOCK 1024
-#endif
-constexpr int kHistBlock = TGBM_HIST_BLOCK;  // threads per histogram workgroup (they share one LDS histogram)
-#ifndef TGBM_FLUSH_EVERY
-#define TGBM_FLUSH_EVERY 8192
-#endif
-constexpr int kHistFlushEvery = TGBM_FLUSH_EVERY;  // timing experiments only; must equal kHistFlushRows
-constexpr int kHistFlushRows = 8192;         // rows a packed 32+32-bit LDS bin may absorb before it is drained
+constexpr int kHistBlock = 1024;      // threads per histogram workgroup (they share one LDS histogram)
+constexpr int kHistFlushRows = 8192;  // rows a packed 32+32-bit LDS bin may absorb before it is drained
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
@@ -434,7 +427,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         // barriers), so the memory pipeline stays busy
         if (base + RPS * U < end) load_rows(base + RPS * U, pk_next, s_next);
         const int step_rows = min(RPS * U, end - base);
-        if (pending + step_rows > kHistFlushEvery) {
+        if (pending + step_rows > kHistFlushRows) {
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < SLOTS; ++k) {
@@ -470,7 +463,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         }
     }
     __syncthreads();
-    if (c.hchunk <= kHistFlushEvery) {
+    if (c.hchunk <= kHistFlushRows) {
         // an item this short was never drained: its packed LDS words are the complete sums and go out as
         // they are (8 bytes per bin instead of 16; k_hist_merge unpacks them)
         unsigned long long *out = reinterpret_cast<unsigned long long *>(partial) + (size_t)item * n_bins + bin0;
@@ -516,7 +509,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
     long long sg = 0, sh = 0;
     if (j < n_bins) {
-        if (tb.ctl[level].hchunk <= kHistFlushEvery) {  // packed 8-byte partials (see k_hist_dense)
+        if (tb.ctl[level].hchunk <= kHistFlushRows) {  // packed 8-byte partials (see k_hist_dense)
             const unsigned long long *packed = reinterpret_cast<const unsigned long long *>(partial);
             for (int it = ib + ig; it < ie; it += kMergeGroups) {
                 const unsigned long long t = packed[(size_t)it * n_bins + j];
@@ -611,7 +604,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb_all, CsrBins
 // no drain is needed; at the end the workgroup adds its non-zero slots to the node's histogram in HBM.
 // 1024 threads (16 wavefronts, one row each, the next row's header prefetched), two workgroups per CU.
 template <bool DIRECT>
-__global__ __launch_bounds__(TGBM_HIST_BLOCK) __attribute__((amdgpu_waves_per_eu(8)))
+__global__ __launch_bounds__(kHistBlock) __attribute__((amdgpu_waves_per_eu(8)))
 void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict__ gh, int n_pairs, int level) {
     extern __shared__ unsigned long long lds[];  // [2 * head_bins]: gradient, hessian of every slot
     __shared__ int s_info[3];
@@ -631,13 +624,13 @@ void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict_
         s_info[1] = min(sg.y, b + c.hchunk);
         s_info[2] = node - ((1 << level) - 1);
     }
-    for (int i = threadIdx.x; i < 2 * bins.head_bins; i += TGBM_HIST_BLOCK) lds[i] = 0ull;
+    for (int i = threadIdx.x; i < 2 * bins.head_bins; i += kHistBlock) lds[i] = 0ull;
     __syncthreads();
     const int begin = s_info[0], end = s_info[1];
     unsigned long long *h = reinterpret_cast<unsigned long long *>(cur_q + (size_t)s_info[2] * tb.n_bins);
     const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    constexpr int NW = TGBM_HIST_BLOCK / 64;
+    constexpr int NW = kHistBlock / 64;
     int pos = begin + w;
     GHPair s{0, 0};
     int e0 = 0, e1 = 0;
@@ -676,7 +669,7 @@ void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict_
         e1 = ne1;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < bins.head_bins; i += TGBM_HIST_BLOCK) {
+    for (int i = threadIdx.x; i < bins.head_bins; i += kHistBlock) {
         const unsigned long long g = lds[2 * i], hh = lds[2 * i + 1];
         if ((g | hh) != 0ull) {
             const size_t b = (size_t)bins.head_bin[i];
