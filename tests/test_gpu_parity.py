@@ -316,7 +316,7 @@ def test_boosting_teacher_forced(T, name, rounds):
 
 
 def test_free_running_c1_matches_oracle(T):
-    """BASELINE config 1 end to end (10 000 x 8, 40 trees, depth 6, lr 0.1) without teacher forcing."""
+    """Benchmark configuration 1 end to end (10 000 x 8, 40 trees, depth 6, lr 0.1) without teacher forcing."""
     X, y = D.config1(10000, 8, seed=0)
     val, rp, col = D.dense_to_csr(X)
     kw = dict(depth=6, n_trees=40, learning_rate=0.1, max_num_bin=255)

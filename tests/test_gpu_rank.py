@@ -106,6 +106,36 @@ def test_rank_gradient_and_metric_parity(T, objective, name, ties):
     s.close()
 
 
+def test_rank_full_size_parity(T):
+    """About a million rows in 8 000 query groups (several thousand radix tiles, 40 000 label runs): order
+    bit-exact, gradients and both metrics against the oracle, which handles this size in a second."""
+    rng = np.random.default_rng(17)
+    groups = rng.integers(40, 200, size=8000)
+    n = int(groups.sum())
+    F = 6
+    X = rng.normal(size=(n, F)).astype(np.float32)
+    rel = X[:, 0] + 0.5 * X[:, 1] + rng.normal(size=n)
+    y = np.digitize(rel, np.quantile(rel, [0.5, 0.75, 0.9, 0.97])).astype(np.float32)
+    rp = np.arange(0, n * F + 1, F, dtype=np.int32)
+    col = np.tile(np.arange(F, dtype=np.int32), n)
+    for objective in ("rank:pairwise", "rank:ndcg"):
+        s = T.Session(X.ravel(), rp, col, y, depth=6, n_trees=3, learning_rate=0.3, objective=objective,
+                      groups=groups)
+        LIBC.srand(9)
+        s.boost(2)  # scores with many distinct values and, from the leaves, many ties
+        score = s.y_pred()
+        draw = _round_seed(31)
+        s.gradient()
+        gh, order = s.gh(), s.get("rank_order", np.int32)
+        ogh, oorder, _ = O.rank_gradient(objective, y, score, groups, draw)
+        assert np.array_equal(order, oorder)
+        assert np.abs(gh.astype(np.float64) - ogh).max() <= 1e-5 * np.abs(ogh).max()
+        assert abs(s.metric() - O.rank_metric(objective, y, score, groups)) <= 1e-5
+        log = s.metric_log()
+        assert log[1] > log[0]
+        s.close()
+
+
 def test_rank_gradient_is_bit_reproducible(T):
     (val, rp, col), y, groups = _ranking_case("many_groups")
     s = T.Session(val, rp, col, y, depth=4, n_trees=2, objective="rank:ndcg", groups=groups)
