@@ -1,4 +1,5 @@
 // extern "C" layer declared in include/thundergbm.h.
+#include <chrono>
 #include <cstring>
 #include <memory>
 
@@ -67,7 +68,10 @@ void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, f
     p.tree_per_rounds = 1;
     set_logger(verbose);
     DataSet ds;
-    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, label, group, num_group, p);
+    auto t0 = std::chrono::steady_clock::now();
+    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, label, group, num_group, p, false);
+    log_debug("host-side dataset checks and label grouping: %.3f s",
+              std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count());
     *num_class = p.num_class;
     std::vector<std::vector<Tree>> boosted = train(p, ds);
     TGBM_CHECK((int)boosted.size() == n_trees, "%d v.s. %zu", n_trees, boosted.size());
@@ -85,7 +89,7 @@ void sparse_predict_scikit(int row_size, float *val, int *row_ptr, int *col_ptr,
     p.num_class = num_class;
     DataSet ds;
     GBMParam load_param = p;
-    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, group, num_group, load_param);
+    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, group, num_group, load_param, false);
     set_logger(verbose);
     ds.label.clear();
     if (group_label != nullptr && objective_needs_group_label(p.objective))
@@ -245,7 +249,7 @@ tgbm_trainer *tgbm_trainer_create_grouped(int row_size, const float *val, const 
     p.num_class = num_class;
     p.verbose = verbose;
     p.tree_method = "hist";
-    t->dataset.load_from_sparse(row_size, val, row_ptr, col_ptr, label, group, num_group, p);
+    t->dataset.load_from_sparse(row_size, val, row_ptr, col_ptr, label, group, num_group, p, false);
     t->impl.reset(new Trainer(t->dataset, p));
     t->dataset.val = nullptr;  // the caller's buffers are not referenced after this call
     t->dataset.col_idx = nullptr;
@@ -303,7 +307,7 @@ void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const 
     GBMParam load_param = p;
     int saved = g_verbose;
     g_verbose = 0;
-    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, nullptr, 0, load_param);
+    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, nullptr, 0, load_param, false);
     g_verbose = saved;
     std::vector<float> r = predict_raw(p, to_nested(model, n_trees, trees_per_iter), ds);
     std::memcpy(out, r.data(), r.size() * sizeof(float));

@@ -250,6 +250,9 @@ struct PairSorter {
 // when the scan scratch has to grow (first call).
 int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
 
+// Largest of n non-negative ints in device memory (synchronises; 0 for n == 0).
+int device_max_int(hipStream_t s, const int *d_v, long n);
+
 // Host -> device copy of a large pageable array through pinned staging buffers (returns when done).
 void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);
 

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstring>
 #include <fstream>
+#include <iterator>
 #include <thread>
 #include <map>
 #include <sstream>
@@ -59,7 +60,8 @@ bool objective_supported(const std::string &o) {
 }
 
 void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr, const int *col_idx,
-                               const float *labels, const int *grp, int num_group, GBMParam &param) {
+                               const float *labels, const int *grp, int num_group, GBMParam &param,
+                               bool count_features) {
     n_features_ = 0;
     y.clear();
     label.clear();
@@ -71,23 +73,26 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
     this->row_ptr = row_ptr;
     this->col_idx = col_idx;
     this->nnz = nnz;
-    // largest column index, on a few threads when the matrix is large
-    const int n_thr = nnz > (1 << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
-    std::vector<int> part_max(n_thr, 0);
-    auto scan = [&](int t) {
-        const long b = (long)nnz * t / n_thr, e = (long)nnz * (t + 1) / n_thr;
-        int m = 0;
-        for (long i = b; i < e; ++i) m = std::max(m, col_idx[i]);
-        part_max[t] = m;
-    };
-    std::vector<std::thread> pool;
-    for (int t = 1; t < n_thr; ++t) pool.emplace_back(scan, t);
-    scan(0);
-    for (auto &th : pool) th.join();
-    int max_col = 0;
-    for (int m : part_max) max_col = std::max(max_col, m);
-    n_features_ = (size_t)max_col + 1;
-    log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
+    features_counted = count_features;
+    if (count_features) {
+        // largest column index, on a few threads when the matrix is large
+        const int n_thr = nnz > (1 << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
+        std::vector<int> part_max(n_thr, 0);
+        auto scan = [&](int t) {
+            const long b = (long)nnz * t / n_thr, e = (long)nnz * (t + 1) / n_thr;
+            int m = 0;
+            for (long i = b; i < e; ++i) m = std::max(m, col_idx[i]);
+            part_max[t] = m;
+        };
+        std::vector<std::thread> pool;
+        for (int t = 1; t < n_thr; ++t) pool.emplace_back(scan, t);
+        scan(0);
+        for (auto &th : pool) th.join();
+        int max_col = 0;
+        for (int m : part_max) max_col = std::max(max_col, m);
+        n_features_ = (size_t)max_col + 1;
+        log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
+    }
     if (labels != nullptr && objective_needs_group_label(param.objective)) {
         group_label();
         param.num_class = (int)label.size();
@@ -111,23 +116,39 @@ void DataSet::load_group_file(const std::string &file_name) {
 }
 
 void DataSet::group_label() {
-    // labels are truncated to int for the label set; the set is small, so it is kept sorted while scanning
-    // (no sort of all rows)
+    // labels are truncated to int for the label set; the set is small, so every thread keeps a sorted set of
+    // its part while scanning (no sort of all rows) and the sets are merged
+    const int n_thr = y.size() > (1u << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
+    std::vector<std::vector<int>> part(n_thr);
+    auto collect = [&](int t) {
+        const size_t b = y.size() * t / n_thr, e = y.size() * (t + 1) / n_thr;
+        std::vector<int> &set = part[t];
+        bool have_last = false;
+        int last = 0;
+        for (size_t i = b; i < e; ++i) {
+            const int iv = (int)y[i];
+            if (have_last && iv == last) continue;
+            have_last = true;
+            last = iv;
+            auto it = std::lower_bound(set.begin(), set.end(), iv);
+            if (it == set.end() || *it != iv) set.insert(it, iv);
+        }
+    };
+    {
+        std::vector<std::thread> pool;
+        for (int t = 1; t < n_thr; ++t) pool.emplace_back(collect, t);
+        collect(0);
+        for (auto &th : pool) th.join();
+    }
     std::vector<int> distinct;
-    bool have_last = false;
-    int last = 0;
-    for (float v : y) {
-        const int iv = (int)v;
-        if (have_last && iv == last) continue;
-        have_last = true;
-        last = iv;
-        auto it = std::lower_bound(distinct.begin(), distinct.end(), iv);
-        if (it == distinct.end() || *it != iv) distinct.insert(it, iv);
+    for (const std::vector<int> &set : part) {
+        std::vector<int> merged;
+        std::set_union(distinct.begin(), distinct.end(), set.begin(), set.end(), std::back_inserter(merged));
+        distinct.swap(merged);
     }
     label.assign(distinct.begin(), distinct.end());
     // a row's class is the position of its label in the set; labels that are not in it (non-integers)
     // read as class 0, like a failed lookup in the reference's map
-    const int n_thr = y.size() > (1u << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
     auto remap = [&](int t) {
         const size_t b = y.size() * t / n_thr, e = y.size() * (t + 1) / n_thr;
         for (size_t i = b; i < e; ++i) {

@@ -22,7 +22,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     hipError_t e = hipGetDeviceCount(&n_dev);
     TGBM_CHECK(e == hipSuccess && n_dev >= 1, "no HIP device available: this library has no CPU path");
     const int n = (int)ds.n_instances();
-    const int F = (int)ds.n_features();
+    int F = (int)ds.n_features();
     const long nnz = ds.nnz;
     TGBM_CHECK(!model.empty() && !model.front().empty(), "empty model");
     const int n_iter = (int)model.size();
@@ -53,6 +53,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
         upload_large(s, d_val, ds.val, sizeof(float) * (size_t)nnz);
         upload_large(s, d_col, ds.col_idx, sizeof(int) * (size_t)nnz);
     }
+    if (!ds.features_counted) F = device_max_int(s, d_col, nnz) + 1;
     HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.row_ptr, sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
     HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));
     launch_fill_f32(s, d_out, 0.f, n_out);

@@ -385,6 +385,28 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     return out;
 }
 
+// Largest element of n non-negative ints (0 for n == 0).
+__global__ __launch_bounds__(256) void k_max_int(const int *__restrict__ v, long n, int *__restrict__ out) {
+    int m = 0;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) m = max(m, v[i]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d));
+    if ((threadIdx.x & 63) == 0) atomicMax(out, m);
+}
+
+int device_max_int(hipStream_t s, const int *d_v, long n) {
+    if (n <= 0) return 0;
+    int *d_out = nullptr;
+    HIP_CHECK(hipMalloc(&d_out, sizeof(int)));
+    HIP_CHECK(hipMemsetAsync(d_out, 0, sizeof(int), s));
+    k_max_int<<<grid_for((size_t)n, 4096), 256, 0, s>>>(d_v, n, d_out);
+    int h = 0;
+    HIP_CHECK(hipMemcpyAsync(&h, d_out, sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipFree(d_out));
+    return h;
+}
+
 void ScanScratch::release() {
     for (Level &lv : levels) {
         if (lv.sums) (void)hipFree(lv.sums);

@@ -132,10 +132,15 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     HIP_CHECK(hipStreamSynchronize(stream_));
     log_debug("upload of %.2f GB: %.3f s", (double)nnz_ * 8e-9,
               std::chrono::duration<double>(std::chrono::steady_clock::now() - t_up).count());
+    if (!ds.features_counted) {  // the number of features = largest column index + 1 (dataset.cpp:40-46)
+        F_ = device_max_int(stream_, d_col, nnz_) + 1;
+        log_info("#instances = %d, #features = %d", n_, F_);
+    }
     log_info("Fast getting cut points...");
     auto t_cut = std::chrono::steady_clock::now();
     cuts_ = build_cut_points(stream_, F_, nnz_, d_val, d_col, param_.max_num_bin);
     log_debug("cut points: %.3f s", std::chrono::duration<double>(std::chrono::steady_clock::now() - t_cut).count());
+    auto t_bin = std::chrono::steady_clock::now();
     n_bins_ = cuts_.n_bins;
     allocs_.push_back(cuts_.cut_row_ptr);
     if (cuts_.cut_val) allocs_.push_back(cuts_.cut_val);
@@ -244,6 +249,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     // ---- labels, predictions, gradients (Booster::init) --------------------------------------
     d_y_ = dalloc<float>(n_);
     upload(stream_, d_y_, ds.y.data(), (size_t)n_);
+    log_debug("bin matrix: %.3f s", std::chrono::duration<double>(std::chrono::steady_clock::now() - t_bin).count());
+    auto t_rest = std::chrono::steady_clock::now();
     n_yp_ = (long)param_.num_class * n_;
     if (param_.num_class == 2) n_yp_ = n_;
     d_yp_ = dalloc<float>((size_t)n_yp_);
@@ -275,6 +282,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     }
     param.base_score = param_.base_score;
     HIP_CHECK(hipStreamSynchronize(stream_));
+    log_debug("training buffers and base score: %.3f s",
+              std::chrono::duration<double>(std::chrono::steady_clock::now() - t_rest).count());
 }
 
 void Trainer::alloc_tree_buffers() {
@@ -750,7 +759,10 @@ std::vector<std::vector<Tree>> train(GBMParam &param, const DataSet &dataset) {
     trainer.sync();
     auto stop = std::chrono::high_resolution_clock::now();
     log_info("training time = %g", std::chrono::duration<float>(stop - start).count());
-    return trainer.model_to_host();
+    std::vector<std::vector<Tree>> model = trainer.model_to_host();
+    log_debug("model to host: %.3f s",
+              std::chrono::duration<double>(std::chrono::high_resolution_clock::now() - stop).count());
+    return model;
 }
 
 }  // namespace tgbm
