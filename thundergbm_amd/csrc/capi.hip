@@ -89,8 +89,11 @@ void sparse_predict_scikit(int row_size, float *val, int *row_ptr, int *col_ptr,
     p.num_class = num_class;
     DataSet ds;
     GBMParam load_param = p;
-    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, group, num_group, load_param, false);
     set_logger(verbose);
+    auto t0 = std::chrono::steady_clock::now();
+    ds.load_from_sparse(row_size, val, row_ptr, col_ptr, nullptr, group, num_group, load_param, false);
+    log_debug("predict: host-side dataset %.3f s",
+              std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count());
     ds.label.clear();
     if (group_label != nullptr && objective_needs_group_label(p.objective))
         for (int i = 0; i < num_class; ++i) ds.label.push_back(group_label[i]);

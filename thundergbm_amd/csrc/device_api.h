@@ -253,13 +253,15 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
 // Largest of n non-negative ints in device memory (synchronises; 0 for n == 0).
 int device_max_int(hipStream_t s, const int *d_v, long n);
 
-// Host -> device copy of a large pageable array through pinned staging buffers (returns when done).
+// Host -> device copy of a pageable array on stream s; large ones go through pinned staging buffers and are
+// complete on return, small ones (< 128 MB) are a plain stream-ordered hipMemcpyAsync.
 void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);
 
-// prediction
+// prediction of the n rows that row_ptr addresses (entry offsets into col / val); out[t * out_stride + i] for
+// class tree t and row i, out_stride = 0 means n (a slice of a larger row set passes the whole set's size)
 void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
                     const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
-                    float *out);
+                    float *out, size_t out_stride = 0);
 void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y);
 
 }  // namespace tgbm

@@ -34,7 +34,7 @@ template <typename ACC, bool INF_IS_MISSING>
 __global__ __launch_bounds__(kBlock) void k_predict(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
                                                    const float *__restrict__ val, const TreeNode *__restrict__ model,
                                                    int n_iter, int n_class_trees, int n_nodes, float lr,
-                                                   float base_score, float *__restrict__ out) {
+                                                   float base_score, float *__restrict__ out, size_t out_stride) {
     const int i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     const int rb = row_ptr[i];
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kBlock) void k_predict(int n, const int *__restrict
             }
             sum += lr * nd[cur].base_weight;
         }
-        out[(size_t)t * n + i] += (float)sum;
+        out[(size_t)t * out_stride + i] += (float)sum;
     }
 }
 
@@ -74,7 +74,8 @@ __global__ __launch_bounds__(kStageBlock) void k_predict_staged(int n, int F, co
                                                                const float *__restrict__ val,
                                                                const TreeNode *__restrict__ model, int n_iter,
                                                                int n_class_trees, int n_nodes, float lr,
-                                                               float base_score, float *__restrict__ out) {
+                                                               float base_score, float *__restrict__ out,
+                                                               size_t out_stride) {
     extern __shared__ float dense[];  // [F][kStageBlock]
     const int i = blockIdx.x * kStageBlock + threadIdx.x;
     for (int f = 0; f < F; ++f) dense[f * kStageBlock + threadIdx.x] = INFINITY;
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(kStageBlock) void k_predict_staged(int n, int F, co
             }
             sum += lr * nd[cur].base_weight;
         }
-        out[(size_t)t * n + i] += (float)sum;
+        out[(size_t)t * out_stride + i] += (float)sum;
     }
 }
 
@@ -142,17 +143,18 @@ __global__ void k_predict_transform(int kind, int n, int K, const float *__restr
 
 void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
                     const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
-                    float *out) {
+                    float *out, size_t out_stride) {
     if (n == 0) return;
+    if (out_stride == 0) out_stride = (size_t)n;
     if (n_class_trees > 1) base_score = 0;  // predictor.cu:81-83
     const bool dense_path = (size_t)F * 128 * sizeof(float) <= 48 * 1024;
     int grid = (n + kBlock - 1) / kBlock;
     if (dense_path)
         k_predict_staged<<<(n + kStageBlock - 1) / kStageBlock, kStageBlock, (size_t)F * kStageBlock * sizeof(float), s>>>(
-            n, F, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr, base_score, out);
+            n, F, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr, base_score, out, out_stride);
     else
         k_predict<float, false><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, model, n_iter, n_class_trees, n_nodes, lr,
-                                                       base_score, out);
+                                                       base_score, out, out_stride);
 }
 
 void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y) {

@@ -1,4 +1,6 @@
 // Host side of prediction: the reference's Predictor (src/thundergbm/predictor.cu:11-86).
+#include <algorithm>
+#include <chrono>
 #include <cstring>
 
 #include "device_api.h"
@@ -38,6 +40,12 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
             ++t;
         }
     }
+    auto t_begin = std::chrono::steady_clock::now();
+    auto lap = [&](const char *what) {
+        auto now = std::chrono::steady_clock::now();
+        log_debug("predict: %s %.3f s", what, std::chrono::duration<double>(now - t_begin).count());
+        t_begin = now;
+    };
     hipStream_t s;
     HIP_CHECK(hipStreamCreate(&s));
     float *d_val = nullptr, *d_out = nullptr, *d_label = nullptr;
@@ -49,16 +57,38 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n + 1)));
     HIP_CHECK(hipMalloc(&d_model, sizeof(TreeNode) * flat.size()));
     HIP_CHECK(hipMalloc(&d_out, sizeof(float) * std::max(n_out, (size_t)1)));
-    if (nnz) {
-        upload_large(s, d_val, ds.val, sizeof(float) * (size_t)nnz);
-        upload_large(s, d_col, ds.col_idx, sizeof(int) * (size_t)nnz);
-    }
-    if (!ds.features_counted) F = device_max_int(s, d_col, nnz) + 1;
     HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.row_ptr, sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
     HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));
     launch_fill_f32(s, d_out, 0.f, n_out);
-    launch_predict(s, n, F, d_row_ptr, d_col, d_val, d_model, n_iter, nct, n_nodes, param.learning_rate,
-                   param.base_score, d_out);
+    // The column indices go up first (the feature count, which selects the traversal kernel, may have to be
+    // taken from them), then the values in slices of whole rows on a second stream: the traversal of a
+    // slice runs while the next slice crosses PCIe.
+    if (nnz) upload_large(s, d_col, ds.col_idx, sizeof(int) * (size_t)nnz);
+    if (!ds.features_counted) F = device_max_int(s, d_col, nnz) + 1;
+    HIP_CHECK(hipStreamSynchronize(s));
+    lap("allocation, model and column indices");
+    {
+        hipStream_t s_up;
+        HIP_CHECK(hipStreamCreate(&s_up));
+        const long slice_entries = 64l << 20;  // ~256 MB of values per slice
+        int r0 = 0;
+        while (r0 < n) {
+            const long e0 = ds.row_ptr[r0];
+            // last row whose entries still fit the slice (at least one row)
+            const int *first = ds.row_ptr + r0 + 1, *last = ds.row_ptr + n + 1;
+            int r1 = (int)(std::upper_bound(first, last, (int)std::min<long>(e0 + slice_entries, nnz)) - ds.row_ptr) - 1;
+            r1 = std::max(r1, r0 + 1);
+            const long e1 = ds.row_ptr[r1];
+            if (e1 > e0) upload_large(s_up, d_val + e0, ds.val + e0, sizeof(float) * (size_t)(e1 - e0));
+            HIP_CHECK(hipStreamSynchronize(s_up));  // small copies return before they are done
+            launch_predict(s, r1 - r0, F, d_row_ptr + r0, d_col, d_val, d_model, n_iter, nct, n_nodes,
+                           param.learning_rate, param.base_score, d_out + r0, (size_t)n);
+            r0 = r1;
+        }
+        HIP_CHECK(hipStreamSynchronize(s));
+        HIP_CHECK(hipStreamDestroy(s_up));
+    }
+    lap("values and traversal");
     size_t n_ret = n_out;
     if (log_metric && objective_needs_groups(param.objective)) {
         // MAP / NDCG need the query groups of the rows that are scored (Predictor::predict configures the
@@ -111,6 +141,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     std::vector<float> out(n_ret);
     if (n_ret) HIP_CHECK(hipMemcpyAsync(out.data(), d_out, sizeof(float) * n_ret, hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));
+    lap("transform and download");
     HIP_CHECK(hipFree(d_val));
     HIP_CHECK(hipFree(d_col));
     HIP_CHECK(hipFree(d_row_ptr));
@@ -118,6 +149,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipFree(d_out));
     if (d_label) HIP_CHECK(hipFree(d_label));
     HIP_CHECK(hipStreamDestroy(s));
+    lap("release");
     return out;
 }
 
