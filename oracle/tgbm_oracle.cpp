@@ -879,13 +879,13 @@ void build_tree(Oracle &o, int k) {
 
 // Booster::boost, include/thundergbm/booster.h:76-93
 void boost_round(Oracle &o) {
-    sample_columns(o);
     if (is_rank(o.objective))
         rank_gradient(o.objective == "rank:ndcg", o.n, o.y.data(), o.y_pred.data(), o.group, (unsigned)std::rand(),
                       o.gh.data(), nullptr, nullptr);
     else
         gradient(o.objective, o.n, o.num_class, o.y.data(), o.y_pred.data(), o.gh.data());
     if (o.bagging) do_bagging(o.gh, std::rand());  // booster.h:84
+    sample_columns(o);  // first step of build_approximate, tree_builder.cu:150-152
     std::vector<Node> round_trees;
     for (int k = 0; k < o.tree_per_rounds; ++k) {
         build_tree(o, k);

@@ -203,6 +203,49 @@ def test_rank_boosting_teacher_forced(T, objective, name):
     s.close()
 
 
+@pytest.mark.parametrize("layout", ["dense", "sparse"])
+def test_rank_with_bagging_and_column_sampling(T, layout):
+    """Everything that draws from rand() in one round, in the reference's order (booster.h:80-84 gradients,
+    then bagging; tree_builder.cu:150-152 column sampling at the start of the tree building): the ranking
+    partner seed, the bagging seed, the shuffle of the columns. Both sides start every round from the same
+    srand() and must build the same trees."""
+    os.environ["TGBM_LAYOUT"] = layout
+    try:
+        (val, rp, col), y, groups = _ranking_case("many_groups")
+        rounds = 4
+        kw = dict(depth=4, n_trees=rounds, learning_rate=0.3, objective="rank:ndcg", min_child_weight=0.05)
+        s = T.Session(val, rp, col, y, groups=groups, **kw)
+        o = O.Oracle(val, rp, col, y, debug=True, groups=groups, **kw).prepare()
+        s.set_option("bagging", 1)
+        s.set_option("column_sampling_rate", 0.5)
+        o.set_bagging(True)
+        o.set_column_sampling_rate(0.5)
+        n = s.n
+        ties = 0
+        for r in range(rounds):
+            o.set_y_pred(s.y_pred())
+            LIBC.srand(900 + r)
+            o.compute_gradient()
+            o.sample_columns()
+            ogh = o.gh()
+            LIBC.srand(900 + r)
+            s.gradient()
+            gh = s.gh()
+            assert np.abs(gh.astype(np.float64) - ogh).max() <= 1e-5 * np.abs(ogh).max()
+            LIBC.srand(900 + r)
+            s.boost(1)
+            o.set_gh(gh)
+            o.build_tree(0)
+            ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
+            d = P.compare_trees(s.model()[r, 0], o.nodes(), 1.0, crp=s.cuts()[1], orc_scores=o.tree_scores(),
+                                abs_scale=(ghk[0], ghk[1]), mcw=0.05)
+            ties += len(d.near_ties)
+        assert ties <= rounds
+        s.close()
+    finally:
+        os.environ.pop("TGBM_LAYOUT", None)
+
+
 def test_ranker_through_the_c_abi(T, tmp_path):
     """sparse_train_scikit / sparse_predict_scikit with group sizes (scikit_tgbm.cpp:26-121 with the group and
     num_group arguments): the model ranks better than the constant score and predicts raw scores."""

@@ -587,8 +587,10 @@ void Trainer::boost(int rounds) {
         // (with bagging the next round's gradients are not the plain ones the fused pass would compute)
         const bool fuse = (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && param_.tree_per_rounds == 1 &&
                           !param_.bagging;
-        sample_columns();
+        // the reference's order of the draws from rand(): gradients (ranking partner seed), bagging seed
+        // (booster.h:80-84), then the column shuffle at the start of build_approximate (tree_builder.cu:150-152)
         if (!next_round_ready_) compute_gradient();
+        sample_columns();
         if (n_sets_ > 1) {
             build_round_together();
         } else {
