@@ -109,7 +109,12 @@ void tgbm_trainer_destroy(tgbm_trainer *t);
  * below 1 every boosting round ignores max(1, int(n_features * rate)) randomly chosen columns in its split
  * search (Shard::column_sampling, builder/shard.cu:8-22; the shuffle draws from the process-wide rand()).
  * "bagging" (common.h:97): non-zero makes every gradient pass multiply the gradient pairs by bootstrap draw
- * counts (RowSampler::do_bagging, row_sampler.cu:9-38; seeded with one rand() per pass). */
+ * counts (RowSampler::do_bagging, row_sampler.cu:9-38; seeded with one rand() per pass).
+ * "reorder_first", "reorder_every", "reorder_min_rows" (no counterpart in the reference): tgbm_trainer_boost
+ * physically re-orders the rows by the leaves of the tree just built after `reorder_first` trees and then
+ * every `reorder_every` trees (defaults 2 and 32; 0 = never) when the dataset has at least
+ * `reorder_min_rows` rows (default 2^20), the layout is dense and a round builds one tree. Results do not
+ * depend on it beyond float round-off, and all per-row buffers keep the caller's row order. */
 void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value);
 /* The column sampling of one round for stage-wise driving (tgbm_trainer_boost does it itself). */
 void tgbm_trainer_sample_columns(tgbm_trainer *t);
@@ -130,7 +135,7 @@ float tgbm_trainer_metric(tgbm_trainer *t);
 
 /* Integer facts: n, n_features, n_bins, num_class, tree_per_rounds, n_nodes, dense_W,
  * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems, n_sets (class trees
- * of a round built by common launches). */
+ * of a round built by common launches), reorders_done. */
 int tgbm_trainer_info(tgbm_trainer *t, const char *key);
 float tgbm_trainer_base_score(tgbm_trainer *t);
 

@@ -361,6 +361,88 @@ def test_bagging_through_the_c_abi(T):
     assert np.sqrt(np.mean((preds[0] - y) ** 2)) < 0.8 * np.std(y)  # still learns
 
 
+@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin")])
+def test_row_reordering_is_invisible(T, objective, kind):
+    """boost() physically re-orders the rows by the leaves of a tree every few rounds (here: after every
+    round) so that the rows of a node lie together. Histograms are exact integer sums, so the trees must not
+    change, and everything handed out per row must stay in the caller's row order."""
+    n, F = 30000, 40  # 40 features: two feature blocks
+    val, rp, col = _ragged(n, F, 9, F)
+    y = _target(val, rp, col, n, F, 9, kind)
+    kw = dict(objective=objective, n_trees=7, depth=6, max_num_bin=64, learning_rate=0.3)
+    runs = []
+    for first, every in ((0, 0), (1, 1), (2, 3)):
+        s = T.Session(val, rp, col, y, **kw)
+        s.set_option("reorder_min_rows", 0)
+        s.set_option("reorder_first", first)
+        s.set_option("reorder_every", every)
+        before = s.binmat().copy()
+        s.boost(7)
+        assert s.info("reorders_done") == {0: 0, 1: 7, 2: 2}[first]
+        runs.append(dict(model=s.model().copy(), yp=s.y_pred().copy(), nid=s.nid().copy(), y=s.y().copy(),
+                         binmat=s.binmat().copy(), metric=s.metric_log().copy(), before=before))
+        s.close()
+    base = runs[0]
+    for r in runs[1:]:
+        assert np.array_equal(r["y"], base["y"]) and np.array_equal(r["binmat"], base["binmat"])
+        assert np.array_equal(r["before"], r["binmat"])
+        # (default_right is left out: without missing values in a node it is decided by the round-off of
+        # node sum - feature total, a float reduction over the rows)
+        for key in ("split_fid", "split_bid", "lch", "rch", "is_valid", "is_leaf", "split_value"):
+            assert np.array_equal(r["model"][key], base["model"][key]), key
+        # node sums hang off float reductions over all rows: another order of additions, the same value up to
+        # round-off at the scale of the largest sums (the root's own sum is a cancellation near zero)
+        scale = float(np.abs(base["model"]["sum_g"]).max())
+        np.testing.assert_allclose(r["model"]["sum_g"], base["model"]["sum_g"], rtol=1e-5, atol=1e-6 * scale)
+        np.testing.assert_allclose(r["model"]["base_weight"], base["model"]["base_weight"], rtol=1e-4, atol=1e-6)
+        assert np.array_equal(r["nid"], base["nid"])
+        np.testing.assert_allclose(r["yp"], base["yp"], rtol=1e-5, atol=2e-6 * float(np.abs(base["yp"]).max()))
+        np.testing.assert_allclose(r["metric"], base["metric"], rtol=1e-5)
+
+
+def test_row_reordering_then_stagewise_and_setters(T):
+    """After a re-ordering, the stage-wise calls, set("y_pred") / set("gh") and the row lists still speak the
+    caller's row order: a lock-step tree against the oracle on top of re-ordered rows."""
+    n, F = 20000, 6
+    val, rp, col = _ragged(n, F, 12, F)
+    y = _target(val, rp, col, n, F, 12, "reg")
+    kw = dict(objective="reg:linear", n_trees=5, depth=5, max_num_bin=32, learning_rate=0.5)
+    s = T.Session(val, rp, col, y, **kw)
+    for key, v in (("reorder_min_rows", 0), ("reorder_first", 1), ("reorder_every", 1)):
+        s.set_option(key, v)
+    s.boost(2)
+    assert s.info("reorders_done") == 2
+    o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    o.set_y_pred(s.y_pred())
+    o.compute_gradient()
+    s.gradient()
+    gh = s.gh()
+    np.testing.assert_allclose(gh, o.gh(), rtol=1e-5, atol=2e-7)
+    s.set("gh", gh)  # round trip through the permutation
+    assert np.array_equal(s.gh(), gh)
+    o.set_gh(gh)
+    s.tree_init(0)
+    o.tree_init(0)
+    for level in range(5):
+        s.find_split(level)
+        o.find_split(level)
+        o.update_tree()
+        o.set_nodes(s.nodes())  # both sides apply the same splits (near ties are the other tests' subject)
+        s.partition(level)
+        o.update_ins2node()
+        assert np.array_equal(s.nid(), o.nid()), level
+        if level < 4:  # the row lists name rows by the caller's ids
+            seg = s.get("seg", np.int32, (-1, 2))
+            lists = s.get("ridx%d" % ((level + 1) & 1), np.int32)
+            nid = s.nid()
+            for x in range((1 << (level + 1)) - 1, (1 << (level + 2)) - 1):
+                a, b = seg[x]
+                if b > a:
+                    assert np.array_equal(np.sort(lists[a:b]), np.flatnonzero(nid == x))
+    s.finish_tree(0)
+    s.close()
+
+
 @pytest.mark.parametrize("layout", ["dense", "sparse"])
 def test_training_is_bit_reproducible(T, layout):
     """Histograms are exact integer sums (LDS and HBM atomics alike) and every float reduction has a fixed

@@ -407,6 +407,82 @@ int device_max_int(hipStream_t s, const int *d_v, long n) {
     return h;
 }
 
+// ---- physical re-ordering of the rows (see Trainer::reorder_rows) ---------------------------------
+// Sort keys: the node a row ended in; payload: the row's current position.
+__global__ __launch_bounds__(256) void k_reorder_keys(int n, const int *__restrict__ nid,
+                                                     unsigned long long *__restrict__ keys, int *__restrict__ vals) {
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= n) return;
+    keys[p] = (unsigned long long)(unsigned)max(nid[p], 0);
+    vals[p] = p;
+}
+
+// dst[p] = src[from[p]] for n rows of `words` dwords; consecutive lanes take consecutive dwords of a row.
+__global__ __launch_bounds__(256) void k_gather_rows(int n, int words, const int *__restrict__ from,
+                                                    const unsigned *__restrict__ src, unsigned *__restrict__ dst) {
+    const size_t total = (size_t)n * words;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t p = i / words, w = i % words;
+        dst[i] = src[(size_t)from[p] * words + w];
+    }
+}
+
+// perm_new[p] = perm_old[from[p]], or from[p] itself while the rows are still in their original order
+__global__ __launch_bounds__(256) void k_gather_perm(int n, const int *__restrict__ from,
+                                                    const int *__restrict__ perm_old, int *__restrict__ perm_new) {
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= n) return;
+    const int f = from[p];
+    perm_new[p] = perm_old != nullptr ? perm_old[f] : f;
+}
+
+// Column-major copy of one feature block from its row-major form: a tile of 256 rows x W bytes goes through
+// LDS so that both the reads (whole rows) and the writes (256 consecutive bytes of one feature) are coalesced.
+__global__ __launch_bounds__(256) void k_cols_from_rows(int n, int W, int F, int block, const uint8_t *__restrict__ rows,
+                                                       uint8_t *__restrict__ colmat, size_t col_stride) {
+    extern __shared__ uint8_t tile[];  // [256][W + 4]: the padding spreads a column's bytes over the banks
+    const int r0 = blockIdx.x * 256;
+    const int pitch = W + 4;
+    const int words = W / 4;
+    for (int i = threadIdx.x; i < 256 * words; i += 256) {
+        const int r = i / words, w = i % words;
+        unsigned v = 0xffffffffu;
+        if (r0 + r < n) v = reinterpret_cast<const unsigned *>(rows + (size_t)(r0 + r) * W)[w];
+        *reinterpret_cast<unsigned *>(tile + r * pitch + w * 4) = v;
+    }
+    __syncthreads();
+    const int r = threadIdx.x;
+    if (r0 + r >= n) return;
+    for (int j = 0; j < W; ++j) {
+        const int f = block * W + j;
+        if (f < F) colmat[(size_t)f * col_stride + r0 + r] = tile[r * pitch + j];
+    }
+}
+
+void launch_reorder_keys(hipStream_t s, int n, const int *nid, unsigned long long *keys, int *vals) {
+    if (n > 0) k_reorder_keys<<<(n + 255) / 256, 256, 0, s>>>(n, nid, keys, vals);
+}
+
+void launch_gather_rows(hipStream_t s, int n, int bytes_per_row, const int *from, const void *src, void *dst) {
+    if (n <= 0) return;
+    TGBM_CHECK(bytes_per_row % 4 == 0, "rows of %d bytes cannot be gathered by dwords", bytes_per_row);
+    const int words = bytes_per_row / 4;
+    k_gather_rows<<<grid_for((size_t)n * words, 65536), 256, 0, s>>>(n, words, from, static_cast<const unsigned *>(src),
+                                                                      static_cast<unsigned *>(dst));
+}
+
+void launch_gather_perm(hipStream_t s, int n, const int *from, const int *perm_old, int *perm_new) {
+    if (n > 0) k_gather_perm<<<(n + 255) / 256, 256, 0, s>>>(n, from, perm_old, perm_new);
+}
+
+void launch_cols_from_rows(hipStream_t s, int n, int W, int F, int n_blocks, const uint8_t *binmat, size_t block_stride,
+                           uint8_t *colmat, size_t col_stride) {
+    if (n <= 0) return;
+    for (int b = 0; b < n_blocks; ++b)
+        k_cols_from_rows<<<(n + 255) / 256, 256, (size_t)256 * (W + 4), s>>>(n, W, F, b, binmat + (size_t)b * block_stride,
+                                                                             colmat, col_stride);
+}
+
 void ScanScratch::release() {
     for (Level &lv : levels) {
         if (lv.sums) (void)hipFree(lv.sums);

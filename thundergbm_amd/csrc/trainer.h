@@ -33,7 +33,8 @@ class Trainer {
     void boost(int rounds);
     // step-wise driving (used by parity tests)
     void sample_columns();  // column sampling of one boosting round (no-op for rate >= 1); boost() calls it
-    void set_option(const std::string &key, double value);  // "column_sampling_rate", "bagging"
+    // "column_sampling_rate", "bagging", "reorder_first", "reorder_every", "reorder_min_rows"
+    void set_option(const std::string &key, double value);
     void compute_gradient();
     void tree_init(int k);
     void find_split(int level);  // histogram, merge/subtract, split search, update_tree
@@ -61,6 +62,9 @@ class Trainer {
     void build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class);
     void build_round_together();
     void log_plan(const TreeBuffers &tb);
+    bool reorder_allowed() const;
+    void reorder_rows();                 // physical re-ordering of the rows by the leaves of the tree just built
+    const std::vector<int> &host_perm();  // original row of every physical position (empty: identity)
     void run_metric(float *slot);
     void alloc_tree_buffers();
     template <typename T>
@@ -94,6 +98,17 @@ class Trainer {
     uint8_t *d_ignored_ = nullptr;
     int cur_class_ = 0;
     std::unique_ptr<RankContext> rank_;  // ranking objectives only
+    // physical row order: position p holds original row d_perm_[p] (nullptr: the original order)
+    int *d_perm_ = nullptr, *d_perm_alt_ = nullptr, *perm_spare_ = nullptr;
+    uint8_t *d_binmat_alt_ = nullptr;
+    float *d_y_alt_ = nullptr, *d_yp_alt_ = nullptr;
+    PairSorter reorder_sorter_;
+    std::vector<int> h_perm_;
+    bool h_perm_valid_ = false;
+    bool nid_materialized_ = false;  // tb_.nid already holds the finished tree's row -> node map (in physical order)
+    int reorder_first_ = 2, reorder_every_ = 32;  // after tree 2, then every 32 trees (0: never); see reorder_allowed()
+    long reorder_min_rows_ = 1l << 20;
+    int reorders_done_ = 0;
     int *d_bag_count_ = nullptr;         // bagging: draws per gradient entry (zero between rounds)
     bool rank_order_fresh_ = false;      // d_yp_ unchanged since the last ranking metric pass
     bool in_boost_ = false;

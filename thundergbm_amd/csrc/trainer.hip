@@ -395,6 +395,7 @@ Trainer::~Trainer() {
         (void)hipEventDestroy(ev.start);
         (void)hipEventDestroy(ev.stop);
     }
+    reorder_sorter_.release();
     for (void *p : allocs_) (void)hipFree(p);
     if (stream_) (void)hipStreamDestroy(stream_);
 }
@@ -450,6 +451,12 @@ void Trainer::set_option(const std::string &key, double value) {
         TGBM_CHECK(value > 0, "column_sampling_rate must be positive");
         param_.column_sampling_rate = (float)value;
         if (!(value < 1)) tb_.ignored = nullptr;
+    } else if (key == "reorder_first") {
+        reorder_first_ = (int)value;
+    } else if (key == "reorder_every") {
+        reorder_every_ = (int)value;
+    } else if (key == "reorder_min_rows") {
+        reorder_min_rows_ = (long)value;
     } else if (key == "bagging") {
         param_.bagging = value != 0;
         next_round_ready_ = false;
@@ -466,6 +473,7 @@ void Trainer::tree_init(int k) {
     launch_tree_init(stream_, set_of(k), d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
     next_round_ready_ = false;
     lookup_level_ = -1;
+    nid_materialized_ = false;
 }
 
 void Trainer::find_split(int level) { find_split_sets(set_of(cur_class_), d_gh_ + (size_t)cur_class_ * n_, level, 1); }
@@ -615,8 +623,87 @@ void Trainer::boost(int rounds) {
             log_info("[%d/%d] %s = %g", rounds_done_ + 1, param_.n_trees, names[metric_kind_], v);
         }
         ++rounds_done_;
+        if (reorder_allowed() && (rounds_done_ == reorder_first_ ||
+                                  (reorder_every_ > 0 && rounds_done_ > reorder_first_ &&
+                                   (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
+            reorder_rows();
     }
     in_boost_ = false;
+}
+
+// Rows that end in the same leaf of one tree tend to travel together through the next trees. Below the root
+// a histogram work item gathers its rows through a row list, one 128-byte line per row for the bin bytes and
+// one for the gradient pair; when the rows of a node sit next to each other those lines are shared. So every
+// few trees the rows are physically re-ordered by the leaf they just ended in (stable: inside a leaf the
+// previous order stays): the row-major and column-major bin matrices, labels and predictions move, the
+// permutation is remembered, and everything the API hands out per row is translated back to the caller's row
+// order. Histograms are exact integer sums, so the trees do not depend on the row order; only the float
+// reductions over all rows (root sums, metric) see another order of additions.
+// Not done for: the sparse layout, several trees per round, ranking (groups are runs of rows) and bagging
+// (the draw counts belong to row indices), small data.
+bool Trainer::reorder_allowed() const {
+    static const bool env_off = [] {
+        const char *e = std::getenv("TGBM_REORDER");
+        return e != nullptr && std::string(e) == "0";
+    }();
+    return !env_off && reorder_first_ > 0 && !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
+           (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && !param_.bagging && (long)n_ >= reorder_min_rows_;
+}
+
+void Trainer::reorder_rows() {
+    const TreeBuffers tb = set_of(0);
+    if (reorder_sorter_.cap < n_) {
+        reorder_sorter_.alloc(n_);
+        d_perm_alt_ = dalloc<int>((size_t)n_);
+        int *second = dalloc<int>((size_t)n_);
+        d_binmat_alt_ = dalloc<uint8_t>((size_t)n_ * bins_.W * bins_.n_blocks);
+        d_y_alt_ = dalloc<float>((size_t)n_);
+        d_yp_alt_ = dalloc<float>((size_t)n_);
+        perm_spare_ = second;
+    }
+    // the finished tree's row -> node map (its row lists are intact until the next tree starts)
+    launch_nid_rebuild(stream_, tb, &bins_, &csr_, lookup_level_);
+    launch_reorder_keys(stream_, n_, tb.nid, reorder_sorter_.keys[0], reorder_sorter_.vals[0]);
+    const int cur = sort_pairs(stream_, reorder_sorter_, n_, param_.depth + 1);
+    const int *from = reorder_sorter_.vals[cur];
+    const size_t blk = (size_t)n_ * bins_.W;
+    for (int b = 0; b < bins_.n_blocks; ++b)
+        launch_gather_rows(stream_, n_, bins_.W, from, d_binmat_ + b * blk, d_binmat_alt_ + b * blk);
+    launch_gather_rows(stream_, n_, 4, from, d_y_, d_y_alt_);
+    launch_gather_rows(stream_, n_, 4, from, d_yp_, d_yp_alt_);
+    int *perm_new = d_perm_ == d_perm_alt_ ? perm_spare_ : d_perm_alt_;
+    launch_gather_perm(stream_, n_, from, d_perm_, perm_new);
+    // the row -> node map moves along, so that it can still be handed out for this tree
+    launch_gather_rows(stream_, n_, 4, from, tb.nid, reorder_sorter_.vals[cur ^ 1]);
+    HIP_CHECK(hipMemcpyAsync(tb.nid, reorder_sorter_.vals[cur ^ 1], sizeof(int) * (size_t)n_, hipMemcpyDeviceToDevice,
+                             stream_));
+    std::swap(d_binmat_, d_binmat_alt_);
+    std::swap(d_y_, d_y_alt_);
+    std::swap(d_yp_, d_yp_alt_);
+    d_perm_ = perm_new;
+    bins_.data = d_binmat_;
+    launch_cols_from_rows(stream_, n_, bins_.W, F_, bins_.n_blocks, d_binmat_, bins_.block_stride,
+                          const_cast<uint8_t *>(bins_.col), bins_.col_stride);
+    h_perm_valid_ = false;
+    nid_materialized_ = true;
+    lookup_level_ = -1;
+    // the gradients of the next round (and their block statistics) were computed in the old order
+    if (next_round_ready_) {
+        next_round_ready_ = false;
+        launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
+    }
+    ++reorders_done_;
+}
+
+const std::vector<int> &Trainer::host_perm() {
+    if (d_perm_ == nullptr) {
+        h_perm_.clear();
+    } else if (!h_perm_valid_) {
+        h_perm_.resize((size_t)n_);
+        HIP_CHECK(hipMemcpy(h_perm_.data(), d_perm_, sizeof(int) * (size_t)n_, hipMemcpyDeviceToHost));
+    }
+    h_perm_valid_ = true;
+    return h_perm_;
 }
 
 std::vector<std::vector<Tree>> Trainer::model_to_host() {
@@ -684,6 +771,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "n_sets") return n_sets_;
     if (key == "sparse") return sparse_ ? 1 : 0;
     if (key == "dense_W") return bins_.W;
+    if (key == "reorders_done") return reorders_done_;
     if (key == "dense_blocks") return bins_.n_blocks;
     if (key == "trees_built") return trees_built_;
     if (key == "rounds_done") return rounds_done_;
@@ -706,8 +794,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
-        // the map is kept as row lists; materialise it on demand
-        launch_nid_rebuild(stream_, cur, &bins_, &csr_, lookup_level_);
+        // the map is kept as row lists; materialise it on demand (a re-ordering of the rows has done so already)
+        if (!nid_materialized_) launch_nid_rebuild(stream_, cur, &bins_, &csr_, lookup_level_);
         sync();
         src = cur.nid, bytes = sizeof(int) * (size_t)n_;
     }
@@ -731,7 +819,31 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
         src = rank_->last_sorted_rows(), bytes = sizeof(int) * (size_t)n_;
     }
     else fatal("unknown buffer %s", name.c_str());
-    if (out != nullptr && cap >= bytes && bytes > 0) HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
+    if (out != nullptr && cap >= bytes && bytes > 0) {
+        HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
+        // per-row buffers are handed out in the caller's row order, whatever the physical order is by now
+        size_t row_bytes = 0, n_planes = 1;
+        if (name == "nid" || name == "y_pred" || name == "y") row_bytes = 4;
+        else if (name == "gh") row_bytes = sizeof(GHPair);
+        else if (name == "binmat") row_bytes = (size_t)bins_.W, n_planes = (size_t)bins_.n_blocks;
+        const bool row_list = name == "ridx0" || name == "ridx1";
+        static const std::vector<int> identity;
+        const std::vector<int> &perm = (row_bytes || row_list) ? host_perm() : identity;
+        if (!perm.empty()) {
+            if (row_bytes) {
+                std::vector<char> phys(static_cast<char *>(out), static_cast<char *>(out) + bytes);
+                for (size_t pl = 0; pl < n_planes; ++pl) {
+                    const char *ps = phys.data() + pl * (size_t)n_ * row_bytes;
+                    char *pd = static_cast<char *>(out) + pl * (size_t)n_ * row_bytes;
+                    for (int p = 0; p < n_; ++p) std::memcpy(pd + (size_t)perm[p] * row_bytes, ps + (size_t)p * row_bytes, row_bytes);
+                }
+            } else if (row_list) {  // row lists: the entries are row positions
+                int *v = static_cast<int *>(out);
+                for (int i = 0; i < n_; ++i)
+                    if (v[i] >= 0 && v[i] < n_) v[i] = perm[v[i]];
+            }
+        }
+    }
     return bytes;
 }
 
@@ -745,6 +857,16 @@ void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     else if (name == "y_pred") dst = d_yp_, want = sizeof(float) * (size_t)n_yp_;
     else fatal("buffer %s cannot be set", name.c_str());
     TGBM_CHECK(bytes == want, "set %s: got %zu bytes, expected %zu", name.c_str(), bytes, want);
+    const std::vector<int> &perm = host_perm();
+    if (!perm.empty()) {  // caller's row order -> physical order (re-ordering only happens with one value per row)
+        const size_t row_bytes = bytes / (size_t)n_;
+        std::vector<char> phys(bytes);
+        for (int p = 0; p < n_; ++p)
+            std::memcpy(phys.data() + (size_t)p * row_bytes, static_cast<const char *>(in) + (size_t)perm[p] * row_bytes,
+                        row_bytes);
+        HIP_CHECK(hipMemcpy(dst, phys.data(), bytes, hipMemcpyHostToDevice));
+        return;
+    }
     HIP_CHECK(hipMemcpy(dst, in, bytes, hipMemcpyHostToDevice));
 }
 
