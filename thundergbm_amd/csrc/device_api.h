@@ -253,7 +253,7 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
 // Pieces of the physical re-ordering of the rows: sort keys (node of a row, payload = its position), gathers
 // dst[p] = src[from[p]] of whole rows, the row permutation, and the column-major copy rebuilt from the
 // row-major blocks.
-void launch_reorder_keys(hipStream_t s, int n, const int *nid, unsigned long long *keys, int *vals);
+void launch_reorder_keys(hipStream_t s, int n, int depth, const int *nid, unsigned long long *keys, int *vals);
 void launch_gather_rows(hipStream_t s, int n, int bytes_per_row, const int *from, const void *src, void *dst);
 void launch_gather_perm(hipStream_t s, int n, const int *from, const int *perm_old, int *perm_new);
 void launch_cols_from_rows(hipStream_t s, int n, int W, int F, int n_blocks, const uint8_t *binmat, size_t block_stride,

@@ -408,12 +408,17 @@ int device_max_int(hipStream_t s, const int *d_v, long n) {
 }
 
 // ---- physical re-ordering of the rows (see Trainer::reorder_rows) ---------------------------------
-// Sort keys: the node a row ended in; payload: the row's current position.
-__global__ __launch_bounds__(256) void k_reorder_keys(int n, const int *__restrict__ nid,
+// Sort keys: the node a row ended in, numbered by its path from the root (left = 0, right = 1, padded to
+// `depth` bits), so that the rows of every subtree - not only of every leaf - end up next to each other;
+// payload: the row's current position.
+__global__ __launch_bounds__(256) void k_reorder_keys(int n, int depth, const int *__restrict__ nid,
                                                      unsigned long long *__restrict__ keys, int *__restrict__ vals) {
     const int p = blockIdx.x * 256 + threadIdx.x;
     if (p >= n) return;
-    keys[p] = (unsigned long long)(unsigned)max(nid[p], 0);
+    const int x = max(nid[p], 0);                       // heap order: children of x are 2x + 1 and 2x + 2
+    const int level = 31 - __clz(x + 1);
+    const unsigned path = (unsigned)(x + 1 - (1 << level));
+    keys[p] = (unsigned long long)(path << max(depth - level, 0));
     vals[p] = p;
 }
 
@@ -459,8 +464,8 @@ __global__ __launch_bounds__(256) void k_cols_from_rows(int n, int W, int F, int
     }
 }
 
-void launch_reorder_keys(hipStream_t s, int n, const int *nid, unsigned long long *keys, int *vals) {
-    if (n > 0) k_reorder_keys<<<(n + 255) / 256, 256, 0, s>>>(n, nid, keys, vals);
+void launch_reorder_keys(hipStream_t s, int n, int depth, const int *nid, unsigned long long *keys, int *vals) {
+    if (n > 0) k_reorder_keys<<<(n + 255) / 256, 256, 0, s>>>(n, depth, nid, keys, vals);
 }
 
 void launch_gather_rows(hipStream_t s, int n, int bytes_per_row, const int *from, const void *src, void *dst) {

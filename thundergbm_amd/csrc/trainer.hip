@@ -663,8 +663,8 @@ void Trainer::reorder_rows() {
     }
     // the finished tree's row -> node map (its row lists are intact until the next tree starts)
     launch_nid_rebuild(stream_, tb, &bins_, &csr_, lookup_level_);
-    launch_reorder_keys(stream_, n_, tb.nid, reorder_sorter_.keys[0], reorder_sorter_.vals[0]);
-    const int cur = sort_pairs(stream_, reorder_sorter_, n_, param_.depth + 1);
+    launch_reorder_keys(stream_, n_, param_.depth, tb.nid, reorder_sorter_.keys[0], reorder_sorter_.vals[0]);
+    const int cur = sort_pairs(stream_, reorder_sorter_, n_, param_.depth);
     const int *from = reorder_sorter_.vals[cur];
     const size_t blk = (size_t)n_ * bins_.W;
     for (int b = 0; b < bins_.n_blocks; ++b)
