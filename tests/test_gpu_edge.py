@@ -287,9 +287,10 @@ def test_column_sampling_matches_oracle(T, objective, kind, rate):
     s.close()
 
 
-@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin"),
-                                            ("multi:softmax", "multi")])
-def test_bagging_matches_oracle(T, objective, kind):
+@pytest.mark.parametrize("objective,kind,reorder", [("reg:linear", "reg", False), ("binary:logistic", "bin", False),
+                                                    ("multi:softmax", "multi", False), ("reg:linear", "reg", True),
+                                                    ("binary:logistic", "bin", True)])
+def test_bagging_matches_oracle(T, objective, kind, reorder):
     """bagging = 1 (RowSampler::do_bagging, row_sampler.cu:9-38; booster.h:84): every round multiplies the
     gradient pairs by bootstrap draw counts from thrust's minstd engine seeded with one rand(). The draw
     counts must be the oracle's exactly (integer work), and boosting on the bagged gradients must build the
@@ -305,6 +306,9 @@ def test_bagging_matches_oracle(T, objective, kind):
     kw = dict(objective=objective, n_trees=4, depth=4, max_num_bin=32, learning_rate=0.5, min_child_weight=0.5)
     s = T.Session(val, rp, col, y, **kw)
     o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
+    if reorder:  # the draw counts belong to the caller's row indices, also after the rows were re-ordered
+        for key, v in (("reorder_min_rows", 0), ("reorder_first", 1), ("reorder_every", 1)):
+            s.set_option(key, v)
     s.gradient()
     plain = s.gh().copy()
     s.set_option("bagging", 1)
@@ -340,6 +344,15 @@ def test_bagging_matches_oracle(T, objective, kind):
     # rows drawn zero times carry no weight, so neighbouring candidates can describe the same partition;
     # compare_trees has checked that every differing choice is such a tie in the oracle's own gains
     assert ties <= 3
+    assert s.info("reorders_done") == (4 if reorder else 0)
+    if reorder:  # counts after re-orderings: still per original row
+        s.gradient()  # plain gradients are not available any more; check through the oracle instead
+        libc.srand(55)
+        o.set_y_pred(s.y_pred())
+        o.compute_gradient()
+        libc.srand(55)
+        s.gradient()
+        np.testing.assert_allclose(s.gh(), o.gh(), rtol=1e-5, atol=2e-6)
     s.close()
 
 

@@ -421,7 +421,9 @@ void Trainer::compute_gradient() {
             d_bag_count_ = dalloc<int>(N);
             HIP_CHECK(hipMemsetAsync(d_bag_count_, 0, sizeof(int) * N, stream_));
         }
-        launch_bagging(stream_, (int)N, (unsigned)std::rand(), d_bag_count_, d_gh_);  // row_sampler.cu:15
+        // row_sampler.cu:15. The gradient array may be longer than the rows (binary:logistic: 2n entries, the
+        // rows use the first n); only the row entries are subject to the permutation.
+        launch_bagging(stream_, (int)N, (unsigned)std::rand(), d_bag_count_, d_gh_, d_perm_, n_);
     }
 }
 
@@ -639,15 +641,15 @@ void Trainer::boost(int rounds) {
 // permutation is remembered, and everything the API hands out per row is translated back to the caller's row
 // order. Histograms are exact integer sums, so the trees do not depend on the row order; only the float
 // reductions over all rows (root sums, metric) see another order of additions.
-// Not done for: the sparse layout, several trees per round, ranking (groups are runs of rows) and bagging
-// (the draw counts belong to row indices), small data.
+// Not done for: the sparse layout, several trees per round, ranking (groups are runs of rows), small data.
+// (Bagging's draw counts belong to original row indices: they are applied through the permutation.)
 bool Trainer::reorder_allowed() const {
     static const bool env_off = [] {
         const char *e = std::getenv("TGBM_REORDER");
         return e != nullptr && std::string(e) == "0";
     }();
     return !env_off && reorder_first_ > 0 && !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
-           (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && !param_.bagging && (long)n_ >= reorder_min_rows_;
+           (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && (long)n_ >= reorder_min_rows_;
 }
 
 void Trainer::reorder_rows() {
@@ -859,8 +861,8 @@ void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     TGBM_CHECK(bytes == want, "set %s: got %zu bytes, expected %zu", name.c_str(), bytes, want);
     const std::vector<int> &perm = host_perm();
     if (!perm.empty()) {  // caller's row order -> physical order (re-ordering only happens with one value per row)
-        const size_t row_bytes = bytes / (size_t)n_;
-        std::vector<char> phys(bytes);
+        const size_t row_bytes = name == "gh" ? sizeof(GHPair) : sizeof(float);
+        std::vector<char> phys(static_cast<const char *>(in), static_cast<const char *>(in) + bytes);  // tail as is
         for (int p = 0; p < n_; ++p)
             std::memcpy(phys.data() + (size_t)p * row_bytes, static_cast<const char *>(in) + (size_t)perm[p] * row_bytes,
                         row_bytes);

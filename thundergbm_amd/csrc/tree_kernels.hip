@@ -155,10 +155,13 @@ __global__ void k_bagging_draw(int N, unsigned seed, int *__restrict__ count) {
     }
 }
 
-__global__ void k_bagging_apply(int N, int *__restrict__ count, GHPair *__restrict__ gh) {
+// perm (may be null): original row of every physical position; the draw counts belong to original rows
+__global__ void k_bagging_apply(int N, int *__restrict__ count, GHPair *__restrict__ gh, const int *__restrict__ perm,
+                                int n_rows) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
-        const int c = count[i];
-        count[i] = 0;  // ready for the next round
+        const int src = (perm != nullptr && i < n_rows) ? perm[i] : i;
+        const int c = count[src];
+        count[src] = 0;  // ready for the next round (perm is a bijection: every counter is cleared once)
         GHPair v = gh[i];
         v.g = v.g * c;
         v.h = v.h * c;
@@ -1706,9 +1709,9 @@ void launch_gradient(hipStream_t s, int objective, int n, int num_class, const f
         k_gradient_pointwise<<<grid_for(n), kBlock, 0, s>>>(objective, n, y, yp, gh);
 }
 
-void launch_bagging(hipStream_t s, int N, unsigned seed, int *count, GHPair *gh) {
+void launch_bagging(hipStream_t s, int N, unsigned seed, int *count, GHPair *gh, const int *perm, int n_rows) {
     k_bagging_draw<<<grid_for(N), kBlock, 0, s>>>(N, seed, count);
-    k_bagging_apply<<<grid_for(N), kBlock, 0, s>>>(N, count, gh);
+    k_bagging_apply<<<grid_for(N), kBlock, 0, s>>>(N, count, gh, perm, n_rows);
 }
 
 // Launchers: `tb` is the first buffer set to use, `n_class` consecutive sets (class trees of one round)
