@@ -484,14 +484,16 @@ def test_full_size_properties_config2(T):
     s.close()
 
 
-def _check_boosted_round(T, val, rp, col, y, n_sample, **kw):
+def _check_boosted_round(T, val, rp, col, y, n_sample, pre_rounds=0, **kw):
     """One production boost() round at full size, checked through properties that need no oracle run:
     every tree's root sum is the fp64 sum of its class's gradients; the rows that ended in a node (last
     class tree) reproduce that node's sums in an fp64 recount; children add up to their parent; the
     predictor on a sample of training rows reproduces the training-time predictions."""
     n = len(rp) - 1
-    s = T.Session(val, rp, col, y, n_trees=2, learning_rate=0.3, **kw)
+    s = T.Session(val, rp, col, y, n_trees=2 + pre_rounds, learning_rate=0.3, **kw)
     K = s.tree_per_rounds
+    if pre_rounds:
+        s.boost(pre_rounds)
     s.gradient()
     gh = s.gh().astype(np.float64)
     s.boost(1)
@@ -499,7 +501,7 @@ def _check_boosted_round(T, val, rp, col, y, n_sample, **kw):
     for k in range(K):
         ghk = gh[k * n:(k + 1) * n]
         Ag, Ah = np.abs(ghk[:, 0]).sum(), np.abs(ghk[:, 1]).sum()
-        nodes = model[0, k]
+        nodes = model[pre_rounds, k]
         assert nodes[0]["is_valid"]
         assert abs(nodes[0]["sum_g"] - ghk[:, 0].sum()) <= 1e-5 * Ag and abs(nodes[0]["sum_h"] - ghk[:, 1].sum()) <= 1e-5 * Ah
         inner = np.flatnonzero((nodes["is_valid"] == 1) & (nodes["split_fid"] >= 0))
@@ -521,10 +523,22 @@ def _check_boosted_round(T, val, rp, col, y, n_sample, **kw):
     out = np.zeros(K * m, np.float32)
     p = lambda a: a.ctypes.data_as(C.c_void_p)
     srp = rp[: m + 1].copy()
-    L.tgbm_predict_raw(m, p(val), p(srp), p(col), handle, 1, K, 0.3, s.base_score if K == 1 else 0.0, p(out))
+    L.tgbm_predict_raw(m, p(val), p(srp), p(col), handle, 1 + pre_rounds, K, 0.3, s.base_score if K == 1 else 0.0,
+                       p(out))
     np.testing.assert_allclose(out.reshape(K, m), yp[:, :m], rtol=1e-5, atol=1e-6)
     L.model_free(C.byref(handle))
     s.close()
+
+
+def test_full_size_properties_config2_reordered_rows(T):
+    """10 M x 28 after the rows were physically re-ordered (boost() does that after the second tree): the
+    fourth tree's sums against an fp64 recount through the row -> node map, which like the gradients and the
+    predictions comes back in the caller's row order, and the predictor against the training predictions."""
+    X, y = D.config2(10_000_000, seed=1)
+    val, rp, col = D.dense_to_csr(X)
+    del X
+    _check_boosted_round(T, val, rp, col, y, 100000, pre_rounds=3, objective="binary:logistic", depth=8,
+                         max_num_bin=255)
 
 
 def test_full_size_properties_config5_softmax(T):
