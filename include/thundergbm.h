@@ -110,9 +110,10 @@ void tgbm_trainer_destroy(tgbm_trainer *t);
  * search (Shard::column_sampling, builder/shard.cu:8-22; the shuffle draws from the process-wide rand()).
  * "bagging" (common.h:97): non-zero makes every gradient pass multiply the gradient pairs by bootstrap draw
  * counts (RowSampler::do_bagging, row_sampler.cu:9-38; seeded with one rand() per pass).
- * "reorder_first", "reorder_every", "reorder_min_rows" (no counterpart in the reference): tgbm_trainer_boost
- * physically re-orders the rows by the leaves of the tree just built after `reorder_first` trees and then
- * every `reorder_every` trees (defaults 2 and 32; 0 = never) when the dataset has at least
+ * "reorder_first", "reorder_burst", "reorder_every", "reorder_min_rows" (no counterpart in the reference):
+ * tgbm_trainer_boost physically re-orders the rows by the leaves of the tree just built after each of the
+ * trees `reorder_first` .. `reorder_first + reorder_burst - 1` and then every `reorder_every` trees
+ * (defaults 2, 2 and 32; reorder_first 0 = never) when the dataset has at least
  * `reorder_min_rows` rows (default 2^20), the layout is dense and a round builds one tree. Results do not
  * depend on it beyond float round-off, and all per-row buffers keep the caller's row order. */
 void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value);

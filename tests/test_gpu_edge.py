@@ -388,6 +388,7 @@ def test_row_reordering_is_invisible(T, objective, kind):
         s = T.Session(val, rp, col, y, **kw)
         s.set_option("reorder_min_rows", 0)
         s.set_option("reorder_first", first)
+        s.set_option("reorder_burst", 1)
         s.set_option("reorder_every", every)
         before = s.binmat().copy()
         s.boost(7)

@@ -33,7 +33,7 @@ class Trainer {
     void boost(int rounds);
     // step-wise driving (used by parity tests)
     void sample_columns();  // column sampling of one boosting round (no-op for rate >= 1); boost() calls it
-    // "column_sampling_rate", "bagging", "reorder_first", "reorder_every", "reorder_min_rows"
+    // "column_sampling_rate", "bagging", "reorder_first", "reorder_burst", "reorder_every", "reorder_min_rows"
     void set_option(const std::string &key, double value);
     void compute_gradient();
     void tree_init(int k);
@@ -106,7 +106,8 @@ class Trainer {
     std::vector<int> h_perm_;
     bool h_perm_valid_ = false;
     bool nid_materialized_ = false;  // tb_.nid already holds the finished tree's row -> node map (in physical order)
-    int reorder_first_ = 2, reorder_every_ = 32;  // after tree 2, then every 32 trees (0: never); see reorder_allowed()
+    // after trees 2 and 3, then every 32 trees (first 0: never); see reorder_allowed()
+    int reorder_first_ = 2, reorder_burst_ = 2, reorder_every_ = 32;
     long reorder_min_rows_ = 1l << 20;
     int reorders_done_ = 0;
     int *d_bag_count_ = nullptr;         // bagging: draws per gradient entry (zero between rounds)

@@ -455,6 +455,8 @@ void Trainer::set_option(const std::string &key, double value) {
         if (!(value < 1)) tb_.ignored = nullptr;
     } else if (key == "reorder_first") {
         reorder_first_ = (int)value;
+    } else if (key == "reorder_burst") {
+        reorder_burst_ = std::max(1, (int)value);
     } else if (key == "reorder_every") {
         reorder_every_ = (int)value;
     } else if (key == "reorder_min_rows") {
@@ -625,9 +627,12 @@ void Trainer::boost(int rounds) {
             log_info("[%d/%d] %s = %g", rounds_done_ + 1, param_.n_trees, names[metric_kind_], v);
         }
         ++rounds_done_;
-        if (reorder_allowed() && (rounds_done_ == reorder_first_ ||
-                                  (reorder_every_ > 0 && rounds_done_ > reorder_first_ &&
-                                   (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
+        // after each of the trees reorder_first_ .. reorder_first_ + reorder_burst_ - 1 (consecutive stable sorts
+        // cluster the rows by the leaves of the last tree, inside those by the leaves of the one before), then
+        // every reorder_every_ trees
+        if (reorder_allowed() &&
+            ((rounds_done_ >= reorder_first_ && rounds_done_ < reorder_first_ + reorder_burst_) ||
+             (reorder_every_ > 0 && rounds_done_ > reorder_first_ && (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
             reorder_rows();
     }
     in_boost_ = false;
