@@ -630,8 +630,10 @@ void Trainer::boost(int rounds) {
         // after each of the trees reorder_first_ .. reorder_first_ + reorder_burst_ - 1 (consecutive stable sorts
         // cluster the rows by the leaves of the last tree, inside those by the leaves of the one before), then
         // every reorder_every_ trees
+        const char *always = std::getenv("TGBM_REORDER");
         if (reorder_allowed() &&
-            ((rounds_done_ >= reorder_first_ && rounds_done_ < reorder_first_ + reorder_burst_) ||
+            ((always != nullptr && std::string(always) == "always") ||
+             (rounds_done_ >= reorder_first_ && rounds_done_ < reorder_first_ + reorder_burst_) ||
              (reorder_every_ > 0 && rounds_done_ > reorder_first_ && (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
             reorder_rows();
     }
@@ -649,10 +651,11 @@ void Trainer::boost(int rounds) {
 // Not done for: the sparse layout, several trees per round, ranking (groups are runs of rows), small data.
 // (Bagging's draw counts belong to original row indices: they are applied through the permutation.)
 bool Trainer::reorder_allowed() const {
-    static const bool env_off = [] {
-        const char *e = std::getenv("TGBM_REORDER");
-        return e != nullptr && std::string(e) == "0";
-    }();
+    const char *e = std::getenv("TGBM_REORDER");  // "0": never; "always": after every tree, any size (tests)
+    const bool env_off = e != nullptr && std::string(e) == "0";
+    if (e != nullptr && std::string(e) == "always")
+        return !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
+               (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC);
     return !env_off && reorder_first_ > 0 && !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
            (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && (long)n_ >= reorder_min_rows_;
 }
