@@ -289,7 +289,7 @@ def test_column_sampling_matches_oracle(T, objective, kind, rate):
 
 @pytest.mark.parametrize("objective,kind,reorder", [("reg:linear", "reg", False), ("binary:logistic", "bin", False),
                                                     ("multi:softmax", "multi", False), ("reg:linear", "reg", True),
-                                                    ("binary:logistic", "bin", True)])
+                                                    ("binary:logistic", "bin", True), ("multi:softmax", "multi", True)])
 def test_bagging_matches_oracle(T, objective, kind, reorder):
     """bagging = 1 (RowSampler::do_bagging, row_sampler.cu:9-38; booster.h:84): every round multiplies the
     gradient pairs by bootstrap draw counts from thrust's minstd engine seeded with one rand(). The draw
@@ -374,7 +374,8 @@ def test_bagging_through_the_c_abi(T):
     assert np.sqrt(np.mean((preds[0] - y) ** 2)) < 0.8 * np.std(y)  # still learns
 
 
-@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin")])
+@pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin"),
+                                            ("multi:softmax", "multi")])
 def test_row_reordering_is_invisible(T, objective, kind):
     """boost() physically re-orders the rows by the leaves of a tree every few rounds (here: after every
     round) so that the rows of a node lie together. Histograms are exact integer sums, so the trees must not

@@ -167,7 +167,7 @@ enum Objective { OBJ_SQUARE = 0, OBJ_LOGISTIC = 1, OBJ_SOFTMAX = 2, OBJ_RANK = 3
 void launch_gradient(hipStream_t s, int objective, int n, int num_class, const float *y, const float *yp, GHPair *gh,
                      GHPair *block_sums, int n_blocks);
 // RowSampler::do_bagging over the N gradient pairs; `count` holds N zeroed ints and is left zeroed. perm (may
-// be null): original row of each of the first n_rows physical positions, entries beyond keep their index
+// be null): original row of each of the n_rows physical positions; the N entries are planes of n_rows rows
 void launch_bagging(hipStream_t s, int N, unsigned seed, int *count, GHPair *gh, const int *perm = nullptr,
                     int n_rows = 0);
 // Tree-building launchers: `tb` is the first buffer set, `n_class` consecutive sets (the class trees of one

@@ -559,6 +559,7 @@ void Trainer::build_round_together() {
     tb.target_hitems = std::max(4, tb_.target_hitems / K);
     launch_tree_init(stream_, tb, d_gh_, param_.lambda, false, K);
     lookup_level_ = -1;
+    nid_materialized_ = false;
     for (int level = 0; level < param_.depth; ++level) {
         find_split_sets(tb, d_gh_, level, K);
         partition_sets(tb, level, K);
@@ -648,27 +649,26 @@ void Trainer::boost(int rounds) {
 // permutation is remembered, and everything the API hands out per row is translated back to the caller's row
 // order. Histograms are exact integer sums, so the trees do not depend on the row order; only the float
 // reductions over all rows (root sums, metric) see another order of additions.
-// Not done for: the sparse layout, several trees per round, ranking (groups are runs of rows), small data.
-// (Bagging's draw counts belong to original row indices: they are applied through the permutation.)
+// With several class trees per round the leaves of the round's last tree give the order (measured on 5 M rows,
+// 4 classes: 2.9 -> 2.35 ms per round). Not done for: the sparse layout, ranking (groups are runs of rows),
+// small data. (Bagging's draw counts belong to original row indices: they are applied through the permutation.)
 bool Trainer::reorder_allowed() const {
     const char *e = std::getenv("TGBM_REORDER");  // "0": never; "always": after every tree, any size (tests)
     const bool env_off = e != nullptr && std::string(e) == "0";
-    if (e != nullptr && std::string(e) == "always")
-        return !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
-               (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC);
-    return !env_off && reorder_first_ > 0 && !sparse_ && param_.tree_per_rounds == 1 && n_sets_ == 1 &&
-           (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && (long)n_ >= reorder_min_rows_;
+    if (e != nullptr && std::string(e) == "always") return !sparse_ && objective_ != OBJ_RANK;
+    return !env_off && reorder_first_ > 0 && !sparse_ && objective_ != OBJ_RANK && (long)n_ >= reorder_min_rows_;
 }
 
 void Trainer::reorder_rows() {
-    const TreeBuffers tb = set_of(0);
+    const TreeBuffers tb = set_of(cur_class_);  // the tree built last (the one whose map the API hands out)
+    const int n_planes = (int)(n_yp_ / n_);     // prediction planes: one per class
     if (reorder_sorter_.cap < n_) {
         reorder_sorter_.alloc(n_);
         d_perm_alt_ = dalloc<int>((size_t)n_);
         int *second = dalloc<int>((size_t)n_);
         d_binmat_alt_ = dalloc<uint8_t>((size_t)n_ * bins_.W * bins_.n_blocks);
         d_y_alt_ = dalloc<float>((size_t)n_);
-        d_yp_alt_ = dalloc<float>((size_t)n_);
+        d_yp_alt_ = dalloc<float>((size_t)n_yp_);
         perm_spare_ = second;
     }
     // the finished tree's row -> node map (its row lists are intact until the next tree starts)
@@ -680,7 +680,8 @@ void Trainer::reorder_rows() {
     for (int b = 0; b < bins_.n_blocks; ++b)
         launch_gather_rows(stream_, n_, bins_.W, from, d_binmat_ + b * blk, d_binmat_alt_ + b * blk);
     launch_gather_rows(stream_, n_, 4, from, d_y_, d_y_alt_);
-    launch_gather_rows(stream_, n_, 4, from, d_yp_, d_yp_alt_);
+    for (int k = 0; k < n_planes; ++k)
+        launch_gather_rows(stream_, n_, 4, from, d_yp_ + (size_t)k * n_, d_yp_alt_ + (size_t)k * n_);
     int *perm_new = d_perm_ == d_perm_alt_ ? perm_spare_ : d_perm_alt_;
     launch_gather_perm(stream_, n_, from, d_perm_, perm_new);
     // the row -> node map moves along, so that it can still be handed out for this tree
@@ -697,11 +698,9 @@ void Trainer::reorder_rows() {
     h_perm_valid_ = false;
     nid_materialized_ = true;
     lookup_level_ = -1;
-    // the gradients of the next round (and their block statistics) were computed in the old order
-    if (next_round_ready_) {
-        next_round_ready_ = false;
-        launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
-    }
+    // gradients (of this or already of the next round) and their block statistics are in the old order
+    next_round_ready_ = false;
+    launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
     ++reorders_done_;
 }
 
@@ -833,8 +832,9 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
         HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
         // per-row buffers are handed out in the caller's row order, whatever the physical order is by now
         size_t row_bytes = 0, n_planes = 1;
-        if (name == "nid" || name == "y_pred" || name == "y") row_bytes = 4;
-        else if (name == "gh") row_bytes = sizeof(GHPair);
+        if (name == "nid" || name == "y") row_bytes = 4;
+        else if (name == "y_pred") row_bytes = 4, n_planes = (size_t)(n_yp_ / n_);
+        else if (name == "gh") row_bytes = sizeof(GHPair), n_planes = (size_t)param_.num_class;
         else if (name == "binmat") row_bytes = (size_t)bins_.W, n_planes = (size_t)bins_.n_blocks;
         const bool row_list = name == "ridx0" || name == "ridx1";
         static const std::vector<int> identity;
@@ -870,10 +870,14 @@ void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     const std::vector<int> &perm = host_perm();
     if (!perm.empty()) {  // caller's row order -> physical order (re-ordering only happens with one value per row)
         const size_t row_bytes = name == "gh" ? sizeof(GHPair) : sizeof(float);
-        std::vector<char> phys(static_cast<const char *>(in), static_cast<const char *>(in) + bytes);  // tail as is
-        for (int p = 0; p < n_; ++p)
-            std::memcpy(phys.data() + (size_t)p * row_bytes, static_cast<const char *>(in) + (size_t)perm[p] * row_bytes,
-                        row_bytes);
+        const size_t n_planes = bytes / ((size_t)n_ * row_bytes);  // one per class
+        std::vector<char> phys(bytes);
+        for (size_t pl = 0; pl < n_planes; ++pl) {
+            const char *src_pl = static_cast<const char *>(in) + pl * (size_t)n_ * row_bytes;
+            char *dst_pl = phys.data() + pl * (size_t)n_ * row_bytes;
+            for (int p = 0; p < n_; ++p)
+                std::memcpy(dst_pl + (size_t)p * row_bytes, src_pl + (size_t)perm[p] * row_bytes, row_bytes);
+        }
         HIP_CHECK(hipMemcpy(dst, phys.data(), bytes, hipMemcpyHostToDevice));
         return;
     }

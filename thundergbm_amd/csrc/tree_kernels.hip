@@ -159,7 +159,8 @@ __global__ void k_bagging_draw(int N, unsigned seed, int *__restrict__ count) {
 __global__ void k_bagging_apply(int N, int *__restrict__ count, GHPair *__restrict__ gh, const int *__restrict__ perm,
                                 int n_rows) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < N; i += gridDim.x * blockDim.x) {
-        const int src = (perm != nullptr && i < n_rows) ? perm[i] : i;
+        // entry i = (plane, position): the plane (class) stays, the position maps to its original row
+        const int src = perm != nullptr ? (i / n_rows) * n_rows + perm[i % n_rows] : i;
         const int c = count[src];
         count[src] = 0;  // ready for the next round (perm is a bijection: every counter is cleared once)
         GHPair v = gh[i];
