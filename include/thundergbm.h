@@ -113,7 +113,7 @@ void tgbm_trainer_destroy(tgbm_trainer *t);
  * "reorder_first", "reorder_burst", "reorder_every", "reorder_min_rows" (no counterpart in the reference):
  * tgbm_trainer_boost physically re-orders the rows by the leaves of the tree just built after each of the
  * trees `reorder_first` .. `reorder_first + reorder_burst - 1` and then every `reorder_every` trees
- * (defaults 2, 2 and 32; reorder_first 0 = never) when the dataset has at least
+ * (defaults 1, 3 and 32; reorder_first 0 = never) when the dataset has at least
  * `reorder_min_rows` rows (default 2^20), the layout is dense and the objective is not a ranking one. Results do not
  * depend on it beyond float round-off, and all per-row buffers keep the caller's row order. */
 void tgbm_trainer_set_option(tgbm_trainer *t, const char *key, double value);

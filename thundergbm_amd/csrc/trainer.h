@@ -106,8 +106,8 @@ class Trainer {
     std::vector<int> h_perm_;
     bool h_perm_valid_ = false;
     bool nid_materialized_ = false;  // tb_.nid already holds the finished tree's row -> node map (in physical order)
-    // after trees 2 and 3, then every 32 trees (first 0: never); see reorder_allowed()
-    int reorder_first_ = 2, reorder_burst_ = 2, reorder_every_ = 32;
+    // after trees 1, 2 and 3, then every 32 trees (first 0: never); see reorder_allowed()
+    int reorder_first_ = 1, reorder_burst_ = 3, reorder_every_ = 32;
     long reorder_min_rows_ = 1l << 20;
     int reorders_done_ = 0;
     int *d_bag_count_ = nullptr;         // bagging: draws per gradient entry (zero between rounds)
