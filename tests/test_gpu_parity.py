@@ -549,6 +549,14 @@ def test_full_size_properties_config5_softmax(T):
     _check_boosted_round(T, val, rp, col, y, 100000, objective="multi:softmax", depth=8, max_num_bin=255)
 
 
+def test_full_size_properties_config3_wide(T):
+    """500k x 2000, depth 6: 63 feature blocks per work item, 4 MB of histogram per node."""
+    X, y = D.config3()
+    val, rp, col = D.dense_to_csr(X)
+    del X
+    _check_boosted_round(T, val, rp, col, y, 20000, objective="reg:linear", depth=6, max_num_bin=255)
+
+
 def test_full_size_properties_config4_sparse(T):
     """2 M x 100k CSR with Zipf-distributed feature ids: sparse layout with the LDS head."""
     val, rp, col, y = D.config4()

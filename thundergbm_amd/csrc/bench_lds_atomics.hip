@@ -39,6 +39,62 @@ __global__ __launch_bounds__(1024) void k(float *out, int iters) {
     if (acc == 123.456f) out[0] = acc;
 }
 
+// The histogram kernel's own instruction mix: every lane holds one dword of four bin bytes per step (eight
+// lanes = one row of 28+4 features, 256 bins of 8 bytes per feature) and issues four 64-bit adds; the bytes
+// are refreshed with one rotate-and-add per dword, so address arithmetic stays at the kernel's two to three
+// vector instructions per add. CHECK adds the kernel's "bin != missing" test (compare + exec mask) per add.
+template <bool CHECK, int WIDTH>
+__global__ __launch_bounds__(1024) void k_mix(float *out, int iters) {
+    extern __shared__ float lds[];
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(lds);
+    for (int i = threadIdx.x; i < NBINS; i += blockDim.x) lds[i] = 0.f;
+    __syncthreads();
+    unsigned w = (blockIdx.x * blockDim.x + threadIdx.x) * 2654435761u + 12345u;
+    w ^= w >> 15; w *= 2246822519u; w ^= w >> 13;
+    const unsigned q = threadIdx.x & 7;
+    const unsigned o0 = (q * 4 + 0) % 28 * 256, o1 = (q * 4 + 1) % 28 * 256, o2 = (q * 4 + 2) % 28 * 256,
+                   o3 = (q * 4 + 3) % 28 * 256;
+    const unsigned long long add = ((unsigned long long)(threadIdx.x + 1) << 32) + 3u;
+    for (int it = 0; it < iters; ++it) {
+        w = ((w >> 8) | (w << 24)) + 0x9e3779b9u;
+        const unsigned b0 = w & 0xff, b1 = (w >> 8) & 0xff, b2 = (w >> 16) & 0xff, b3 = w >> 24;
+        if (WIDTH == 8) {
+            if (!CHECK || b0 != 255u) atomicAdd(h + o0 + b0, add);
+            if (!CHECK || b1 != 255u) atomicAdd(h + o1 + b1, add);
+            if (!CHECK || b2 != 255u) atomicAdd(h + o2 + b2, add);
+            if (!CHECK || b3 != 255u) atomicAdd(h + o3 + b3, add);
+        } else {
+            unsigned *h32 = reinterpret_cast<unsigned *>(lds);
+            if (!CHECK || b0 != 255u) atomicAdd(h32 + o0 + b0, (unsigned)add);
+            if (!CHECK || b1 != 255u) atomicAdd(h32 + o1 + b1, (unsigned)add);
+            if (!CHECK || b2 != 255u) atomicAdd(h32 + o2 + b2, (unsigned)add);
+            if (!CHECK || b3 != 255u) atomicAdd(h32 + o3 + b3, (unsigned)add);
+        }
+    }
+    __syncthreads();
+    float acc = 0;
+    for (int i = threadIdx.x; i < NBINS; i += blockDim.x) acc += lds[i];
+    if (acc == 123.456f) out[0] = acc;
+}
+
+template <bool CHECK, int WIDTH>
+int run_mix(const char *name, float *d_out) {
+    hipEvent_t a, b;
+    CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+    const int grid = 512, block = 1024, iters = ITERS / 4;
+    k_mix<CHECK, WIDTH><<<grid, block, NBINS * 4>>>(d_out, 16);
+    CK(hipDeviceSynchronize());
+    CK(hipEventRecord(a));
+    k_mix<CHECK, WIDTH><<<grid, block, NBINS * 4>>>(d_out, iters);
+    CK(hipEventRecord(b));
+    CK(hipEventSynchronize(b));
+    float ms; CK(hipEventElapsedTime(&ms, a, b));
+    double ops = (double)grid * block * iters * 4;
+    printf("%-40s %8.3f ms  %8.1f G lane-ops/s  %.2f lane-ops/clk/CU (2.4GHz, 256 CU)\n", name, ms, ops / ms / 1e6,
+           ops / (ms * 1e-3) / 256 / 2.4e9);
+    return 0;
+}
+
 template <int MODE>
 int run(const char *name, float *d_out, int block = 256) {
     hipEvent_t a, b;
@@ -77,5 +133,9 @@ int main() {
     run<12>("u64 add, conflict free, block 1024", d, 1024);
     run<1>("uint add, random, block 1024", d, 1024);
     run<0>("float add, random, block 1024", d, 1024);
+    run_mix<true, 8>("histogram mix, u64, missing check", d);
+    run_mix<false, 8>("histogram mix, u64, no check", d);
+    run_mix<true, 4>("histogram mix, u32, missing check", d);
+    run_mix<false, 4>("histogram mix, u32, no check", d);
     return 0;
 }
