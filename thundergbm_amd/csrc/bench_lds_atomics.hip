@@ -77,6 +77,51 @@ __global__ __launch_bounds__(1024) void k_mix(float *out, int iters) {
     if (acc == 123.456f) out[0] = acc;
 }
 
+// The same work with the histogram interleaved by feature (slot = bin * 32 + feature, so a feature owns one
+// pair of banks) and the four features of a lane taken in an order rotated by the row's position in the
+// wavefront: every instruction then touches each of the 32 features from exactly two lanes.
+__global__ __launch_bounds__(1024) void k_mix_rotated(float *out, int iters) {
+    extern __shared__ float lds[];
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(lds);
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) lds[i] = 0.f;
+    __syncthreads();
+    unsigned w = (blockIdx.x * blockDim.x + threadIdx.x) * 2654435761u + 12345u;
+    w ^= w >> 15; w *= 2246822519u; w ^= w >> 13;
+    const unsigned q = threadIdx.x & 7, r = (threadIdx.x >> 3) & 7;
+    const unsigned k0 = r & 3, k1 = (r + 1) & 3, k2 = (r + 2) & 3, k3 = (r + 3) & 3;
+    const unsigned f0 = q * 4 + k0, f1 = q * 4 + k1, f2 = q * 4 + k2, f3 = q * 4 + k3;
+    const unsigned s0 = k0 * 8, s1 = k1 * 8, s2 = k2 * 8, s3 = k3 * 8;
+    const unsigned long long add = ((unsigned long long)(threadIdx.x + 1) << 32) + 3u;
+    for (int it = 0; it < iters; ++it) {
+        w = ((w >> 8) | (w << 24)) + 0x9e3779b9u;
+        atomicAdd(h + ((w >> s0) & 0xff) * 32 + f0, add);
+        atomicAdd(h + ((w >> s1) & 0xff) * 32 + f1, add);
+        atomicAdd(h + ((w >> s2) & 0xff) * 32 + f2, add);
+        atomicAdd(h + ((w >> s3) & 0xff) * 32 + f3, add);
+    }
+    __syncthreads();
+    float acc = 0;
+    for (int i = threadIdx.x; i < 16384; i += blockDim.x) acc += lds[i];
+    if (acc == 123.456f) out[0] = acc;
+}
+
+int run_mix_rotated(const char *name, float *d_out) {
+    hipEvent_t a, b;
+    CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+    const int grid = 512, block = 1024, iters = ITERS / 4;
+    k_mix_rotated<<<grid, block, 65536>>>(d_out, 16);
+    CK(hipDeviceSynchronize());
+    CK(hipEventRecord(a));
+    k_mix_rotated<<<grid, block, 65536>>>(d_out, iters);
+    CK(hipEventRecord(b));
+    CK(hipEventSynchronize(b));
+    float ms; CK(hipEventElapsedTime(&ms, a, b));
+    double ops = (double)grid * block * iters * 4;
+    printf("%-40s %8.3f ms  %8.1f G lane-ops/s  %.2f lane-ops/clk/CU (2.4GHz, 256 CU)\n", name, ms, ops / ms / 1e6,
+           ops / (ms * 1e-3) / 256 / 2.4e9);
+    return 0;
+}
+
 template <bool CHECK, int WIDTH>
 int run_mix(const char *name, float *d_out) {
     hipEvent_t a, b;
@@ -137,5 +182,6 @@ int main() {
     run_mix<false, 8>("histogram mix, u64, no check", d);
     run_mix<true, 4>("histogram mix, u32, missing check", d);
     run_mix<false, 4>("histogram mix, u32, no check", d);
+    run_mix_rotated("histogram mix, u64, one bank pair per feature", d);
     return 0;
 }
