@@ -12,7 +12,9 @@
  * calls (the benchmark) or drive the stages one by one (the parity tests).
  *
  * Failures abort the process after printing a FATAL line, as the reference's CHECK macros do.
- * The library is not re-entrant; one call trains on one GPU and blocks until done.
+ * One call trains on one GPU and blocks until done. The training and prediction calls of part 1 hold a
+ * process-wide lock (the reference serialises Booster::boost with a global mutex, booster.h:17,78), so calls
+ * from several threads run one after the other; a session of part 2 belongs to one thread at a time.
  */
 #ifndef THUNDERGBM_H
 #define THUNDERGBM_H

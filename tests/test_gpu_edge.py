@@ -17,7 +17,10 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def T():
     import thundergbm_amd
-    thundergbm_amd.load()
+    L = thundergbm_amd.load()
+    # the first GPU call of a process initialises the runtime (which may draw from rand() itself): do it here,
+    # so that no test's random stream depends on which test runs first
+    L.tgbm_calibration_copy(1 << 20, 1)
     return thundergbm_amd
 
 
@@ -364,6 +367,8 @@ def test_bagging_through_the_c_abi(T):
     X = rng.standard_normal((2000, 6)).astype(np.float32)
     y = (X[:, 0] - X[:, 1] + 0.3 * rng.standard_normal(2000)).astype(np.float32)
     preds = []
+    # the first GPU call of a process initialises the runtime, which may draw from rand() itself
+    T.TGBMRegressor(depth=2, n_trees=1, verbose=0).fit(X, y)
     for bagging, seed in ((1, 5), (1, 5), (1, 6), (0, 5)):
         libc.srand(seed)
         m = T.TGBMRegressor(depth=4, n_trees=6, learning_rate=0.5, bagging=bagging, verbose=0).fit(X, y)
@@ -372,6 +377,34 @@ def test_bagging_through_the_c_abi(T):
     assert not np.array_equal(preds[0], preds[2])
     assert not np.array_equal(preds[0], preds[3])
     assert np.sqrt(np.mean((preds[0] - y) ** 2)) < 0.8 * np.std(y)  # still learns
+
+
+def test_fits_from_two_threads_are_serialised(T):
+    """sparse_train_scikit / sparse_predict_scikit hold a process-wide lock (the reference serialises
+    Booster::boost with a global mutex, booster.h:17,78): four threads fitting and predicting at once get the
+    models and predictions of the same calls made one after the other."""
+    import threading
+    rng = np.random.default_rng(8)
+    sets = []
+    for i in range(4):
+        X = rng.standard_normal((3000 + 500 * i, 5 + i)).astype(np.float32)
+        y = (X[:, 0] * (i + 1) - X[:, 1] + 0.2 * rng.standard_normal(len(X))).astype(np.float32)
+        sets.append((X, y))
+    fit = lambda X, y: np.asarray(T.TGBMRegressor(depth=5, n_trees=8, learning_rate=0.4, verbose=0).fit(X, y).predict(X),
+                                  np.float32).copy()
+    serial = [fit(X, y) for X, y in sets]
+    out = [None] * 4
+
+    def work(i):
+        out[i] = fit(*sets[i])
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for a, b in zip(serial, out):
+        assert np.array_equal(a, b)
 
 
 @pytest.mark.parametrize("objective,kind", [("reg:linear", "reg"), ("binary:logistic", "bin"),

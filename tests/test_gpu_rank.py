@@ -20,7 +20,10 @@ LIBC.rand.restype = C.c_int
 @pytest.fixture(scope="module")
 def T():
     import thundergbm_amd
-    thundergbm_amd.load()
+    L = thundergbm_amd.load()
+    # the first GPU call of a process initialises the runtime (which may draw from rand() itself): do it here,
+    # so that no test's random stream depends on which test runs first
+    L.tgbm_calibration_copy(1 << 20, 1)
     return thundergbm_amd
 
 

@@ -2,6 +2,7 @@
 #include <chrono>
 #include <cstring>
 #include <memory>
+#include <mutex>
 
 #include "../../include/thundergbm.h"
 #include "trainer.h"
@@ -19,6 +20,11 @@ struct tgbm_trainer {
 };
 
 namespace {
+
+// Training and prediction calls of the reference's interface are serialised process-wide, as the reference's
+// global mutex does for Booster::boost (include/thundergbm/booster.h:17,78): two threads that call fit() at
+// once run one after the other instead of competing for the device.
+std::mutex g_call_mutex;
 
 std::vector<std::vector<Tree>> to_nested(const tgbm_model *m, int n_trees, int per_iter) {
     TGBM_CHECK(m != nullptr, "model is null!");
@@ -48,6 +54,7 @@ void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, f
                          int verbose, float column_sampling_rate, int bagging, int n_parallel_trees,
                          float learning_rate, char *obj_type, int *num_class, char *tree_method, tgbm_model **model,
                          int *tree_per_iter, float *group_label, int *group, int num_group) {
+    std::lock_guard<std::mutex> lock(g_call_mutex);
     GBMParam p;
     p.depth = depth;
     p.n_trees = n_trees;
@@ -83,6 +90,7 @@ void sparse_train_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, f
 void sparse_predict_scikit(int row_size, float *val, int *row_ptr, int *col_ptr, float *y_pred, tgbm_model **model,
                            int n_trees, int trees_per_iter, char *objective, int num_class, float learning_rate,
                            float *group_label, int *group, int num_group, int verbose) {
+    std::lock_guard<std::mutex> lock(g_call_mutex);
     GBMParam p;  // base_score stays 0 on this path, as in the reference (scikit_tgbm.cpp:87-90)
     p.objective = objective;
     p.learning_rate = learning_rate;
@@ -184,6 +192,7 @@ void train_R(int *depth, int *n_trees, int *n_gpus, int *verbose, int *profiling
              double *column_sampling_rate, int *bagging, int *n_parallel_trees, double *learning_rate,
              char **objective, int *num_class, int *min_child_weight, double *lambda_tgbm, double *gamma,
              char **tree_method, char **model_out) {
+    std::lock_guard<std::mutex> lock(g_call_mutex);
     set_logger(*verbose);
     GBMParam p;
     p.depth = *depth;
@@ -212,6 +221,7 @@ void train_R(int *depth, int *n_trees, int *n_gpus, int *verbose, int *profiling
 }
 
 void predict_R(char **data, char **model_in, int *verbose) {
+    std::lock_guard<std::mutex> lock(g_call_mutex);
     set_logger(*verbose);
     GBMParam p;
     DataSet dataset;
