@@ -138,7 +138,7 @@ float tgbm_trainer_metric(tgbm_trainer *t);
 
 /* Integer facts: n, n_features, n_bins, num_class, tree_per_rounds, n_nodes, dense_W,
  * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems, n_sets (class trees
- * of a round built by common launches), reorders_done. */
+ * of a round built by common launches), reorders_done, device_free_mb (free device memory in MiB). */
 int tgbm_trainer_info(tgbm_trainer *t, const char *key);
 float tgbm_trainer_base_score(tgbm_trainer *t);
 

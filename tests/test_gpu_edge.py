@@ -379,6 +379,43 @@ def test_bagging_through_the_c_abi(T):
     assert np.sqrt(np.mean((preds[0] - y) ** 2)) < 0.8 * np.std(y)  # still learns
 
 
+def test_sessions_release_their_device_memory(T):
+    """Every layout's session (dense with row re-ordering, sparse, ranking, class trees built together) gives
+    its device memory back when it is closed: free memory after ten open/boost/close cycles is what it was."""
+    rng = np.random.default_rng(12)
+    n = 1_200_000  # above the row count from which rows are re-ordered
+    X = rng.standard_normal((n, 6)).astype(np.float32)
+    y = (X[:, 0] - X[:, 1] > 0).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    ym = rng.integers(0, 3, n).astype(np.float32)
+    yr = rng.integers(0, 4, n).astype(np.float32)
+    groups = np.full(n // 100, 100, np.int32)
+
+    def cycle():
+        s = T.Session(val, rp, col, y, depth=4, n_trees=4, objective="binary:logistic")
+        s.boost(4)
+        assert s.info("reorders_done") >= 1
+        free = s.info("device_free_mb")
+        s.close()
+        os.environ["TGBM_LAYOUT"] = "sparse"
+        s = T.Session(val, rp, col, y, depth=4, n_trees=2, objective="binary:logistic")
+        s.boost(2)
+        s.close()
+        os.environ.pop("TGBM_LAYOUT")
+        s = T.Session(val, rp, col, ym, depth=4, n_trees=2, objective="multi:softmax", num_class=3)
+        s.boost(2)
+        s.close()
+        s = T.Session(val, rp, col, yr, depth=4, n_trees=2, objective="rank:ndcg", groups=groups)
+        s.boost(2)
+        s.close()
+        return free
+
+    first = cycle()
+    for _ in range(9):
+        last = cycle()
+    assert abs(first - last) <= 64, (first, last)
+
+
 def test_fits_from_two_threads_are_serialised(T):
     """sparse_train_scikit / sparse_predict_scikit hold a process-wide lock (the reference serialises
     Booster::boost with a global mutex, booster.h:17,78): four threads fitting and predicting at once get the

@@ -781,6 +781,11 @@ int Trainer::info(const std::string &key) const {
     if (key == "sparse") return sparse_ ? 1 : 0;
     if (key == "dense_W") return bins_.W;
     if (key == "reorders_done") return reorders_done_;
+    if (key == "device_free_mb") {
+        size_t free_b = 0, total_b = 0;
+        HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        return (int)(free_b >> 20);
+    }
     if (key == "dense_blocks") return bins_.n_blocks;
     if (key == "trees_built") return trees_built_;
     if (key == "rounds_done") return rounds_done_;
