@@ -26,10 +26,10 @@ def T():
 
 @pytest.fixture(autouse=True)
 def _default_layout():
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT"):
         os.environ.pop(k, None)
     yield
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT"):
         os.environ.pop(k, None)
 
 
@@ -544,6 +544,36 @@ def test_training_is_bit_reproducible(T, layout):
         runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.metric_log().tobytes()))
         s.close()
     assert runs[0] == runs[1] == runs[2]
+
+
+@pytest.mark.parametrize("head", ["1", "0"])
+@pytest.mark.parametrize("objective,kind", [("binary:logistic", "bin"), ("multi:softmax", "multi")])
+def test_sparse_root_histogram_from_either_copy(T, objective, kind, head):
+    """Sparse layout: the root histogram summed over the bin-major copy of the stored values and accumulated row
+    by row with atomics (TGBM_CSC_ROOT=0; with and without the LDS head) are the same integers: same bytes."""
+    os.environ["TGBM_LAYOUT"] = "sparse"
+    os.environ["TGBM_CSR_HEAD"] = head
+    n, F = 30000, 300
+    val, rp, col = _ragged(n, F, 9, 12)
+    y = _target(val, rp, col, n, F, 9, kind)
+    kw = dict(objective=objective, n_trees=4, depth=5, max_num_bin=16, learning_rate=0.3)
+    if kind == "multi":
+        kw["num_class"] = int(y.max()) + 1
+    runs = []
+    for csc in ("1", "0"):
+        os.environ["TGBM_CSC_ROOT"] = csc
+        s = T.Session(val, rp, col, y, **kw)
+        s.gradient()
+        s.tree_init(0)
+        s.find_split(0)
+        root_hist = s.level_hist(0).tobytes()
+        s.close()
+        s = T.Session(val, rp, col, y, **kw)
+        s.boost(4)
+        runs.append((root_hist, s.model().tobytes(), s.y_pred().tobytes()))
+        s.close()
+    os.environ.pop("TGBM_CSC_ROOT")
+    assert runs[0] == runs[1]
 
 
 def test_predict_transforms_through_the_c_abi(T):

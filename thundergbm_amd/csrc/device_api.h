@@ -80,6 +80,11 @@ struct CsrBins {
     const int *hist_word = nullptr;  // [nnz]
     const int *head_bin = nullptr;   // [head_bins] global bin id of every head slot
     int head_bins = 0;
+    // The same stored values sorted by global bin id (rows ascending inside a bin): the root histogram, where
+    // every row takes part, is a segmented sum over this copy instead of atomics to random bins. nullptr: none.
+    const int *csc_bin = nullptr;  // [nnz]
+    const int *csc_row = nullptr;  // [nnz]
+    long nnz = 0;
 };
 
 struct TreeBuffers {
@@ -251,6 +256,12 @@ struct PairSorter {
 // ascending. Returns which of the two buffer pairs (0 or 1) holds the result. Stream-ordered; allocates only
 // when the scan scratch has to grow (first call).
 int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
+
+// Bin-major copy of CSR bin ids: sort keys (global bin, payload = row) of every stored value, and the sorted
+// pairs split into the two int arrays the root histogram reads.
+void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, unsigned long long *keys, int *vals);
+void launch_csc_unpack(hipStream_t s, long nnz, const unsigned long long *keys, const int *vals, int *csc_bin,
+                       int *csc_row);
 
 // Pieces of the physical re-ordering of the rows: sort keys (node of a row, payload = its position), gathers
 // dst[p] = src[from[p]] of whole rows, the row permutation, and the column-major copy rebuilt from the

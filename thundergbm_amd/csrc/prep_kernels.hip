@@ -283,6 +283,28 @@ __global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *_
     }
 }
 
+// One wavefront per row: (global bin, row) of every stored value, for the bin-major copy.
+__global__ __launch_bounds__(kBlock) void k_csc_keys(int n_rows, const int *__restrict__ row_ptr,
+                                                    const int *__restrict__ bin, unsigned long long *__restrict__ keys,
+                                                    int *__restrict__ vals) {
+    const int r = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (r >= n_rows) return;
+    const int e1 = row_ptr[r + 1];
+    for (int e = row_ptr[r] + (threadIdx.x & 63); e < e1; e += 64) {
+        keys[e] = (unsigned long long)(unsigned)bin[e];
+        vals[e] = r;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_csc_unpack(long nnz, const unsigned long long *__restrict__ keys,
+                                                      const int *__restrict__ vals, int *__restrict__ csc_bin,
+                                                      int *__restrict__ csc_row) {
+    for (long e = (long)blockIdx.x * kBlock + threadIdx.x; e < nnz; e += (long)gridDim.x * kBlock) {
+        csc_bin[e] = (int)keys[e];
+        csc_row[e] = vals[e];
+    }
+}
+
 __global__ void k_bin_csr(long nnz, const int *__restrict__ col, const float *__restrict__ val,
                           const float *__restrict__ cut_val, const int *__restrict__ cut_row_ptr,
                           int *__restrict__ bin_id, const int *__restrict__ feat_slot, int *__restrict__ hist_word) {
@@ -554,6 +576,19 @@ void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, 
                       size_t col_stride) {
     k_bin_dense<<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride,
                                               colmat, col_stride);
+}
+
+void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, unsigned long long *keys,
+                     int *vals) {
+    if (n_rows == 0) return;
+    const int rows_per_block = kBlock / 64;
+    k_csc_keys<<<(n_rows + rows_per_block - 1) / rows_per_block, kBlock, 0, s>>>(n_rows, row_ptr, bin, keys, vals);
+}
+
+void launch_csc_unpack(hipStream_t s, long nnz, const unsigned long long *keys, const int *vals, int *csc_bin,
+                       int *csc_row) {
+    if (nnz == 0) return;
+    k_csc_unpack<<<grid_for(nnz), kBlock, 0, s>>>(nnz, keys, vals, csc_bin, csc_row);
 }
 
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,

@@ -207,6 +207,24 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         allocs_.push_back(d_row_ptr);  // kept for the whole session
         csr_.row_ptr = d_row_ptr;
         csr_.bin = d_bin;
+        // bin-major copy for the root histogram (TGBM_CSC_ROOT=0: without, the root goes through the row-major
+        // kernels like every other level; tests of both)
+        const char *ce = std::getenv("TGBM_CSC_ROOT");
+        if (nnz_ > 0 && !(ce != nullptr && std::string(ce) == "0")) {
+            PairSorter ps;
+            ps.alloc(nnz_);
+            launch_csc_keys(stream_, n_, d_row_ptr, d_bin, ps.keys[0], ps.vals[0]);
+            int bits = 1;
+            while (bits < 31 && (1l << bits) < (long)n_bins_) ++bits;
+            const int cur = sort_pairs(stream_, ps, nnz_, bits);
+            int *d_cbin = dalloc<int>((size_t)nnz_), *d_crow = dalloc<int>((size_t)nnz_);
+            launch_csc_unpack(stream_, nnz_, ps.keys[cur], ps.vals[cur], d_cbin, d_crow);
+            HIP_CHECK(hipStreamSynchronize(stream_));
+            ps.release();
+            csr_.csc_bin = d_cbin;
+            csr_.csc_row = d_crow;
+            csr_.nnz = nnz_;
+        }
         bins_.W = 4;
         bins_.n_blocks = 1;
         HIP_CHECK(hipStreamSynchronize(stream_));
