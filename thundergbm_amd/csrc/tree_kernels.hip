@@ -693,7 +693,7 @@ void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict_
 // bin is the sum over a contiguous run of the copy. A wavefront reduces 64 consecutive values by bin (segmented
 // scan over sorted keys) and the last lane of every run adds it to the histogram: one pair of atomics per run
 // and wavefront, to addresses that ascend with the position, instead of one pair per stored value to random
-// lines of a histogram far larger than the caches (4.3 ms -> 0.5 ms at 69 M values, 6.3 M bins). Same integers
+// lines of a histogram far larger than the caches (4.3 ms -> 1.1 ms at 69 M values, 6.3 M bins). Same integers
 // as k_hist_csr, in another order: the histogram is bit-identical.
 __global__ __launch_bounds__(kBlock) void k_hist_root_csc(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict__ gh) {
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
