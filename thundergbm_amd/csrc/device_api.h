@@ -14,6 +14,15 @@
                                             hipGetErrorString(e_));                                  \
     } while (0)
 
+// A kernel launch reports a bad configuration (too much LDS, an empty or oversized grid) only through
+// hipGetLastError; the host stages call this after their launches so that such a failure aborts with the
+// stage's name instead of leaving stale results behind.
+#define HIP_CHECK_LAUNCHES(stage)                                                                    \
+    do {                                                                                             \
+        hipError_t e_ = hipGetLastError();                                                           \
+        if (e_ != hipSuccess) ::tgbm::fatal("kernel launch failed in %s: %s", stage, hipGetErrorString(e_)); \
+    } while (0)
+
 namespace tgbm {
 
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row

@@ -83,6 +83,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
             HIP_CHECK(hipStreamSynchronize(s_up));  // small copies return before they are done
             launch_predict(s, r1 - r0, F, d_row_ptr + r0, d_col, d_val, d_model, n_iter, nct, n_nodes,
                            param.learning_rate, param.base_score, d_out + r0, (size_t)n);
+            HIP_CHECK_LAUNCHES("predict");
             r0 = r1;
         }
         HIP_CHECK(hipStreamSynchronize(s));
@@ -138,6 +139,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
         launch_predict_transform(s, kind, n, kind == 2 || kind == 3 ? nct : param.num_class, d_label, d_out);
         if (kind == 1 || kind == 2) n_ret = (size_t)n;
     }
+    HIP_CHECK_LAUNCHES("predict (metric, transform)");
     std::vector<float> out(n_ret);
     if (n_ret) HIP_CHECK(hipMemcpyAsync(out.data(), d_out, sizeof(float) * n_ret, hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));

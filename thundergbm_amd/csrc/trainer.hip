@@ -405,6 +405,7 @@ void Trainer::alloc_tree_buffers() {
     d_model_ = dalloc<TreeNode>((size_t)model_cap_trees_ * tb.n_nodes);
     d_metric_ = dalloc<float>((size_t)std::max(1, param_.n_trees));
     d_metric_scratch_ = dalloc<double>((size_t)row_blocks(n_));
+    HIP_CHECK_LAUNCHES("set-up (cut points, bin matrix)");
 }
 
 Trainer::~Trainer() {
@@ -492,6 +493,7 @@ TreeBuffers Trainer::set_of(int k) const { return tb_.for_class(n_sets_ > 1 ? k 
 
 void Trainer::tree_init(int k) {
     cur_class_ = k;
+    HIP_CHECK_LAUNCHES("the stages before tree_init");  // gradients, bagging, column sampling, metric, re-ordering
     launch_tree_init(stream_, set_of(k), d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
     next_round_ready_ = false;
     lookup_level_ = -1;
@@ -520,6 +522,7 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
                       !(in_boost_ && level == param_.depth - 1));
     launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
+    HIP_CHECK_LAUNCHES("find_split");
 }
 
 void Trainer::build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class) {
@@ -538,6 +541,7 @@ void Trainer::partition_sets(const TreeBuffers &tb, int level, int n_class) {
         launch_partition_csr(stream_, tb, csr_, level, n_class);
     else
         launch_partition_dense(stream_, tb, bins_, level, n_class);
+    HIP_CHECK_LAUNCHES("partition");
 }
 
 void Trainer::log_plan(const TreeBuffers &tb) {
@@ -566,6 +570,7 @@ void Trainer::finish_tree(int k, bool fuse_round_end) {
                              sizeof(TreeNode) * (size_t)tb.n_nodes, hipMemcpyDeviceToDevice, stream_));
     if (profiling_) log_plan(tb);
     ++trees_built_;
+    HIP_CHECK_LAUNCHES("finish_tree");
 }
 
 // All class trees of a round through the same launches (class = blockIdx.z): the trees are independent
@@ -591,6 +596,7 @@ void Trainer::build_round_together() {
         for (int k = 0; k < K; ++k) log_plan(tb.for_class(k));
     trees_built_ += K;
     cur_class_ = K - 1;
+    HIP_CHECK_LAUNCHES("build_round_together");
 }
 
 void Trainer::run_metric(float *slot) {
@@ -655,6 +661,7 @@ void Trainer::boost(int rounds) {
              (rounds_done_ >= reorder_first_ && rounds_done_ < reorder_first_ + reorder_burst_) ||
              (reorder_every_ > 0 && rounds_done_ > reorder_first_ && (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
             reorder_rows();
+        HIP_CHECK_LAUNCHES("boost");
     }
     in_boost_ = false;
 }
