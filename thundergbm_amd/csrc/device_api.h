@@ -124,6 +124,8 @@ struct TreeBuffers {
     int n_grad_blocks = 0;
     // split finder packing: wavefront w scans global bins [pack_begin[w], pack_begin[w+1]) (whole features)
     const int *pack_begin = nullptr;
+    // per bin: distance to the last bin of its feature (low byte) and whether it is the feature's first bin (bit 8)
+    const unsigned short *bin_meta = nullptr;  // [n_bins]
     int n_packs = 0;
     const uint8_t *ignored = nullptr;  // [F] columns whose candidates score 0 this round (nullptr: none)
     const int *cut_row_ptr = nullptr;

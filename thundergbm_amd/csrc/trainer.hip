@@ -377,6 +377,13 @@ void Trainer::alloc_tree_buffers() {
     int *d_pack = dalloc<int>(pack_begin.size());
     upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
     tb.pack_begin = d_pack;
+    std::vector<unsigned short> bin_meta((size_t)n_bins_);
+    for (int f = 0; f < F_; ++f)
+        for (int b = h_cut_row_ptr_[f]; b < h_cut_row_ptr_[f + 1]; ++b)
+            bin_meta[(size_t)b] = (unsigned short)((h_cut_row_ptr_[f + 1] - 1 - b) | (b == h_cut_row_ptr_[f] ? 0x100 : 0));
+    unsigned short *d_meta = dalloc<unsigned short>(bin_meta.size());
+    upload(stream_, d_meta, bin_meta.data(), bin_meta.size());
+    tb.bin_meta = d_meta;
     tb.cand = dalloc<SplitCand>(S * max_level_nodes * tb.n_packs);
 
     // dense block tables

@@ -873,12 +873,13 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
         incg[j] = inch[j] = 0;
         if (valid[j]) {
             const longlong2 v = s_v[w][lane * 4 + j];
-            const int f = tb.cut_fid[b];
-            ign[j] = tb.ignored != nullptr && tb.ignored[f] != 0;
-            const int fend = tb.cut_row_ptr[f + 1];
-            head[j] = tb.cut_row_ptr[f] == b;
-            last[j] = fend == b + 1;
-            lastb[j] = fend - 1 - b_begin;
+            // one word per bin instead of the chain bin -> feature -> feature's bin range
+            const unsigned meta = tb.bin_meta[b];  // low byte: bins up to the feature's last one, bit 8: first bin
+            ign[j] = tb.ignored != nullptr && tb.ignored[tb.cut_fid[b]] != 0;
+            const int to_last = (int)(meta & 0xffu);
+            head[j] = (meta & 0x100u) != 0;
+            last[j] = to_last == 0;
+            lastb[j] = b + to_last - b_begin;
             if (head[j]) {
                 rung = v.x;
                 runh = v.y;
