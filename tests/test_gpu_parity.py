@@ -435,6 +435,13 @@ def test_full_size_properties_config2(T):
     n = int(os.environ.get("TGBM_TEST_FULL_ROWS", "10000000"))
     X, y = D.config2(n, seed=1)
     val, rp, col = D.dense_to_csr(X)
+    # the cut rule in closed form on three full-size columns (hist_cut.cu:259-265): sorted distinct stored values,
+    # all of them when fewer than max_num_bin, else every (n_unique / max_num_bin)-th, max_num_bin of them
+    expected_cuts, columns = {}, {}
+    for f in (0, 13, 27):
+        columns[f] = X[:, f].copy()
+        u = np.unique(X[:, f][X[:, f] != 0])
+        expected_cuts[f] = u if len(u) < 255 else u[np.arange(255) * (len(u) // 255)]
     del X
     s = T.Session(val, rp, col, y, depth=8, n_trees=2, objective="binary:logistic", learning_rate=0.3)
     _, crp, cf = s.cuts()
@@ -443,6 +450,17 @@ def test_full_size_properties_config2(T):
     for f in range(s.F):
         seg = cv[crp[f]:crp[f + 1]]
         assert len(seg) <= 255 and np.all(np.diff(seg) > 0)
+    binmat = s.binmat()  # [blocks, n, W] bytes, in the caller's row order
+    W = s.info("dense_W")
+    for f, exp in expected_cuts.items():
+        assert np.array_equal(cv[crp[f]:crp[f + 1]].view(np.uint32), exp.astype(np.float32).view(np.uint32))
+        # bin id of every row of the column: min(#{cuts <= v}, k - 1), 255 where nothing is stored
+        # (hist_tree_builder_single.cu:81-92, :113-119)
+        x = columns[f]
+        want = np.minimum(np.searchsorted(exp, x, side="right"), len(exp) - 1).astype(np.uint8)
+        want[x == 0] = 255
+        assert np.array_equal(binmat[f // W, :, f % W], want)
+    del binmat, columns
     s.gradient()
     s.tree_init(0)
     gh = s.gh()[:n].astype(np.float64)
