@@ -957,23 +957,22 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
             }
         }
     }
-    // wavefront arg-max: larger |score| wins, ties go to the smaller bin index
+    // wavefront arg-max: larger |score| wins, ties go to the smaller bin index. Only the key travels through the
+    // butterfly; the lane that holds the winner writes its candidate itself.
+    float win = best;
+    int win_idx = best_idx;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
-        float oa = __shfl_xor(best, d);
-        float os = __shfl_xor(best_score, d);
-        int oi = __shfl_xor(best_idx, d);
-        float omg = __shfl_xor(best_miss.g, d), omh = __shfl_xor(best_miss.h, d);
-        float olg = __shfl_xor(best_left.g, d), olh = __shfl_xor(best_left.h, d);
-        if (oa > best || (oa == best && oi < best_idx)) {
-            best = oa;
-            best_score = os;
-            best_idx = oi;
-            best_miss = GHPair{omg, omh};
-            best_left = GHPair{olg, olh};
+        const float oa = __shfl_xor(win, d);
+        const int oi = __shfl_xor(win_idx, d);
+        if (oa > win || (oa == win && oi < win_idx)) {
+            win = oa;
+            win_idx = oi;
         }
     }
-    if (active && lane == 0) {
+    // (without any candidate every lane still holds the initial key and the first one writes the empty record)
+    const unsigned long long owners = __ballot(best == win && best_idx == win_idx);
+    if (active && lane == __ffsll((long long)owners) - 1) {
         SplitCand c;
         c.score = best_score;
         c.index = best_idx;
