@@ -1820,7 +1820,12 @@ void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bi
 
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class) {
     const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
-    if (n_pairs * n_class <= 4) {
+    if (tb.target_hitems <= 16) {
+        // wide data: many feature blocks, so a node has only a handful of work items and very long histograms;
+        // one thread per bin walks them (a block of 8 bins would leave most of its 32 groups without an item)
+        dim3 grid((tb.n_bins + kBlock - 1) / kBlock, n_pairs, n_class);
+        k_hist_merge<kBlock><<<grid, kBlock, 0, s>>>(tb, level);
+    } else if (n_pairs * n_class <= 4) {
         dim3 grid((tb.n_bins + 7) / 8, n_pairs, n_class);
         k_hist_merge<8><<<grid, kBlock, 0, s>>>(tb, level);
     } else {
