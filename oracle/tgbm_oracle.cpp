@@ -12,6 +12,7 @@
 //   cut points      closed-form rule on hand inputs, invariants, the a1a fixture (one cut = 1.0 per feature)
 //   bin ids         brute force min(#cuts<=v, k-1) against numpy searchsorted
 //   gradients       float64 closed forms
+//   base score      mean(y) for reg:linear, the logit closed form for binary:logistic, 0 for softmax / ranking
 //   histogram       brute-force float64 accumulation; bin counts for squared loss (the oracle itself
 //                   accumulates in float64 and rounds once: the reference's float atomics have no defined
 //                   order, so their result is only defined up to float round-off)

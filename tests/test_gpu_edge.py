@@ -601,3 +601,23 @@ def test_predict_transforms_through_the_c_abi(T):
             assert np.mean(got == exp) > 0.99
         else:
             np.testing.assert_allclose(got, exp, rtol=1e-4, atol=1e-5)
+
+
+def test_negative_column_index_is_rejected_before_any_kernel_uses_it(T):
+    """The C ABI takes the caller's column indices as they are; the largest and smallest are taken on the device
+    right after the upload, and a negative one (e.g. a 0-based file read as 1-based) stops the call with a
+    message instead of indexing device memory with it. Runs in a child process: the library aborts like the
+    reference's CHECK."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import ctypes as C, sys\nimport numpy as np\nsys.path.insert(0, %r)\nimport thundergbm_amd\n"
+        "L = thundergbm_amd.load()\n"
+        "val = np.ones(6, np.float32); col = np.array([0, 1, -1, 1, 0, 2], np.int32)\n"
+        "rp = np.array([0, 2, 4, 6], np.int32); y = np.zeros(3, np.float32)\n"
+        "p = lambda a: a.ctypes.data_as(C.c_void_p)\n"
+        "L.tgbm_trainer_create_grouped(3, p(val), p(rp), p(col), p(y), 3, 1, 1.0, 1.0, 1.0, 16, 1.0, b'reg:linear',"
+        " 1, 0, None, 0)\n" % root)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode != 0 and "negative column index -1" in out.stderr, out.stderr

@@ -141,3 +141,54 @@ def test_estimator_parameters_follow_the_reference_defaults():
     assert set(r.get_params()) >= {"depth", "n_trees", "n_gpus", "bagging", "column_sampling_rate"}
     with pytest.raises(ValueError):
         r.predict(np.zeros((2, 2)))
+
+
+def test_zero_based_libsvm_file_is_rejected_with_its_line(tmp_path):
+    """LIBSVM feature ids are 1-based (dataset.cpp:243 stores fid - 1); a 0-based file (what sklearn's
+    dump_svmlight_file writes by default) must stop on the host with the offending line, not index column -1."""
+    if not os.path.exists(TRAIN):
+        pytest.skip("CLI not built")
+    data = tmp_path / "zero_based.txt"
+    data.write_text("# comment line\n1 1:0.5 3:1.5\n0 2:1.0\n1 0:2.0 4:1.0\n0 1:1.0\n")
+    out = subprocess.run([TRAIN, "data=%s" % data, "n_trees=1"], capture_output=True, text=True, cwd=str(tmp_path))
+    assert out.returncode != 0
+    assert "line 4" in out.stderr and "feature id 0" in out.stderr and "1-based" in out.stderr
+
+
+_BAD_CSR = r"""
+import ctypes as C, sys
+import numpy as np
+sys.path.insert(0, %r)
+import thundergbm_amd
+L = thundergbm_amd.load()
+val = np.ones(4, np.float32); col = np.array([0, 1, 0, 1], np.int32); y = np.zeros(3, np.float32)
+rp = np.array(%s, np.int32)
+p = lambda a: a.ctypes.data_as(C.c_void_p)
+L.tgbm_trainer_create_grouped(3, p(val), p(rp), p(col), p(y), 3, 1, 1.0, 1.0, 1.0, 16, 1.0, b"reg:linear", 1, 0, None, 0)
+"""
+
+
+@pytest.mark.parametrize("row_ptr,msg", [("[0, 2, 1, 4]", "row_ptr decreases at row 1"), ("[1, 2, 3, 4]", "row_ptr[0] is 1")])
+def test_malformed_row_ptr_is_rejected_on_the_host(lib, row_ptr, msg):
+    import sys
+    out = subprocess.run([sys.executable, "-c", _BAD_CSR % (ROOT, row_ptr)], capture_output=True, text=True)
+    assert out.returncode != 0 and msg in out.stderr, out.stderr
+
+
+def test_load_model_with_one_label_per_training_row(lib, tmp_path):
+    """Model files written by the CLI for reg:* objectives store every training label (dataset.cpp:290-291,
+    parser.cpp:156-157); load_config copies them all, so the Python side must size its buffer from the file."""
+    import sys
+    sys.path.insert(0, ROOT)
+    import thundergbm_amd as T
+    labels = tuple(float(i % 7) for i in range(5000))
+    data, _ = _toy_model_bytes(objective=b"reg:linear", labels=labels, n_iter=2)
+    # num_class of a regression model is 1 whatever the label count
+    olen = 4 + len(b"reg:linear")
+    data = data[:olen + 4] + struct.pack("<i", 1) + data[olen + 8:]
+    path = tmp_path / "cli_reg.model"
+    path.write_bytes(data)
+    m = T.TGBMRegressor()
+    m.load_model(str(path))
+    assert m.num_class == 1 and m.n_trees == 2 and m.group_label == [0.0]
+    assert len(m.get_trees()) == 2

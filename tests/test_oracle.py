@@ -560,6 +560,22 @@ def test_base_score_binary_closed_form():
     assert np.all(o.y_pred() == np.float32(o.base_score))
 
 
+def test_base_score_regression_and_softmax_closed_form():
+    """init_base_score: reg:linear starts from -G/max(H, 1e-6) at a zero prediction = mean(y)
+    (regression_obj.h:35-53); objectives that do not override it start from 0 (objective_function.h:21-24)."""
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((700, 4)).astype(np.float32)
+    y = (3.0 + 2.0 * rng.standard_normal(700)).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    o = O.Oracle(val, rp, col, y, objective="reg:linear").prepare()
+    np.testing.assert_allclose(o.base_score, y.astype(np.float64).mean(), rtol=1e-6)
+    assert np.all(o.y_pred() == np.float32(o.base_score))
+    yc = rng.integers(0, 4, 700).astype(np.float32)
+    o = O.Oracle(val, rp, col, yc, objective="multi:softmax", num_class=4).prepare()
+    assert o.base_score == 0.0
+    assert np.all(o.y_pred() == 0.0)
+
+
 def test_softprob_transform_sums_to_one():
     rng = np.random.default_rng(9)
     raw = rng.standard_normal(5 * 40).astype(np.float32)

@@ -53,9 +53,6 @@ def build(force=True):
     for name, src in (("thundergbm-train", "cli_train.cpp"), ("thundergbm-predict", "cli_predict.cpp")):
         _run([HIPCC, "-O2", "-std=c++17", os.path.join(CSRC, src), "-o", os.path.join(BIN_DIR, name),
               "-L" + HERE, "-lthundergbm", "-Wl,-rpath,$ORIGIN/.."])
-    _run([HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "-munsafe-fp-atomics",
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-          os.path.join(CSRC, "bench_lds_atomics.hip"), "-o", os.path.join(BIN_DIR, "bench_lds_atomics")])
     return LIB
 
 

@@ -283,7 +283,7 @@ void launch_gather_perm(hipStream_t s, int n, const int *from, const int *perm_o
 void launch_cols_from_rows(hipStream_t s, int n, int W, int F, int n_blocks, const uint8_t *binmat, size_t block_stride,
                            uint8_t *colmat, size_t col_stride);
 
-// Largest of n non-negative ints in device memory (synchronises; 0 for n == 0).
+// Largest of n ints in device memory (synchronises; 0 for n == 0); aborts when one of them is negative.
 int device_max_int(hipStream_t s, const int *d_v, long n);
 
 // Host -> device copy of a pageable array on stream s; large ones go through pinned staging buffers and are

@@ -66,6 +66,11 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
     y.clear();
     label.clear();
     group.clear();
+    TGBM_CHECK(n_rows >= 0 && row_ptr != nullptr, "CSR input: %d rows", n_rows);
+    TGBM_CHECK(row_ptr[0] == 0, "CSR input: row_ptr[0] is %d, expected 0", row_ptr[0]);
+    for (int i = 0; i < n_rows; ++i)
+        TGBM_CHECK(row_ptr[i + 1] >= row_ptr[i], "CSR input: row_ptr decreases at row %d (%d -> %d)", i, row_ptr[i],
+                   row_ptr[i + 1]);
     const int nnz = row_ptr[n_rows];
     y.assign(n_rows, 0.f);
     if (labels != nullptr) std::copy(labels, labels + n_rows, y.begin());
@@ -77,12 +82,16 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
     if (count_features) {
         // largest column index, on a few threads when the matrix is large
         const int n_thr = nnz > (1 << 22) ? (int)std::min(8u, std::max(1u, std::thread::hardware_concurrency())) : 1;
-        std::vector<int> part_max(n_thr, 0);
+        std::vector<int> part_max(n_thr, 0), part_min(n_thr, 0);
         auto scan = [&](int t) {
             const long b = (long)nnz * t / n_thr, e = (long)nnz * (t + 1) / n_thr;
-            int m = 0;
-            for (long i = b; i < e; ++i) m = std::max(m, col_idx[i]);
+            int m = 0, lo = 0;
+            for (long i = b; i < e; ++i) {
+                m = std::max(m, col_idx[i]);
+                lo = std::min(lo, col_idx[i]);
+            }
             part_max[t] = m;
+            part_min[t] = lo;
         };
         std::vector<std::thread> pool;
         for (int t = 1; t < n_thr; ++t) pool.emplace_back(scan, t);
@@ -90,6 +99,8 @@ void DataSet::load_from_sparse(int n_rows, const float *val, const int *row_ptr,
         for (auto &th : pool) th.join();
         int max_col = 0;
         for (int m : part_max) max_col = std::max(max_col, m);
+        for (int lo : part_min) TGBM_CHECK(lo >= 0, "CSR input: negative column index %d", lo);
+        TGBM_CHECK(max_col < 2147483647, "CSR input: column index %d leaves no room for the feature count", max_col);
         n_features_ = (size_t)max_col + 1;
         log_info("#instances = %zu, #features = %zu", n_instances(), n_features());
     }
@@ -169,6 +180,9 @@ struct LibsvmChunk {
     std::vector<float> y, val;
     std::vector<int> col, row_len;
     size_t max_fid = 0;
+    size_t lines = 0;       // text lines of the chunk (data rows, comments and blank lines)
+    size_t bad_line = 0;    // 1-based line of the chunk that holds a feature id outside 1 .. 2^31 - 1 (0: none)
+    long bad_fid = 0;
 };
 
 void parse_libsvm_chunk(const char *b, const char *e, LibsvmChunk &out) {
@@ -178,6 +192,7 @@ void parse_libsvm_chunk(const char *b, const char *e, LibsvmChunk &out) {
         if (eol == nullptr) eol = e;
         const char *p = line;
         line = eol + 1;
+        ++out.lines;
         while (p < eol && (*p == ' ' || *p == '\t')) ++p;
         if (p >= eol || *p == '#' || *p == '\r') continue;
         char *end = nullptr;
@@ -196,6 +211,11 @@ void parse_libsvm_chunk(const char *b, const char *e, LibsvmChunk &out) {
             float v = std::strtof(p, &end);
             if (end == p) break;
             p = end;
+            // LIBSVM feature ids are 1-based (dataset.cpp:243 stores fid - 1): a 0-based file would index column -1
+            if ((fid < 1 || fid > 2147483647l) && out.bad_line == 0) {
+                out.bad_line = out.lines;
+                out.bad_fid = fid;
+            }
             out.col.push_back((int)fid - 1);
             out.val.push_back(v);
             ++len;
@@ -238,8 +258,12 @@ void DataSet::load_from_file(const std::string &file_name, GBMParam &param) {
     csr_col_idx.clear();
     csr_row_ptr.assign(1, 0);
     n_features_ = 0;
-    size_t rows = 0, entries = 0;
+    size_t rows = 0, entries = 0, lines_before = 0;
     for (const LibsvmChunk &c : chunks) {
+        TGBM_CHECK(c.bad_line == 0,
+                   "%s line %zu: feature id %ld is outside 1 .. 2^31 - 1 (LIBSVM feature ids are 1-based)",
+                   file_name.c_str(), lines_before + c.bad_line, c.bad_fid);
+        lines_before += c.lines;
         rows += c.y.size();
         entries += c.val.size();
     }

@@ -407,26 +407,39 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
     return out;
 }
 
-// Largest element of n non-negative ints (0 for n == 0).
-__global__ __launch_bounds__(256) void k_max_int(const int *__restrict__ v, long n, int *__restrict__ out) {
-    int m = 0;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) m = max(m, v[i]);
+// Largest element of n ints, with a check that none is negative (the values are column indices that the
+// callers are about to use as array indices): returns 0 for n == 0 and aborts on a negative entry.
+__global__ __launch_bounds__(256) void k_min_max_int(const int *__restrict__ v, long n, int *__restrict__ out) {
+    int m = 0, lo = 0;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int x = v[i];
+        m = max(m, x);
+        lo = min(lo, x);
+    }
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) m = max(m, __shfl_xor(m, d));
-    if ((threadIdx.x & 63) == 0) atomicMax(out, m);
+    for (int d = 32; d >= 1; d >>= 1) {
+        m = max(m, __shfl_xor(m, d));
+        lo = min(lo, __shfl_xor(lo, d));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicMax(out, m);
+        atomicMin(out + 1, lo);
+    }
 }
 
 int device_max_int(hipStream_t s, const int *d_v, long n) {
     if (n <= 0) return 0;
     int *d_out = nullptr;
-    HIP_CHECK(hipMalloc(&d_out, sizeof(int)));
-    HIP_CHECK(hipMemsetAsync(d_out, 0, sizeof(int), s));
-    k_max_int<<<grid_for((size_t)n, 4096), 256, 0, s>>>(d_v, n, d_out);
-    int h = 0;
-    HIP_CHECK(hipMemcpyAsync(&h, d_out, sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipMalloc(&d_out, 2 * sizeof(int)));
+    HIP_CHECK(hipMemsetAsync(d_out, 0, 2 * sizeof(int), s));
+    k_min_max_int<<<grid_for((size_t)n, 4096), 256, 0, s>>>(d_v, n, d_out);
+    int h[2] = {0, 0};
+    HIP_CHECK(hipMemcpyAsync(h, d_out, 2 * sizeof(int), hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));
     HIP_CHECK(hipFree(d_out));
-    return h;
+    TGBM_CHECK(h[1] >= 0, "CSR input: negative column index %d", h[1]);
+    TGBM_CHECK(h[0] < 2147483647, "CSR input: column index %d leaves no room for the feature count", h[0]);
+    return h[0];
 }
 
 // ---- physical re-ordering of the rows (see Trainer::reorder_rows) ---------------------------------

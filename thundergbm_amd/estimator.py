@@ -34,6 +34,23 @@ def _ptr(a):
     return a.ctypes.data_as(C.c_void_p)
 
 
+def _stored_label_count(model_path):
+    """Number of labels a model file stores (read from its header, nothing else is parsed)."""
+    import struct
+    with open(model_path, "rb") as f:
+        (olen,) = struct.unpack("<i", f.read(4))
+        if olen < 0 or olen >= 4096:
+            raise ValueError("model file %s: bad objective length" % model_path)
+        f.seek(olen + 16, 1)
+        raw = f.read(4)
+        if len(raw) != 4:
+            raise ValueError("model file %s is truncated" % model_path)
+        (n_label,) = struct.unpack("<i", raw)
+    if n_label < 0:
+        raise ValueError("model file %s: bad label count" % model_path)
+    return n_label
+
+
 class TGBMModel(BaseEstimator):
     def __init__(self, depth=6, n_trees=40, n_gpus=1, min_child_weight=1.0, lambda_tgbm=1.0, gamma=1.0,
                  max_num_bin=255, verbose=1, column_sampling_rate=1.0, bagging=0, n_parallel_trees=1,
@@ -136,7 +153,12 @@ class TGBMModel(BaseEstimator):
         self.num_class = n_class[0]
         self.n_trees = n_trees[0]
         self.tree_per_iter = per_iter[0]
-        labels = (C.c_float * max(self.num_class, 1))()
+        # load_config copies every label the file stores (scikit_tgbm.cpp:173-182) and has no capacity argument:
+        # files written by the CLI for reg:* / rank:* objectives hold one label per training row, so the buffer is
+        # sized from the file's own label count (header: i32 objective length, objective, f32 learning rate,
+        # i32 num_class, i32 n_trees, f32 base_score, i32 label count; parser.cpp:146-157)
+        n_stored = _stored_label_count(model_path)
+        labels = (C.c_float * max(n_stored, self.num_class, 1))()
         lib.load_config(model_path.encode("utf-8"), C.cast(labels, C.c_void_p))
         self.group_label = [labels[i] for i in range(self.num_class)]
 
