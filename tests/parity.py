@@ -9,20 +9,65 @@ import numpy as np
 REL = 1e-5
 
 
-def abs_hist(bins, rows, gh, n_bins):
-    """Per-bin sum of |g| and |h| over all stored entries: the scale a relative error refers to."""
-    out = np.zeros((n_bins, 2))
-    np.add.at(out, bins, np.abs(gh[rows].astype(np.float64)))
-    return out
+def node_hist_refs(bins, rows, gh, n_bins, node_of_row, first, count):
+    """For the nodes first .. first + count - 1: per-bin sums of |g|, |h| over the node's own rows
+    ([count, n_bins, 2]) and the number of stored entries per bin ([count, n_bins])."""
+    x = node_of_row[rows] - first
+    m = (x >= 0) & (x < count)
+    idx = x[m].astype(np.int64) * n_bins + bins[m]
+    a = np.abs(gh[rows[m]].astype(np.float64))
+    S = np.zeros((count * n_bins, 2))
+    S[:, 0] = np.bincount(idx, weights=a[:, 0], minlength=count * n_bins)
+    S[:, 1] = np.bincount(idx, weights=a[:, 1], minlength=count * n_bins)
+    cnt = np.bincount(idx, minlength=count * n_bins)
+    return S.reshape(count, n_bins, 2), cnt.reshape(count, n_bins)
 
 
-def assert_hist_close(got, ref64, scale, what="", rel=REL):
-    """|got - ref64| <= rel * scale, scale = per-bin sum of absolute contributions."""
+def item_shift(qmax, rows, bits):
+    """The library's rule (k_hist_dense): smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits."""
+    lim = 2.0 ** bits / rows * (1 - 1e-6) - 0.5
+    if not qmax >= lim:
+        return 0
+    return int(np.floor(np.log2(qmax / lim))) + 1
+
+
+def node_quantum(quant, node_rows, sparse, flush_rows=8192):
+    """Coarsest (g, h) step at which a row of a node with node_rows rows is counted. The library sums
+    round(g * scale) as exact 64-bit integers; a dense work item coarsens the tree's scale by a power of two
+    that depends on the rows it adds between two drains of its packed LDS bins (at most min(node rows, 8192)).
+    Every histogram built from rows is therefore exact up to half a step per stored entry."""
+    qg, qh = float(quant["inv_g"]), float(quant["inv_h"])
+    if sparse:
+        return np.array([qg, qh])
+    r = max(1, min(int(node_rows), flush_rows))
+    sg = item_shift(float(quant["gq_max"]), r, 63 - int(quant["h_bits"]))
+    sh = 0 if quant["h_integer"] else item_shift(float(quant["hq_max"]), r, int(quant["h_bits"]))
+    return np.array([qg * 2.0 ** sg, qh * 2.0 ** sh])
+
+
+def hist_tolerance(S_own, cnt, quantum, rel=REL):
+    """rel x (the node's own per-bin sum of |g|, |h|) + half a quantisation step per stored entry of the bin."""
+    return rel * S_own + 0.5 * cnt[:, None] * quantum[None, :]
+
+
+def assert_hist_close(got, ref64, tol, what=""):
     err = np.abs(got.astype(np.float64) - ref64)
-    tol = rel * scale + 1e-30
-    bad = err > tol
-    assert not bad.any(), "%s: %d bins off, worst err/scale %.3g" % (
-        what, int(bad.sum()), float((err / np.maximum(scale, 1e-30)).max()))
+    bad = err > tol + 1e-30
+    assert not bad.any(), "%s: %d bins off, worst err/tol %.3g" % (
+        what, int(bad.sum()), float((err / np.maximum(tol, 1e-300)).max()))
+    return err
+
+
+def sum_bounds(abs_scale, rel=REL):
+    """Bounds on a node's gradient / hessian sum: node sums are float32 results of a chain of histogram
+    subtractions that starts at the root, so their error is relative to the root-level sums of |g| and |h|."""
+    return rel * abs_scale[0] + 1e-7, rel * abs_scale[1] + 1e-7
+
+
+def gain_tolerance(weights, gain, dG, dH, rel=REL):
+    """First-order propagation of |dG|, |dH| into a gain built from the terms G^2 / (H + lambda) of the nodes with
+    the given weights w = -G / (H + lambda): d term / dG = -2 w, d term / dH = -w^2."""
+    return sum(2 * abs(w) * dG + w * w * dH for w in weights) + rel * max(1.0, abs(float(gain)))
 
 
 def gain_scale(node_sum, left_sum, lam):
@@ -78,13 +123,13 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     stack = [0]
     if abs_scale is None:
         abs_scale = (max(1.0, abs(float(orc[0]["sum_g"])) + float(orc[0]["sum_h"])),) * 2
-    dG, dH = rel * abs_scale[0] + 1e-7, rel * abs_scale[1] + 1e-7
+    dG, dH = sum_bounds(abs_scale, rel)
 
     def gain_tol(x, o):
         ws = [float(orc[x]["base_weight"])]
         if o["lch"] >= 0:
             ws += [float(orc[o["lch"]]["base_weight"]), float(orc[o["rch"]]["base_weight"])]
-        return sum(2 * abs(w) * dG + w * w * dH for w in ws) + rel * max(1.0, abs(float(o["gain"])))
+        return gain_tolerance(ws, o["gain"], dG, dH, rel)
 
     while stack:
         x = stack.pop()
@@ -153,5 +198,5 @@ def pred_tolerance(nodes, nid, lr, lam, abs_scale, y_pred, rel=REL):
     leaf = leaf_of(nodes, nid)
     w = np.abs(nodes["base_weight"][leaf].astype(np.float64))
     H = nodes["sum_h"][leaf].astype(np.float64)
-    dG, dH = rel * abs_scale[0] + 1e-7, rel * abs_scale[1] + 1e-7
+    dG, dH = sum_bounds(abs_scale, rel)
     return lr * ((dG + w * dH) / (H + lam) + rel * np.maximum(1.0, w)) + rel * np.abs(y_pred) + 1e-6

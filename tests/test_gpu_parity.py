@@ -41,13 +41,28 @@ def _missing_dataset(n, F, seed, frac=0.3, round_to=1):
     return X, y
 
 
+def _outlier_dataset(n, F, seed):
+    """Gaussian regression target with five labels 1e4 times larger than the rest: the gradients of reg:linear
+    inherit the outliers, so max|g| is ~1e4 times a typical |g|."""
+    rng = np.random.default_rng(seed)
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[X == 0] = 0.25
+    y = (X[:, 0] - 0.5 * X[:, 3] + 0.3 * rng.standard_normal(n)).astype(np.float32)
+    y[rng.choice(n, size=5, replace=False)] *= 1e4
+    return X, y
+
+
 def _cases():
     X1, y1 = D.config1(10000, 8, seed=0)
     X2, y2 = _missing_dataset(6000, 11, 3)
     X3, y3 = D.config2(20000, seed=1)
     X5, y5 = D.config5(8000, seed=4)
     v4, rp4, c4, y4 = D.config4(n=20000, F=3000, nnz_per_row=20, seed=3)
+    Xw, yw = D.config3(n=20000, F=200, seed=2)
+    Xo, yo = _outlier_dataset(20000, 12, 6)
     return {
+        "c3_wide_heavy_tails": (D.dense_to_csr(Xw), yw, dict(objective="reg:linear", depth=6, max_num_bin=255)),
+        "outlier_regression": (D.dense_to_csr(Xo), yo, dict(objective="reg:linear", depth=6, max_num_bin=255)),
         "c4_sparse": ((v4, rp4, c4), y4, dict(objective="binary:logistic", depth=6, max_num_bin=63)),
         "c1_regression": (D.dense_to_csr(X1), y1, dict(objective="reg:linear", depth=6, max_num_bin=255)),
         "missing_regression": (D.dense_to_csr(X2), y2, dict(objective="reg:linear", depth=5, max_num_bin=16)),
@@ -68,8 +83,8 @@ def case(name):
     return CASES[name.split("@")[0]]
 
 
-CASE_NAMES = ["c1_regression", "missing_regression", "c2_binary", "c5_softmax", "c4_sparse", "missing_regression@sparse",
-              "c5_softmax@sparse"]
+CASE_NAMES = ["c1_regression", "missing_regression", "c2_binary", "c3_wide_heavy_tails", "outlier_regression",
+              "c5_softmax", "c4_sparse", "missing_regression@sparse", "c5_softmax@sparse"]
 
 
 # ----------------------------------------------------------------------- cuts and bin ids (exact)
@@ -195,11 +210,22 @@ def test_tree_lockstep(T, name):
     gh_all = s.gh()
     o.set_gh(gh_all)  # both sides build from bit-identical gradients
     lam = 1.0
+    sparse = bool(s.info("sparse"))
     for k in range(s.tree_per_rounds):
         gh = gh_all[k * n:(k + 1) * n]
-        scale_root = P.abs_hist(gbins, rows, gh, nb)
+        ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
+        dG, dH = P.sum_bounds(ghk)
         s.tree_init(k)
         o.tree_init(k)
+        quant = s.quant()
+        # resolution of the fixed-point plan: the coarsest step (8192 rows between two drains) against the largest
+        # |g| of the tree; 50-bit gradient fields when every hessian is an integer (squared loss), 32 otherwise
+        if not sparse:
+            gmax = float(np.abs(gh[:, 0]).max())
+            assert bool(quant["h_integer"]) == (kw["objective"] == "reg:linear")
+            assert P.node_quantum(quant, n, False)[0] <= gmax * 2.0 ** (-34 if quant["h_integer"] else -17)
+        node_of_row = np.zeros(n, np.int64)
+        tol_prev = None  # tolerance arrays of the previous level's nodes
         diverged = False
         for level in range(depth):
             s.find_split(level)
@@ -210,27 +236,52 @@ def test_tree_lockstep(T, name):
             gnodes = s.nodes()
             off = (1 << level) - 1
             sp_g, sp_o = s.splits(level), o.splits()
+            # Tolerance of a node built from rows: 1e-5 of its own per-bin sum of |g|, |h| plus half a fixed-point
+            # step per stored entry; of a node derived as parent - sibling: the sum of the two operands' tolerances.
+            S_own, cnt = P.node_hist_refs(gbins, rows, gh, nb, node_of_row, off, 1 << level)
+            loc = node_of_row - off
+            n_rows = np.bincount(loc[(loc >= 0) & (loc < (1 << level))], minlength=1 << level)
+            # built from rows: the root, then of every sibling pair the child with fewer rows, ties the left one
+            # (hist_tree_builder_single.cu:466-467)
+            built = [level == 0 or n_rows[x] < n_rows[x ^ 1] or (n_rows[x] == n_rows[x ^ 1] and x % 2 == 0)
+                     for x in range(1 << level)]
+            tol_level = [None] * (1 << level)
+            for x in range(1 << level):
+                if built[x]:
+                    tol_level[x] = P.hist_tolerance(S_own[x], cnt[x], P.node_quantum(quant, n_rows[x], sparse))
+            for x in range(1 << level):
+                if tol_level[x] is None:
+                    tol_level[x] = tol_prev[x >> 1] + tol_level[x ^ 1]
             for x in range(1 << level):
                 if not onodes[off + x]["is_valid"]:
                     assert sp_g[x]["nid"] == -1 and sp_o[x]["nid"] == -1
                     continue
                 _, h64 = o.level_hist(x)
-                P.assert_hist_close(gh_level[x], h64, scale_root, "tree %d level %d node %d" % (k, level, x))
+                what = "tree %d level %d node %d" % (k, level, x)
+                err = P.assert_hist_close(gh_level[x], h64, tol_level[x], what)
+                if built[x] and (sparse or quant["h_integer"]):
+                    # wide fixed-point fields (64-bit sums in the sparse layout, 50-bit gradient fields for squared
+                    # loss): also without the half-step allowance, every bin whose entries are not far below the
+                    # node's typical |g| is within 1e-5 of its own sum
+                    typical = S_own[x][:, 0].sum() / max(1, cnt[x].sum())
+                    judged = S_own[x][:, 0] >= 1e-3 * typical * cnt[x]
+                    assert np.all(err[judged, 0] <= 1e-5 * S_own[x][judged, 0] + 1e-30), what
                 a, b = sp_g[x], sp_o[x]
+                ws = [float(onodes[off + x]["base_weight"])]
+                if onodes[off + x]["lch"] >= 0:
+                    ws += [float(onodes[2 * (off + x) + 1]["base_weight"]), float(onodes[2 * (off + x) + 2]["base_weight"])]
                 if a["best_index"] != b["best_index"]:
                     sc = o.tree_scores()[off + x]
                     best = abs(sc).max()
-                    assert best - abs(sc[a["best_index"]]) <= 1e-4 * max(1.0, best), \
+                    assert best - abs(sc[a["best_index"]]) <= 2 * P.gain_tolerance(ws, best, dG, dH), \
                         "level %d node %d picks %d vs %d" % (level, x, a["best_index"], b["best_index"])
                     diverged = True
                     continue
                 assert a["fid"] == b["fid"] and a["bid"] == b["bid"] and a["fval"] == b["fval"]
-                S = (float(onodes[off + x]["sum_g"]), float(onodes[off + x]["sum_h"]))
-                gs = max(1.0, P.gain_scale(S, (float(b["lch_g"]), float(b["lch_h"])), lam))
-                assert abs(a["gain"] - b["gain"]) <= 1e-4 * gs
-                nsc = max(1.0, abs(S[0]) + abs(S[1]))
-                for key in ("lch_g", "lch_h", "miss_g", "miss_h"):
-                    assert abs(a[key] - b[key]) <= 1e-4 * nsc, (key, a[key], b[key])
+                assert abs(a["gain"] - b["gain"]) <= P.gain_tolerance(ws, b["gain"], dG, dH), what
+                for key, d in (("lch_g", dG), ("lch_h", dH), ("miss_g", dG), ("miss_h", dH)):
+                    assert abs(a[key] - b[key]) <= d, (key, a[key], b[key])
+            tol_prev = tol_level
             if diverged:
                 break
             # same splits -> node arrays agree and the partition must be bit-identical
@@ -239,11 +290,13 @@ def test_tree_lockstep(T, name):
             assert np.array_equal(gnodes["split_value"], onodes["split_value"])
             # default direction matters only where values are missing; force agreement for the rest
             # by copying the GPU's nodes into the oracle (sums differ in the last ulps only)
-            np.testing.assert_allclose(gnodes["sum_g"], onodes["sum_g"], rtol=0, atol=1e-4 * max(1, abs(gh[:, 0]).sum()))
+            np.testing.assert_allclose(gnodes["sum_g"], onodes["sum_g"], rtol=0, atol=dG)
+            np.testing.assert_allclose(gnodes["sum_h"], onodes["sum_h"], rtol=0, atol=dH)
             o.set_nodes(gnodes)
             s.partition(level)
             has = o.update_ins2node()
             assert np.array_equal(s.nid(), o.nid()), "node assignment differs at level %d" % level
+            node_of_row = s.nid().astype(np.int64)
             # row lists: every node's segment holds exactly its rows in ascending order
             seg = s.get("seg", np.int32, (-1, 2))
             ridx = s.get("ridx%d" % ((level + 1) & 1), np.int32)
@@ -263,7 +316,6 @@ def test_tree_lockstep(T, name):
         s.finish_tree(k)
         o.prune()
         o.predict_in_training(k)
-        ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
         d = P.compare_trees(s.nodes(), o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(), abs_scale=(ghk[0], ghk[1]))
         assert not d.near_ties
         sl = slice(k * n, (k + 1) * n)
@@ -274,7 +326,7 @@ def test_tree_lockstep(T, name):
 
 # -------------------------------------------------------------------- boosting, tree by tree
 @pytest.mark.parametrize("name,rounds", [("c1_regression", 40), ("missing_regression", 10), ("c2_binary", 10),
-                                         ("c5_softmax", 3), ("c4_sparse", 10), ("missing_regression@sparse", 10),
+                                         ("c3_wide_heavy_tails", 6), ("outlier_regression", 8), ("c5_softmax", 3), ("c4_sparse", 10), ("missing_regression@sparse", 10),
                                          ("c1_regression@sparse", 5)])
 def test_boosting_teacher_forced(T, name, rounds):
     """Each round both sides start from the GPU's predictions, so every tree is compared on its own."""
@@ -307,7 +359,9 @@ def test_boosting_teacher_forced(T, name, rounds):
             d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(),
                                 missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
                                 abs_scale=(ghk[0], ghk[1]))
-            total_ties += len(d.near_ties)
+            # candidates that cut a node's rows into the same two sets have equal gains in exact arithmetic and
+            # differ by float round-off only (wide data, nodes of a few rows): those are not counted
+            total_ties += sum(1 for (_, best, alt) in d.near_ties if not best - alt <= 2e-6 * best)
             ok_round &= not d.near_ties
             sl = slice(k * n, (k + 1) * n)
             tol[sl] = P.pred_tolerance(o.nodes(), final_nid, kw["learning_rate"], 1.0, (ghk[0], ghk[1]), o.y_pred()[sl])

@@ -40,21 +40,32 @@ struct LevelCtl {
     int rows_built;  // rows visited by the histogram build of the level
 };
 
-// Fixed-point scales of one tree. Gradients and hessians are accumulated in LDS as one packed
-// 64-bit integer per bin (gradient in the high, hessian in the low 32 bits) because gfx950 executes
-// 64-bit integer LDS atomics about 15x faster than float ones; scales are powers of two chosen so
-// that the sums of a few thousand rows cannot leave their 32-bit fields; the LDS bins are drained
-// into 64-bit integers before that many rows were added. All further sums are 64-bit integers, so
-// histograms (and sibling subtraction) are exact in the quantised values and bit-reproducible.
+// Fixed-point plan of one tree. Histograms are exact 64-bit integer sums of round(g * scale_g), round(h * scale_h);
+// the scales are the largest powers of two that keep the sum over all n rows below 2^62, so the quantum is about
+// max|g| * n / 2^62 (2^-38 of the largest gradient at 10 M rows).
+//   Dense layout: a work item (a run of rows of one node) accumulates in LDS with one 64-bit integer atomic per
+// (row, feature) - gfx950 executes those about 15x faster than float LDS atomics - into a packed bin: gradient in
+// the high 64 - h_bits bits (signed), hessian in the low h_bits bits. The fields must hold the sum of the
+// min(rows of the item, kHistFlushRows) rows added between two drains of the LDS bins into 64-bit registers, so an
+// item coarsens the tree's scales by its own power of two (shift): the fewer rows an item has, the finer it counts;
+// k_hist_merge shifts every item's sums back to the tree's scale. h_bits: 32 in general; when every hessian of the
+// tree is a small non-negative integer (squared loss: 1, or the draw count under bagging) the hessian field gets
+// exactly the bits that kHistFlushRows * max h needs and the gradient field the rest (50 bits for h = 1), which
+// is what keeps heavy-tailed regression residuals at float-like resolution (2^-36 of the largest |g| per row).
+// All sums after the LDS stage are 64-bit integers: exact, order-independent, bit-reproducible.
 struct QuantCtl {
-    float scale_g, scale_h;  // value -> integer
+    float scale_g, scale_h;  // value -> integer of the tree's histograms (powers of two)
     float inv_g, inv_h;      // integer -> value
+    float gq_max, hq_max;    // max|g| * scale_g, max h * scale_h: the most one row can add
+    int h_bits;              // width of the hessian field of a packed LDS bin
+    int h_integer;           // 1: every hessian is an integer, scale_h = 1 and no item shifts it
 };
 
 // Block result of the per-tree gradient reduction.
 struct GradStats {
     float g, h;        // sums
     float gmax, hmax;  // max |g|, max h
+    float hfrac;       // max |h - round(h)|: 0 when every hessian is an integer
 };
 
 // Candidate produced by one wavefront of the split finder.
@@ -108,6 +119,7 @@ struct TreeBuffers {
                                                 // of the nodes of a level, ping-pong by level parity
     longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
     QuantCtl *quant = nullptr;     // scales of the current tree
+    int2 *hitem_shift = nullptr;   // [max_hitems] powers of two by which a dense work item coarsened (g, h)
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
     float *leaf_value = nullptr;   // [n_nodes] prediction increment of a row that ended in the node (after pruning)
     int *end_bound = nullptr;      // [(row_blocks(n) + 1) x (2^depth - 1)] list positions of the row block boundaries
@@ -161,6 +173,7 @@ struct TreeBuffers {
         t.hist_q[1] += K * max_level_nodes * n_bins;
         t.partial += K * n_partial;
         t.quant += K;
+        t.hitem_shift += K * max_hitems;
         t.leaf_value += K * n_nodes;
         t.end_bound += K * n_end_bound;
         t.hpair_begin += K * (max_level_nodes + 1);

@@ -343,6 +343,7 @@ void Trainer::alloc_tree_buffers() {
     tb.hist_q[1] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
     tb.partial = dalloc<longlong2>(S * tb.n_partial);
     tb.quant = dalloc<QuantCtl>(S);
+    tb.hitem_shift = dalloc<int2>(S * (size_t)tb.max_hitems);
     tb.hpair_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
     tb.leaf_value = dalloc<float>(S * tb.n_nodes);
     tb.end_bound = dalloc<int>(S * tb.n_end_bound);

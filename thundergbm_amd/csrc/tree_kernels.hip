@@ -175,38 +175,44 @@ __global__ void k_bagging_apply(int N, int *__restrict__ count, GHPair *__restri
 // gradient statistics or metric partials follows this order, so fused and separate passes give the
 // same bits.
 struct RowStats {
-    float g = 0, h = 0, gm = 0, hm = 0;
+    float g = 0, h = 0, gm = 0, hm = 0, hf = 0;
     __device__ __forceinline__ void add(GHPair v) {
         g += v.g;
         h += v.h;
         gm = fmaxf(gm, fabsf(v.g));
         hm = fmaxf(hm, v.h);
+        hf = fmaxf(hf, fabsf(v.h - rintf(v.h)));
     }
 };
 
-// lds: 4 * kWaves floats; every thread of the block must call
+constexpr int kStatsLds = 5 * kWaves;  // floats of LDS that store_block_stats needs
+
+// lds: kStatsLds floats; every thread of the block must call
 __device__ void store_block_stats(RowStats r, float *lds, GradStats *out) {
-    float *sg = lds, *sh = lds + kWaves, *mg = lds + 2 * kWaves, *mh = lds + 3 * kWaves;
-    float g = wave_sum_f(r.g), h = wave_sum_f(r.h), gm = r.gm, hm = r.hm;
+    float *sg = lds, *sh = lds + kWaves, *mg = lds + 2 * kWaves, *mh = lds + 3 * kWaves, *fh = lds + 4 * kWaves;
+    float g = wave_sum_f(r.g), h = wave_sum_f(r.h), gm = r.gm, hm = r.hm, hf = r.hf;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
         gm = fmaxf(gm, __shfl_xor(gm, d));
         hm = fmaxf(hm, __shfl_xor(hm, d));
+        hf = fmaxf(hf, __shfl_xor(hf, d));
     }
     if (lane_id() == 0) {
         sg[wave_id()] = g;
         sh[wave_id()] = h;
         mg[wave_id()] = gm;
         mh[wave_id()] = hm;
+        fh[wave_id()] = hf;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        GradStats o{0, 0, 0, 0};
+        GradStats o{0, 0, 0, 0, 0};
         for (int i = 0; i < kWaves; ++i) {
             o.g += sg[i];
             o.h += sh[i];
             o.gmax = fmaxf(o.gmax, mg[i]);
             o.hmax = fmaxf(o.hmax, mh[i]);
+            o.hfrac = fmaxf(o.hfrac, fh[i]);
         }
         *out = o;
     }
@@ -228,7 +234,7 @@ __device__ void store_block_sum_d(double acc, double *lds, double *out) {
 // Block sums of (g,h) and block maxima of |g|, h for one tree.
 // Class trees of a round: blockIdx.z selects the class (gradients and outputs are class-major).
 __global__ __launch_bounds__(kBlock) void k_sum_gh(int n, const GHPair *__restrict__ gh, GradStats *__restrict__ out) {
-    __shared__ float lds[4 * kWaves];
+    __shared__ float lds[kStatsLds];
     gh += (size_t)blockIdx.z * n;
     out += (size_t)blockIdx.z * gridDim.x;
     const int r0 = blockIdx.x * kRowBlock, r1 = min(n, r0 + kRowBlock);
@@ -247,11 +253,29 @@ __device__ float pow2_scale(float vmax, int rows, float limit) {
     return ldexpf(1.f, e - 1);     // 2^(e-1) <= bound
 }
 
+// Power of two by which a dense work item that adds `rows` rows between two drains coarsens one of the tree's
+// scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
+// scale, bits: magnitude bits of the packed field).
+__device__ int item_shift(float qmax, int rows, int bits) {
+    const double lim = ldexp(1.0, bits) / (double)rows * (1.0 - 1e-6) - 0.5;
+    const double q = (double)qmax;
+    if (!(q >= lim)) return 0;
+    return ilogb(q / lim) + 1;  // 2^s > q / lim
+}
+
+// Round-to-nearest-even of a float (|x| < 2^51) as a 64-bit integer: the integer sits in the low mantissa bits of
+// x + 1.5 * 2^52 (bit pattern 0x4338000000000000, whose low word is zero: only the high word is corrected).
+__device__ __forceinline__ long long round_to_ll(float x) {
+    const long long b = __double_as_longlong((double)x + 6755399441055744.0);
+    const unsigned hi = (unsigned)((unsigned long long)b >> 32) - 0x43380000u;
+    return (long long)(((unsigned long long)hi << 32) | (unsigned)b);
+}
+
 // ------------------------------------------------------------------------------- tree init
 // Node array initialisation of the reference's Tree::init2 (src/thundergbm/tree.cu:8-39), root sum
 // from the block partials, root segment and the histogram plan of level 0. One workgroup.
 __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float lambda) {
-    __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves];
+    __shared__ float sg[kWaves], sh[kWaves], mg[kWaves], mh[kWaves], fh[kWaves];
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     const GradStats *__restrict__ block_sums = tb.root_partial;
     const int nn = tb.n_nodes;
@@ -283,12 +307,13 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         tb.nodes[i] = nd;
         tb.seg[i] = make_int2(0, 0);
     }
-    float g = 0, h = 0, gm = 0, hm = 0;
+    float g = 0, h = 0, gm = 0, hm = 0, hf = 0;
     for (int i = threadIdx.x; i < tb.n_grad_blocks; i += kBlock) {
         g += block_sums[i].g;
         h += block_sums[i].h;
         gm = fmaxf(gm, block_sums[i].gmax);
         hm = fmaxf(hm, block_sums[i].hmax);
+        hf = fmaxf(hf, block_sums[i].hfrac);
     }
     g = wave_sum_f(g);
     h = wave_sum_f(h);
@@ -296,23 +321,27 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
     for (int d = 32; d >= 1; d >>= 1) {
         gm = fmaxf(gm, __shfl_xor(gm, d));
         hm = fmaxf(hm, __shfl_xor(hm, d));
+        hf = fmaxf(hf, __shfl_xor(hf, d));
     }
     if (lane_id() == 0) {
         sg[wave_id()] = g;
         sh[wave_id()] = h;
         mg[wave_id()] = gm;
         mh[wave_id()] = hm;
+        fh[wave_id()] = hf;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         GHPair s{0, 0};
         gm = 0;
         hm = 0;
+        hf = 0;
         for (int i = 0; i < kWaves; ++i) {
             s.g += sg[i];
             s.h += sh[i];
             gm = fmaxf(gm, mg[i]);
             hm = fmaxf(hm, mh[i]);
+            hf = fmaxf(hf, fh[i]);
         }
         TreeNode &root = tb.nodes[0];
         root.sum_gh_pair = s;
@@ -332,20 +361,25 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         c.rows_built = tb.n;
         tb.ctl[0] = c;
         tb.ctl[tb.depth] = LevelCtl{0, 0, 0, 0};  // the last level plans no further one
-        // One pair of scales serves the whole tree: between two drains of the LDS histogram at most
-        // kHistFlushRows rows are added, which keeps a bin's gradient sum inside a signed and its
-        // hessian sum inside an unsigned 32-bit field.
+        // The tree's scales keep the 64-bit sums over all n rows below 2^62; a dense work item coarsens them by its
+        // own power of two so that its packed LDS fields hold the rows between two drains (item_shifts).
         QuantCtl q;
-        if (tb.sparse) {
-            // sums go straight into 64-bit integers: the whole dataset must fit below 2^62
-            q.scale_g = pow2_scale(gm, tb.n, 4.6e18f);
-            q.scale_h = pow2_scale(hm, tb.n, 4.6e18f);
-        } else {
-            q.scale_g = pow2_scale(gm, kHistFlushRows, 2147483520.f);  // largest float below 2^31
-            q.scale_h = pow2_scale(hm, kHistFlushRows, 4294967040.f);  // largest float below 2^32
+        q.scale_g = pow2_scale(gm, tb.n, 4.6e18f);
+        q.scale_h = pow2_scale(hm, tb.n, 4.6e18f);
+        q.h_bits = 32;
+        q.h_integer = 0;
+        // every hessian a non-negative integer (squared loss; bagging multiplies by draw counts): the hessian field
+        // takes the bits that kHistFlushRows such rows need, the gradient field the rest
+        const float hrows = hm * (float)kHistFlushRows;
+        if (!tb.sparse && hf == 0.f && hm >= 1.f && hrows < 4.0e9f) {
+            q.h_integer = 1;
+            q.h_bits = ilogbf(hrows) + 1;
+            q.scale_h = 1.f;
         }
         q.inv_g = 1.f / q.scale_g;
         q.inv_h = 1.f / q.scale_h;
+        q.gq_max = gm * q.scale_g;
+        q.hq_max = hm * q.scale_h;
         *tb.quant = q;
     }
 }
@@ -353,11 +387,12 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
 // ------------------------------------------------------------------------- dense histogram
 // One workgroup = one work item (a run of rows of one node) x one feature block. The block's
 // histogram lives in LDS as one 64-bit integer per bin holding the fixed-point gradient sum in the
-// high and the hessian sum in the low half; a row contributes with a single ds_add_u64 per feature
-// (float LDS atomics run at ~0.3 lanes/clk/CU on gfx950, 64-bit integer ones at ~5). The 32-bit
-// fields are safe for kHistFlushRows rows (that bound sets the fixed-point scales), so after at most
-// that many rows every thread drains the bins it owns into 64-bit register accumulators and clears
-// them; at the end the registers go to the item's slot of `partial`.
+// high and the hessian sum in the low field (QuantCtl::h_bits wide); a row contributes with a single
+// ds_add_u64 per feature (float LDS atomics run at ~0.3 lanes/clk/CU on gfx950, 64-bit integer ones at ~5).
+// The fields are safe for the rows added between two drains (at most kHistFlushRows; fewer for a short item,
+// which therefore counts finer: item_shift), so after at most that many rows every thread drains the bins it
+// owns into 64-bit register accumulators and clears them; at the end the registers go to the item's slot of
+// `partial`, at the item's scale (k_hist_merge shifts them to the tree's).
 // LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
 // instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
 // (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
@@ -367,7 +402,7 @@ template <int LPR, bool DIRECT, int BLK, int SLOTS>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
-    __shared__ int s_range[2];
+    __shared__ int s_range[4];
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     gh += (size_t)blockIdx.z * tb.n;
     const int *__restrict__ ridx = tb.list(level);
@@ -386,18 +421,30 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     const int bin0 = blk_bin_begin[fb];
     const int nb = blk_bin_begin[fb + 1] - bin0;
     if (nb == 0) return;
+    const int h_bits = quant->h_bits;
     if (threadIdx.x == 0) {
         int p = find_owner(hpair_begin, n_pairs, item);
         int node = hpair_built[p];
         int2 sg = seg[node];
         int b = sg.x + (item - hpair_begin[p]) * c.hchunk;
+        int e = min(sg.y, b + c.hchunk);
         s_range[0] = b;
-        s_range[1] = min(sg.y, b + c.hchunk);
+        s_range[1] = e;
+        const int rows = max(1, min(e - b, kHistFlushRows));
+        const int2 shift = make_int2(item_shift(quant->gq_max, rows, 63 - h_bits),
+                                     quant->h_integer ? 0 : item_shift(quant->hq_max, rows, h_bits));
+        s_range[2] = shift.x;
+        s_range[3] = shift.y;
+        if (fb == 0) tb.hitem_shift[item] = shift;
     }
     for (int i = threadIdx.x; i < nb; i += BLK) lds[i] = 0ull;
     __syncthreads();
-    const int begin = s_range[0], end = s_range[1];
-    const float scale_g = quant->scale_g, scale_h = quant->scale_h;
+    // (values that are the same for every lane are moved to scalar registers)
+    const int begin = __builtin_amdgcn_readfirstlane(s_range[0]), end = __builtin_amdgcn_readfirstlane(s_range[1]);
+    // the item's scales: powers of two well inside the float range, so the products below are exact
+    const float scale_g = ldexpf(quant->scale_g, -__builtin_amdgcn_readfirstlane(s_range[2]));
+    const float scale_h = ldexpf(quant->scale_h, -__builtin_amdgcn_readfirstlane(s_range[3]));
+    const unsigned long long h_mask = (1ull << h_bits) - 1ull;  // h_bits <= 32
     constexpr int RPS = BLK / LPR;  // rows per step of the whole block
     // steps in flight per thread: three keep the 64-register variants (8 waves per SIMD) free of spills
     constexpr int U = SLOTS <= 8 ? 3 : 4;
@@ -439,9 +486,9 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
                 if (i < nb) {
                     const unsigned long long t = lds[i];
                     lds[i] = 0ull;
-                    const unsigned lo = (unsigned)t;
-                    accg[k] += (int)((long long)(t - lo) >> 32);
-                    acch[k] += lo;
+                    const unsigned long long lo = t & h_mask;
+                    accg[k] += (long long)(t - lo) >> h_bits;
+                    acch[k] += (long long)lo;
                 }
             }
             __syncthreads();
@@ -451,9 +498,10 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const unsigned v = pk[u];
-            const int gq = __float2int_rn(s[u].g * scale_g);
-            const unsigned hq = __float2uint_rn(s[u].h * scale_h);
-            const unsigned long long add = ((unsigned long long)(long long)gq << 32) + hq;
+            // exact products (the scales are powers of two), rounded once to the nearest integer
+            const long long gq = round_to_ll(s[u].g * scale_g);
+            const long long hq = round_to_ll(fmaxf(s[u].h, 0.f) * scale_h);
+            const unsigned long long add = ((unsigned long long)gq << h_bits) + (unsigned long long)hq;
             const unsigned b0 = v & 0xff, b1 = (v >> 8) & 0xff, b2 = (v >> 16) & 0xff, b3 = v >> 24;
             if (b0 != kMissingBin) atomicAdd(lds + o0 + b0, add);
             if (b1 != kMissingBin) atomicAdd(lds + o1 + b1, add);
@@ -480,8 +528,8 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         const int i = threadIdx.x + k * BLK;
         if (i < nb) {
             const unsigned long long t = lds[i];
-            const unsigned lo = (unsigned)t;
-            out[i] = make_longlong2(accg[k] + (int)((long long)(t - lo) >> 32), acch[k] + lo);
+            const unsigned long long lo = t & h_mask;
+            out[i] = make_longlong2(accg[k] + ((long long)(t - lo) >> h_bits), acch[k] + (long long)lo);
         }
     }
 }
@@ -513,19 +561,25 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
     long long sg = 0, sh = 0;
     if (j < n_bins) {
+        // every item counted at its own scale (item_shift): shift its sums to the tree's
+        const int2 *__restrict__ shift = tb.hitem_shift;
         if (tb.ctl[level].hchunk <= kHistFlushRows) {  // packed 8-byte partials (see k_hist_dense)
             const unsigned long long *packed = reinterpret_cast<const unsigned long long *>(partial);
+            const int h_bits = tb.quant->h_bits;
+            const unsigned long long h_mask = (1ull << h_bits) - 1ull;
             for (int it = ib + ig; it < ie; it += kMergeGroups) {
                 const unsigned long long t = packed[(size_t)it * n_bins + j];
-                const unsigned lo = (unsigned)t;
-                sg += (int)((long long)(t - lo) >> 32);
-                sh += lo;
+                const int2 s = shift[it];
+                const unsigned long long lo = t & h_mask;
+                sg += ((long long)(t - lo) >> h_bits) << s.x;
+                sh += (long long)lo << s.y;
             }
         } else {
             for (int it = ib + ig; it < ie; it += kMergeGroups) {
                 longlong2 v = partial[(size_t)it * n_bins + j];
-                sg += v.x;
-                sh += v.y;
+                const int2 s = shift[it];
+                sg += v.x << s.x;
+                sh += v.y << s.y;
             }
         }
     }
@@ -1519,7 +1573,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
     __shared__ int s_off[kEndListCap];
     __shared__ int s_scan[kWaves];
     __shared__ int s_n;
-    __shared__ float s_f[4 * kWaves];
+    __shared__ float s_f[kStatsLds];
     __shared__ double s_d[kWaves];
     const int r0 = blockIdx.x * kRowBlock, r1 = min(tb.n, r0 + kRowBlock);
     for (int i = threadIdx.x; i < kRowBlock; i += kBlock) s_leaf[i] = -1;

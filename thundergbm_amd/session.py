@@ -20,6 +20,8 @@ SPLIT_DTYPE = np.dtype(
         ("best_index", "<i4"), ("pad", "<i4"),
     ]
 )
+QUANT_DTYPE = np.dtype([("scale_g", "<f4"), ("scale_h", "<f4"), ("inv_g", "<f4"), ("inv_h", "<f4"),
+                        ("gq_max", "<f4"), ("hq_max", "<f4"), ("h_bits", "<i4"), ("h_integer", "<i4")])
 CTL_DTYPE = np.dtype([("hchunk", "<i4"), ("n_hitems", "<i4"), ("n_pitems", "<i4"), ("rows_built", "<i4")])
 
 
@@ -148,11 +150,15 @@ class Session:
         return self.get("sp", SPLIT_DTYPE)[: 1 << level]
 
     def level_hist(self, level):
-        """Raw histograms of the nodes of `level`: [2^level, n_bins, 2] (exact fixed-point sums as float32)."""
+        """Raw histograms of the nodes of `level`: [2^level, n_bins, 2] (exact fixed-point sums as float64)."""
         q = self.get("hist_q%d" % (level & 1), np.int64)
         q = q[: (1 << level) * self.n_bins * 2].reshape(1 << level, self.n_bins, 2)
-        sc = self.get("quant", np.float32)  # scale_g, scale_h, inv_g, inv_h
-        return (q.astype(np.float64) * sc[2:4].astype(np.float64)).astype(np.float32)
+        sc = self.quant()
+        return q.astype(np.float64) * np.array([float(sc["inv_g"]), float(sc["inv_h"])])
+
+    def quant(self):
+        """Fixed-point plan of the current tree (QuantCtl)."""
+        return self.get("quant", QUANT_DTYPE)[0]
 
     def ctl(self):
         return self.get("ctl", CTL_DTYPE)
