@@ -81,10 +81,18 @@ def gain_scale(node_sum, left_sum, lam):
 class TreeDiff:
     def __init__(self):
         self.compared = 0
-        self.near_ties = []  # (node, oracle best |gain|, oracle |gain| of the GPU's choice)
+        # (node, oracle best |gain|, oracle |gain| of the GPU's choice, magnitude of the oracle gain's terms)
+        self.near_ties = []
 
     def __repr__(self):
         return "TreeDiff(compared=%d, near_ties=%r)" % (self.compared, self.near_ties)
+
+
+def significant_ties(near_ties):
+    """Near ties that are more than float round-off between two candidates: candidates that cut a node's rows into
+    the same two sets have equal gains in exact arithmetic, and which of them a float implementation prefers is
+    decided by the order of its additions (in the reference: by the order of its atomics)."""
+    return [t for t in near_ties if not t[1] - t[2] <= 2e-6 * max(t[1], t[3])]
 
 
 def rows_in_node(final_nid, x):
@@ -161,21 +169,25 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
             if has:
                 hmin = min(float(t[int(t[x]["lch"])]["sum_h"]), float(t[int(t[x]["rch"])]["sum_h"]))
                 on_gate |= abs(hmin - mcw) <= dH
-        if on_gate:
-            diff.near_ties.append((x, float("nan"), float("nan")))
-            continue
         sc = orc_scores[x]
         best = float(np.abs(sc).max())
         tol = 2 * gain_tol(x, o)
         if split_g:
             alt = abs(float(sc[int(crp[g["split_fid"]]) + int(g["split_bid"])]))
-            assert best - alt <= tol, \
-                "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d), tol %g" % (
-                    x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"], tol)
+            ok = best - alt <= tol
+            msg = "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d), tol %g" % (
+                x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"], tol)
         else:
             alt = 0.0  # gpu made a leaf where the oracle split: the gain must sit at the rt_eps edge
-            assert best <= 1e-6 + tol, "node %d: gpu leaf, oracle split gain %g" % (x, best)
-        diff.near_ties.append((x, best, alt))
+            ok = best <= 1e-6 + tol
+            msg = "node %d: gpu leaf, oracle split gain %g" % (x, best)
+        if not ok:
+            assert on_gate, msg
+            diff.near_ties.append((x, float("nan"), float("nan"), 0.0))
+            continue
+        # magnitude of the three terms whose difference the gain is (float cancellation noise scales with it)
+        terms = gain_scale(S, (float(orc[int(o["lch"])]["sum_g"]), float(orc[int(o["lch"])]["sum_h"])), lam) if split_o else 0.0
+        diff.near_ties.append((x, best, alt, terms))
     if not diff.near_ties:
         for key in ("is_leaf", "is_pruned", "final_id", "lch", "rch", "parent"):
             valid = orc["is_valid"] == 1

@@ -361,7 +361,7 @@ def test_boosting_teacher_forced(T, name, rounds):
                                 abs_scale=(ghk[0], ghk[1]))
             # candidates that cut a node's rows into the same two sets have equal gains in exact arithmetic and
             # differ by float round-off only (wide data, nodes of a few rows): those are not counted
-            total_ties += sum(1 for (_, best, alt) in d.near_ties if not best - alt <= 2e-6 * best)
+            total_ties += len(P.significant_ties(d.near_ties))
             ok_round &= not d.near_ties
             sl = slice(k * n, (k + 1) * n)
             tol[sl] = P.pred_tolerance(o.nodes(), final_nid, kw["learning_rate"], 1.0, (ghk[0], ghk[1]), o.y_pred()[sl])

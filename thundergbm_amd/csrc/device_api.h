@@ -46,8 +46,10 @@ struct LevelCtl {
 //   Dense layout: a work item (a run of rows of one node) accumulates in LDS with one 64-bit integer atomic per
 // (row, feature) - gfx950 executes those about 15x faster than float LDS atomics - into a packed bin: gradient in
 // the high 64 - h_bits bits (signed), hessian in the low h_bits bits. The fields must hold the sum of the
-// min(rows of the item, kHistFlushRows) rows added between two drains of the LDS bins into 64-bit registers, so an
-// item coarsens the tree's scales by its own power of two (shift): the fewer rows an item has, the finer it counts;
+// rows added between two drains of the LDS bins into 64-bit registers, at most min(rows of the node,
+// kHistFlushRows), so the items of a node coarsen the tree's scales by a power of two (shift) that depends on the
+// node's row count only: the fewer rows a node has, the finer it counts, and what a row adds to a node does not
+// depend on the order of the rows;
 // k_hist_merge shifts every item's sums back to the tree's scale. h_bits: 32 in general; when every hessian of the
 // tree is a small non-negative integer (squared loss: 1, or the draw count under bagging) the hessian field gets
 // exactly the bits that kHistFlushRows * max h needs and the gradient field the rest (50 bits for h = 1), which
@@ -119,7 +121,11 @@ struct TreeBuffers {
                                                 // of the nodes of a level, ping-pong by level parity
     longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
     QuantCtl *quant = nullptr;     // scales of the current tree
-    int2 *hitem_shift = nullptr;   // [max_hitems] powers of two by which a dense work item coarsened (g, h)
+    int2 *hitem_shift = nullptr;   // [max_hitems] powers of two by which a dense work item (its node) coarsened (g, h)
+    // Root sums as exact integers at the tree's scales (what a row order cannot change): [0], [1] the sums,
+    // [2] a ticket counter of the kernel that adds them up (all zeroed by k_tree_init)
+    long long *root_total = nullptr;
+    int complete_feature = -1;     // dense layout: a feature stored in every row (its bins add up to the root), or -1
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
     float *leaf_value = nullptr;   // [n_nodes] prediction increment of a row that ended in the node (after pruning)
     int *end_bound = nullptr;      // [(row_blocks(n) + 1) x (2^depth - 1)] list positions of the row block boundaries
@@ -174,6 +180,7 @@ struct TreeBuffers {
         t.partial += K * n_partial;
         t.quant += K;
         t.hitem_shift += K * max_hitems;
+        t.root_total += K * 4;
         t.leaf_value += K * n_nodes;
         t.end_bound += K * n_end_bound;
         t.hpair_begin += K * (max_level_nodes + 1);
@@ -207,6 +214,11 @@ void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_cla
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level,
                        int n_class = 1);
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class = 1);
+// After the root histogram exists: replaces the root's float sums (whose last bits depend on the order of the rows)
+// by the exact fixed-point totals, from the bins of tb.complete_feature or, without one, from the gradients.
+void launch_root_sum(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, int n_class = 1);
+// Number of bytes equal to `value` among n bytes in device memory (synchronises).
+long device_count_bytes(hipStream_t s, const uint8_t *d_v, size_t n, uint8_t value);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
                      int n_class = 1);
 void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);

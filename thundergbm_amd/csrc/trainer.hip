@@ -344,6 +344,16 @@ void Trainer::alloc_tree_buffers() {
     tb.partial = dalloc<longlong2>(S * tb.n_partial);
     tb.quant = dalloc<QuantCtl>(S);
     tb.hitem_shift = dalloc<int2>(S * (size_t)tb.max_hitems);
+    tb.root_total = dalloc<long long>(S * 4);
+    // a feature that is stored in every row (checked on the bin matrix itself: a row with a repeated column index
+    // would make the stored-value count lie): its bins add up to the root's sums
+    tb.complete_feature = -1;
+    if (!sparse_) {
+        for (int f = 0; f < F_ && tb.complete_feature < 0; ++f)
+            if (cuts_.feature_nnz[f] == (long)n_ &&
+                device_count_bytes(stream_, bins_.col + (size_t)f * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
+                tb.complete_feature = f;
+    }
     tb.hpair_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
     tb.leaf_value = dalloc<float>(S * tb.n_nodes);
     tb.end_bound = dalloc<int>(S * tb.n_end_bound);
@@ -525,6 +535,7 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
         build_level_hist(tb, level, gh, n_class);
     }
     if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
+    if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
     // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them)
     launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
                       !(in_boost_ && level == param_.depth - 1));

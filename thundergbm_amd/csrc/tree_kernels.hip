@@ -253,8 +253,8 @@ __device__ float pow2_scale(float vmax, int rows, float limit) {
     return ldexpf(1.f, e - 1);     // 2^(e-1) <= bound
 }
 
-// Power of two by which a dense work item that adds `rows` rows between two drains coarsens one of the tree's
-// scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
+// Power of two by which the dense work items of a node that add at most `rows` rows between two drains coarsen one
+// of the tree's scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
 // scale, bits: magnitude bits of the packed field).
 __device__ int item_shift(float qmax, int rows, int bits) {
     const double lim = ldexp(1.0, bits) / (double)rows * (1.0 - 1e-6) - 0.5;
@@ -381,6 +381,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         q.gq_max = gm * q.scale_g;
         q.hq_max = hm * q.scale_h;
         *tb.quant = q;
+        tb.root_total[0] = tb.root_total[1] = tb.root_total[2] = 0;
     }
 }
 
@@ -389,10 +390,10 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
 // histogram lives in LDS as one 64-bit integer per bin holding the fixed-point gradient sum in the
 // high and the hessian sum in the low field (QuantCtl::h_bits wide); a row contributes with a single
 // ds_add_u64 per feature (float LDS atomics run at ~0.3 lanes/clk/CU on gfx950, 64-bit integer ones at ~5).
-// The fields are safe for the rows added between two drains (at most kHistFlushRows; fewer for a short item,
-// which therefore counts finer: item_shift), so after at most that many rows every thread drains the bins it
-// owns into 64-bit register accumulators and clears them; at the end the registers go to the item's slot of
-// `partial`, at the item's scale (k_hist_merge shifts them to the tree's).
+// The fields are safe for the rows added between two drains (at most kHistFlushRows; fewer in a node with fewer
+// rows, whose items therefore count finer: item_shift), so after at most that many rows every thread drains the
+// bins it owns into 64-bit register accumulators and clears them; at the end the registers go to the item's slot
+// of `partial`, at the item's scale (k_hist_merge shifts them to the tree's).
 // LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
 // instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
 // (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
@@ -430,7 +431,9 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         int e = min(sg.y, b + c.hchunk);
         s_range[0] = b;
         s_range[1] = e;
-        const int rows = max(1, min(e - b, kHistFlushRows));
+        // (the node's rows, not the item's: what a row adds must not depend on the item it falls into, or the sums
+        // would change with the order of the rows)
+        const int rows = max(1, min(sg.y - sg.x, kHistFlushRows));
         const int2 shift = make_int2(item_shift(quant->gq_max, rows, 63 - h_bits),
                                      quant->h_integer ? 0 : item_shift(quant->hq_max, rows, h_bits));
         s_range[2] = shift.x;
@@ -599,6 +602,100 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
         const longlong2 par = prev_q[(size_t)p * n_bins + j];
         cur_q[(size_t)(sib - off) * n_bins + j] = make_longlong2(par.x - sg, par.y - sh);
     }
+}
+
+// ------------------------------------------------------------------------------ exact root sums
+// k_tree_init sets the root's sums from a float reduction over the rows, whose last bits depend on the physical
+// order of the rows; every later quantity of a tree (child sums, weights, gains, predictions, the next gradients)
+// derives from it. These kernels replace it by the exact fixed-point total - the same integers in any order - so
+// that a tree does not depend on the row order at all.
+__device__ __forceinline__ long long wave_sum_ll(long long v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const int lo = __shfl_xor((int)(unsigned)(unsigned long long)v, d);
+        const int hi = __shfl_xor((int)((unsigned long long)v >> 32), d);
+        v += (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+    }
+    return v;
+}
+
+__device__ void set_root_sums(const TreeBuffers &tb, long long G, long long H, float lambda) {
+    GHPair s{(float)((double)G * (double)tb.quant->inv_g), (float)((double)H * (double)tb.quant->inv_h)};
+    TreeNode &root = tb.nodes[0];
+    root.sum_gh_pair = s;
+    root.base_weight = -s.g / (s.h + lambda);
+}
+
+// From the root histogram: the bins of a feature that is stored in every row add up to the root. One workgroup.
+__global__ __launch_bounds__(kBlock) void k_root_sum_bins(TreeBuffers tb_all, float lambda) {
+    __shared__ long long s_g[kWaves], s_h[kWaves];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const longlong2 *__restrict__ h = tb.hist(0);
+    const int b0 = tb.cut_row_ptr[tb.complete_feature], b1 = tb.cut_row_ptr[tb.complete_feature + 1];
+    long long g = 0, hh = 0;
+    for (int b = b0 + threadIdx.x; b < b1; b += kBlock) {
+        const longlong2 v = h[b];
+        g += v.x;
+        hh += v.y;
+    }
+    g = wave_sum_ll(g);
+    hh = wave_sum_ll(hh);
+    if (lane_id() == 0) {
+        s_g[wave_id()] = g;
+        s_h[wave_id()] = hh;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < kWaves; ++i) {
+            g += s_g[i];
+            hh += s_h[i];
+        }
+        set_root_sums(tb, g, hh, lambda);
+    }
+}
+
+// From the gradients (no feature is stored in every row): every row's pair rounded at the tree's scales, block sums
+// added to two 64-bit counters; the last workgroup to arrive applies the totals.
+__global__ __launch_bounds__(kBlock) void k_root_sum_rows(TreeBuffers tb_all, const GHPair *__restrict__ gh, float lambda) {
+    __shared__ long long s_g[kWaves], s_h[kWaves];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    gh += (size_t)blockIdx.z * tb.n;
+    const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
+    long long g = 0, hh = 0;
+    for (int i = blockIdx.x * kBlock + threadIdx.x; i < tb.n; i += gridDim.x * kBlock) {
+        const GHPair v = gh[i];
+        g += __float2ll_rn(v.g * scale_g);
+        hh += __float2ll_rn(fmaxf(v.h, 0.f) * scale_h);
+    }
+    g = wave_sum_ll(g);
+    hh = wave_sum_ll(hh);
+    if (lane_id() == 0) {
+        s_g[wave_id()] = g;
+        s_h[wave_id()] = hh;
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    for (int i = 1; i < kWaves; ++i) {
+        g += s_g[i];
+        hh += s_h[i];
+    }
+    unsigned long long *tot = reinterpret_cast<unsigned long long *>(tb.root_total);
+    atomicAdd(tot, (unsigned long long)g);
+    atomicAdd(tot + 1, (unsigned long long)hh);
+    __threadfence();
+    if (atomicAdd(tot + 2, 1ull) == (unsigned long long)gridDim.x - 1ull) {
+        __threadfence();
+        const long long G = (long long)atomicAdd(tot, 0ull), H = (long long)atomicAdd(tot + 1, 0ull);
+        set_root_sums(tb, G, H, lambda);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_count_bytes(const uint8_t *__restrict__ v, size_t n, uint8_t value,
+                                                       unsigned long long *__restrict__ out) {
+    unsigned long long c = 0;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) c += v[i] == value;
+    c = (unsigned long long)wave_sum_ll((long long)c);
+    if (lane_id() == 0 && c) atomicAdd(out, c);
 }
 
 __device__ __forceinline__ long long shfl_up_ll(long long v, int d) {
@@ -1886,6 +1983,25 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_cl
         dim3 grid((tb.n_bins + 31) / 32, n_pairs, n_class);
         k_hist_merge<32><<<grid, kBlock, 0, s>>>(tb, level);
     }
+}
+
+void launch_root_sum(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, int n_class) {
+    if (tb.complete_feature >= 0) {
+        k_root_sum_bins<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, lambda);
+    } else {
+        k_root_sum_rows<<<dim3(grid_for((size_t)tb.n, 1024), 1, n_class), kBlock, 0, s>>>(tb, gh_class, lambda);
+    }
+}
+
+long device_count_bytes(hipStream_t s, const uint8_t *d_v, size_t n, uint8_t value) {
+    unsigned long long *d_out = nullptr, h = 0;
+    HIP_CHECK(hipMalloc(&d_out, sizeof(unsigned long long)));
+    HIP_CHECK(hipMemsetAsync(d_out, 0, sizeof(unsigned long long), s));
+    k_count_bytes<<<grid_for(n, 2048), kBlock, 0, s>>>(d_v, n, value, d_out);
+    HIP_CHECK(hipMemcpyAsync(&h, d_out, sizeof(h), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipFree(d_out));
+    return (long)h;
 }
 
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
