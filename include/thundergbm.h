@@ -165,6 +165,20 @@ tgbm_model *tgbm_trainer_export_model(tgbm_trainer *t);
 void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const int *col_ptr, tgbm_model *model,
                       int n_trees, int trees_per_iter, float learning_rate, float base_score, float *out);
 
+/* tgbm_predict_raw for callers that cannot allocate (tight serving loops, harnesses that forbid hipMalloc, code that
+ * records the call's device work into a HIP graph). It has no counterpart in the reference. Same arguments, same
+ * scores bit for bit, but no hipMalloc / hipFree / stream creation: the device copies of the rows, the model and
+ * the scores live in a file-scope device array of about 34 MiB that every GPU used by the library holds until the
+ * process ends (its address is resolved on the first call on a device). Limits per call: row_size <= 65536,
+ * stored values <= 2^20, row_size * trees_per_iter <= 2^19, nodes of the trees used <= 2^19 (e.g. 800 trees of
+ * depth 8). Returns 0, or 1 with a message on stderr when a limit is exceeded (nothing is computed then). Calls
+ * share the device's array, which keeps the last call's contents; they are serialised inside one process, and
+ * calls from several processes on one GPU do not interfere (every process has its own copy). The work runs on
+ * the default stream and the call returns after the scores were copied to `out`. */
+int tgbm_predict_raw_noalloc(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
+                             tgbm_model *model, int n_trees, int trees_per_iter, float learning_rate,
+                             float base_score, float *out);
+
 /* Cut points and global bin ids of a CSR matrix (HistCut::get_cut_points_single, hist_cut.cu:232-286;
  * get_bin_ids, hist_tree_builder_single.cu:49-130), computed on the GPU. cut_val / cut_fid need one
  * slot per stored value at most (row_ptr[row_size]); returns the number of cut points. */

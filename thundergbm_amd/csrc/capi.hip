@@ -5,13 +5,10 @@
 #include <mutex>
 
 #include "../../include/thundergbm.h"
+#include "model_handle.h"
 #include "trainer.h"
 
 using namespace tgbm;
-
-struct tgbm_model {
-    std::vector<Tree> trees;  // iteration-major, class inside
-};
 
 struct tgbm_trainer {
     std::unique_ptr<Trainer> impl;
