@@ -1,10 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the boosting loop on one MI355X.
 
-A step is one boosting iteration (gradients, one depth-8 tree, prediction update, training metric)
-on the 10M x 28 dense binary-logistic configuration with 255 bins; data, cut points and the bin matrix
-are resident in HBM before the timed region starts (the reference's "training time" span,
-src/thundergbm/trainer.cu:42-50, also excludes them). Prints one JSON line.
+A step is one boosting iteration (gradients, the trees of the round, prediction update, training metric);
+data, cut points and the bin matrix are resident in HBM before the timed region starts (the reference's
+"training time" span, src/thundergbm/trainer.cu:42-50, also excludes them). The K timed steps are one
+boosting call of K rounds, as in a training run, bracketed by device synchronisations. Prints one JSON line.
+
+The default workload is benchmark configuration 2 (10M x 28 dense, binary:logistic, depth 8, 255 bins), the one
+the headline metric is quoted on; --config 3, 4, 5 time the other full-size configurations the same way.
 """
 import argparse
 import json
@@ -18,18 +21,69 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 import numpy as np  # noqa: E402
 
+# objective, depth, bins, learning rate, trees of the configuration, histogram kernel
+CONFIGS = {
+    2: dict(objective="binary:logistic", depth=8, max_num_bin=255, learning_rate=0.1, n_trees=100,
+            kernel="k_hist_dense", name="config 2: %d rows x %d dense features, binary:logistic, depth %d, 255 bins"),
+    3: dict(objective="reg:linear", depth=6, max_num_bin=255, learning_rate=0.1, n_trees=50,
+            kernel="k_hist_dense", name="config 3: %d rows x %d dense features (5%% heavy-tailed), reg:linear, depth %d, 255 bins"),
+    4: dict(objective="binary:logistic", depth=8, max_num_bin=63, learning_rate=0.1, n_trees=100,
+            kernel="sparse histogram kernels", name="config 4: %d rows x %d features CSR (~40 per row, Zipf), binary:logistic, depth %d, 63 bins"),
+    5: dict(objective="multi:softmax", depth=8, max_num_bin=255, learning_rate=0.1, n_trees=100,
+            kernel="k_hist_dense", name="config 5: %d rows x %d features, 8-class softmax (8 trees per step), depth %d, 255 bins"),
+}
 
-def measured_traffic_per_launch():
-    """HBM bytes per k_hist_dense launch from the committed rocprofv3 --pmc summary (FETCH_SIZE and
-    WRITE_SIZE runs, calibrated against a plain copy kernel); None when the summary is absent."""
-    path = os.path.join(ROOT, "profiles", "k_hist_dense_config2_pmc.txt")
+
+KERNEL_SOURCES = ["thundergbm_amd/csrc/tree_kernels.hip", "thundergbm_amd/csrc/trainer.hip",
+                  "thundergbm_amd/csrc/device_api.h"]
+
+
+def kernel_sources_sha1():
+    """Fingerprint of the histogram kernels' sources; the counter summaries under profiles/ carry the one they
+    were measured with."""
+    import hashlib
+    h = hashlib.sha1()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def traffic_from_profile(config):
+    """HBM bytes per histogram launch from the committed rocprofv3 --pmc summary of this configuration (FETCH_SIZE
+    and WRITE_SIZE runs, calibrated against a plain copy kernel), with where it comes from. The figure is only
+    passed on when the summary was measured with the kernel sources as they are now; else it would be stale."""
+    rel = os.path.join("profiles", "k_hist_dense_config%d_pmc.txt" % config)
+    value = sha = None
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             if line.startswith("traffic_bytes_per_launch:"):
-                return float(line.split(":")[1])
+                value = float(line.split(":")[1])
+            if line.startswith("kernel_sources_sha1:"):
+                sha = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, None
+    if value is None:
+        return None, None
+    if sha != kernel_sources_sha1():
+        return None, "%s was measured with other kernel sources (%s): not used" % (rel, sha)
+    return value, "%s (kernel sources %s)" % (rel, sha[:12])
+
+
+def make_data(config, rows):
+    import datasets as D
+    if config == 2:
+        X, y = D.config2(rows or 10_000_000, seed=1)
+    elif config == 3:
+        X, y = D.config3(rows or 500_000, 2000, seed=2)
+    elif config == 5:
+        X, y = D.config5(rows or 1_000_000, seed=4)
+    else:
+        val, rp, col, y = D.config4(rows or 2_000_000, 100_000, 40, seed=3)
+        return val, rp, col, y, len(rp) - 1, 100_000
+    n, F = X.shape
+    val, rp, col = D.dense_to_csr(X)
+    return val, rp, col, y, n, F
 
 
 def main():
@@ -37,13 +91,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--rows", type=int, default=10_000_000)
-    ap.add_argument("--depth", type=int, default=8)
+    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
+    ap.add_argument("--rows", type=int, default=0, help="rows of the synthetic matrix (0 = the configuration's own)")
+    ap.add_argument("--depth", type=int, default=0, help="tree depth (0 = the configuration's own)")
     ap.add_argument("--profile-steps", type=int, default=5)
     ap.add_argument("--cpu-steps", type=int, default=2, help="boosting iterations of the CPU baseline (0 = skip)")
+    ap.add_argument("--full-run", type=int, default=1,
+                    help="config 2: also time one training call of all the configuration's trees (0 = skip)")
     ap.add_argument("--calibration-copy-mb", type=int, default=0,
                     help="also run 3 launches of a plain copy kernel of this many MiB (profiler counter calibration)")
-    ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU baseline sample (0 = all rows)")
+    ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU baseline sample (0 = a default per config)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build trains on one GPU; --gpus %d is not supported (no multi-GPU path exists)"
@@ -51,28 +108,26 @@ def main():
         sys.exit(2)
 
     import torch  # device synchronisation only; the library manages its own HBM buffers
-    import datasets as D
     import thundergbm_amd as T
 
     assert torch.cuda.is_available(), "no GPU visible"
     T.load()
+    cfg = CONFIGS[args.config]
+    depth = args.depth or cfg["depth"]
     t0 = time.perf_counter()
-    X, y = D.config2(args.rows, seed=1)
-    val, rp, col = D.dense_to_csr(X)
-    n, F = X.shape
-    del X
+    val, rp, col, y, n, F = make_data(args.config, args.rows)
     t_gen = time.perf_counter() - t0
+    kw = dict(depth=depth, objective=cfg["objective"], learning_rate=cfg["learning_rate"],
+              max_num_bin=cfg["max_num_bin"], verbose=0)
     total_rounds = args.warmup + args.steps + args.profile_steps
     t0 = time.perf_counter()
-    s = T.Session(val, rp, col, y, depth=args.depth, n_trees=total_rounds, objective="binary:logistic",
-                  learning_rate=0.1, max_num_bin=255, verbose=0)
+    s = T.Session(val, rp, col, y, n_trees=total_rounds, **kw)
     t_prep = time.perf_counter() - t0
-    for _ in range(args.warmup):
-        s.boost(1)
+    if args.warmup:
+        s.boost(args.warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        s.boost(1)  # returns after the GPU finished the iteration
+    s.boost(args.steps)  # K rounds enqueued back to back; returns after the GPU finished the last one
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
@@ -81,52 +136,68 @@ def main():
     roofline = None
     if args.profile_steps > 0:
         s.set_profiling(True)
-        for _ in range(args.profile_steps):
-            s.boost(1)
+        s.boost(args.profile_steps)
         prof = s.profile()
         s.set_profiling(False)
         if prof["launches"] > 0 and prof["hist_ms"] > 0:
             achieved = prof["bytes"] / (prof["hist_ms"] * 1e-3) / 1e9
-            roofline = {"bound": "hbm", "kernel": "k_hist_dense", "achieved": round(achieved, 2), "peak": 8000.0,
+            full_size = args.rows == 0 and args.depth == 0
+            traffic, source = traffic_from_profile(args.config) if full_size else (None, None)
+            roofline = {"bound": "hbm", "kernel": cfg["kernel"], "achieved": round(achieved, 2), "peak": 8000.0,
                         "unit": "GB/s", "frac": round(achieved / 8000.0, 4),
-                        "traffic": measured_traffic_per_launch() if args.rows == 10_000_000 else None,
+                        "traffic": traffic, "traffic_source": source,
                         "bytes_per_launch": round(prof["bytes"] / prof["launches"], 1),
                         "avg_launch_us": round(prof["hist_ms"] * 1e3 / prof["launches"], 2),
-                        "hist_ms_per_tree": round(prof["hist_ms"] / args.profile_steps, 4),
-                        "rows_built_per_tree": prof["rows_built"] // args.profile_steps}
+                        "hist_ms_per_step": round(prof["hist_ms"] / args.profile_steps, 4),
+                        "rows_built_per_step": prof["rows_built"] // args.profile_steps}
     metric_log = s.metric_log()
+    reorders = s.info("reorders_done")
     s.close()
+
+    aux = {"data_gen_s": round(t_gen, 2), "prep_s_upload_cuts_bins": round(t_prep, 3),
+           "train_metric_last": float(metric_log[-1]) if len(metric_log) else None,
+           "row_reorderings_before_or_inside_the_timed_steps": reorders}
+    if args.config == 2 and args.full_run and args.rows == 0:
+        # the whole configuration as one training call: every row re-ordering pass is inside the timed span
+        s = T.Session(val, rp, col, y, n_trees=cfg["n_trees"], **kw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        s.boost(cfg["n_trees"])
+        torch.cuda.synchronize()
+        t_full = time.perf_counter() - t0
+        aux["iters_per_s_100_trees"] = round(cfg["n_trees"] / t_full, 2)
+        aux["reorderings_in_100_trees"] = s.info("reorders_done")
+        s.close()
     if args.calibration_copy_mb > 0:
         T.load().tgbm_calibration_copy(args.calibration_copy_mb << 20, 3)
 
     cpu = None
     if args.cpu_steps > 0:
         import oracle_lib as O
-        m = args.cpu_rows if args.cpu_rows > 0 else n
+        default_rows = {2: n, 3: 25_000, 4: 200_000, 5: 200_000}[args.config]
+        m = min(n, args.cpu_rows if args.cpu_rows > 0 else default_rows)
         crp = rp[: m + 1]
         nnz = int(crp[-1])
-        o = O.Oracle(val[:nnz], crp, col[:nnz], y[:m], depth=args.depth, n_trees=args.cpu_steps,
-                     objective="binary:logistic", learning_rate=0.1, max_num_bin=255).prepare()
+        o = O.Oracle(val[:nnz], crp, col[:nnz], y[:m], depth=depth, n_trees=args.cpu_steps, objective=cfg["objective"],
+                     learning_rate=cfg["learning_rate"], max_num_bin=cfg["max_num_bin"]).prepare()
         t0 = time.perf_counter()
         o.boost(args.cpu_steps)
         cdt = time.perf_counter() - t0
         cpu_value = args.cpu_steps / cdt * (m / n)  # iterations/s scaled to the full row count
         cpu = {"value": round(cpu_value, 4), "unit": "boosting iters/s", "cores": O.lib().orc_num_threads(),
                "kind": "port",
-               "sample": "%d boosting iterations of the OpenMP oracle on %d of %d rows (linear in rows), "
-                         "boost loop only" % (args.cpu_steps, m, n)}
+               "sample": "%d boosting iterations of the OpenMP oracle on the first %d of %d rows (scaled linearly "
+                         "in rows), boost loop only" % (args.cpu_steps, m, n)}
 
     out = {
-        "metric": "boosting iters/sec (depth 8, 255 bins, 1 GPU)", "value": round(value, 3),
+        "metric": "boosting iters/sec (depth %d, %d bins, 1 GPU)" % (depth, cfg["max_num_bin"]), "value": round(value, 3),
         "unit": "boosting iters/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config 2: %d rows x %d dense features, binary:logistic, depth %d, 255 bins"
-                               % (n, F, args.depth),
-                   "rows": n, "features": F, "depth": args.depth, "max_num_bin": 255, "learning_rate": 0.1},
-        "roofline": roofline, "cpu_baseline": cpu,
-        "aux": {"data_gen_s": round(t_gen, 2), "prep_s_upload_cuts_bins": round(t_prep, 3),
-                "train_error_last": float(metric_log[-1]) if len(metric_log) else None},
+        "config": {"workload": cfg["name"] % (n, F, depth), "rows": n, "features": F, "depth": depth,
+                   "max_num_bin": cfg["max_num_bin"], "learning_rate": cfg["learning_rate"],
+                   "objective": cfg["objective"]},
+        "roofline": roofline, "cpu_baseline": cpu, "aux": aux,
     }
     print(json.dumps(out))
 
