@@ -131,7 +131,7 @@ struct TreeBuffers {
     int *end_bound = nullptr;      // [(row_blocks(n) + 1) x (2^depth - 1)] list positions of the row block boundaries
     int *hpair_begin = nullptr;    // [max_pairs + 1] first histogram item of every sibling pair
     int *hpair_built = nullptr;    // [max_pairs] heap id of the node built from rows, -1 = inactive pair
-    int *pitem_begin = nullptr;    // [max_level_nodes + 1]
+    int *pitem_begin = nullptr;    // [2][max_level_nodes + 1] first partition item of every node of a level, by level parity
     int *pitem_nleft = nullptr;    // [max_pitems]
     int *pitem_loff = nullptr;     // [max_pitems]
     int *node_nleft = nullptr;     // [max_level_nodes]
@@ -163,6 +163,7 @@ struct TreeBuffers {
     // kernel's local copy of this struct would otherwise be placed in scratch memory).
     __host__ __device__ int *list(int level) const { return (level & 1) ? ridx[1] : ridx[0]; }
     __host__ __device__ longlong2 *hist(int level) const { return (level & 1) ? hist_q[1] : hist_q[0]; }
+    __host__ __device__ int *pbegin(int level) const { return pitem_begin + (level & 1) * (max_level_nodes + 1); }
 
     // The buffers of set k (k = 0: this object itself).
     __host__ __device__ TreeBuffers for_class(int k) const {
@@ -185,7 +186,7 @@ struct TreeBuffers {
         t.end_bound += K * n_end_bound;
         t.hpair_begin += K * (max_level_nodes + 1);
         t.hpair_built += K * max_level_nodes;
-        t.pitem_begin += K * (max_level_nodes + 1);
+        t.pitem_begin += K * 2 * (max_level_nodes + 1);
         t.pitem_nleft += K * ((size_t)max_pitems + 1);
         t.pitem_loff += K * ((size_t)max_pitems + 1);
         t.node_nleft += K * max_level_nodes;

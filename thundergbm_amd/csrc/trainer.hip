@@ -358,7 +358,7 @@ void Trainer::alloc_tree_buffers() {
     tb.leaf_value = dalloc<float>(S * tb.n_nodes);
     tb.end_bound = dalloc<int>(S * tb.n_end_bound);
     tb.hpair_built = dalloc<int>(S * max_level_nodes);
-    tb.pitem_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
+    tb.pitem_begin = dalloc<int>(S * 2 * ((size_t)max_level_nodes + 1));
     tb.pitem_nleft = dalloc<int>(S * ((size_t)tb.max_pitems + 1));
     tb.pitem_loff = dalloc<int>(S * ((size_t)tb.max_pitems + 1));
     tb.node_nleft = dalloc<int>(S * max_level_nodes);

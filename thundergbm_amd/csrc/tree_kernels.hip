@@ -62,6 +62,10 @@ __device__ __forceinline__ float wave_sum_f(float v) {
     return v;
 }
 
+__device__ __forceinline__ bool node_splits(const TreeNode &nd) {
+    return nd.is_valid && !nd.is_leaf && nd.split_feature_id >= 0;
+}
+
 // Largest p in [0, n) with begin[p] <= item (begin is non-decreasing, begin[0] <= item < begin[n]).
 __device__ int find_owner(const int *begin, int n, int item) {
     int lo = 0, hi = n;
@@ -357,9 +361,11 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         LevelCtl c;
         c.hchunk = chunk;
         c.n_hitems = items;
-        c.n_pitems = 0;
+        c.n_pitems = (tb.n + kPartChunk - 1) / kPartChunk;  // the root's partition items (used if it splits)
         c.rows_built = tb.n;
         tb.ctl[0] = c;
+        tb.pbegin(0)[0] = 0;
+        tb.pbegin(0)[1] = c.n_pitems;
         tb.ctl[tb.depth] = LevelCtl{0, 0, 0, 0};  // the last level plans no further one
         // The tree's scales keep the 64-bit sums over all n rows below 2^62; a dense work item coarsens them by its
         // own power of two so that its packed LDS fields hold the rows between two drains (item_shifts).
@@ -911,12 +917,16 @@ __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, C
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
-    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    if (threadIdx.x == 0) s_x = find_owner(tb.pbegin(level), nl, item);
     __syncthreads();
     const int x_in = s_x;
     const TreeNode &nd = tb.nodes[off + x_in];
+    if (!node_splits(nd)) {
+        if (threadIdx.x == 0) tb.pitem_nleft[item] = 0;
+        return;
+    }
     const int2 sg = tb.seg[off + x_in];
-    const int pb = sg.x + (item - tb.pitem_begin[x_in]) * kPartChunk;
+    const int pb = sg.x + (item - tb.pbegin(level)[x_in]) * kPartChunk;
     const int pe = min(sg.y, pb + kPartChunk);
     const int f = nd.split_feature_id;
     const int cb = tb.cut_row_ptr[f], ce = tb.cut_row_ptr[f + 1];
@@ -1241,35 +1251,10 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
 }
 
 // ------------------------------------------------------------------------------ partition
-__device__ __forceinline__ bool node_splits(const TreeNode &nd) {
-    return nd.is_valid && !nd.is_leaf && nd.split_feature_id >= 0;
-}
 
-// Partition work items: every node of the level that was split gets ceil(rows / kPartChunk) items.
-__global__ __launch_bounds__(kBlock) void k_part_plan(TreeBuffers tb_all, int level) {
-    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
-    __shared__ int lds[kWaves];
-    const int nl = 1 << level, off = nl - 1;
-    int carry = 0;
-    for (int base = 0; base < nl; base += kBlock) {
-        int x_in = base + threadIdx.x;
-        int cnt = 0;
-        if (x_in < nl) {
-            const TreeNode &nd = tb.nodes[off + x_in];
-            int2 sg = tb.seg[off + x_in];
-            if (node_splits(nd)) cnt = (sg.y - sg.x + kPartChunk - 1) / kPartChunk;
-        }
-        int tot;
-        int ex = block_excl_scan(cnt, lds, &tot);
-        if (x_in < nl) tb.pitem_begin[x_in] = carry + ex;
-        carry += tot;
-    }
-    if (threadIdx.x == 0) {
-        tb.pitem_begin[nl] = carry;
-        tb.ctl[level].n_pitems = carry;
-    }
-}
-
+// Partition work items: every node of a level that holds rows owns ceil(rows / kPartChunk) items, planned one level
+// ahead (k_tree_init for the root, k_part_scan_plan for the children it creates) so that no planning step sits
+// between the split search and the partition; the items of a node that did not split return at once.
 // Decide left/right for every row of a work item from the split feature's column of the bin matrix
 // (missing -> default direction, else right iff bin >= split bin; the reference's rule at
 // hist_tree_builder_single.cu:986-1011) and count the rows that go left.
@@ -1282,12 +1267,16 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
-    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    if (threadIdx.x == 0) s_x = find_owner(tb.pbegin(level), nl, item);
     __syncthreads();
     const int x_in = s_x;
     const TreeNode &nd = tb.nodes[off + x_in];
+    if (!node_splits(nd)) {
+        if (threadIdx.x == 0) tb.pitem_nleft[item] = 0;
+        return;
+    }
     const int2 sg = tb.seg[off + x_in];
-    const int pb = sg.x + (item - tb.pitem_begin[x_in]) * kPartChunk;
+    const int pb = sg.x + (item - tb.pbegin(level)[x_in]) * kPartChunk;
     const int pe = min(sg.y, pb + kPartChunk);
     const int f = nd.split_feature_id;
     const int sbid = nd.split_bid;
@@ -1325,6 +1314,8 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
     __shared__ int lds[kWaves];
     const int nl = 1 << level, off = nl - 1;
     const int n_p = tb.ctl[level].n_pitems;
+    const int *pb_cur = tb.pbegin(level);
+    int *pb_next = tb.pbegin(level + 1);
     int carry = 0;
     constexpr int IPT = 20;  // items per thread and step (10 M rows are 4 883 items: one step)
     for (int base = 0; base < n_p; base += kBlock * IPT) {
@@ -1351,17 +1342,20 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         // the usual case (levels up to 8): one node per thread, everything after the scan stays in registers
         const int x_in = threadIdx.x;
         int built = -1, rows = 0;
+        int pl = 0, pr = 0;  // partition items of the two children
         if (x_in < nl) {
             const TreeNode &nd = tb.nodes[off + x_in];
             const int2 sg = tb.seg[off + x_in];
             if (node_splits(nd)) {
-                const int nleft = tb.pitem_loff[tb.pitem_begin[x_in + 1]] - tb.pitem_loff[tb.pitem_begin[x_in]];
+                const int nleft = tb.pitem_loff[pb_cur[x_in + 1]] - tb.pitem_loff[pb_cur[x_in]];
                 const int nright = (sg.y - sg.x) - nleft;
                 tb.node_nleft[x_in] = nleft;
                 tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
                 tb.seg[nd.rch_index] = make_int2(sg.x + nleft, sg.y);
                 built = (nleft <= nright) ? nd.lch_index : nd.rch_index;
                 rows = min(nleft, nright);
+                pl = (nleft + kPartChunk - 1) / kPartChunk;
+                pr = (nright + kPartChunk - 1) / kPartChunk;
             } else {
                 tb.node_nleft[x_in] = 0;
                 tb.seg[nd.lch_index] = make_int2(0, 0);
@@ -1375,15 +1369,21 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         int chunk = (total_rows + room - 1) / room;
         chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
         const int cnt = built >= 0 ? (rows + chunk - 1) / chunk : 0;
-        int tot;
+        int tot, ptot;
         const int ex = block_excl_scan(cnt, lds, &tot);
-        if (x_in < nl) tb.hpair_begin[x_in] = ex;
+        const int pex = block_excl_scan(pl + pr, lds, &ptot);
+        if (x_in < nl) {
+            tb.hpair_begin[x_in] = ex;
+            pb_next[2 * x_in] = pex;
+            pb_next[2 * x_in + 1] = pex + pl;
+        }
         if (threadIdx.x == 0) {
             tb.hpair_begin[nl] = tot;
+            pb_next[2 * nl] = ptot;
             LevelCtl c;
             c.hchunk = chunk;
             c.n_hitems = tot;
-            c.n_pitems = 0;
+            c.n_pitems = ptot;
             c.rows_built = total_rows;
             tb.ctl[level + 1] = c;
         }
@@ -1396,7 +1396,7 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         const int2 sg = tb.seg[off + x_in];
         int built = -1;
         if (node_splits(nd)) {
-            int nleft = tb.pitem_loff[tb.pitem_begin[x_in + 1]] - tb.pitem_loff[tb.pitem_begin[x_in]];
+            int nleft = tb.pitem_loff[pb_cur[x_in + 1]] - tb.pitem_loff[pb_cur[x_in]];
             int nright = (sg.y - sg.x) - nleft;
             tb.node_nleft[x_in] = nleft;
             tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
@@ -1435,12 +1435,32 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         if (x_in < nl) tb.hpair_begin[x_in] = carry + ex;
         carry += tot;
     }
+    // partition items of the next level: every child that received rows
+    int pcarry = 0;
+    for (int base = 0; base < nl; base += kBlock) {
+        const int x_in = base + threadIdx.x;
+        int pl = 0, pr = 0;
+        if (x_in < nl) {
+            const TreeNode &nd = tb.nodes[off + x_in];
+            const int2 sl = tb.seg[nd.lch_index], sr = tb.seg[nd.rch_index];
+            pl = (sl.y - sl.x + kPartChunk - 1) / kPartChunk;
+            pr = (sr.y - sr.x + kPartChunk - 1) / kPartChunk;
+        }
+        int ptot;
+        const int pex = block_excl_scan(pl + pr, lds, &ptot);
+        if (x_in < nl) {
+            pb_next[2 * x_in] = pcarry + pex;
+            pb_next[2 * x_in + 1] = pcarry + pex + pl;
+        }
+        pcarry += ptot;
+    }
     if (threadIdx.x == 0) {
         tb.hpair_begin[nl] = carry;
+        pb_next[2 * nl] = pcarry;
         LevelCtl c;
         c.hchunk = chunk;
         c.n_hitems = carry;
-        c.n_pitems = 0;
+        c.n_pitems = pcarry;
         c.rows_built = total_rows;
         tb.ctl[level + 1] = c;
     }
@@ -1461,11 +1481,12 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int
     const int item = blockIdx.x;
     if (item >= tb.ctl[level].n_pitems) return;
     const int nl = 1 << level, off = nl - 1;
-    if (threadIdx.x == 0) s_x = find_owner(tb.pitem_begin, nl, item);
+    if (threadIdx.x == 0) s_x = find_owner(tb.pbegin(level), nl, item);
     __syncthreads();
     const int x_in = s_x;
+    if (!node_splits(tb.nodes[off + x_in])) return;
     const int2 sg = tb.seg[off + x_in];
-    const int first_item = tb.pitem_begin[x_in];
+    const int first_item = tb.pbegin(level)[x_in];
     const int pb = sg.x + (item - first_item) * kPartChunk;
     const int pe = min(sg.y, pb + kPartChunk);
     const int loff = tb.pitem_loff[item] - tb.pitem_loff[first_item];
@@ -2051,7 +2072,6 @@ void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float r
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class) {
     if (level == tb.depth - 1) return;  // the last level's children never get row lists (see k_tree_end)
     const dim3 one(1, 1, n_class), items(tb.max_pitems, 1, n_class);
-    k_part_plan<<<one, kBlock, 0, s>>>(tb, level);
     if (level == 0) {
         k_part_count_dense<true><<<items, kBlock, 0, s>>>(tb, bins, level);
         k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
@@ -2066,7 +2086,6 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
 void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class) {
     if (level == tb.depth - 1) return;
     const dim3 one(1, 1, n_class), items(tb.max_pitems, 1, n_class);
-    k_part_plan<<<one, kBlock, 0, s>>>(tb, level);
     if (level == 0) {
         k_part_count_csr<true><<<items, kBlock, 0, s>>>(tb, bins, level);
         k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
