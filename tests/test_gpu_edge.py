@@ -26,10 +26,10 @@ def T():
 
 @pytest.fixture(autouse=True)
 def _default_layout():
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS"):
         os.environ.pop(k, None)
     yield
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS"):
         os.environ.pop(k, None)
 
 
@@ -544,8 +544,10 @@ def test_training_is_bit_reproducible(T, layout):
 @pytest.mark.parametrize("head", ["1", "0"])
 @pytest.mark.parametrize("objective,kind", [("binary:logistic", "bin"), ("multi:softmax", "multi")])
 def test_sparse_root_histogram_from_either_copy(T, objective, kind, head):
-    """Sparse layout: the root histogram summed over the bin-major copy of the stored values and accumulated row
-    by row with atomics (TGBM_CSC_ROOT=0; with and without the LDS head) are the same integers: same bytes."""
+    """Sparse layout: the level pass over the bin-major copy (tables in LDS, no per-node histogram in HBM) and the
+    row-list kernels with per-node histograms (TGBM_SPARSE_PASS=0; root from the bin-major copy or row by row with
+    atomics, TGBM_CSC_ROOT; with and without the LDS head) sum the same integers: same root histogram, same model,
+    same predictions, byte for byte."""
     os.environ["TGBM_LAYOUT"] = "sparse"
     os.environ["TGBM_CSR_HEAD"] = head
     n, F = 30000, 300
@@ -555,20 +557,25 @@ def test_sparse_root_histogram_from_either_copy(T, objective, kind, head):
     if kind == "multi":
         kw["num_class"] = int(y.max()) + 1
     runs = []
-    for csc in ("1", "0"):
-        os.environ["TGBM_CSC_ROOT"] = csc
-        s = T.Session(val, rp, col, y, **kw)
-        s.gradient()
-        s.tree_init(0)
-        s.find_split(0)
-        root_hist = s.level_hist(0).tobytes()
-        s.close()
-        s = T.Session(val, rp, col, y, **kw)
-        s.boost(4)
-        runs.append((root_hist, s.model().tobytes(), s.y_pred().tobytes()))
-        s.close()
-    os.environ.pop("TGBM_CSC_ROOT")
-    assert runs[0] == runs[1]
+    try:
+        for level_pass, csc in (("1", "1"), ("0", "1"), ("0", "0")):
+            os.environ["TGBM_SPARSE_PASS"] = level_pass
+            os.environ["TGBM_CSC_ROOT"] = csc
+            s = T.Session(val, rp, col, y, **kw)
+            assert s.info("sparse_pass") == int(level_pass)
+            s.gradient()
+            s.tree_init(0)
+            s.find_split(0)
+            root_hist = s.level_hist(0).tobytes()
+            s.close()
+            s = T.Session(val, rp, col, y, **kw)
+            s.boost(4)
+            runs.append((root_hist, s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        os.environ.pop("TGBM_CSC_ROOT", None)
+        os.environ.pop("TGBM_SPARSE_PASS", None)
+    assert runs[0] == runs[1] == runs[2]
 
 
 def test_predict_transforms_through_the_c_abi(T):

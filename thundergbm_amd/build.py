@@ -8,7 +8,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libthundergbm.so")
 BIN_DIR = os.path.join(HERE, "bin")
 
-HIP_SOURCES = ["tree_kernels.hip", "prep_kernels.hip", "predict_kernels.hip", "rank_kernels.hip", "trainer.hip",
+HIP_SOURCES = ["tree_kernels.hip", "sparse_kernels.hip", "prep_kernels.hip", "predict_kernels.hip", "rank_kernels.hip", "trainer.hip",
                "predictor.hip", "capi.hip", "predict_noalloc.hip"]
 CPP_SOURCES = ["host_io.cpp"]
 

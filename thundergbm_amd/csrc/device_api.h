@@ -109,6 +109,37 @@ struct CsrBins {
     long nnz = 0;
 };
 
+// Sparse layout, level pass: one pass per level over the bin-major copy of the stored values (sorted by global bin,
+// rows ascending inside a bin). A task is a run of whole features, or a chunk of one feature that has too many
+// values for one workgroup ("big" feature); a task accumulates (node, bin) tables of its features in LDS and
+// searches them for every node's best candidate right there, so no per-node histogram exists in HBM.
+constexpr int kSparseCells = 8192;      // (node, bin) cells of 16 bytes an LDS table holds
+constexpr int kSparseMaxLevelNodes = 1024;  // deepest level the pass serves (depth <= 11)
+constexpr int kSparseBatchFeatures = 2047;  // features whose tables share one LDS batch at most
+constexpr int kSparseTaskValues = 32768;    // stored values per task (and per chunk of a big feature)
+struct SparseTask {
+    int f_begin, f_end;  // features [f_begin, f_end) (a chunk task: one feature)
+    int v_begin, v_end;  // positions of the bin-major copy
+    int cand_slot;       // candidate slot the task fills, -1: a chunk (its feature's slot is filled by k_sparse_big)
+    int partial_slot;    // chunk: where its table goes in SparsePass::partial, else -1
+};
+struct SparseBig {
+    int feature;
+    int slot_begin, slot_end;  // partial slots of its chunks
+    int cand_slot;
+};
+struct SparsePass {
+    const SparseTask *tasks = nullptr;
+    int n_tasks = 0;
+    const SparseBig *big = nullptr;
+    int n_big = 0;
+    const int *feat_val_begin = nullptr;  // [F + 1] first position of every feature in the bin-major copy
+    longlong2 *partial = nullptr;         // [n_sets][n_partial_slots][partial_stride] chunk tables, (bin, node) cells
+    size_t partial_stride = 0;            // cells per slot: most bins of a big feature x kSparseMaxLevelNodes at most
+    int n_partial_slots = 0;
+    int n_cand_slots = 0;
+};
+
 struct TreeBuffers {
     int n = 0, n_bins = 0, F = 0, depth = 0, n_nodes = 0;
     int sparse = 0;                // 1: CSR layout, histograms accumulated directly in hist_q
@@ -124,6 +155,9 @@ struct TreeBuffers {
     int2 *hitem_shift = nullptr;   // [max_hitems] powers of two by which a dense work item (its node) coarsened (g, h)
     // Root sums as exact integers at the tree's scales (what a row order cannot change): [0], [1] the sums,
     // [2] a ticket counter of the kernel that adds them up (all zeroed by k_tree_init)
+    // sparse level pass only (else nullptr): node every row has reached (heap id) and rows per node
+    unsigned short *nid16 = nullptr;  // [n + 2]
+    int *node_rows = nullptr;         // [n_nodes]
     long long *root_total = nullptr;
     int complete_feature = -1;     // dense layout: a feature stored in every row (its bins add up to the root), or -1
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
@@ -182,6 +216,10 @@ struct TreeBuffers {
         t.quant += K;
         t.hitem_shift += K * max_hitems;
         t.root_total += K * 4;
+        if (nid16 != nullptr) {
+            t.nid16 += K * (((size_t)n + 2) / 2 * 2);
+            t.node_rows += K * n_nodes;
+        }
         t.leaf_value += K * n_nodes;
         t.end_bound += K * n_end_bound;
         t.hpair_begin += K * (max_level_nodes + 1);
@@ -229,6 +267,12 @@ void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mc
                        bool store_sibling = true);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class = 1);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class = 1);
+// Sparse level pass (tb.nid16 set): split search of a level (candidates into tb.cand, one slot per task / big
+// feature; launch_best_update follows) and the row -> node update. dump_hist: also store the (node, bin) tables
+// into tb.hist(level) (stage-wise driving and tests; needs tb.hist_q).
+void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
+                         const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1);
+void launch_sparse_partition(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
 // Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level
 // whose split nodes still hold their children's rows (-1: none).
 void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,

@@ -87,6 +87,11 @@ class Trainer {
     DenseBins bins_;
     bool sparse_ = false;
     CsrBins csr_;
+    // sparse layout: one pass per level over the bin-major copy instead of per-node histograms (depth <= 11)
+    bool sparse_pass_ = false;
+    SparsePass sp_;
+    void build_sparse_tasks();
+    void ensure_hist_arena();  // per-node histograms for stage-wise inspection (the level pass itself keeps none)
     TreeBuffers tb_;      // buffer set 0; set k = tb_.for_class(k)
     int n_sets_ = 1;      // tree_per_rounds when the class trees of a round are built together, else 1
     // model

@@ -165,6 +165,9 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
     log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
     if (sparse_) {
+        // TGBM_SPARSE_PASS=0 keeps the row-list kernels with per-node histograms in HBM (tests compare the two)
+        const char *pe = std::getenv("TGBM_SPARSE_PASS");
+        sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && !(pe != nullptr && std::string(pe) == "0");
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
         // Head of the histogram: the most frequent features whose bins fit the LDS slots. Worth it when
         // they carry a real share of the stored values (skewed, e.g. Zipf-distributed, feature usage).
@@ -184,7 +187,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
                 head_nnz += cuts_.feature_nnz[f];
             }
             const char *he = std::getenv("TGBM_CSR_HEAD");  // "0" disables the head (tests of both kernels)
-            if (head_nnz * 10 < nnz_ || (he != nullptr && std::string(he) == "0")) head_bin.clear();
+            if (head_nnz * 10 < nnz_ || (he != nullptr && std::string(he) == "0") || sparse_pass_) head_bin.clear();
             log_info("sparse histogram head: %zu bins in LDS carry %.1f%% of the stored values", head_bin.size(),
                      nnz_ > 0 ? 100.0 * (double)head_nnz / (double)nnz_ : 0.0);
         }
@@ -210,7 +213,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         // bin-major copy for the root histogram (TGBM_CSC_ROOT=0: without, the root goes through the row-major
         // kernels like every other level; tests of both)
         const char *ce = std::getenv("TGBM_CSC_ROOT");
-        if (nnz_ > 0 && !(ce != nullptr && std::string(ce) == "0")) {
+        if (nnz_ > 0 && (sparse_pass_ || !(ce != nullptr && std::string(ce) == "0"))) {
             PairSorter ps;
             ps.alloc(nnz_);
             launch_csc_keys(stream_, n_, d_row_ptr, d_bin, ps.keys[0], ps.vals[0]);
@@ -325,8 +328,12 @@ void Trainer::alloc_tree_buffers() {
     // One set of buffers per class tree of a round when that fits comfortably: the trees of a round are
     // independent and are then built together (class = blockIdx.z of every launch).
     const int K = param_.tree_per_rounds;
-    const size_t set_bytes = (size_t)n_ * 13 + ((size_t)2 * max_level_nodes * n_bins_ + tb.n_partial) * sizeof(longlong2) +
-                             tb.n_end_bound * sizeof(int);
+    if (sparse_pass_) build_sparse_tasks();
+    const size_t set_bytes =
+        sparse_pass_ ? (size_t)n_ * 15 + (size_t)sp_.n_partial_slots * sp_.partial_stride * sizeof(longlong2) +
+                           (size_t)max_level_nodes * sp_.n_cand_slots * sizeof(SplitCand)
+                     : (size_t)n_ * 13 + ((size_t)2 * max_level_nodes * n_bins_ + tb.n_partial) * sizeof(longlong2) +
+                           tb.n_end_bound * sizeof(int);
     size_t free_b = 0, total_b = 0;
     HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
     const char *be = std::getenv("TGBM_BATCH_CLASSES");  // "0": build the trees of a round one after the other
@@ -339,8 +346,13 @@ void Trainer::alloc_tree_buffers() {
     tb.ridx[0] = dalloc<int>(S * n_);
     tb.ridx[1] = dalloc<int>(S * n_);
     tb.goes_right = dalloc<uint8_t>(S * ((size_t)n_ + 4));
-    tb.hist_q[0] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
-    tb.hist_q[1] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+    if (!sparse_pass_) {
+        tb.hist_q[0] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+        tb.hist_q[1] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+    } else {
+        tb.nid16 = dalloc<unsigned short>(S * (((size_t)n_ + 2) / 2 * 2));
+        tb.node_rows = dalloc<int>(S * tb.n_nodes);
+    }
     tb.partial = dalloc<longlong2>(S * tb.n_partial);
     tb.quant = dalloc<QuantCtl>(S);
     tb.hitem_shift = dalloc<int2>(S * (size_t)tb.max_hitems);
@@ -384,7 +396,9 @@ void Trainer::alloc_tree_buffers() {
         cur += k;
     }
     pack_begin.push_back(n_bins_);
-    tb.n_packs = (int)pack_begin.size() - 1;
+    tb.n_packs = sparse_pass_ ? sp_.n_cand_slots : (int)pack_begin.size() - 1;  // candidates per node
+    if (sparse_pass_)
+        sp_.partial = dalloc<longlong2>(S * (size_t)sp_.n_partial_slots * sp_.partial_stride);
     int *d_pack = dalloc<int>(pack_begin.size());
     upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
     tb.pack_begin = d_pack;
@@ -518,9 +532,89 @@ void Trainer::tree_init(int k) {
     nid_materialized_ = false;
 }
 
-void Trainer::find_split(int level) { find_split_sets(set_of(cur_class_), d_gh_ + (size_t)cur_class_ * n_, level, 1); }
+void Trainer::find_split(int level) {
+    if (sparse_pass_ && !in_boost_) ensure_hist_arena();
+    find_split_sets(set_of(cur_class_), d_gh_ + (size_t)cur_class_ * n_, level, 1);
+}
+
+// The sparse level pass keeps no per-node histogram; callers that drive the stages one by one can look at them,
+// so the first such call allocates the two level arenas the other layouts always have.
+void Trainer::ensure_hist_arena() {
+    if (tb_.hist_q[0] != nullptr) return;
+    const size_t cells = (size_t)n_sets_ * tb_.max_level_nodes * n_bins_;
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    TGBM_CHECK(cells * 2 * sizeof(longlong2) < free_b / 2,
+               "per-node histograms for stage-wise inspection need %zu bytes (free %zu); use tgbm_trainer_boost",
+               cells * 2 * sizeof(longlong2), free_b);
+    tb_.hist_q[0] = dalloc<longlong2>(cells);
+    tb_.hist_q[1] = dalloc<longlong2>(cells);
+}
+
+// Work list of the sparse level pass: runs of whole features with about kSparseTaskValues stored values each;
+// a feature with more values than that is cut into chunks (its own tasks) whose tables k_sparse_big adds up.
+void Trainer::build_sparse_tasks() {
+    std::vector<int> fvb(F_ + 1, 0);
+    for (int f = 0; f < F_; ++f) fvb[f + 1] = fvb[f] + (int)cuts_.feature_nnz[f];
+    std::vector<SparseTask> tasks;
+    std::vector<SparseBig> big;
+    int n_small = 0, n_partial = 0, max_big_bins = 0;
+    // first pass: small tasks get candidate slots 0 .. n_small - 1, big features the slots after them
+    int f = 0;
+    while (f < F_) {
+        const long m = cuts_.feature_nnz[f];
+        if (m > kSparseTaskValues) {
+            SparseBig b;
+            b.feature = f;
+            b.slot_begin = n_partial;
+            for (long v = 0; v < m; v += kSparseTaskValues) {
+                SparseTask t{f, f + 1, fvb[f] + (int)v, fvb[f] + (int)std::min(m, v + kSparseTaskValues), -1, n_partial++};
+                tasks.push_back(t);
+            }
+            b.slot_end = n_partial;
+            b.cand_slot = -1;  // numbered below
+            big.push_back(b);
+            max_big_bins = std::max(max_big_bins, h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f]);
+            ++f;
+            continue;
+        }
+        int fe = f;
+        long vals = 0;
+        while (fe < F_ && cuts_.feature_nnz[fe] <= kSparseTaskValues && vals + cuts_.feature_nnz[fe] <= kSparseTaskValues) {
+            vals += cuts_.feature_nnz[fe];
+            ++fe;
+        }
+        if (vals > 0) {
+            SparseTask t{f, fe, fvb[f], fvb[fe], n_small++, -1};
+            tasks.push_back(t);
+        }
+        f = std::max(fe, f + 1);
+    }
+    for (size_t i = 0; i < big.size(); ++i) big[i].cand_slot = n_small + (int)i;
+    // the biggest tasks first: they decide when the level is done
+    std::stable_sort(tasks.begin(), tasks.end(),
+                     [](const SparseTask &a, const SparseTask &b) { return a.v_end - a.v_begin > b.v_end - b.v_begin; });
+    sp_.n_tasks = (int)tasks.size();
+    sp_.n_big = (int)big.size();
+    sp_.n_cand_slots = std::max(1, n_small + (int)big.size());
+    sp_.n_partial_slots = n_partial;
+    sp_.partial_stride = (size_t)max_big_bins * (size_t)tb_.max_level_nodes;
+    SparseTask *d_tasks = dalloc<SparseTask>(tasks.size());
+    SparseBig *d_big = dalloc<SparseBig>(big.size());
+    int *d_fvb = dalloc<int>(fvb.size());
+    upload(stream_, d_tasks, tasks.data(), tasks.size());
+    upload(stream_, d_big, big.data(), big.size());
+    upload(stream_, d_fvb, fvb.data(), fvb.size());
+    HIP_CHECK(hipStreamSynchronize(stream_));  // the host vectors go out of scope
+    sp_.tasks = d_tasks;
+    sp_.big = d_big;
+    sp_.feat_val_begin = d_fvb;
+    log_info("sparse level pass: %d tasks, %d features in chunks (%d chunks), %d candidate slots per node", sp_.n_tasks,
+             sp_.n_big, n_partial, sp_.n_cand_slots);
+}
 
 void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level, int n_class) {
+    if (sparse_pass_ && level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
     if (profiling_) {
         HistEvent ev;
         HIP_CHECK(hipEventCreate(&ev.start));
@@ -534,18 +628,24 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
     } else {
         build_level_hist(tb, level, gh, n_class);
     }
-    if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
-    if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
-    // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them)
-    launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
-                      !(in_boost_ && level == param_.depth - 1));
+    if (!sparse_pass_) {
+        if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
+        if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
+        // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them)
+        launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
+                          !(in_boost_ && level == param_.depth - 1));
+    }
     launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
     HIP_CHECK_LAUNCHES("find_split");
 }
 
 void Trainer::build_level_hist(const TreeBuffers &tb, int level, const GHPair *gh, int n_class) {
-    if (sparse_)
+    if (sparse_pass_) {
+        // histogram and split search of the level in one pass; stage-wise driving also gets the per-node histograms
+        launch_sparse_level(stream_, tb, csr_, sp_, gh, level, param_.min_child_weight, param_.lambda,
+                            !in_boost_ && tb_.hist_q[0] != nullptr, n_class);
+    } else if (sparse_)
         launch_hist_csr(stream_, tb, csr_, gh, level, n_class);
     else
         launch_hist_dense(stream_, tb, bins_, gh, level, n_class);
@@ -556,7 +656,10 @@ void Trainer::partition(int level) { partition_sets(set_of(cur_class_), level, 1
 void Trainer::partition_sets(const TreeBuffers &tb, int level, int n_class) {
     // the last level is not partitioned: its split nodes keep their rows until the tree's final pass
     if (level < param_.depth - 1) lookup_level_ = -1;
-    if (sparse_)
+    if (sparse_pass_) {
+        launch_sparse_partition(stream_, tb, csr_, level, n_class);  // every level: the map is the only row state
+        lookup_level_ = -1;
+    } else if (sparse_)
         launch_partition_csr(stream_, tb, csr_, level, n_class);
     else
         launch_partition_dense(stream_, tb, bins_, level, n_class);
@@ -566,6 +669,19 @@ void Trainer::partition_sets(const TreeBuffers &tb, int level, int n_class) {
 void Trainer::log_plan(const TreeBuffers &tb) {
     size_t off = ctl_log_.size();
     ctl_log_.resize(off + param_.depth + 1);
+    if (sparse_pass_) {
+        // rows of the nodes the reference would build from rows: the root, then the smaller child of every pair
+        std::vector<int> rows((size_t)tb.n_nodes);
+        HIP_CHECK(hipMemcpyAsync(rows.data(), tb.node_rows, sizeof(int) * rows.size(), hipMemcpyDeviceToHost, stream_));
+        HIP_CHECK(hipStreamSynchronize(stream_));
+        for (int level = 0; level <= param_.depth; ++level) {
+            long built = level == 0 ? n_ : 0;
+            if (level > 0 && level < param_.depth)
+                for (int x = (1 << level) - 1; x < (2 << level) - 1; x += 2) built += std::min(rows[x], rows[x + 1]);
+            ctl_log_[off + level] = LevelCtl{0, 0, 0, (int)built};
+        }
+        return;
+    }
     HIP_CHECK(hipMemcpyAsync(ctl_log_.data() + off, tb.ctl, sizeof(LevelCtl) * (size_t)(param_.depth + 1),
                              hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
@@ -823,6 +939,8 @@ int Trainer::info(const std::string &key) const {
     if (key == "n_nodes") return tb_.n_nodes;
     if (key == "n_sets") return n_sets_;
     if (key == "sparse") return sparse_ ? 1 : 0;
+    if (key == "sparse_pass") return sparse_pass_ ? 1 : 0;
+    if (key == "row_lists") return sparse_pass_ ? 0 : 1;  // the sparse level pass keeps a row -> node map only
     if (key == "dense_W") return bins_.W;
     if (key == "reorders_done") return reorders_done_;
     if (key == "device_free_mb") {
@@ -862,8 +980,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "y") src = d_y_, bytes = sizeof(float) * (size_t)n_;
     else if (name == "nodes") src = cur.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
     else if (name == "sp") src = cur.sp, bytes = sizeof(SplitPoint) * (size_t)max_level_nodes;
-    else if (name == "hist_q0") src = cur.hist_q[0], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
-    else if (name == "hist_q1") src = cur.hist_q[1], bytes = sizeof(longlong2) * (size_t)max_level_nodes * n_bins_;
+    else if (name == "hist_q0") src = cur.hist_q[0], bytes = tb_.hist_q[0] ? sizeof(longlong2) * (size_t)max_level_nodes * n_bins_ : 0;
+    else if (name == "hist_q1") src = cur.hist_q[1], bytes = tb_.hist_q[1] ? sizeof(longlong2) * (size_t)max_level_nodes * n_bins_ : 0;
     else if (name == "quant") src = cur.quant, bytes = sizeof(QuantCtl);
     else if (name == "ctl") src = cur.ctl, bytes = sizeof(LevelCtl) * (size_t)(param_.depth + 1);
     else if (name == "seg") src = cur.seg, bytes = sizeof(int2) * (size_t)tb_.n_nodes;

@@ -5,6 +5,7 @@
 #include <algorithm>
 
 #include "device_api.h"
+#include "kernel_common.h"
 
 namespace tgbm {
 namespace {
@@ -14,12 +15,6 @@ constexpr int kWaves = kBlock / 64;
 constexpr int kHistMinChunk = 1024;
 constexpr int kHistBlock = 1024;      // threads per histogram workgroup (they share one LDS histogram)
 constexpr int kHistFlushRows = 8192;  // rows a packed 32+32-bit LDS bin may absorb before it is drained
-
-__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
-__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
-__device__ __forceinline__ int lanes_below(unsigned long long mask) {
-    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0));
-}
 
 // Exclusive scan of one int per thread over a 256-thread block; lds needs kWaves ints.
 __device__ int block_excl_scan(int v, int *lds, int *total) {
@@ -60,10 +55,6 @@ __device__ __forceinline__ float wave_sum_f(float v) {
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
     return v;
-}
-
-__device__ __forceinline__ bool node_splits(const TreeNode &nd) {
-    return nd.is_valid && !nd.is_leaf && nd.split_feature_id >= 0;
 }
 
 // Largest p in [0, n) with begin[p] <= item (begin is non-decreasing, begin[0] <= item < begin[n]).
@@ -310,6 +301,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         raw[9] &= 0x000000ffu;  // bytes 37..39 are padding (byte 36 = is_pruned)
         tb.nodes[i] = nd;
         tb.seg[i] = make_int2(0, 0);
+        if (tb.node_rows != nullptr) tb.node_rows[i] = i == 0 ? tb.n : 0;
     }
     float g = 0, h = 0, gm = 0, hm = 0, hf = 0;
     for (int i = threadIdx.x; i < tb.n_grad_blocks; i += kBlock) {
@@ -615,16 +607,6 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
 // order of the rows; every later quantity of a tree (child sums, weights, gains, predictions, the next gradients)
 // derives from it. These kernels replace it by the exact fixed-point total - the same integers in any order - so
 // that a tree does not depend on the row order at all.
-__device__ __forceinline__ long long wave_sum_ll(long long v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) {
-        const int lo = __shfl_xor((int)(unsigned)(unsigned long long)v, d);
-        const int hi = __shfl_xor((int)((unsigned long long)v >> 32), d);
-        v += (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
-    }
-    return v;
-}
-
 __device__ void set_root_sums(const TreeBuffers &tb, long long G, long long H, float lambda) {
     GHPair s{(float)((double)G * (double)tb.quant->inv_g), (float)((double)H * (double)tb.quant->inv_h)};
     TreeNode &root = tb.nodes[0];
@@ -702,12 +684,6 @@ __global__ __launch_bounds__(kBlock) void k_count_bytes(const uint8_t *__restric
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) c += v[i] == value;
     c = (unsigned long long)wave_sum_ll((long long)c);
     if (lane_id() == 0 && c) atomicAdd(out, c);
-}
-
-__device__ __forceinline__ long long shfl_up_ll(long long v, int d) {
-    int lo = __shfl_up((int)(unsigned)(unsigned long long)v, d);
-    int hi = __shfl_up((int)((unsigned long long)v >> 32), d);
-    return (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
 }
 
 // --------------------------------------------------------------------------- sparse histogram
@@ -886,28 +862,6 @@ __global__ __launch_bounds__(kBlock) void k_hist_root_csc(TreeBuffers tb_all, Cs
     }
 }
 
-// Left/right decision of the sparse layout: binary search of the row's bin ids for the one inside
-// the split feature's bin range (absent = missing), hist_tree_builder_single.cu:941-1011.
-// Does the row go right at a split of the feature whose global bins are [cb, ce)? Binary search of the
-// row's ascending bin ids for one inside the feature's range; none = missing -> default direction.
-__device__ __forceinline__ bool csr_goes_right(const CsrBins &bins, int row, int cb, int ce, int sbid, bool dr) {
-    int lo = bins.row_ptr[row], hi = bins.row_ptr[row + 1];
-    int found = -1;
-    while (lo < hi) {
-        int mid = lo + (hi - lo) / 2;
-        int b = bins.bin[mid];
-        if (b >= cb && b < ce) {
-            found = b;
-            break;
-        }
-        if (b < cb)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    return found < 0 ? dr : (found >= sbid);
-}
-
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, CsrBins bins, int level) {
     __shared__ int lds[kWaves];
@@ -948,16 +902,6 @@ __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, C
 }
 
 // ------------------------------------------------------------------------ split finding
-__device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float lambda) {
-#pragma clang fp contract(off)
-    GHPair r{f.g - l.g, f.h - l.h};
-    float gain = 0.f;
-    if (l.h >= mcw && r.h >= mcw)
-        gain = (l.g * l.g) / (l.h + lambda) + (r.g * r.g) / (r.h + lambda) - (f.g * f.g) / (f.h + lambda);
-    return fmaxf(0.f, gain);
-}
-
-
 // Split search. One wavefront scans one pack of whole features (at most 256 bins, 4 consecutive bins
 // per lane) of one node with a segmented inclusive prefix sum over the exact 64-bit fixed-point
 // histogram: integer sums are associative, so the parallel scan returns bit-for-bit what a
@@ -1694,6 +1638,11 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
     __shared__ float s_f[kStatsLds];
     __shared__ double s_d[kWaves];
     const int r0 = blockIdx.x * kRowBlock, r1 = min(tb.n, r0 + kRowBlock);
+    constexpr int U = 4;
+    if (tb.nid16 != nullptr) {
+        // sparse level pass: the row -> node map is kept per row, nothing to look up
+        for (int i = threadIdx.x; i < kRowBlock; i += kBlock) s_leaf[i] = r0 + i < r1 ? (short)tb.nid16[r0 + i] : (short)-1;
+    } else {
     for (int i = threadIdx.x; i < kRowBlock; i += kBlock) s_leaf[i] = -1;
     if (threadIdx.x == 0) s_n = 0;
     __syncthreads();
@@ -1735,7 +1684,6 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
         total += tot;
     }
     __syncthreads();
-    constexpr int U = 4;
     for (int j0 = threadIdx.x; j0 < total; j0 += kBlock * U) {
         int node[U], row[U], split[U];
 #pragma unroll
@@ -1779,6 +1727,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
             }
         }
     }
+    }  // row lists
     __syncthreads();
     if (MODE == 0) {
         for (int i = r0 + threadIdx.x; i < r1; i += kBlock) {
@@ -1936,6 +1885,11 @@ void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_cla
     if (!stats_ready)  // n_grad_blocks == row_blocks(n)
         k_sum_gh<<<dim3(tb.n_grad_blocks, 1, n_class), kBlock, 0, s>>>(tb.n, gh_class, tb.root_partial);
     k_tree_init<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, lambda);
+    if (tb.nid16 != nullptr) {
+        // sparse level pass: every row starts in the root (the n_class maps lie back to back)
+        const size_t words = ((size_t)tb.n + 2) / 2 * (size_t)n_class;
+        k_fill_u32<<<grid_for(words), kBlock, 0, s>>>(reinterpret_cast<unsigned *>(tb.nid16), 0u, words);
+    }
 }
 
 template <int LPR, int SLOTS>
@@ -2110,7 +2064,8 @@ static void tree_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbin
                      const TreeEndArgs &a, int n_class = 1) {
     const int n_blocks = row_blocks(tb.n);
     const size_t entries = (size_t)((1 << tb.depth) - 1) * (n_blocks + 1);
-    k_end_bounds<<<dim3(grid_for(entries, 8192), 1, n_class), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
+    if (tb.nid16 == nullptr)
+        k_end_bounds<<<dim3(grid_for(entries, 8192), 1, n_class), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
     if (tb.sparse) tree_end_launch<true>(s, tb, DenseBins{}, *cbins, mode, a, n_class);
     else tree_end_launch<false>(s, tb, *dbins, CsrBins{}, mode, a, n_class);
 }
