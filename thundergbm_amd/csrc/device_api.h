@@ -123,6 +123,15 @@ struct SparseTask {
     int cand_slot;       // candidate slot the task fills, -1: a chunk (its feature's slot is filled by k_sparse_big)
     int partial_slot;    // chunk: where its table goes in SparsePass::partial, else -1
 };
+// Features with at most kSparseTailValues stored values are searched by one wavefront each, which sorts the
+// feature's values by node and scans them: the work follows the values, not the (bin, node) cells of a table.
+constexpr int kSparseTailValues = 512;
+constexpr int kSparseTailWaves = 4;          // wavefronts (and candidate slots) of a tail task
+constexpr int kSparseTailTaskValues = 16384; // stored values per tail task
+struct SparseTailTask {
+    int i_begin, i_end;  // entries of SparsePass::tail_feat
+    int cand_slot;       // first of the kSparseTailWaves candidate slots of the task
+};
 struct SparseBig {
     int feature;
     int slot_begin, slot_end;  // partial slots of its chunks
@@ -133,7 +142,14 @@ struct SparsePass {
     int n_tasks = 0;
     const SparseBig *big = nullptr;
     int n_big = 0;
+    const SparseTailTask *tail_tasks = nullptr;
+    int n_tail_tasks = 0;
+    const int *tail_feat = nullptr;       // feature ids served by the tail tasks
     const int *feat_val_begin = nullptr;  // [F + 1] first position of every feature in the bin-major copy
+    // [n_sets][nnz] the gradient pair of every stored value's row, in the order of the bin-major copy, refreshed once
+    // per tree: the level passes then stream it instead of fetching a cache line per value (nullptr: no room, gather)
+    GHPair *csc_gh = nullptr;
+    long nnz = 0;
     longlong2 *partial = nullptr;         // [n_sets][n_partial_slots][partial_stride] chunk tables, (bin, node) cells
     size_t partial_stride = 0;            // cells per slot: most bins of a big feature x kSparseMaxLevelNodes at most
     int n_partial_slots = 0;
@@ -273,6 +289,9 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                          const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1);
 void launch_sparse_partition(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
+// csc_gh[e] = gh[csc_row[e]] for the n_class gradient planes (once per tree, before its first level)
+void launch_sparse_gh_refresh(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
+                              const GHPair *gh, int n_class = 1);
 // Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level
 // whose split nodes still hold their children's rows (-1: none).
 void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,

@@ -397,8 +397,15 @@ void Trainer::alloc_tree_buffers() {
     }
     pack_begin.push_back(n_bins_);
     tb.n_packs = sparse_pass_ ? sp_.n_cand_slots : (int)pack_begin.size() - 1;  // candidates per node
-    if (sparse_pass_)
+    if (sparse_pass_) {
         sp_.partial = dalloc<longlong2>(S * (size_t)sp_.n_partial_slots * sp_.partial_stride);
+        // per-value gradient pairs in the order of the bin-major copy, when they fit comfortably
+        sp_.nnz = nnz_;
+        HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        const char *ge = std::getenv("TGBM_SPARSE_GH_COPY");  // "0": gather the pairs per value instead (tests)
+        if (S * (size_t)nnz_ * sizeof(GHPair) < free_b / 4 && !(ge != nullptr && std::string(ge) == "0"))
+            sp_.csc_gh = dalloc<GHPair>(S * (size_t)nnz_);
+    }
     int *d_pack = dalloc<int>(pack_begin.size());
     upload(stream_, d_pack, pack_begin.data(), pack_begin.size());
     tb.pack_begin = d_pack;
@@ -551,18 +558,31 @@ void Trainer::ensure_hist_arena() {
     tb_.hist_q[1] = dalloc<longlong2>(cells);
 }
 
-// Work list of the sparse level pass: runs of whole features with about kSparseTaskValues stored values each;
-// a feature with more values than that is cut into chunks (its own tasks) whose tables k_sparse_big adds up.
+// Work lists of the sparse level pass. Features with at most kSparseTailValues stored values go to the tail tasks
+// (one wavefront per feature); the others to table tasks: runs of consecutive such features with about
+// kSparseTaskValues values, a feature with more values than that cut into chunks (tasks of their own) whose tables
+// k_sparse_big adds up. The feature that owns global bin 0 is always a table feature (its table is searched for
+// every node even without values: the arg-max of a node without any positive gain ends there).
 void Trainer::build_sparse_tasks() {
     std::vector<int> fvb(F_ + 1, 0);
     for (int f = 0; f < F_; ++f) fvb[f + 1] = fvb[f] + (int)cuts_.feature_nnz[f];
+    int bin0_owner = -1;
+    for (int f = 0; f < F_ && bin0_owner < 0; ++f)
+        if (h_cut_row_ptr_[f + 1] > h_cut_row_ptr_[f]) bin0_owner = f;
+    auto is_table = [&](int f) { return cuts_.feature_nnz[f] > kSparseTailValues || f == bin0_owner; };
     std::vector<SparseTask> tasks;
     std::vector<SparseBig> big;
+    std::vector<SparseTailTask> tail_tasks;
+    std::vector<int> tail_feat;
     int n_small = 0, n_partial = 0, max_big_bins = 0;
-    // first pass: small tasks get candidate slots 0 .. n_small - 1, big features the slots after them
     int f = 0;
     while (f < F_) {
         const long m = cuts_.feature_nnz[f];
+        if (!is_table(f)) {
+            if (m > 0) tail_feat.push_back(f);
+            ++f;
+            continue;
+        }
         if (m > kSparseTaskValues) {
             SparseBig b;
             b.feature = f;
@@ -580,41 +600,61 @@ void Trainer::build_sparse_tasks() {
         }
         int fe = f;
         long vals = 0;
-        while (fe < F_ && cuts_.feature_nnz[fe] <= kSparseTaskValues && vals + cuts_.feature_nnz[fe] <= kSparseTaskValues) {
+        while (fe < F_ && is_table(fe) && cuts_.feature_nnz[fe] <= kSparseTaskValues &&
+               vals + cuts_.feature_nnz[fe] <= kSparseTaskValues) {
             vals += cuts_.feature_nnz[fe];
             ++fe;
         }
-        if (vals > 0) {
-            SparseTask t{f, fe, fvb[f], fvb[fe], n_small++, -1};
-            tasks.push_back(t);
-        }
-        f = std::max(fe, f + 1);
+        SparseTask t{f, fe, fvb[f], fvb[fe], n_small++, -1};
+        tasks.push_back(t);
+        f = fe;
     }
     for (size_t i = 0; i < big.size(); ++i) big[i].cand_slot = n_small + (int)i;
+    int next_slot = n_small + (int)big.size();
+    for (size_t i = 0; i < tail_feat.size();) {
+        size_t e = i;
+        long vals = 0;
+        while (e < tail_feat.size() && (e == i || vals + cuts_.feature_nnz[tail_feat[e]] <= kSparseTailTaskValues))
+            vals += cuts_.feature_nnz[tail_feat[e++]];
+        tail_tasks.push_back(SparseTailTask{(int)i, (int)e, next_slot});
+        next_slot += kSparseTailWaves;
+        i = e;
+    }
     // the biggest tasks first: they decide when the level is done
     std::stable_sort(tasks.begin(), tasks.end(),
                      [](const SparseTask &a, const SparseTask &b) { return a.v_end - a.v_begin > b.v_end - b.v_begin; });
     sp_.n_tasks = (int)tasks.size();
     sp_.n_big = (int)big.size();
-    sp_.n_cand_slots = std::max(1, n_small + (int)big.size());
+    sp_.n_tail_tasks = (int)tail_tasks.size();
+    sp_.n_cand_slots = std::max(1, next_slot);
     sp_.n_partial_slots = n_partial;
     sp_.partial_stride = (size_t)max_big_bins * (size_t)tb_.max_level_nodes;
     SparseTask *d_tasks = dalloc<SparseTask>(tasks.size());
     SparseBig *d_big = dalloc<SparseBig>(big.size());
+    SparseTailTask *d_tail = dalloc<SparseTailTask>(tail_tasks.size());
+    int *d_tail_feat = dalloc<int>(tail_feat.size());
     int *d_fvb = dalloc<int>(fvb.size());
     upload(stream_, d_tasks, tasks.data(), tasks.size());
     upload(stream_, d_big, big.data(), big.size());
+    upload(stream_, d_tail, tail_tasks.data(), tail_tasks.size());
+    upload(stream_, d_tail_feat, tail_feat.data(), tail_feat.size());
     upload(stream_, d_fvb, fvb.data(), fvb.size());
     HIP_CHECK(hipStreamSynchronize(stream_));  // the host vectors go out of scope
     sp_.tasks = d_tasks;
     sp_.big = d_big;
+    sp_.tail_tasks = d_tail;
+    sp_.tail_feat = d_tail_feat;
     sp_.feat_val_begin = d_fvb;
-    log_info("sparse level pass: %d tasks, %d features in chunks (%d chunks), %d candidate slots per node", sp_.n_tasks,
-             sp_.n_big, n_partial, sp_.n_cand_slots);
+    log_info("sparse level pass: %d table tasks, %d features in chunks (%d chunks), %zu tail features in %d tasks, "
+             "%d candidate slots per node", sp_.n_tasks, sp_.n_big, n_partial, tail_feat.size(), sp_.n_tail_tasks,
+             sp_.n_cand_slots);
 }
 
 void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level, int n_class) {
-    if (sparse_pass_ && level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
+    if (sparse_pass_ && level == 0) {
+        launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
+        launch_sparse_gh_refresh(stream_, tb, csr_, sp_, gh, n_class);
+    }
     if (profiling_) {
         HistEvent ev;
         HIP_CHECK(hipEventCreate(&ev.start));
