@@ -26,10 +26,12 @@ def T():
 
 @pytest.fixture(autouse=True)
 def _default_layout():
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
+              "TGBM_SPARSE_SORTED"):
         os.environ.pop(k, None)
     yield
-    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS"):
+    for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
+              "TGBM_SPARSE_SORTED"):
         os.environ.pop(k, None)
 
 
@@ -558,9 +560,10 @@ def test_sparse_root_histogram_from_either_copy(T, objective, kind, head):
         kw["num_class"] = int(y.max()) + 1
     runs = []
     try:
-        for level_pass, csc in (("1", "1"), ("0", "1"), ("0", "0")):
+        for level_pass, csc, srt in (("1", "1", "1"), ("1", "1", "0"), ("0", "1", "1"), ("0", "0", "1")):
             os.environ["TGBM_SPARSE_PASS"] = level_pass
             os.environ["TGBM_CSC_ROOT"] = csc
+            os.environ["TGBM_SPARSE_SORTED"] = srt  # "0": every feature through the (bin, node) tables
             s = T.Session(val, rp, col, y, **kw)
             assert s.info("sparse_pass") == int(level_pass)
             s.gradient()
@@ -575,7 +578,45 @@ def test_sparse_root_histogram_from_either_copy(T, objective, kind, head):
     finally:
         os.environ.pop("TGBM_CSC_ROOT", None)
         os.environ.pop("TGBM_SPARSE_PASS", None)
-    assert runs[0] == runs[1] == runs[2]
+        os.environ.pop("TGBM_SPARSE_SORTED", None)
+    assert runs[0] == runs[1] == runs[2] == runs[3]
+
+
+@pytest.mark.parametrize("mcw,gamma", [(1.0, 0.0), (40.0, 0.0), (1.0, 30.0)])
+def test_sparse_sorted_pass_equals_table_pass_on_deep_uneven_trees(T, mcw, gamma):
+    """Sparse level pass: features of a few thousand values are searched through their values kept sorted by
+    (feature, node, bin) from level to level, the frequent ones through (bin, node) tables; TGBM_SPARSE_SORTED=0
+    sends every feature through the tables. Same integers either way: identical models, predictions and row -> node
+    maps, on trees whose nodes stop at different levels (min_child_weight) and with frequent and rare features
+    mixed (a few columns in nearly every row, many in a handful of rows)."""
+    os.environ["TGBM_LAYOUT"] = "sparse"
+    rng = np.random.default_rng(21)
+    n, F = 40000, 900
+    # Zipf-like column usage: columns 0..5 in most rows (more than one tile of values), the rest rare
+    cols = []
+    rp = np.zeros(n + 1, np.int32)
+    for i in range(n):
+        c = set(np.flatnonzero(rng.random(6) < 0.7).tolist())
+        c.update((6 + rng.integers(0, F - 6, rng.integers(0, 7))).tolist())
+        cols.append(np.sort(np.fromiter(c, np.int32, len(c))))
+        rp[i + 1] = rp[i] + len(c)
+    col = np.concatenate(cols).astype(np.int32)
+    val = rng.lognormal(0, 1, len(col)).astype(np.float32)
+    y = _target(val, rp, col, n, F, 21, "bin")
+    kw = dict(objective="binary:logistic", n_trees=5, depth=8, max_num_bin=32, learning_rate=0.4,
+              min_child_weight=mcw, gamma=gamma)
+    runs = []
+    try:
+        for srt in ("1", "0"):
+            os.environ["TGBM_SPARSE_SORTED"] = srt
+            s = T.Session(val, rp, col, y, **kw)
+            assert s.info("sparse_pass") == 1
+            s.boost(5)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        os.environ.pop("TGBM_SPARSE_SORTED", None)
+    assert runs[0] == runs[1]
 
 
 def test_predict_transforms_through_the_c_abi(T):

@@ -123,15 +123,23 @@ struct SparseTask {
     int cand_slot;       // candidate slot the task fills, -1: a chunk (its feature's slot is filled by k_sparse_big)
     int partial_slot;    // chunk: where its table goes in SparsePass::partial, else -1
 };
-// Features with at most kSparseTailValues stored values are searched by one wavefront each, which sorts the
-// feature's values by node and scans them: the work follows the values, not the (bin, node) cells of a table.
-constexpr int kSparseTailValues = 512;
-constexpr int kSparseTailWaves = 4;          // wavefronts (and candidate slots) of a tail task
-constexpr int kSparseTailTaskValues = 16384; // stored values per tail task
-struct SparseTailTask {
-    int i_begin, i_end;  // entries of SparsePass::tail_feat
-    int cand_slot;       // first of the kSparseTailWaves candidate slots of the task
+// Features with at most kSortedTile stored values are not searched through tables: their values are kept sorted by
+// (feature, node, bin) from level to level - a stable two-way partition of every (feature, node) run when the node
+// splits - and the split search is a segmented scan of that order, so the work follows the stored values and not
+// the (bin, node) cells. A task is a run of whole features whose values fit one workgroup tile.
+constexpr int kSortedBlock = 512;                        // threads of a sorted-pass workgroup
+constexpr int kSortedPerThread = 8;                      // consecutive values a thread owns
+constexpr int kSortedTile = kSortedBlock * kSortedPerThread;  // values per task at most
+constexpr int kSortedLevels = 12;                        // levels the pass serves (depth <= 11, one spare)
+struct SortedTask {
+    int v_begin;     // first position of the task's tile in the sorted-pass arrays
+    int count;       // stored values of its features (= live values at the root)
+    int meta_begin;  // first entry of its features in SparsePass::sorted_meta / sorted_fid
+    int n_feat;      // features of the task
+    int cand_slot;   // candidate slot the task fills
 };
+// Key of a stored value in the sorted pass: feature (index inside its task) << 20 | node of the level << 8 | local bin
+constexpr int kSortedNodeShift = 8, kSortedFeatShift = 20;
 struct SparseBig {
     int feature;
     int slot_begin, slot_end;  // partial slots of its chunks
@@ -142,9 +150,20 @@ struct SparsePass {
     int n_tasks = 0;
     const SparseBig *big = nullptr;
     int n_big = 0;
-    const SparseTailTask *tail_tasks = nullptr;
-    int n_tail_tasks = 0;
-    const int *tail_feat = nullptr;       // feature ids served by the tail tasks
+    // sorted pass (features of at most kSortedTile values)
+    const SortedTask *sorted_tasks = nullptr;
+    int n_sorted_tasks = 0;
+    const int2 *sorted_meta = nullptr;    // per feature of a task: (first global bin, number of bins)
+    const int *sorted_fid = nullptr;      // its feature id
+    const int *sorted_row0 = nullptr;     // [n_sorted] rows and keys in the static order (feature, bin, row): the
+    const unsigned *sorted_key0 = nullptr;  // root level's input
+    const unsigned short *sorted_start0 = nullptr;  // [n_sorted] tile position where the value's feature starts
+    long n_sorted = 0;
+    // per set: the order of the previous and of the current level, ping-pong by level parity
+    int *sorted_row[2] = {nullptr, nullptr};
+    unsigned *sorted_key[2] = {nullptr, nullptr};
+    GHPair *sorted_gh[2] = {nullptr, nullptr};
+    int *sorted_live = nullptr;           // [n_sets][kSortedLevels][n_sorted_tasks] live values of a tile after a level
     const int *feat_val_begin = nullptr;  // [F + 1] first position of every feature in the bin-major copy
     // [n_sets][nnz] the gradient pair of every stored value's row, in the order of the bin-major copy, refreshed once
     // per tree: the level passes then stream it instead of fetching a cache line per value (nullptr: no room, gather)
@@ -154,6 +173,11 @@ struct SparsePass {
     size_t partial_stride = 0;            // cells per slot: most bins of a big feature x kSparseMaxLevelNodes at most
     int n_partial_slots = 0;
     int n_cand_slots = 0;
+
+    // the sorted pass's order of a level (selected without indexing an array member dynamically)
+    __host__ __device__ int *srow(int level) const { return (level & 1) ? sorted_row[1] : sorted_row[0]; }
+    __host__ __device__ unsigned *skey(int level) const { return (level & 1) ? sorted_key[1] : sorted_key[0]; }
+    __host__ __device__ GHPair *sgh(int level) const { return (level & 1) ? sorted_gh[1] : sorted_gh[0]; }
 };
 
 struct TreeBuffers {
@@ -174,6 +198,10 @@ struct TreeBuffers {
     // sparse level pass only (else nullptr): node every row has reached (heap id) and rows per node
     unsigned short *nid16 = nullptr;  // [n + 2]
     int *node_rows = nullptr;         // [n_nodes]
+    // sparse level pass: best candidate key of every node of the level over all tasks, and the candidate slot of
+    // the task that searches a feature (k_best_update reads the winner's record from that slot)
+    unsigned long long *best_key = nullptr;  // [max_level_nodes]
+    const int *feat_slot = nullptr;          // [F]
     long long *root_total = nullptr;
     int complete_feature = -1;     // dense layout: a feature stored in every row (its bins add up to the root), or -1
     int max_hitems = 0, target_hitems = 0, max_pitems = 0;
@@ -235,6 +263,7 @@ struct TreeBuffers {
         if (nid16 != nullptr) {
             t.nid16 += K * (((size_t)n + 2) / 2 * 2);
             t.node_rows += K * n_nodes;
+            t.best_key += K * max_level_nodes;
         }
         t.leaf_value += K * n_nodes;
         t.end_bound += K * n_end_bound;
@@ -289,7 +318,10 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                          const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1);
 void launch_sparse_partition(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
-// csc_gh[e] = gh[csc_row[e]] for the n_class gradient planes (once per tree, before its first level)
+// Fills the static order of the sorted pass (row0 / key0, sp.n_sorted entries) from the bin-major copy.
+void launch_sorted_setup(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp, int *row0,
+                         unsigned *key0, unsigned short *start0);
+// csc_gh[e] = gh[csc_row[e]] for the values of the table tasks, n_class gradient planes (once per tree)
 void launch_sparse_gh_refresh(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                               const GHPair *gh, int n_class = 1);
 // Row-ordered passes over the row lists (one of dbins / cbins by tb.sparse). lookup_level: the level
@@ -358,8 +390,10 @@ struct PairSorter {
 int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits);
 
 // Bin-major copy of CSR bin ids: sort keys (global bin, payload = row) of every stored value, and the sorted
-// pairs split into the two int arrays the root histogram reads.
-void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, unsigned long long *keys, int *vals);
+// pairs split into the two int arrays the root histogram reads. sort_key (may be null): the key a bin sorts by
+// (the bin itself stays in the key's high half and is what csc_bin receives).
+void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, const int *sort_key,
+                     unsigned long long *keys, int *vals);
 void launch_csc_unpack(hipStream_t s, long nnz, const unsigned long long *keys, const int *vals, int *csc_bin,
                        int *csc_row);
 

@@ -285,13 +285,14 @@ __global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *_
 
 // One wavefront per row: (global bin, row) of every stored value, for the bin-major copy.
 __global__ __launch_bounds__(kBlock) void k_csc_keys(int n_rows, const int *__restrict__ row_ptr,
-                                                    const int *__restrict__ bin, unsigned long long *__restrict__ keys,
-                                                    int *__restrict__ vals) {
+                                                    const int *__restrict__ bin, const int *__restrict__ sort_key,
+                                                    unsigned long long *__restrict__ keys, int *__restrict__ vals) {
     const int r = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
     if (r >= n_rows) return;
     const int e1 = row_ptr[r + 1];
     for (int e = row_ptr[r] + (threadIdx.x & 63); e < e1; e += 64) {
-        keys[e] = (unsigned long long)(unsigned)bin[e];
+        const unsigned b = (unsigned)bin[e];
+        keys[e] = ((unsigned long long)b << 32) | (sort_key != nullptr ? (unsigned)sort_key[b] : b);
         vals[e] = r;
     }
 }
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(kBlock) void k_csc_unpack(long nnz, const unsigned 
                                                       const int *__restrict__ vals, int *__restrict__ csc_bin,
                                                       int *__restrict__ csc_row) {
     for (long e = (long)blockIdx.x * kBlock + threadIdx.x; e < nnz; e += (long)gridDim.x * kBlock) {
-        csc_bin[e] = (int)keys[e];
+        csc_bin[e] = (int)(keys[e] >> 32);
         csc_row[e] = vals[e];
     }
 }
@@ -591,11 +592,12 @@ void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, 
                                               colmat, col_stride);
 }
 
-void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, unsigned long long *keys,
-                     int *vals) {
+void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, const int *sort_key,
+                     unsigned long long *keys, int *vals) {
     if (n_rows == 0) return;
     const int rows_per_block = kBlock / 64;
-    k_csc_keys<<<(n_rows + rows_per_block - 1) / rows_per_block, kBlock, 0, s>>>(n_rows, row_ptr, bin, keys, vals);
+    k_csc_keys<<<(n_rows + rows_per_block - 1) / rows_per_block, kBlock, 0, s>>>(n_rows, row_ptr, bin, sort_key, keys,
+                                                                                vals);
 }
 
 void launch_csc_unpack(hipStream_t s, long nnz, const unsigned long long *keys, const int *vals, int *csc_bin,

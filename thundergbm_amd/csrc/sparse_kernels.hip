@@ -11,6 +11,7 @@
 // Sums are 64-bit integers at the tree's scales: exact, so the candidates are the very numbers a per-node histogram
 // would give.
 #include <algorithm>
+#include <cstdlib>
 
 #include "device_api.h"
 #include "kernel_common.h"
@@ -135,16 +136,26 @@ struct SpShared {
     int ctl[8];  // batch: first feature, end feature, first bin, bins, node range begin, nodes in range, first value, end value
 };
 
-// Level-wide state every task starts from: node sums and validity into LDS, keys cleared, the task's candidate slot
-// marked empty for every node.
-__device__ void sp_begin(const TreeBuffers &tb, SpShared &sh, int level, int cand_slot) {
+// Level-wide state every task starts from: node sums and validity into LDS, keys cleared.
+__device__ void sp_begin(const TreeBuffers &tb, SpShared &sh, int level) {
     const int nl = 1 << level, off = nl - 1;
     for (int x = threadIdx.x; x < nl; x += kSpBlock) {
         const TreeNode &nd = tb.nodes[off + x];
         sh.S[x] = nd.sum_gh_pair;
         sh.ok[x] = nd.is_valid ? 1 : 0;
         sh.key[x] = 0ull;
-        if (cand_slot >= 0) tb.cand[(size_t)x * tb.n_packs + cand_slot].index = 0x7fffffff;
+    }
+}
+
+// End of a task: its best key of every node competes with the other tasks' (the record already sits in the task's
+// candidate slot, where k_best_update finds it through the winning bin's feature).
+__device__ void sp_publish(const TreeBuffers &tb, SpShared &sh, int level) {
+    const int nl = 1 << level;
+    __syncthreads();
+    for (int x = threadIdx.x; x < nl; x += kSpBlock) {
+        const unsigned long long k = sh.key[x];
+        if (k != 0ull && k > __hip_atomic_load(&tb.best_key[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+            atomicMax(&tb.best_key[x], k);
     }
 }
 
@@ -207,10 +218,11 @@ __device__ void sp_search_batch(const TreeBuffers &tb, SpShared &sh, const longl
 
 // One task = a run of whole features (batched so that their tables fit the LDS) or one chunk of a big feature (its
 // table goes to the partial buffer, k_sparse_big adds the chunks up and searches them).
-__global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
+__global__ __launch_bounds__(kSpBlock) __attribute__((amdgpu_waves_per_eu(8)))  // two workgroups per CU
+void k_sparse_level(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
                                                           const GHPair *__restrict__ gh, int level, float mcw,
-                                                          float lambda, int dump_hist) {
-    extern __shared__ longlong2 cells[];  // [kSparseCells]
+                                                          float lambda, int dump_hist, int n_cells) {
+    extern __shared__ longlong2 cells[];  // [n_cells]
     __shared__ SpShared sh;
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     gh += (size_t)blockIdx.z * tb.n;
@@ -220,7 +232,7 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, C
     const int *__restrict__ crp = tb.cut_row_ptr;
     const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
     const GHPair *__restrict__ csc_gh = sp.csc_gh != nullptr ? sp.csc_gh + (size_t)blockIdx.z * sp.nnz : nullptr;
-    sp_begin(tb, sh, level, task.cand_slot);
+    sp_begin(tb, sh, level);
     longlong2 *dump = (dump_hist && task.cand_slot >= 0) ? tb.hist(level) : nullptr;
     longlong2 *partial = task.partial_slot >= 0
                              ? sp.partial + ((size_t)blockIdx.z * sp.n_partial_slots + task.partial_slot) * sp.partial_stride
@@ -232,17 +244,17 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, C
             // next batch: as many whole features as fit with all nodes of the level, or one feature with a node range
             int kf = crp[f + 1] - crp[f];
             int fb = f + 1, nn = nl;
-            if ((long)kf * nl <= kSparseCells) {
+            if ((long)kf * nl <= n_cells) {
                 int total = kf;
                 while (fb < task.f_end && fb - f < kSparseBatchFeatures) {
                     const int k = crp[fb + 1] - crp[fb];
-                    if ((long)(total + k) * nl > kSparseCells) break;
+                    if ((long)(total + k) * nl > n_cells) break;
                     total += k;
                     ++fb;
                 }
                 kf = total;
             } else {
-                nn = kSparseCells / kf;
+                nn = n_cells / kf;
             }
             sh.ctl[0] = f;
             sh.ctl[1] = fb;
@@ -300,11 +312,12 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, C
         }
         f = fb;
     }
+    if (partial == nullptr) sp_publish(tb, sh, level);
 }
 
 // A big feature: the tables of its chunks are added up (node range by node range) and searched.
 __global__ __launch_bounds__(kSpBlock) void k_sparse_big(TreeBuffers tb_all, SparsePass sp, int level, float mcw,
-                                                        float lambda, int dump_hist) {
+                                                        float lambda, int dump_hist, int n_cells) {
     extern __shared__ longlong2 cells[];
     __shared__ SpShared sh;
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
@@ -312,14 +325,14 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_big(TreeBuffers tb_all, Spa
     const int nl = 1 << level;
     const int f = big.feature;
     const int bin0 = tb.cut_row_ptr[f], kf = tb.cut_row_ptr[f + 1] - bin0;
-    sp_begin(tb, sh, level, big.cand_slot);
+    sp_begin(tb, sh, level);
     if (threadIdx.x == 0) {
         sh.fbin[0] = 0;
         sh.fbin[1] = kf;
     }
     const longlong2 *base = sp.partial + (size_t)blockIdx.z * sp.n_partial_slots * sp.partial_stride;
     longlong2 *dump = dump_hist ? tb.hist(level) : nullptr;
-    const int nn_max = (long)kf * nl <= kSparseCells ? nl : kSparseCells / kf;
+    const int nn_max = (long)kf * nl <= n_cells ? nl : n_cells / kf;
     for (int n0 = 0; n0 < nl; n0 += nn_max) {
         const int nn = min(nn_max, nl - n0);
         const int n_cells = kf * nn;
@@ -336,330 +349,451 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_big(TreeBuffers tb_all, Spa
         __syncthreads();
         sp_search_batch(tb, sh, cells, level, f, 1, bin0, n0, nn, big.cand_slot, mcw, lambda, dump);
     }
+    sp_publish(tb, sh, level);
 }
 
-// ------------------------------------------------------------------------------------ tail features
-// A feature with a few hundred stored values touches a few hundred (bin, node) cells of the thousands a table of
-// a deep level has. One wavefront takes such a feature: it loads the values (already ascending by bin), sorts them
-// stably by the node of their row (counting sort in LDS, ranks from ballots), and scans the sorted run: a forward
-// and a backward segmented sum per node give every position the node's sum up to it and after it, hence the left
-// sum and the feature total (missing = node sum - total). Candidates exist only where the left sum changes: the
-// feature's first bin (left empty) and the bin after every bin that holds a value - all bins in between repeat the
-// previous candidate's gain and lose the tie on the smaller index - so the result is what the scan of a complete
-// (bin, node) table gives. Every wavefront keeps its best key per node in LDS and owns one candidate slot in HBM.
-constexpr int kTailBlock = 64 * kSparseTailWaves;
-constexpr int kTailR = kSparseTailValues / 64;  // values per lane
+// ------------------------------------------------------------------------------------ sorted pass
+// Features with at most kSortedTile stored values. A task (one workgroup) owns a run of whole features and a tile of
+// the sorted-pass arrays; the tile holds the features' values in the order (feature, node of the level, bin), rows
+// in arrival order inside a bin. A level reads the previous level's order, looks up the node every value's row has
+// moved to, and partitions every (feature, node) run stably into the values of the left and of the right child;
+// the runs of nodes that did not split drop out (all rows of a node split or none, so a run is all live or all
+// dead). The new order goes back to HBM for the next level and is scanned right away: a forward and a backward
+// segmented sum per (feature, node) run give every position the run's sum up to it and after it, hence the left
+// sum and the feature's total in the node (missing = node sum - total). Candidates exist only where the left sum
+// changes: the feature's first bin (left side empty) and the bin after every bin that holds a value - the bins in
+// between repeat the previous candidate's gain and lose the tie on the smaller index - so the result is what the
+// scan of a complete (bin, node) table gives. The root level reads the static order and fetches the gradient pairs.
+constexpr int kSoV = kSortedPerThread;
+constexpr int kSoWaves = kSortedBlock / 64;
+constexpr unsigned kSoNodeMask = 0xfffu << kSortedNodeShift;
+// LDS position of tile position i: one element of padding after every 32, so that neither the lanes of a wavefront
+// that each own eight consecutive positions nor lanes at consecutive positions collide in a bank
+constexpr int kSoLds = kSortedTile + kSortedTile / 32;
+__device__ __forceinline__ int so_phys(int i) { return i + (i >> 5); }
 
-__device__ __forceinline__ long long shfl_down_ll(long long v, int d) {
-    int lo = __shfl_down((int)(unsigned)(unsigned long long)v, d);
-    int hi = __shfl_down((int)((unsigned long long)v >> 32), d);
+struct SoCount {
+    int seg;    // since the run began: values << 16 | values that go left
+    int plain;  // over the whole tile: dead values
+};
+struct SoSum {
+    long long g, h;
+};
+__device__ __forceinline__ void so_zero_seg(SoCount &a) { a.seg = 0; }
+__device__ __forceinline__ void so_add_seg(SoCount &a, const SoCount &b) { a.seg += b.seg; }
+__device__ __forceinline__ void so_add_plain(SoCount &a, const SoCount &b) { a.plain += b.plain; }
+__device__ __forceinline__ void so_zero_seg(SoSum &a) { a.g = a.h = 0; }
+__device__ __forceinline__ void so_add_seg(SoSum &a, const SoSum &b) {
+    a.g += b.g;
+    a.h += b.h;
+}
+__device__ __forceinline__ void so_add_plain(SoSum &, const SoSum &) {}
+
+template <bool FWD>
+__device__ __forceinline__ int so_shfl(int v, int d) {
+    return FWD ? __shfl_up(v, d) : __shfl_down(v, d);
+}
+template <bool FWD>
+__device__ __forceinline__ long long so_shfl(long long v, int d) {
+    const int lo = so_shfl<FWD>((int)(unsigned)(unsigned long long)v, d);
+    const int hi = so_shfl<FWD>((int)((unsigned long long)v >> 32), d);
     return (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
 }
-
-struct TailCand {
-    float score;
-    int index;
-    GHPair left;
-    unsigned long long key;
-};
-
-__device__ __forceinline__ TailCand tail_candidate(GHPair S, GHPair m, GHPair l, int index, bool ignored, float mcw,
-                                                   float lambda) {
-#pragma clang fp contract(off)
-    const float gr = split_gain(S, l, mcw, lambda);
-    const GHPair l2{l.g + m.g, l.h + m.h};
-    const float gl = split_gain(S, l2, mcw, lambda);
-    TailCand c;
-    c.score = (gl > gr) ? gl : -gr;
-    if (ignored) c.score = 0.f;
-    c.index = index;
-    c.left = l;
-    c.key = cand_key(fabsf(c.score), index);
-    return c;
+template <bool FWD>
+__device__ __forceinline__ SoCount so_shfl(SoCount v, int d) {
+    return SoCount{so_shfl<FWD>(v.seg, d), so_shfl<FWD>(v.plain, d)};
+}
+template <bool FWD>
+__device__ __forceinline__ SoSum so_shfl(SoSum v, int d) {
+    return SoSum{so_shfl<FWD>(v.g, d), so_shfl<FWD>(v.h, d)};
 }
 
-__global__ __launch_bounds__(kTailBlock) void k_sparse_tail(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
-                                                          const GHPair *__restrict__ gh, int level, float mcw,
-                                                          float lambda, int dump_hist) {
-#pragma clang fp contract(off)
-    extern __shared__ unsigned char dyn[];
-    __shared__ GHPair s_S[kSparseMaxLevelNodes];
-    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
-    gh += (size_t)blockIdx.z * tb.n;
-    const SparseTailTask task = sp.tail_tasks[blockIdx.x];
-    const int nl = 1 << level, off = nl - 1;
-    const int w = threadIdx.x >> 6, lane = lane_id();
-    // per wavefront: sorted sums (2 x 8 B), sorted (node << 8 | bin) keys, node counters, best keys
-    const size_t wave_bytes = (size_t)kSparseTailValues * 20 + (size_t)nl * 12;
-    unsigned char *base = dyn + (size_t)w * ((wave_bytes + 15) / 16 * 16);
-    long long *s_g = reinterpret_cast<long long *>(base);
-    long long *s_h = s_g + kSparseTailValues;
-    unsigned long long *s_key = reinterpret_cast<unsigned long long *>(s_h + kSparseTailValues);  // [nl]
-    unsigned *s_k = reinterpret_cast<unsigned *>(s_key + nl);                                   // [kSparseTailValues]
-    int *s_cnt = reinterpret_cast<int *>(s_k + kSparseTailValues);                              // [nl]
-    const int slot = task.cand_slot + w;
-    for (int x = threadIdx.x; x < nl; x += kTailBlock) s_S[x] = tb.nodes[off + x].sum_gh_pair;
-    for (int x = lane; x < nl; x += 64) {
-        s_key[x] = 0ull;
-        tb.cand[(size_t)x * tb.n_packs + slot].index = 0x7fffffff;
+// Inclusive segmented scan over the tile (thread t owns positions t * kSoV ..). FWD: v[j] becomes the sum from the
+// start of its run (brk = a run starts here) up to j; !FWD: from j to the end of its run (brk = a run ends here).
+// The `plain` part of T ignores the breaks. Two barriers; s_agg / s_flag are free again afterwards.
+template <typename T, bool FWD>
+__device__ void so_block_scan(T (&v)[kSoV], const bool (&brk)[kSoV], T *s_agg, int *s_flag) {
+    const int lane = lane_id(), w = wave_id();
+    T run{};
+    bool any = false;
+#pragma unroll
+    for (int jj = 0; jj < kSoV; ++jj) {
+        const int j = FWD ? jj : kSoV - 1 - jj;
+        if (brk[j]) {
+            so_zero_seg(run);
+            any = true;
+        }
+        so_add_seg(run, v[j]);
+        so_add_plain(run, v[j]);
+        v[j] = run;
+    }
+    T agg = run;
+    int flag = any ? 1 : 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const T o = so_shfl<FWD>(agg, d);
+        const int of = so_shfl<FWD>(flag, d);
+        const bool has = FWD ? lane >= d : lane + d < 64;
+        if (has) {
+            if (!flag) so_add_seg(agg, o);
+            so_add_plain(agg, o);
+            flag |= of;
+        }
+    }
+    T carry = so_shfl<FWD>(agg, 1);
+    int cflag = so_shfl<FWD>(flag, 1);
+    if (FWD ? lane == 0 : lane == 63) {
+        carry = T{};
+        cflag = 0;
+    }
+    if (FWD ? lane == 63 : lane == 0) {
+        s_agg[w] = agg;
+        s_flag[w] = flag;
     }
     __syncthreads();
-    const unsigned short *__restrict__ nid16 = tb.nid16;
+    T wc{};
+    if (FWD) {
+        for (int u = 0; u < w; ++u) {
+            if (s_flag[u]) so_zero_seg(wc);
+            so_add_seg(wc, s_agg[u]);
+            so_add_plain(wc, s_agg[u]);
+        }
+    } else {
+        for (int u = kSoWaves - 1; u > w; --u) {
+            if (s_flag[u]) so_zero_seg(wc);
+            so_add_seg(wc, s_agg[u]);
+            so_add_plain(wc, s_agg[u]);
+        }
+    }
+    if (!cflag) so_add_seg(carry, wc);
+    so_add_plain(carry, wc);
+    bool open = true;
+#pragma unroll
+    for (int jj = 0; jj < kSoV; ++jj) {
+        const int j = FWD ? jj : kSoV - 1 - jj;
+        if (brk[j]) open = false;
+        if (open) so_add_seg(v[j], carry);
+        so_add_plain(v[j], carry);
+    }
+    __syncthreads();
+}
+
+// split_gain with the node's own term (f.g^2 / (f.h + lambda), the same for every candidate of the node) taken from
+// a table: the same operations in the same order, hence the same bits
+__device__ __forceinline__ float so_gain(GHPair f, float fterm, GHPair l, float mcw, float lambda) {
+#pragma clang fp contract(off)
+    const GHPair r{f.g - l.g, f.h - l.h};
+    float gain = 0.f;
+    if (l.h >= mcw && r.h >= mcw) gain = (l.g * l.g) / (l.h + lambda) + (r.g * r.g) / (r.h + lambda) - fterm;
+    return fmaxf(0.f, gain);
+}
+
+// Upper estimate of so_gain from the hardware reciprocal (1 ulp) instead of divisions; -1: the weight gate closes
+__device__ __forceinline__ float so_gain_estimate(GHPair f, float fterm, GHPair l, float mcw, float lambda) {
+    const GHPair r{f.g - l.g, f.h - l.h};
+    if (!(l.h >= mcw && r.h >= mcw)) return -1.f;
+    const float a = l.g * l.g * __builtin_amdgcn_rcpf(l.h + lambda), b = r.g * r.g * __builtin_amdgcn_rcpf(r.h + lambda);
+    return (a + b - fterm) + (a + b + fabsf(fterm)) * 3.8146973e-6f;  // + 2^-18 of the terms: far above the roundings
+}
+
+// Signed score of a candidate (> 0: missing values go left), hist_tree_builder_single.cu:300-323. `floor`: the
+// largest |score| the candidate's node has seen so far; a candidate whose estimate stays below it cannot become the
+// node's best and is not evaluated (0 = no candidate).
+__device__ __forceinline__ float so_score(GHPair S, float fterm, GHPair m, GHPair l, bool ignored, float mcw,
+                                          float lambda, float floor) {
+#pragma clang fp contract(off)
+    const GHPair l2{l.g + m.g, l.h + m.h};
+    const float er = so_gain_estimate(S, fterm, l, mcw, lambda), el = so_gain_estimate(S, fterm, l2, mcw, lambda);
+    if (fmaxf(er, el) < floor || ignored) return 0.f;  // (column sampling: hist_tree_builder_single.cu:304 / :663)
+    const float gr = so_gain(S, fterm, l, mcw, lambda);
+    const float gl = so_gain(S, fterm, l2, mcw, lambda);
+    return (gl > gr) ? gl : -gr;
+}
+
+template <bool LEVEL0>
+__global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_all, SparsePass sp,
+                                                               const GHPair *__restrict__ gh, int level, float mcw,
+                                                               float lambda, int dump_hist) {
+#pragma clang fp contract(off)
+    extern __shared__ unsigned char so_dyn[];  // per node of the level: best key (8 bytes), sums (8), own gain term (4)
+    __shared__ int s_row[kSoLds];
+    __shared__ unsigned s_key[kSoLds];
+    __shared__ GHPair s_gh[kSoLds];
+    __shared__ unsigned short s_aux[kSoLds];  // first the left counts of the old runs, then the start of every value's run
+    __shared__ SoSum s_agg_sum[kSoWaves];
+    __shared__ SoCount s_agg_cnt[kSoWaves];
+    __shared__ int s_flag[kSoWaves];
+    __shared__ int s_dead;
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const SortedTask task = sp.sorted_tasks[blockIdx.x];
+    const int nl = 1 << level, off = nl - 1;
+    unsigned long long *s_best = reinterpret_cast<unsigned long long *>(so_dyn);
+    GHPair *s_S = reinterpret_cast<GHPair *>(s_best + nl);
+    float *s_P = reinterpret_cast<float *>(s_S + nl);
+    const size_t base = (size_t)blockIdx.z * (size_t)sp.n_sorted + (size_t)task.v_begin;
+    int *live = sp.sorted_live + ((size_t)blockIdx.z * kSortedLevels + level) * sp.n_sorted_tasks;
+    const int M = LEVEL0 ? task.count : live[(long)blockIdx.x - sp.n_sorted_tasks];
+    gh += (size_t)blockIdx.z * tb.n;
+    const int *__restrict__ in_row = LEVEL0 ? sp.sorted_row0 + task.v_begin : sp.srow(level - 1) + base;
+    const unsigned *__restrict__ in_key = LEVEL0 ? sp.sorted_key0 + task.v_begin : sp.skey(level - 1) + base;
+    const GHPair *__restrict__ in_gh = LEVEL0 ? nullptr : sp.sgh(level - 1) + base;
+    int *__restrict__ out_row = sp.srow(level) + base;
+    unsigned *__restrict__ out_key = sp.skey(level) + base;
+    GHPair *__restrict__ out_gh = sp.sgh(level) + base;
+    if (M == 0) {
+        if (threadIdx.x == 0) live[blockIdx.x] = 0;
+        return;
+    }
+    for (int x = threadIdx.x; x < nl; x += kSortedBlock) {
+        const GHPair S = tb.nodes[off + x].sum_gh_pair;
+        // what the other tasks have published so far: a candidate below it need not be looked at
+        s_best[x] = __hip_atomic_load(&tb.best_key[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_S[x] = S;
+        s_P[x] = (S.g * S.g) / (S.h + lambda);
+    }
+    // ---- the previous order into LDS with coalesced loads (position q = k * block + thread), every load of the
+    // thread in flight before the first one is used; the root level also fetches the gradient pair of every value's
+    // row here and takes the run starts (= feature starts) from the static arrays
+    {
+        int lrow[kSoV];
+        unsigned lkey[kSoV];
+        GHPair lgh[kSoV];
+        unsigned short lst[kSoV];
+#pragma unroll
+        for (int k = 0; k < kSoV; ++k) {
+            const int q = k * kSortedBlock + threadIdx.x;
+            lrow[k] = q < M ? in_row[q] : 0;
+            lkey[k] = q < M ? in_key[q] : 0u;
+            if (!LEVEL0) lgh[k] = q < M ? in_gh[q] : GHPair{0, 0};
+            if (LEVEL0) lst[k] = q < M ? sp.sorted_start0[task.v_begin + q] : (unsigned short)0;
+        }
+        if (LEVEL0) {
+#pragma unroll
+            for (int k = 0; k < kSoV; ++k) lgh[k] = gh[lrow[k]];  // (row 0 for the positions past the end)
+        }
+#pragma unroll
+        for (int k = 0; k < kSoV; ++k) {
+            const int q = k * kSortedBlock + threadIdx.x;
+            if (q < M) {
+                s_row[so_phys(q)] = lrow[k];
+                s_key[so_phys(q)] = lkey[k];
+                s_gh[so_phys(q)] = lgh[k];
+                if (LEVEL0) s_aux[so_phys(q)] = lst[k];
+            }
+        }
+    }
+    __syncthreads();
+    const int i0 = threadIdx.x * kSoV;
+    int Mn = M;  // values of the new order
+    if (!LEVEL0) {
+        const unsigned short *__restrict__ nid16 = tb.nid16;
+        int row[kSoV];
+        unsigned key[kSoV];
+        GHPair pair[kSoV];
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j) {
+            const int i = i0 + j;
+            row[j] = i < M ? s_row[so_phys(i)] : -1;
+            key[j] = i < M ? s_key[so_phys(i)] : 0xffffffffu;
+            pair[j] = i < M ? s_gh[so_phys(i)] : GHPair{0, 0};
+        }
+        const unsigned prevk = (i0 > 0 && i0 - 1 < M) ? s_key[so_phys(i0 - 1)] : 0xffffffffu;
+        const unsigned nextk = (i0 + kSoV < M) ? s_key[so_phys(i0 + kSoV)] : 0xffffffffu;
+        int xn[kSoV];
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j) {
+            xn[j] = row[j] >= 0 ? (int)nid16[row[j]] - off : -1;          // < 0: its node is a leaf
+            if ((key[j] & kSoNodeMask) == kSoNodeMask) xn[j] = -1;       // its run left the pass at the level above
+        }
+        SoCount fw[kSoV];
+        bool head[kSoV], tail[kSoV];
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j) {
+            const int i = i0 + j;
+            const bool valid = i < M;
+            const unsigned pk = j == 0 ? prevk : key[j > 0 ? j - 1 : 0];
+            const unsigned nk = j == kSoV - 1 ? nextk : key[j < kSoV - 1 ? j + 1 : 0];
+            head[j] = valid && (i == 0 || (pk >> kSortedNodeShift) != (key[j] >> kSortedNodeShift));
+            tail[j] = valid && (i == M - 1 || (nk >> kSortedNodeShift) != (key[j] >> kSortedNodeShift));
+            const bool alive = valid && xn[j] >= 0;
+            fw[j].seg = alive ? ((1 << 16) | ((xn[j] & 1) ? 0 : 1)) : 0;
+            fw[j].plain = (valid && !alive) ? 1 : 0;
+        }
+        // (the scan's barriers also make sure that every thread has taken its values out of the LDS arrays before
+        // the new order is written over them)
+        so_block_scan<SoCount, true>(fw, head, s_agg_cnt, s_flag);
+        if (threadIdx.x == kSortedBlock - 1) s_dead = fw[kSoV - 1].plain;  // (positions past the end add nothing)
+        // the last value of a run knows how many of the run go left: it leaves the count at the run's start
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j)
+            if (tail[j] && xn[j] >= 0)
+                s_aux[so_phys(i0 + j - ((fw[j].seg >> 16) - 1))] = (unsigned short)(fw[j].seg & 0xffff);
+        __syncthreads();
+        Mn = M - s_dead;
+        int pos[kSoV], start[kSoV];
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j) {
+            pos[j] = -1;
+            const int i = i0 + j;
+            if (i < M && xn[j] >= 0) {
+                const int cnt = fw[j].seg >> 16, lefts = fw[j].seg & 0xffff;  // inclusive
+                const int nleft = s_aux[so_phys(i - (cnt - 1))];               // of the whole run
+                const int s_new = i - (cnt - 1) - fw[j].plain;                 // the run's start once the dead are gone
+                const bool l = !(xn[j] & 1);
+                start[j] = l ? s_new : s_new + nleft;
+                pos[j] = l ? s_new + lefts - 1 : s_new + nleft + (cnt - 1) - lefts;
+            }
+        }
+        __syncthreads();  // every left count has been read: s_aux takes the run starts of the new order
+#pragma unroll
+        for (int j = 0; j < kSoV; ++j) {
+            if (pos[j] >= 0) {
+                const int pp = so_phys(pos[j]);
+                s_row[pp] = row[j];
+                s_key[pp] = (key[j] & ~kSoNodeMask) | ((unsigned)xn[j] << kSortedNodeShift);
+                s_gh[pp] = pair[j];
+                s_aux[pp] = (unsigned short)start[j];
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) live[blockIdx.x] = Mn;
+    if (Mn == 0) return;
+    // ---- rows and gradient pairs of the new order back to HBM (coalesced); the keys follow once the runs that leave
+    // the pass are marked
+    for (int q = threadIdx.x; q < Mn; q += kSortedBlock) {
+        out_row[q] = s_row[so_phys(q)];
+        out_gh[q] = s_gh[so_phys(q)];
+    }
+    unsigned key[kSoV];
+    SoSum fs[kSoV];
+    bool head[kSoV], tail[kSoV], last_of_bin[kSoV];
     const float scale_g = tb.quant->scale_g, scale_h = tb.quant->scale_h;
     const double inv_g = tb.quant->inv_g, inv_h = tb.quant->inv_h;
-    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    const GHPair *__restrict__ csc_gh = sp.csc_gh != nullptr ? sp.csc_gh + (size_t)blockIdx.z * sp.nnz : nullptr;
-    for (int fi = task.i_begin + w; fi < task.i_end; fi += kSparseTailWaves) {
-        const int f = sp.tail_feat[fi];
-        const int v0 = sp.feat_val_begin[f], m = sp.feat_val_begin[f + 1] - v0;
-        const int fbegin = tb.cut_row_ptr[f], kf = tb.cut_row_ptr[f + 1] - fbegin;
-        const bool ign = tb.ignored != nullptr && tb.ignored[f] != 0;
-        const int R = (m + 63) >> 6;  // rounds that hold values (the loops below stop there)
-        // ---- load: value a = r * 64 + lane of the feature, ascending by bin
-        int xs[kTailR], lbs[kTailR], posn[kTailR];
-        long long gq[kTailR], hq[kTailR];
-        {
-            int row[kTailR];
 #pragma unroll
-            for (int r = 0; r < kTailR; ++r) {
-                const int a = r * 64 + lane;
-                const bool in = r < R && a < m;
-                lbs[r] = in ? bins.csc_bin[v0 + a] - fbegin : 0;
-                row[r] = in ? bins.csc_row[v0 + a] : -1;
-            }
+    for (int j = 0; j < kSoV; ++j) {
+        const int p = i0 + j;
+        const bool in = p < Mn;
+        key[j] = in ? s_key[so_phys(p)] : 0xffffffffu;
+        fs[j] = SoSum{0, 0};
+        if (in) {
+            const GHPair s = s_gh[so_phys(p)];
+            fs[j].g = __float2ll_rn(s.g * scale_g);
+            fs[j].h = __float2ll_rn(s.h * scale_h);
+        }
+    }
+    {
+        const unsigned prevk = (i0 > 0 && i0 - 1 < Mn) ? s_key[so_phys(i0 - 1)] : 0xffffffffu;
+        const unsigned nextk = (i0 + kSoV < Mn) ? s_key[so_phys(i0 + kSoV)] : 0xffffffffu;
 #pragma unroll
-            for (int r = 0; r < kTailR; ++r) {
-                xs[r] = -1;
-                if (r < R && row[r] >= 0) xs[r] = (int)nid16[row[r]] - off;  // < 0: a leaf above
-            }
+        for (int j = 0; j < kSoV; ++j) {
+            const int p = i0 + j;
+            const bool in = p < Mn;
+            const unsigned pk = j == 0 ? prevk : key[j > 0 ? j - 1 : 0];
+            const unsigned nk = j == kSoV - 1 ? nextk : key[j < kSoV - 1 ? j + 1 : 0];
+            head[j] = in && (p == 0 || (pk >> kSortedNodeShift) != (key[j] >> kSortedNodeShift));
+            tail[j] = in && (p + 1 == Mn || (nk >> kSortedNodeShift) != (key[j] >> kSortedNodeShift));
+            last_of_bin[j] = in && (p + 1 == Mn || nk != key[j]);
+        }
+    }
+    if (dump_hist) {
+        // stage-wise inspection: the per-node histograms of the level (zeroed before the launch) get the values
+        unsigned long long *hist = reinterpret_cast<unsigned long long *>(tb.hist(level));
 #pragma unroll
-            for (int r = 0; r < kTailR; ++r) {
-                gq[r] = hq[r] = 0;
-                if (r < R && xs[r] >= 0) {
-                    const GHPair s = csc_gh != nullptr ? csc_gh[v0 + r * 64 + lane] : gh[row[r]];
-                    gq[r] = __float2ll_rn(s.g * scale_g);
-                    hq[r] = __float2ll_rn(s.h * scale_h);
-                }
+        for (int j = 0; j < kSoV; ++j) {
+            if (i0 + j < Mn) {
+                const int x = (int)((key[j] >> kSortedNodeShift) & 0xfffu), lb = (int)(key[j] & 0xffu);
+                const int fbegin = sp.sorted_meta[task.meta_begin + (int)(key[j] >> kSortedFeatShift)].x;
+                unsigned long long *cell = hist + 2 * ((size_t)x * tb.n_bins + fbegin + lb);
+                atomicAdd(cell, (unsigned long long)fs[j].g);
+                atomicAdd(cell + 1, (unsigned long long)fs[j].h);
             }
         }
-        if (dump_hist) {
-            // stage-wise inspection: the per-node histograms of the level (zeroed before the launch) get the values
-            unsigned long long *hist = reinterpret_cast<unsigned long long *>(tb.hist(level));
+    }
+    // (the scan's barriers: the stores above have read s_gh, which now takes the run totals)
+    so_block_scan<SoSum, true>(fs, head, s_agg_sum, s_flag);
+    // the last value of a run holds the run's sums = the feature's total in the node: as floats to the run's start
+    int start[kSoV];
 #pragma unroll
-            for (int r = 0; r < kTailR; ++r) {
-                if (xs[r] >= 0) {
-                    unsigned long long *cell = hist + 2 * ((size_t)xs[r] * tb.n_bins + fbegin + lbs[r]);
-                    atomicAdd(cell, (unsigned long long)gq[r]);
-                    atomicAdd(cell + 1, (unsigned long long)hq[r]);
-                }
-            }
+    for (int j = 0; j < kSoV; ++j) {
+        start[j] = (i0 + j < Mn) ? (int)s_aux[so_phys(i0 + j)] : 0;
+        if (tail[j])
+            s_gh[so_phys(start[j])] = GHPair{(float)((double)fs[j].g * inv_g), (float)((double)fs[j].h * inv_h)};
+    }
+    __syncthreads();
+    // ---- A (feature, node) run whose hessians add up to less than min_child_weight cannot yield a split, here or
+    // in any node below (hessians are not negative, so every left or right side taken from the run's values, and
+    // every run of a child node, weighs less still; the margin covers the float roundings of the missing-value
+    // arithmetic, a few ulps of the node's hessian sum). Such runs leave the pass: their keys get the node field's
+    // all-ones mark, which the next level reads as "dead". Not when the per-node histograms are being recorded.
+    GHPair tot[kSoV];
+    bool drop[kSoV];
+#pragma unroll
+    for (int j = 0; j < kSoV; ++j) {
+        drop[j] = false;
+        tot[j] = GHPair{0, 0};
+        const int p = i0 + j;
+        if (p < Mn) {
+            tot[j] = s_gh[so_phys(start[j])];
+            const float Sh = s_S[(key[j] >> kSortedNodeShift) & 0xfffu].h;
+            drop[j] = !dump_hist && tot[j].h + Sh * 4.76837158e-7f < mcw;  // 2^-21
+            if (drop[j]) s_key[so_phys(p)] = key[j] | kSoNodeMask;
         }
-        // ---- stable counting sort by node: rank inside the node from ballots, in arrival order
-        for (int x = lane; x < nl; x += 64) s_cnt[x] = 0;
-        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    for (int q = threadIdx.x; q < Mn; q += kSortedBlock) out_key[q] = s_key[so_phys(q)];
+    // ---- candidates: raise the node's key in LDS, then the winners publish. A candidate without gain never
+    // competes: the node's candidate at global bin 0 (a table feature's) has at least its key.
+    float sc_head[kSoV], sc_bin[kSoV];
 #pragma unroll
-        for (int r = 0; r < kTailR; ++r) {
-            if (r >= R) break;
-            const bool act = xs[r] >= 0;
-            unsigned long long mask = __ballot(act);
-            for (int bit = 0; bit < level; ++bit) {
-                const bool b = (xs[r] >> bit) & 1;
-                const unsigned long long bm = __ballot(act && b);
-                mask &= b ? bm : ~bm;
-            }
-            int first = 0;
-            if (act) {
-                const int rank = __popcll(mask & below);
-                if (rank == 0) {
-                    first = s_cnt[xs[r]];
-                    s_cnt[xs[r]] = first + __popcll(mask);
-                }
-                posn[r] = rank;
-            }
-            const int leader = act ? __ffsll((long long)mask) - 1 : lane;
-            first = __shfl(first, leader);
-            if (act) posn[r] += first;
-            __builtin_amdgcn_wave_barrier();
+    for (int j = 0; j < kSoV; ++j) {
+        sc_head[j] = sc_bin[j] = 0.f;
+        if (!(head[j] || last_of_bin[j]) || drop[j]) continue;
+        const int x = (int)((key[j] >> kSortedNodeShift) & 0xfffu), lb = (int)(key[j] & 0xffu);
+        const int fi = task.meta_begin + (int)(key[j] >> kSortedFeatShift);
+        const int2 meta = sp.sorted_meta[fi];
+        const bool ign = tb.ignored != nullptr && tb.ignored[sp.sorted_fid[fi]] != 0;
+        const GHPair S = s_S[x];
+        const float P = s_P[x];
+        const GHPair mm{S.g - tot[j].g, S.h - tot[j].h};
+        const float floor = __uint_as_float((unsigned)(s_best[x] >> 32));
+        if (head[j]) {
+            sc_head[j] = so_score(S, P, mm, GHPair{0, 0}, ign, mcw, lambda, floor);
+            if (sc_head[j] != 0.f) atomicMax(&s_best[x], cand_key(fabsf(sc_head[j]), meta.x));
         }
-        // exclusive scan of the node counters (a run of counters per lane)
-        int M;
-        {
-            const int per = (nl + 63) / 64;
-            const int i0 = lane * per, i1 = min(nl, i0 + per);
-            int local = 0;
-            for (int i = i0; i < i1; ++i) local += s_cnt[i];
-            int inc = local;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int t = __shfl_up(inc, d);
-                if (lane >= d) inc += t;
-            }
-            M = __shfl(inc, 63);
-            int run = inc - local;
-            for (int i = i0; i < i1; ++i) {
-                const int c = s_cnt[i];
-                s_cnt[i] = run;
-                run += c;
-            }
+        if (last_of_bin[j] && lb < meta.y - 1) {
+            const GHPair l{(float)((double)fs[j].g * inv_g), (float)((double)fs[j].h * inv_h)};
+            sc_bin[j] = so_score(S, P, mm, l, ign, mcw, lambda, floor);
+            if (sc_bin[j] != 0.f) atomicMax(&s_best[x], cand_key(fabsf(sc_bin[j]), meta.x + lb + 1));
         }
-        if (M == 0) continue;  // every value sits in a row that stopped in a leaf above this level
-        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
 #pragma unroll
-        for (int r = 0; r < kTailR; ++r) {
-            if (r >= R) break;
-            if (xs[r] >= 0) {
-                const int d = s_cnt[xs[r]] + posn[r];
-                s_g[d] = gq[r];
-                s_h[d] = hq[r];
-                s_k[d] = ((unsigned)xs[r] << 8) | (unsigned)lbs[r];
-            }
+    for (int j = 0; j < kSoV; ++j) {
+        if (sc_head[j] == 0.f && sc_bin[j] == 0.f) continue;
+        const int x = (int)((key[j] >> kSortedNodeShift) & 0xfffu), lb = (int)(key[j] & 0xffu);
+        const int fbegin = sp.sorted_meta[task.meta_begin + (int)(key[j] >> kSortedFeatShift)].x;
+        const unsigned long long best = s_best[x];
+        const bool win_head = sc_head[j] != 0.f && best == cand_key(fabsf(sc_head[j]), fbegin);
+        const bool win_bin = sc_bin[j] != 0.f && best == cand_key(fabsf(sc_bin[j]), fbegin + lb + 1);
+        if (!(win_head || win_bin)) continue;
+        // the tile's best of the node: worth publishing only if it beats what other tasks have published so far
+        if (best <= __hip_atomic_load(&tb.best_key[x], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) continue;
+        const GHPair S = s_S[x];
+        SplitCand o;
+        o.miss = GHPair{S.g - tot[j].g, S.h - tot[j].h};
+        o.pad[0] = o.pad[1] = 0;
+        if (win_head) {
+            o.score = sc_head[j];
+            o.index = fbegin;
+            o.left = GHPair{0, 0};  // the first bin records an empty left side (hist_tree_builder_single.cu:378)
+        } else {
+            o.score = sc_bin[j];
+            o.index = fbegin + lb + 1;
+            o.left = GHPair{(float)((double)fs[j].g * inv_g), (float)((double)fs[j].h * inv_h)};
         }
-        __builtin_amdgcn_wave_barrier();
-        // ---- scans over the sorted run: lane l owns positions [l * Rm, (l + 1) * Rm)
-        const int Rm = (M + 63) / 64;
-        const int p0 = lane * Rm;
-        unsigned k[kTailR];
-        long long Ig[kTailR], Ih[kTailR], Bg[kTailR], Bh[kTailR];
-        bool head[kTailR], tail[kTailR], last_of_bin[kTailR];
-        {
-            long long rg = 0, rh = 0;
-            bool any_head = false;
-#pragma unroll
-            for (int j = 0; j < kTailR; ++j) {
-                const int p = p0 + j;
-                const bool in = j < Rm && p < M;
-                k[j] = in ? s_k[p] : 0xffffffffu;
-                gq[j] = in ? s_g[p] : 0;
-                hq[j] = in ? s_h[p] : 0;
-                const unsigned prev = (in && p > 0) ? s_k[p - 1] : 0xffffffffu;
-                const unsigned next = (in && p + 1 < M) ? s_k[p + 1] : 0xffffffffu;
-                head[j] = in && (p == 0 || (prev >> 8) != (k[j] >> 8));
-                tail[j] = in && (p + 1 == M || (next >> 8) != (k[j] >> 8));
-                last_of_bin[j] = in && (p + 1 == M || next != k[j]);
-                if (head[j]) {
-                    rg = rh = 0;
-                    any_head = true;
-                }
-                rg += gq[j];
-                rh += hq[j];
-                Ig[j] = rg;
-                Ih[j] = rh;
-            }
-            long long ag = rg, ah = rh;
-            int flag = any_head ? 1 : 0;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const long long pg = shfl_up_ll(ag, d), ph = shfl_up_ll(ah, d);
-                const int pf = __shfl_up(flag, d);
-                if (lane >= d) {
-                    if (!flag) {
-                        ag += pg;
-                        ah += ph;
-                    }
-                    flag |= pf;
-                }
-            }
-            long long cg = shfl_up_ll(ag, 1), ch = shfl_up_ll(ah, 1);
-            if (lane == 0) cg = ch = 0;
-            bool seen = false;
-#pragma unroll
-            for (int j = 0; j < kTailR; ++j) {
-                if (head[j]) seen = true;
-                if (!seen) {
-                    Ig[j] += cg;
-                    Ih[j] += ch;
-                }
-            }
-        }
-        {
-            long long rg = 0, rh = 0;
-            bool any_tail = false;
-#pragma unroll
-            for (int j = kTailR - 1; j >= 0; --j) {
-                if (tail[j]) {
-                    rg = rh = 0;
-                    any_tail = true;
-                }
-                Bg[j] = rg;
-                Bh[j] = rh;
-                rg += gq[j];
-                rh += hq[j];
-            }
-            long long ag = rg, ah = rh;
-            int flag = any_tail ? 1 : 0;
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const long long pg = shfl_down_ll(ag, d), ph = shfl_down_ll(ah, d);
-                const int pf = __shfl_down(flag, d);
-                if (lane + d < 64) {
-                    if (!flag) {
-                        ag += pg;
-                        ah += ph;
-                    }
-                    flag |= pf;
-                }
-            }
-            long long cg = shfl_down_ll(ag, 1), ch = shfl_down_ll(ah, 1);
-            if (lane == 63) cg = ch = 0;
-            bool seen = false;
-#pragma unroll
-            for (int j = kTailR - 1; j >= 0; --j) {
-                if (tail[j]) seen = true;
-                if (!seen) {
-                    Bg[j] += cg;
-                    Bh[j] += ch;
-                }
-            }
-        }
-        // ---- candidates: raise the wavefront's key of the node, then the winners write their record. A candidate
-        // without gain never wins: the node's candidate at global bin 0 (a table feature's) has at least its key.
-        float sc_head[kTailR], sc_bin[kTailR];
-#pragma unroll
-        for (int j = 0; j < kTailR; ++j) {
-            sc_head[j] = sc_bin[j] = 0.f;
-            if (j >= Rm) break;
-            if (!(head[j] || last_of_bin[j])) continue;
-            const int x = (int)(k[j] >> 8), lb = (int)(k[j] & 0xffu);
-            const GHPair S = s_S[x];
-            const GHPair mm{S.g - (float)((double)(Ig[j] + Bg[j]) * inv_g), S.h - (float)((double)(Ih[j] + Bh[j]) * inv_h)};
-            if (head[j]) {
-                const TailCand c = tail_candidate(S, mm, GHPair{0, 0}, fbegin, ign, mcw, lambda);
-                sc_head[j] = c.score;
-                if (c.score != 0.f) atomicMax(&s_key[x], c.key);
-            }
-            if (last_of_bin[j] && lb < kf - 1) {
-                const GHPair l{(float)((double)Ig[j] * inv_g), (float)((double)Ih[j] * inv_h)};
-                const TailCand c = tail_candidate(S, mm, l, fbegin + lb + 1, ign, mcw, lambda);
-                sc_bin[j] = c.score;
-                if (c.score != 0.f) atomicMax(&s_key[x], c.key);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int j = 0; j < kTailR; ++j) {
-            if (j >= Rm) break;
-            if (sc_head[j] == 0.f && sc_bin[j] == 0.f) continue;
-            const int x = (int)(k[j] >> 8), lb = (int)(k[j] & 0xffu);
-            const unsigned long long best = s_key[x];
-            const bool win_head = sc_head[j] != 0.f && best == cand_key(fabsf(sc_head[j]), fbegin);
-            const bool win_bin = sc_bin[j] != 0.f && best == cand_key(fabsf(sc_bin[j]), fbegin + lb + 1);
-            if (!(win_head || win_bin)) continue;
-            const GHPair S = s_S[x];
-            SplitCand o;
-            o.miss = GHPair{S.g - (float)((double)(Ig[j] + Bg[j]) * inv_g), S.h - (float)((double)(Ih[j] + Bh[j]) * inv_h)};
-            o.pad[0] = o.pad[1] = 0;
-            if (win_head) {
-                o.score = sc_head[j];
-                o.index = fbegin;
-                o.left = GHPair{0, 0};  // the first bin records an empty left side (hist_tree_builder_single.cu:378)
-            } else {
-                o.score = sc_bin[j];
-                o.index = fbegin + lb + 1;
-                o.left = GHPair{(float)((double)Ig[j] * inv_g), (float)((double)Ih[j] * inv_h)};
-            }
-            tb.cand[(size_t)x * tb.n_packs + slot] = o;
-        }
-        __builtin_amdgcn_wave_barrier();
+        tb.cand[(size_t)x * tb.n_packs + task.cand_slot] = o;
+        atomicMax(&tb.best_key[x], best);
     }
 }
 
@@ -687,56 +821,85 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_partition(TreeBuffers tb_al
         if (cnt[i] != 0) atomicAdd(&tb.node_rows[2 * off + 1 + i], cnt[i]);  // children of level node x: 2 (off + x) + 1, + 2
 }
 
-__global__ __launch_bounds__(256) void k_sparse_gh_refresh(int n, long nnz, const int *__restrict__ csc_row,
-                                                          const GHPair *__restrict__ gh, GHPair *__restrict__ out) {
+// csc_gh[e] = gh[csc_row[e]] for the stored values of the table tasks (the sorted pass fetches its pairs itself)
+__global__ __launch_bounds__(256) void k_sparse_gh_refresh(int n, SparsePass sp, const int *__restrict__ csc_row,
+                                                          const GHPair *__restrict__ gh) {
     gh += (size_t)blockIdx.z * n;
-    out += (size_t)blockIdx.z * nnz;
-    for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < nnz; e += (long)gridDim.x * 256) out[e] = gh[csc_row[e]];
+    GHPair *__restrict__ out = sp.csc_gh + (size_t)blockIdx.z * sp.nnz;
+    const SparseTask task = sp.tasks[blockIdx.x];
+    for (int e = task.v_begin + threadIdx.x; e < task.v_end; e += 256) out[e] = gh[csc_row[e]];
+}
+
+// Static order of a sorted task's tile: its features one after the other, each in the order of the bin-major copy.
+__global__ __launch_bounds__(256) void k_sorted_setup(SparsePass sp, CsrBins bins, const int *__restrict__ cut_row_ptr,
+                                                     int *__restrict__ row0, unsigned *__restrict__ key0,
+                                                     unsigned short *__restrict__ start0) {
+    const SortedTask task = sp.sorted_tasks[blockIdx.x];
+    int dst = task.v_begin;
+    for (int fi = 0; fi < task.n_feat; ++fi) {
+        const int f = sp.sorted_fid[task.meta_begin + fi];
+        const int v0 = sp.feat_val_begin[f], m = sp.feat_val_begin[f + 1] - v0;
+        const int fbegin = cut_row_ptr[f];
+        for (int a = threadIdx.x; a < m; a += 256) {
+            row0[dst + a] = bins.csc_row[v0 + a];
+            key0[dst + a] = ((unsigned)fi << kSortedFeatShift) | (unsigned)(bins.csc_bin[v0 + a] - fbegin);
+            start0[dst + a] = (unsigned short)(dst - task.v_begin);
+        }
+        dst += m;
+    }
 }
 
 }  // namespace
 
+void launch_sorted_setup(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp, int *row0,
+                         unsigned *key0, unsigned short *start0) {
+    if (sp.n_sorted_tasks == 0) return;
+    k_sorted_setup<<<sp.n_sorted_tasks, 256, 0, s>>>(sp, bins, tb.cut_row_ptr, row0, key0, start0);
+}
+
 void launch_sparse_gh_refresh(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                               const GHPair *gh, int n_class) {
-    if (sp.csc_gh == nullptr || sp.nnz == 0) return;
-    const int grid = (int)std::min<long>(16384, (sp.nnz + 255) / 256);
-    k_sparse_gh_refresh<<<dim3(grid, 1, n_class), 256, 0, s>>>(tb.n, sp.nnz, bins.csc_row, gh, sp.csc_gh);
+    if (sp.csc_gh == nullptr || sp.n_tasks == 0) return;
+    k_sparse_gh_refresh<<<dim3(sp.n_tasks, 1, n_class), 256, 0, s>>>(tb.n, sp, bins.csc_row, gh);
 }
 
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                          const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class) {
-    const size_t lds = sizeof(longlong2) * (size_t)kSparseCells;
+    // LDS table of a table task: room for one feature of 255 bins with every node of the level, at least 2048 and at
+    // most kSparseCells cells (shallow levels: small tables, two workgroups per CU; deep levels: node ranges)
+    int n_cells = 2048;
+    while (n_cells < kSparseCells && n_cells < 256 * (1 << level)) n_cells *= 2;
+    const size_t lds = sizeof(longlong2) * (size_t)n_cells;
     if (dump_hist) {
-        // the table kernels store the cells of their features, the tail kernel adds its values: start from zero
+        // the table kernels store the cells of their features, the sorted pass adds its values: start from zero
         for (int k = 0; k < n_class; ++k)
             launch_fill_f32(s, reinterpret_cast<float *>(tb.for_class(k).hist(level)), 0.f,
                             (size_t)(1 << level) * tb.n_bins * 4);
     }
     static bool opted = false;
     if (!opted) {  // more than the default dynamic LDS window: opt in once
+        const size_t lds_max = sizeof(longlong2) * (size_t)kSparseCells;
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_sparse_level),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max));
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_sparse_big),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_max));
         opted = true;
     }
     if (sp.n_tasks > 0)
         k_sparse_level<<<dim3(sp.n_tasks, 1, n_class), kSpBlock, lds, s>>>(tb, bins, sp, gh, level, mcw, lambda,
-                                                                          dump_hist ? 1 : 0);
+                                                                          dump_hist ? 1 : 0, n_cells);
     if (sp.n_big > 0)
-        k_sparse_big<<<dim3(sp.n_big, 1, n_class), kSpBlock, lds, s>>>(tb, sp, level, mcw, lambda, dump_hist ? 1 : 0);
-    if (sp.n_tail_tasks > 0) {
-        const int nl = 1 << level;
-        const size_t wave_bytes = ((size_t)kSparseTailValues * 20 + (size_t)nl * 12 + 15) / 16 * 16;
-        const size_t tail_lds = wave_bytes * kSparseTailWaves;
-        static size_t tail_opted = 0;
-        if (tail_lds > 64 * 1024 && tail_lds > tail_opted) {
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_sparse_tail),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)tail_lds));
-            tail_opted = tail_lds;
-        }
-        k_sparse_tail<<<dim3(sp.n_tail_tasks, 1, n_class), kTailBlock, tail_lds, s>>>(tb, bins, sp, gh, level, mcw, lambda,
-                                                                                     dump_hist ? 1 : 0);
+        k_sparse_big<<<dim3(sp.n_big, 1, n_class), kSpBlock, lds, s>>>(tb, sp, level, mcw, lambda, dump_hist ? 1 : 0,
+                                                                      n_cells);
+    if (sp.n_sorted_tasks > 0) {
+        const int dh = dump_hist ? 1 : 0;
+        const size_t so_lds = (size_t)(1 << level) * 20;
+        if (level == 0)
+            k_sparse_sorted<true><<<dim3(sp.n_sorted_tasks, 1, n_class), kSortedBlock, so_lds, s>>>(
+                tb, sp, gh, level, mcw, lambda, dh);
+        else
+            k_sparse_sorted<false><<<dim3(sp.n_sorted_tasks, 1, n_class), kSortedBlock, so_lds, s>>>(
+                tb, sp, gh, level, mcw, lambda, dh);
     }
 }
 

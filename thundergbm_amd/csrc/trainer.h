@@ -89,6 +89,9 @@ class Trainer {
     CsrBins csr_;
     // sparse layout: one pass per level over the bin-major copy instead of per-node histograms (depth <= 11)
     bool sparse_pass_ = false;
+    int sparse_bin0_owner_ = -2;    // -2: not looked up yet
+    bool sparse_sorted_on_ = true;
+    bool sparse_feature_in_tables(int f);
     SparsePass sp_;
     void build_sparse_tasks();
     void ensure_hist_arena();  // per-node histograms for stage-wise inspection (the level pass itself keeps none)

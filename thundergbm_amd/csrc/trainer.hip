@@ -216,7 +216,21 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         if (nnz_ > 0 && (sparse_pass_ || !(ce != nullptr && std::string(ce) == "0"))) {
             PairSorter ps;
             ps.alloc(nnz_);
-            launch_csc_keys(stream_, n_, d_row_ptr, d_bin, ps.keys[0], ps.vals[0]);
+            // Sort key of every bin. The features that the level pass serves through (bin, node) tables need no bin
+            // order: all their bins share one key, so the stable sort leaves their values in row order - the row ->
+            // node map and the gradient pairs are then fetched at ascending, for frequent features nearly consecutive
+            // addresses, and neighbouring lanes add to different table cells.
+            int *d_sort_key = nullptr;
+            if (sparse_pass_) {
+                std::vector<int> sort_key((size_t)n_bins_);
+                for (int f = 0; f < F_; ++f)
+                    for (int b = h_cut_row_ptr_[f]; b < h_cut_row_ptr_[f + 1]; ++b)
+                        sort_key[(size_t)b] = sparse_feature_in_tables(f) ? h_cut_row_ptr_[f] : b;
+                HIP_CHECK(hipMalloc(&d_sort_key, sizeof(int) * (size_t)n_bins_));
+                upload(stream_, d_sort_key, sort_key.data(), sort_key.size());
+                HIP_CHECK(hipStreamSynchronize(stream_));
+            }
+            launch_csc_keys(stream_, n_, d_row_ptr, d_bin, d_sort_key, ps.keys[0], ps.vals[0]);
             int bits = 1;
             while (bits < 31 && (1l << bits) < (long)n_bins_) ++bits;
             const int cur = sort_pairs(stream_, ps, nnz_, bits);
@@ -224,6 +238,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
             launch_csc_unpack(stream_, nnz_, ps.keys[cur], ps.vals[cur], d_cbin, d_crow);
             HIP_CHECK(hipStreamSynchronize(stream_));
             ps.release();
+            if (d_sort_key != nullptr) HIP_CHECK(hipFree(d_sort_key));
             csr_.csc_bin = d_cbin;
             csr_.csc_row = d_crow;
             csr_.nnz = nnz_;
@@ -331,7 +346,8 @@ void Trainer::alloc_tree_buffers() {
     if (sparse_pass_) build_sparse_tasks();
     const size_t set_bytes =
         sparse_pass_ ? (size_t)n_ * 15 + (size_t)sp_.n_partial_slots * sp_.partial_stride * sizeof(longlong2) +
-                           (size_t)max_level_nodes * sp_.n_cand_slots * sizeof(SplitCand)
+                           (size_t)max_level_nodes * sp_.n_cand_slots * sizeof(SplitCand) +
+                           (size_t)sp_.n_sorted * 32 + (size_t)nnz_ * sizeof(GHPair)
                      : (size_t)n_ * 13 + ((size_t)2 * max_level_nodes * n_bins_ + tb.n_partial) * sizeof(longlong2) +
                            tb.n_end_bound * sizeof(int);
     size_t free_b = 0, total_b = 0;
@@ -398,6 +414,26 @@ void Trainer::alloc_tree_buffers() {
     pack_begin.push_back(n_bins_);
     tb.n_packs = sparse_pass_ ? sp_.n_cand_slots : (int)pack_begin.size() - 1;  // candidates per node
     if (sparse_pass_) {
+        tb.best_key = dalloc<unsigned long long>(S * (size_t)max_level_nodes);
+        HIP_CHECK(hipMemsetAsync(tb.best_key, 0, sizeof(unsigned long long) * S * (size_t)max_level_nodes, stream_));
+        if (sp_.n_sorted_tasks > 0) {
+            // static order of the sorted pass, then per set the two level orders and the live counts
+            int *row0 = dalloc<int>((size_t)sp_.n_sorted);
+            unsigned *key0 = dalloc<unsigned>((size_t)sp_.n_sorted);
+            unsigned short *start0 = dalloc<unsigned short>((size_t)sp_.n_sorted);
+            launch_sorted_setup(stream_, tb, csr_, sp_, row0, key0, start0);
+            sp_.sorted_row0 = row0;
+            sp_.sorted_key0 = key0;
+            sp_.sorted_start0 = start0;
+            for (int b = 0; b < 2; ++b) {
+                sp_.sorted_row[b] = dalloc<int>(S * (size_t)sp_.n_sorted);
+                sp_.sorted_key[b] = dalloc<unsigned>(S * (size_t)sp_.n_sorted);
+                sp_.sorted_gh[b] = dalloc<GHPair>(S * (size_t)sp_.n_sorted);
+            }
+            sp_.sorted_live = dalloc<int>(S * (size_t)kSortedLevels * sp_.n_sorted_tasks);
+            HIP_CHECK(hipMemsetAsync(sp_.sorted_live, 0, sizeof(int) * S * (size_t)kSortedLevels * sp_.n_sorted_tasks,
+                                     stream_));
+        }
         sp_.partial = dalloc<longlong2>(S * (size_t)sp_.n_partial_slots * sp_.partial_stride);
         // per-value gradient pairs in the order of the bin-major copy, when they fit comfortably
         sp_.nnz = nnz_;
@@ -558,28 +594,44 @@ void Trainer::ensure_hist_arena() {
     tb_.hist_q[1] = dalloc<longlong2>(cells);
 }
 
-// Work lists of the sparse level pass. Features with at most kSparseTailValues stored values go to the tail tasks
-// (one wavefront per feature); the others to table tasks: runs of consecutive such features with about
-// kSparseTaskValues values, a feature with more values than that cut into chunks (tasks of their own) whose tables
-// k_sparse_big adds up. The feature that owns global bin 0 is always a table feature (its table is searched for
-// every node even without values: the arg-max of a node without any positive gain ends there).
+// Which features the sparse level pass serves through (bin, node) tables: those with more values than a sorted-pass
+// tile holds, and the feature that owns global bin 0 (its table is searched for every node even without values: the
+// arg-max of a node without any positive gain ends there).
+bool Trainer::sparse_feature_in_tables(int f) {
+    if (sparse_bin0_owner_ == -2) {
+        sparse_bin0_owner_ = -1;
+        for (int q = 0; q < F_ && sparse_bin0_owner_ < 0; ++q)
+            if (h_cut_row_ptr_[q + 1] > h_cut_row_ptr_[q]) sparse_bin0_owner_ = q;
+        const char *se = std::getenv("TGBM_SPARSE_SORTED");  // "0": every feature through the tables (tests)
+        sparse_sorted_on_ = !(se != nullptr && std::string(se) == "0");
+    }
+    return !sparse_sorted_on_ || cuts_.feature_nnz[f] > kSortedTile || f == sparse_bin0_owner_;
+}
+
+// Work lists of the sparse level pass. Features with at most kSortedTile stored values go to the sorted pass (tasks:
+// runs of such features whose values fit one tile); the others to table tasks: runs of consecutive such features
+// with about kSparseTaskValues values, a feature with more values than that cut into chunks (tasks of their own)
+// whose tables k_sparse_big adds up. The feature that owns global bin 0 is always a table feature (its table is
+// searched for every node even without values: the arg-max of a node without any positive gain ends there).
 void Trainer::build_sparse_tasks() {
     std::vector<int> fvb(F_ + 1, 0);
     for (int f = 0; f < F_; ++f) fvb[f + 1] = fvb[f] + (int)cuts_.feature_nnz[f];
-    int bin0_owner = -1;
-    for (int f = 0; f < F_ && bin0_owner < 0; ++f)
-        if (h_cut_row_ptr_[f + 1] > h_cut_row_ptr_[f]) bin0_owner = f;
-    auto is_table = [&](int f) { return cuts_.feature_nnz[f] > kSparseTailValues || f == bin0_owner; };
+    auto is_table = [&](int f) { return sparse_feature_in_tables(f); };
     std::vector<SparseTask> tasks;
     std::vector<SparseBig> big;
-    std::vector<SparseTailTask> tail_tasks;
-    std::vector<int> tail_feat;
+    std::vector<SortedTask> sorted_tasks;
+    std::vector<int> sorted_fid;
+    std::vector<int2> sorted_meta;
+    std::vector<int> feat_slot(F_, -1);
     int n_small = 0, n_partial = 0, max_big_bins = 0;
     int f = 0;
     while (f < F_) {
         const long m = cuts_.feature_nnz[f];
         if (!is_table(f)) {
-            if (m > 0) tail_feat.push_back(f);
+            if (m > 0) {
+                sorted_fid.push_back(f);
+                sorted_meta.push_back(make_int2(h_cut_row_ptr_[f], h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f]));
+            }
             ++f;
             continue;
         }
@@ -605,19 +657,26 @@ void Trainer::build_sparse_tasks() {
             vals += cuts_.feature_nnz[fe];
             ++fe;
         }
+        for (int q = f; q < fe; ++q) feat_slot[q] = n_small;
         SparseTask t{f, fe, fvb[f], fvb[fe], n_small++, -1};
         tasks.push_back(t);
         f = fe;
     }
-    for (size_t i = 0; i < big.size(); ++i) big[i].cand_slot = n_small + (int)i;
+    for (size_t i = 0; i < big.size(); ++i) {
+        big[i].cand_slot = n_small + (int)i;
+        feat_slot[big[i].feature] = big[i].cand_slot;
+    }
     int next_slot = n_small + (int)big.size();
-    for (size_t i = 0; i < tail_feat.size();) {
+    long n_sorted = 0;
+    for (size_t i = 0; i < sorted_fid.size();) {
         size_t e = i;
         long vals = 0;
-        while (e < tail_feat.size() && (e == i || vals + cuts_.feature_nnz[tail_feat[e]] <= kSparseTailTaskValues))
-            vals += cuts_.feature_nnz[tail_feat[e++]];
-        tail_tasks.push_back(SparseTailTask{(int)i, (int)e, next_slot});
-        next_slot += kSparseTailWaves;
+        while (e < sorted_fid.size() && e - i < ((size_t)1 << (32 - kSortedFeatShift)) &&
+               vals + cuts_.feature_nnz[sorted_fid[e]] <= kSortedTile)
+            vals += cuts_.feature_nnz[sorted_fid[e++]];
+        for (size_t q = i; q < e; ++q) feat_slot[sorted_fid[q]] = next_slot;
+        sorted_tasks.push_back(SortedTask{(int)n_sorted, (int)vals, (int)i, (int)(e - i), next_slot++});
+        n_sorted += vals;
         i = e;
     }
     // the biggest tasks first: they decide when the level is done
@@ -625,29 +684,36 @@ void Trainer::build_sparse_tasks() {
                      [](const SparseTask &a, const SparseTask &b) { return a.v_end - a.v_begin > b.v_end - b.v_begin; });
     sp_.n_tasks = (int)tasks.size();
     sp_.n_big = (int)big.size();
-    sp_.n_tail_tasks = (int)tail_tasks.size();
+    sp_.n_sorted_tasks = (int)sorted_tasks.size();
+    sp_.n_sorted = n_sorted;
     sp_.n_cand_slots = std::max(1, next_slot);
     sp_.n_partial_slots = n_partial;
     sp_.partial_stride = (size_t)max_big_bins * (size_t)tb_.max_level_nodes;
     SparseTask *d_tasks = dalloc<SparseTask>(tasks.size());
     SparseBig *d_big = dalloc<SparseBig>(big.size());
-    SparseTailTask *d_tail = dalloc<SparseTailTask>(tail_tasks.size());
-    int *d_tail_feat = dalloc<int>(tail_feat.size());
+    SortedTask *d_sorted = dalloc<SortedTask>(sorted_tasks.size());
+    int *d_sorted_fid = dalloc<int>(sorted_fid.size());
+    int2 *d_sorted_meta = dalloc<int2>(sorted_meta.size());
+    int *d_feat_slot = dalloc<int>(feat_slot.size());
     int *d_fvb = dalloc<int>(fvb.size());
     upload(stream_, d_tasks, tasks.data(), tasks.size());
     upload(stream_, d_big, big.data(), big.size());
-    upload(stream_, d_tail, tail_tasks.data(), tail_tasks.size());
-    upload(stream_, d_tail_feat, tail_feat.data(), tail_feat.size());
+    upload(stream_, d_sorted, sorted_tasks.data(), sorted_tasks.size());
+    upload(stream_, d_sorted_fid, sorted_fid.data(), sorted_fid.size());
+    upload(stream_, d_sorted_meta, sorted_meta.data(), sorted_meta.size());
+    upload(stream_, d_feat_slot, feat_slot.data(), feat_slot.size());
     upload(stream_, d_fvb, fvb.data(), fvb.size());
     HIP_CHECK(hipStreamSynchronize(stream_));  // the host vectors go out of scope
     sp_.tasks = d_tasks;
     sp_.big = d_big;
-    sp_.tail_tasks = d_tail;
-    sp_.tail_feat = d_tail_feat;
+    sp_.sorted_tasks = d_sorted;
+    sp_.sorted_fid = d_sorted_fid;
+    sp_.sorted_meta = d_sorted_meta;
     sp_.feat_val_begin = d_fvb;
-    log_info("sparse level pass: %d table tasks, %d features in chunks (%d chunks), %zu tail features in %d tasks, "
-             "%d candidate slots per node", sp_.n_tasks, sp_.n_big, n_partial, tail_feat.size(), sp_.n_tail_tasks,
-             sp_.n_cand_slots);
+    tb_.feat_slot = d_feat_slot;
+    log_info("sparse level pass: %d table tasks, %d features in chunks (%d chunks), %zu features (%ld values) in %d "
+             "sorted tasks, %d candidate slots per node", sp_.n_tasks, sp_.n_big, n_partial, sorted_fid.size(), n_sorted,
+             sp_.n_sorted_tasks, sp_.n_cand_slots);
 }
 
 void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level, int n_class) {

@@ -1110,6 +1110,19 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
     }
     float best = -1.f;
     int best_idx = 0x7fffffff, best_pack = -1;
+    if (tb.best_key != nullptr) {
+        // sparse level pass: the tasks have already reduced their candidates to one key per node (larger |gain|,
+        // then smaller bin index); the record sits in the slot of the task that searches the winning bin's feature
+        if (threadIdx.x == 0) {
+            const unsigned long long key = tb.best_key[x_in];
+            tb.best_key[x_in] = 0ull;  // ready for the next level
+            if (key != 0ull) {
+                best_idx = (int)(0xffffffffu - (unsigned)key);
+                best_pack = tb.feat_slot[tb.cut_fid[best_idx]];
+                best = __uint_as_float((unsigned)(key >> 32));
+            }
+        }
+    } else
     for (int p = threadIdx.x; p < tb.n_packs; p += kBlock) {
         const SplitCand &c = tb.cand[(size_t)x_in * tb.n_packs + p];
         if (c.index == 0x7fffffff) continue;  // a wavefront whose features have no bins
@@ -1144,6 +1157,16 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
             best_idx = s_idx[i];
             best_pack = s_pack[i];
         }
+    }
+    if (best_pack < 0) {  // no candidate at all (a node none of whose rows stores a value): a leaf
+        SplitPoint z{};
+        z.nid = x;
+        z.split_fea_id = -1;
+        sp = z;
+        node.is_leaf = true;
+        tb.nodes[node.lch_index].is_valid = false;
+        tb.nodes[node.rch_index].is_valid = false;
+        return;
     }
     const SplitCand c = tb.cand[(size_t)x_in * tb.n_packs + best_pack];
     const int f = tb.cut_fid[c.index];
