@@ -27,11 +27,11 @@ def T():
 @pytest.fixture(autouse=True)
 def _default_layout():
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
-              "TGBM_SPARSE_SORTED"):
+              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS"):
         os.environ.pop(k, None)
     yield
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
-              "TGBM_SPARSE_SORTED"):
+              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS"):
         os.environ.pop(k, None)
 
 
@@ -607,8 +607,11 @@ def test_sparse_sorted_pass_equals_table_pass_on_deep_uneven_trees(T, mcw, gamma
               min_child_weight=mcw, gamma=gamma)
     runs = []
     try:
-        for srt in ("1", "0"):
+        # (TGBM_SPARSE_COLS=0: the row -> node update searches every row's bin ids instead of reading the frequent
+        # features' byte columns)
+        for srt, cols in (("1", "1"), ("0", "1"), ("1", "0")):
             os.environ["TGBM_SPARSE_SORTED"] = srt
+            os.environ["TGBM_SPARSE_COLS"] = cols
             s = T.Session(val, rp, col, y, **kw)
             assert s.info("sparse_pass") == 1
             s.boost(5)
@@ -616,7 +619,8 @@ def test_sparse_sorted_pass_equals_table_pass_on_deep_uneven_trees(T, mcw, gamma
             s.close()
     finally:
         os.environ.pop("TGBM_SPARSE_SORTED", None)
-    assert runs[0] == runs[1]
+        os.environ.pop("TGBM_SPARSE_COLS", None)
+    assert runs[0] == runs[1] == runs[2]
 
 
 def test_predict_transforms_through_the_c_abi(T):

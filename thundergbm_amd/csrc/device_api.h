@@ -107,6 +107,11 @@ struct CsrBins {
     const int *csc_bin = nullptr;  // [nnz]
     const int *csc_row = nullptr;  // [nnz]
     long nnz = 0;
+    // Sparse level pass: byte columns of the frequent features (local bin id of the row, kMissingBin = no stored
+    // value), column col_of_feature[f] at colbin + col * col_stride; col_of_feature[f] < 0: the feature has none
+    const uint8_t *colbin = nullptr;
+    const int *col_of_feature = nullptr;  // [F]
+    size_t col_stride = 0;
 };
 
 // Sparse layout, level pass: one pass per level over the bin-major copy of the stored values (sorted by global bin,
@@ -318,6 +323,9 @@ void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBin
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
                          const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1);
 void launch_sparse_partition(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
+// Byte columns of the frequent features (CsrBins::colbin, pre-filled with kMissingBin) from the bin-major copy.
+void launch_sparse_cols(hipStream_t s, long nnz, const int *csc_bin, const int *csc_row, const int *cut_fid,
+                        const int *cut_row_ptr, const int *col_of_feature, uint8_t *colbin, size_t col_stride);
 // Fills the static order of the sorted pass (row0 / key0, sp.n_sorted entries) from the bin-major copy.
 void launch_sorted_setup(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp, int *row0,
                          unsigned *key0, unsigned short *start0);

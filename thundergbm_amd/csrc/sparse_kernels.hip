@@ -332,13 +332,18 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_big(TreeBuffers tb_all, Spa
     }
     const longlong2 *base = sp.partial + (size_t)blockIdx.z * sp.n_partial_slots * sp.partial_stride;
     longlong2 *dump = dump_hist ? tb.hist(level) : nullptr;
-    const int nn_max = (long)kf * nl <= n_cells ? nl : n_cells / kf;
-    for (int n0 = 0; n0 < nl; n0 += nn_max) {
-        const int nn = min(nn_max, nl - n0);
+    // the level's nodes are shared out over gridDim.y workgroups (a feature of many chunks would otherwise add up
+    // megabytes of tables in one workgroup)
+    const int per = (nl + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int ny0 = min(nl, (int)blockIdx.y * per), ny1 = min(nl, ny0 + per);
+    const int nn_max = (long)kf * per <= n_cells ? per : n_cells / kf;
+    for (int n0 = ny0; n0 < ny1; n0 += nn_max) {
+        const int nn = min(nn_max, ny1 - n0);
         const int n_cells = kf * nn;
         __syncthreads();
         for (int c = threadIdx.x; c < n_cells; c += kSpBlock) {
             long long g = 0, h = 0;
+#pragma unroll 4
             for (int slot = big.slot_begin; slot < big.slot_end; ++slot) {
                 const longlong2 v = base[(size_t)slot * sp.partial_stride + (size_t)n0 * kf + c];
                 g += v.x;
@@ -811,8 +816,17 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_partition(TreeBuffers tb_al
         if (node < off) continue;  // the row stays in a leaf of an earlier level
         const TreeNode &nd = tb.nodes[node];
         if (!node_splits(nd)) continue;
-        const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
-        const bool right = csr_goes_right(bins, r, cb, ce, cb + nd.split_bid, nd.default_right);
+        const int col = bins.col_of_feature != nullptr ? bins.col_of_feature[nd.split_feature_id] : -1;
+        bool right;
+        if (col >= 0) {
+            // a frequent feature: the row's local bin id is one byte away (same rule: missing -> default direction,
+            // else right iff the bin is not below the split bin)
+            const int b = bins.colbin[(size_t)col * bins.col_stride + r];
+            right = b == kMissingBin ? (bool)nd.default_right : (b >= (int)nd.split_bid);
+        } else {
+            const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
+            right = csr_goes_right(bins, r, cb, ce, cb + nd.split_bid, nd.default_right);
+        }
         tb.nid16[r] = (unsigned short)(right ? nd.rch_index : nd.lch_index);
         atomicAdd(&cnt[2 * (node - off) + (right ? 1 : 0)], 1);
     }
@@ -828,6 +842,19 @@ __global__ __launch_bounds__(256) void k_sparse_gh_refresh(int n, SparsePass sp,
     GHPair *__restrict__ out = sp.csc_gh + (size_t)blockIdx.z * sp.nnz;
     const SparseTask task = sp.tasks[blockIdx.x];
     for (int e = task.v_begin + threadIdx.x; e < task.v_end; e += 256) out[e] = gh[csc_row[e]];
+}
+
+__global__ __launch_bounds__(256) void k_sparse_cols(long nnz, const int *__restrict__ csc_bin,
+                                                    const int *__restrict__ csc_row, const int *__restrict__ cut_fid,
+                                                    const int *__restrict__ cut_row_ptr,
+                                                    const int *__restrict__ col_of_feature, uint8_t *__restrict__ colbin,
+                                                    size_t col_stride) {
+    for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < nnz; e += (long)gridDim.x * 256) {
+        const int b = csc_bin[e];
+        const int f = cut_fid[b];
+        const int c = col_of_feature[f];
+        if (c >= 0) colbin[(size_t)c * col_stride + csc_row[e]] = (uint8_t)(b - cut_row_ptr[f]);
+    }
 }
 
 // Static order of a sorted task's tile: its features one after the other, each in the order of the bin-major copy.
@@ -850,6 +877,13 @@ __global__ __launch_bounds__(256) void k_sorted_setup(SparsePass sp, CsrBins bin
 }
 
 }  // namespace
+
+void launch_sparse_cols(hipStream_t s, long nnz, const int *csc_bin, const int *csc_row, const int *cut_fid,
+                        const int *cut_row_ptr, const int *col_of_feature, uint8_t *colbin, size_t col_stride) {
+    if (nnz == 0) return;
+    const int grid = (int)std::min<long>(16384, (nnz + 255) / 256);
+    k_sparse_cols<<<grid, 256, 0, s>>>(nnz, csc_bin, csc_row, cut_fid, cut_row_ptr, col_of_feature, colbin, col_stride);
+}
 
 void launch_sorted_setup(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp, int *row0,
                          unsigned *key0, unsigned short *start0) {
@@ -889,8 +923,8 @@ void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bi
         k_sparse_level<<<dim3(sp.n_tasks, 1, n_class), kSpBlock, lds, s>>>(tb, bins, sp, gh, level, mcw, lambda,
                                                                           dump_hist ? 1 : 0, n_cells);
     if (sp.n_big > 0)
-        k_sparse_big<<<dim3(sp.n_big, 1, n_class), kSpBlock, lds, s>>>(tb, sp, level, mcw, lambda, dump_hist ? 1 : 0,
-                                                                      n_cells);
+        k_sparse_big<<<dim3(sp.n_big, std::min(1 << level, 16), n_class), kSpBlock, lds, s>>>(
+            tb, sp, level, mcw, lambda, dump_hist ? 1 : 0, n_cells);
     if (sp.n_sorted_tasks > 0) {
         const int dh = dump_hist ? 1 : 0;
         const size_t so_lds = (size_t)(1 << level) * 20;

@@ -243,6 +243,37 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
             csr_.csc_row = d_crow;
             csr_.nnz = nnz_;
         }
+        if (sparse_pass_) {
+            // One byte per row (local bin id, 255 = no stored value) for the frequent features - the ones that win
+            // most splits: the row -> node update then takes a row's side from one byte instead of searching the
+            // row's bin ids. As many of the table features, most frequent first, as fit an eighth of the free memory.
+            std::vector<int> order;
+            for (int f = 0; f < F_; ++f)
+                if (cuts_.feature_nnz[f] > 0 && cuts_.feature_nnz[f] > kSortedTile) order.push_back(f);
+            std::stable_sort(order.begin(), order.end(),
+                             [&](int a, int b) { return cuts_.feature_nnz[a] > cuts_.feature_nnz[b]; });
+            HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+            const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
+            const char *ce2 = std::getenv("TGBM_SPARSE_COLS");  // "0": none (tests of the search path)
+            size_t n_cols = std::min(order.size(), free_b / 8 / col_stride);
+            if (ce2 != nullptr && std::string(ce2) == "0") n_cols = 0;
+            if (n_cols > 0) {
+                std::vector<int> col_of(F_, -1);
+                for (size_t c = 0; c < n_cols; ++c) col_of[order[c]] = (int)c;
+                int *d_col_of = dalloc<int>((size_t)F_);
+                upload(stream_, d_col_of, col_of.data(), col_of.size());
+                uint8_t *d_cols = dalloc<uint8_t>(n_cols * col_stride);
+                launch_fill_u8(stream_, d_cols, (uint8_t)kMissingBin, n_cols * col_stride);
+                launch_sparse_cols(stream_, nnz_, csr_.csc_bin, csr_.csc_row, cuts_.cut_fid, cuts_.cut_row_ptr, d_col_of,
+                                   d_cols, col_stride);
+                HIP_CHECK(hipStreamSynchronize(stream_));
+                csr_.col_of_feature = d_col_of;
+                csr_.colbin = d_cols;
+                csr_.col_stride = col_stride;
+                log_info("sparse level pass: %zu frequent features have a byte column (%.1f MB)", n_cols,
+                         (double)(n_cols * col_stride) * 1e-6);
+            }
+        }
         bins_.W = 4;
         bins_.n_blocks = 1;
         HIP_CHECK(hipStreamSynchronize(stream_));
