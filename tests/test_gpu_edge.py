@@ -668,3 +668,28 @@ def test_negative_column_index_is_rejected_before_any_kernel_uses_it(T):
         " 1, 0, None, 0)\n" % root)
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert out.returncode != 0 and "negative column index -1" in out.stderr, out.stderr
+
+
+def test_histogram_arena_that_cannot_fit_is_reported_with_the_depth_that_would(T):
+    """The per-node histogram paths keep two whole levels of node histograms. Wide data at depth 14 can ask for more
+    memory than the device has (here 1.2 M cut points: 2 x 8192 nodes x 1.2 M bins x 16 bytes = 315 GB): the trainer
+    says so, with the largest depth that fits, before it allocates anything. Runs in a child process: the library
+    aborts like the reference's CHECK."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import ctypes as C, sys, os\nimport numpy as np\nsys.path.insert(0, %r)\n"
+        "os.environ['TGBM_LAYOUT'] = 'sparse'\nimport thundergbm_amd\n"
+        "L = thundergbm_amd.load()\n"
+        "F, per = 20000, 60\n"
+        "col = np.tile(np.arange(F, dtype=np.int32), per)\n"
+        "val = np.repeat(np.arange(1, per + 1, dtype=np.float32), F)\n"
+        "n = 30000; nnz = F * per\n"
+        "rp = np.linspace(0, nnz, n + 1).astype(np.int32)\n"
+        "y = np.arange(n, dtype=np.float32) %% 7\n"
+        "p = lambda a: a.ctypes.data_as(C.c_void_p)\n"
+        "L.tgbm_trainer_create_grouped(n, p(val), p(rp), p(col), p(y), 14, 1, 1.0, 1.0, 1.0, 255, 1.0, b'reg:linear',"
+        " 1, 0, None, 0)\n" % root)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert out.returncode != 0 and "largest depth that fits" in out.stderr, out.stderr[-2000:]

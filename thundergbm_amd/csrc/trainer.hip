@@ -383,6 +383,21 @@ void Trainer::alloc_tree_buffers() {
                            tb.n_end_bound * sizeof(int);
     size_t free_b = 0, total_b = 0;
     HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    // The per-node paths keep the histograms of two whole levels (the reference sizes its `last_hist` against the
+    // free memory and rebuilds both siblings beyond the depth that fits, hist_tree_builder_single.cu:811-832; that
+    // fallback is not built here): say what is needed and which depth would fit instead of failing in hipMalloc.
+    if (set_bytes > free_b - free_b / 16) {
+        int fit = depth;
+        size_t need = set_bytes;
+        while (fit > 1 && need > free_b - free_b / 16) {
+            --fit;
+            const size_t ln = (size_t)1 << (fit - 1);
+            need = sparse_pass_ ? set_bytes : (size_t)n_ * 13 + ((size_t)2 * ln * n_bins_ + tb.n_partial) * sizeof(longlong2);
+        }
+        fatal("the tree buffers for depth %d need %.1f GB (two levels of %d node histograms x %d bins x 16 bytes), "
+              "%.1f GB are free; the largest depth that fits this data is %d", depth, (double)set_bytes * 1e-9,
+              max_level_nodes, n_bins_, (double)free_b * 1e-9, fit);
+    }
     const char *be = std::getenv("TGBM_BATCH_CLASSES");  // "0": build the trees of a round one after the other
     n_sets_ = (K > 1 && set_bytes * K < free_b / 2 && !(be != nullptr && std::string(be) == "0")) ? K : 1;
     tb.n_sets = n_sets_;
