@@ -198,8 +198,8 @@ struct TreeBuffers {
     longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
     QuantCtl *quant = nullptr;     // scales of the current tree
     int2 *hitem_shift = nullptr;   // [max_hitems] powers of two by which a dense work item (its node) coarsened (g, h)
-    // Root sums as exact integers at the tree's scales (what a row order cannot change): [0], [1] the sums,
-    // [2] a ticket counter of the kernel that adds them up (all zeroed by k_tree_init)
+    // Root sums as exact integers at the tree's scales (what a row order cannot change), from the gradients when no
+    // feature is stored in every row: [2 i], [2 i + 1] the sums of workgroup i of k_root_sum_rows (up to 256)
     // sparse level pass only (else nullptr): node every row has reached (heap id) and rows per node
     unsigned short *nid16 = nullptr;  // [n + 2]
     int *node_rows = nullptr;         // [n_nodes]
@@ -264,7 +264,7 @@ struct TreeBuffers {
         t.partial += K * n_partial;
         t.quant += K;
         t.hitem_shift += K * max_hitems;
-        t.root_total += K * 4;
+        t.root_total += K * 512;
         if (nid16 != nullptr) {
             t.nid16 += K * (((size_t)n + 2) / 2 * 2);
             t.node_rows += K * n_nodes;

@@ -290,6 +290,10 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         } else {
             W = 32;
         }
+        if (const char *we = std::getenv("TGBM_DENSE_W")) {  // block width override (measurements)
+            const int w = atoi(we);
+            if (w == 4 || w == 8 || w == 16 || w == 32 || w == 64) W = w;
+        }
         const int n_blocks = (F_ + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;
@@ -418,7 +422,7 @@ void Trainer::alloc_tree_buffers() {
     tb.partial = dalloc<longlong2>(S * tb.n_partial);
     tb.quant = dalloc<QuantCtl>(S);
     tb.hitem_shift = dalloc<int2>(S * (size_t)tb.max_hitems);
-    tb.root_total = dalloc<long long>(S * 4);
+    tb.root_total = dalloc<long long>(S * 512);
     // a feature that is stored in every row (checked on the bin matrix itself: a row with a repeated column index
     // would make the stored-value count lie): its bins add up to the root's sums
     tb.complete_feature = -1;
