@@ -240,6 +240,29 @@ struct TreeBuffers {
     // boosting round, so that the trees of a round can be built by the same launches, class = blockIdx.z).
     int n_sets = 1;
     int max_level_nodes = 0;
+    // Histogram arena smaller than the deepest level (it is sized against the free memory; the reference does the
+    // same with its last_hist buffer and builds both siblings from rows beyond the depth that fits,
+    // hist_tree_builder_single.cu:811-832, :544-570): hist_nodes node histograms per buffer. A level with more nodes
+    // is served in batches of nodes [lvl_x0, lvl_x1) (the buffer pointer is shifted so that node x still sits at
+    // x * n_bins); from level singles_from on no parent histogram exists any more, so every child of a split node
+    // is built from its own rows and the "pairs" of the work-item plan are single nodes.
+    int hist_nodes = 0;
+    int lvl_x0 = 0, lvl_x1 = 1 << 30;
+    int singles_from = 1 << 30;
+    __host__ __device__ bool singles(int level) const { return level >= singles_from; }
+    __host__ __device__ int n_hpairs(int level) const {
+        return level == 0 ? 1 : (singles(level) ? (1 << level) : (1 << (level - 1)));
+    }
+    __host__ __device__ int hpair_lo(int level) const { return singles(level) ? lvl_x0 : (lvl_x0 >> 1); }
+    __host__ __device__ int hpair_hi(int level) const {  // end of the pairs of the served nodes
+        const int n = n_hpairs(level);
+        const long hi = singles(level) ? (long)lvl_x1 : (((long)lvl_x1 + 1) >> 1);
+        return hi < n ? (int)hi : n;
+    }
+    __host__ __device__ int nodes_served(int level) const {
+        const int nl = 1 << level;
+        return (lvl_x1 < nl ? lvl_x1 : nl) - lvl_x0;
+    }
     size_t n_end_bound = 0, n_partial = 0;
 
     // Row list / histogram buffer of a level (selected without indexing an array member dynamically: a
@@ -259,8 +282,8 @@ struct TreeBuffers {
         t.ridx[0] += K * n;
         t.ridx[1] += K * n;
         t.goes_right += K * ((size_t)n + 4);
-        t.hist_q[0] += K * max_level_nodes * n_bins;
-        t.hist_q[1] += K * max_level_nodes * n_bins;
+        t.hist_q[0] += K * hist_nodes * n_bins;
+        t.hist_q[1] += K * hist_nodes * n_bins;
         t.partial += K * n_partial;
         t.quant += K;
         t.hitem_shift += K * max_hitems;

@@ -89,6 +89,7 @@ class Trainer {
     CsrBins csr_;
     // sparse layout: one pass per level over the bin-major copy instead of per-node histograms (depth <= 11)
     bool sparse_pass_ = false;
+    int hist_cap_level_ = -1;       // first level with more nodes than the histogram arena holds (-1: none)
     int sparse_bin0_owner_ = -2;    // -2: not looked up yet
     bool sparse_sorted_on_ = true;
     bool sparse_feature_in_tables(int f);

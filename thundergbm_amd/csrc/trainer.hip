@@ -379,29 +379,47 @@ void Trainer::alloc_tree_buffers() {
     // independent and are then built together (class = blockIdx.z of every launch).
     const int K = param_.tree_per_rounds;
     if (sparse_pass_) build_sparse_tasks();
+    // The per-node paths keep the node histograms of two levels. The reference sizes its `last_hist` buffer against
+    // the free memory and builds both siblings from rows beyond the depth that fits
+    // (hist_tree_builder_single.cu:811-832, :544-570); same here: the arena holds `hist_nodes` node histograms per
+    // buffer - all of the deepest level when that fits, else the largest power of two that does - and deeper levels
+    // are served in batches of that many nodes (find_split_sets). TGBM_HIST_ARENA_NODES caps it (tests).
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    int hist_nodes = max_level_nodes;
+    const size_t fixed_bytes = sparse_pass_ ? 0 : (size_t)n_ * 13 + tb.n_end_bound * sizeof(int);
+    auto arena_bytes = [&](int nodes) {  // two buffers + the work items' partial histograms (dense layout)
+        const size_t items = sparse_ ? 0 : (size_t)tb.target_hitems + (nodes < max_level_nodes ? nodes : max_pairs) + 2;
+        return ((size_t)2 * nodes + items) * (size_t)n_bins_ * sizeof(longlong2);
+    };
+    if (!sparse_pass_) {
+        if (const char *ae = std::getenv("TGBM_HIST_ARENA_NODES")) hist_nodes = std::max(2, std::min(hist_nodes, atoi(ae)));
+        const size_t budget = free_b - free_b / 8;
+        while (hist_nodes > 2 && fixed_bytes + arena_bytes(hist_nodes) > budget) hist_nodes /= 2;
+        int p2 = 1;
+        while (p2 * 2 <= hist_nodes) p2 *= 2;
+        hist_nodes = std::max(max_level_nodes >= 2 ? 2 : 1, p2);
+        TGBM_CHECK(fixed_bytes + arena_bytes(hist_nodes) <= free_b - free_b / 16,
+                   "the histograms of %d bins need %.1f GB for a %d-node arena, %.1f GB are free", n_bins_,
+                   (double)arena_bytes(hist_nodes) * 1e-9, hist_nodes, (double)free_b * 1e-9);
+        if (hist_nodes < max_level_nodes) {
+            // first level that does not fit: still has its parents (batches of sibling pairs); below it single nodes
+            int lc = 0;
+            while ((1 << lc) <= hist_nodes) ++lc;
+            hist_cap_level_ = lc;
+            tb.singles_from = lc + 1;
+            tb.max_hitems = tb.target_hitems + max_level_nodes + 1;  // every node of a level may add a partly filled item
+            tb.n_partial = sparse_ ? 1 : ((size_t)tb.target_hitems + hist_nodes + 2) * n_bins_;
+            log_info("histogram arena: %d node histograms per buffer (%.2f GB); levels from %d on are built in batches, "
+                     "both siblings from rows below level %d", hist_nodes, (double)arena_bytes(hist_nodes) * 1e-9, lc, lc);
+        }
+    }
+    tb.hist_nodes = hist_nodes;
     const size_t set_bytes =
         sparse_pass_ ? (size_t)n_ * 15 + (size_t)sp_.n_partial_slots * sp_.partial_stride * sizeof(longlong2) +
                            (size_t)max_level_nodes * sp_.n_cand_slots * sizeof(SplitCand) +
                            (size_t)sp_.n_sorted * 32 + (size_t)nnz_ * sizeof(GHPair)
-                     : (size_t)n_ * 13 + ((size_t)2 * max_level_nodes * n_bins_ + tb.n_partial) * sizeof(longlong2) +
-                           tb.n_end_bound * sizeof(int);
-    size_t free_b = 0, total_b = 0;
-    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-    // The per-node paths keep the histograms of two whole levels (the reference sizes its `last_hist` against the
-    // free memory and rebuilds both siblings beyond the depth that fits, hist_tree_builder_single.cu:811-832; that
-    // fallback is not built here): say what is needed and which depth would fit instead of failing in hipMalloc.
-    if (set_bytes > free_b - free_b / 16) {
-        int fit = depth;
-        size_t need = set_bytes;
-        while (fit > 1 && need > free_b - free_b / 16) {
-            --fit;
-            const size_t ln = (size_t)1 << (fit - 1);
-            need = sparse_pass_ ? set_bytes : (size_t)n_ * 13 + ((size_t)2 * ln * n_bins_ + tb.n_partial) * sizeof(longlong2);
-        }
-        fatal("the tree buffers for depth %d need %.1f GB (two levels of %d node histograms x %d bins x 16 bytes), "
-              "%.1f GB are free; the largest depth that fits this data is %d", depth, (double)set_bytes * 1e-9,
-              max_level_nodes, n_bins_, (double)free_b * 1e-9, fit);
-    }
+                     : fixed_bytes + arena_bytes(hist_nodes);
     const char *be = std::getenv("TGBM_BATCH_CLASSES");  // "0": build the trees of a round one after the other
     n_sets_ = (K > 1 && set_bytes * K < free_b / 2 && !(be != nullptr && std::string(be) == "0")) ? K : 1;
     tb.n_sets = n_sets_;
@@ -413,8 +431,8 @@ void Trainer::alloc_tree_buffers() {
     tb.ridx[1] = dalloc<int>(S * n_);
     tb.goes_right = dalloc<uint8_t>(S * ((size_t)n_ + 4));
     if (!sparse_pass_) {
-        tb.hist_q[0] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
-        tb.hist_q[1] = dalloc<longlong2>(S * max_level_nodes * n_bins_);
+        tb.hist_q[0] = dalloc<longlong2>(S * (size_t)hist_nodes * n_bins_);
+        tb.hist_q[1] = dalloc<longlong2>(S * (size_t)hist_nodes * n_bins_);
     } else {
         tb.nid16 = dalloc<unsigned short>(S * (((size_t)n_ + 2) / 2 * 2));
         tb.node_rows = dalloc<int>(S * tb.n_nodes);
@@ -642,6 +660,7 @@ void Trainer::ensure_hist_arena() {
                cells * 2 * sizeof(longlong2), free_b);
     tb_.hist_q[0] = dalloc<longlong2>(cells);
     tb_.hist_q[1] = dalloc<longlong2>(cells);
+    tb_.hist_nodes = tb_.max_level_nodes;
 }
 
 // Which features the sparse level pass serves through (bin, node) tables: those with more values than a sorted-pass
@@ -771,6 +790,26 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
         launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
         launch_sparse_gh_refresh(stream_, tb, csr_, sp_, gh, n_class);
     }
+    if (hist_cap_level_ >= 0 && level >= hist_cap_level_) {
+        // the level has more nodes than the histogram arena: batches of hist_nodes nodes, each through the whole
+        // chain histogram -> merge -> split search -> update before the next one overwrites the arena
+        const int nl = 1 << level;
+        for (int x0 = 0; x0 < nl; x0 += tb.hist_nodes) {
+            TreeBuffers tbb = tb;
+            tbb.lvl_x0 = x0;
+            tbb.lvl_x1 = std::min(nl, x0 + tb.hist_nodes);
+            // node x of the batch sits at (x - x0) * n_bins of the level's buffer (for every class set alike)
+            longlong2 *&cur = (level & 1) ? tbb.hist_q[1] : tbb.hist_q[0];
+            cur -= (size_t)x0 * n_bins_;
+            build_level_hist(tbb, level, gh, n_class);
+            if (!sparse_) launch_hist_merge(stream_, tbb, level, n_class);
+            launch_eval_split(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
+            launch_best_update(stream_, tbb, level, param_.rt_eps, param_.lambda, n_class);
+        }
+        lookup_level_ = level;
+        HIP_CHECK_LAUNCHES("find_split");
+        return;
+    }
     if (profiling_) {
         HistEvent ev;
         HIP_CHECK(hipEventCreate(&ev.start));
@@ -787,7 +826,8 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
     if (!sparse_pass_) {
         if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
         if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
-        // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them)
+        // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them); the
+        // last level that fits a capped arena keeps them for the batches of the next one
         launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
                           !(in_boost_ && level == param_.depth - 1));
     }

@@ -400,7 +400,7 @@ template <int LPR, bool DIRECT, int BLK, int SLOTS>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
-    __shared__ int s_range[4];
+    __shared__ int s_range[5];
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     gh += (size_t)blockIdx.z * tb.n;
     const int *__restrict__ ridx = tb.list(level);
@@ -435,12 +435,17 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
                                      quant->h_integer ? 0 : item_shift(quant->hq_max, rows, h_bits));
         s_range[2] = shift.x;
         s_range[3] = shift.y;
-        if (fb == 0) tb.hitem_shift[item] = shift;
+        const int x_in = node - ((1 << level) - 1);
+        s_range[4] = (x_in < tb.lvl_x0 || x_in >= tb.lvl_x1) ? 1 : 0;  // not in the batch of nodes this launch serves
+        if (fb == 0 && !s_range[4]) tb.hitem_shift[item] = shift;
     }
     for (int i = threadIdx.x; i < nb; i += BLK) lds[i] = 0ull;
     __syncthreads();
+    if (s_range[4]) return;
     // (values that are the same for every lane are moved to scalar registers)
     const int begin = __builtin_amdgcn_readfirstlane(s_range[0]), end = __builtin_amdgcn_readfirstlane(s_range[1]);
+    // (slots of `partial` count from the first item of the served batch of nodes: item 0 unless the arena is capped)
+    const int item0 = hpair_begin[tb.hpair_lo(level)];
     // the item's scales: powers of two well inside the float range, so the products below are exact
     const float scale_g = ldexpf(quant->scale_g, -__builtin_amdgcn_readfirstlane(s_range[2]));
     const float scale_h = ldexpf(quant->scale_h, -__builtin_amdgcn_readfirstlane(s_range[3]));
@@ -518,11 +523,11 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     if (c.hchunk <= kHistFlushRows) {
         // an item this short was never drained: its packed LDS words are the complete sums and go out as
         // they are (8 bytes per bin instead of 16; k_hist_merge unpacks them)
-        unsigned long long *out = reinterpret_cast<unsigned long long *>(partial) + (size_t)item * n_bins + bin0;
+        unsigned long long *out = reinterpret_cast<unsigned long long *>(partial) + (size_t)(item - item0) * n_bins + bin0;
         for (int i = threadIdx.x; i < nb; i += BLK) out[i] = lds[i];
         return;
     }
-    longlong2 *out = partial + (size_t)item * n_bins + bin0;
+    longlong2 *out = partial + (size_t)(item - item0) * n_bins + bin0;
 #pragma unroll
     for (int k = 0; k < SLOTS; ++k) {
         const int i = threadIdx.x + k * BLK;
@@ -553,12 +558,13 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     const int *__restrict__ hpair_begin = tb.hpair_begin;
     const int *__restrict__ hpair_built = tb.hpair_built;
     const int n_bins = tb.n_bins;
-    const int p = blockIdx.y;
+    const int p = blockIdx.y + tb.hpair_lo(level);
     const int built = hpair_built[p];
     if (built < 0) return;
     const int jl = threadIdx.x % kMergeBins, ig = threadIdx.x / kMergeBins;
     const int j = blockIdx.x * kMergeBins + jl;
     const int ib = hpair_begin[p], ie = hpair_begin[p + 1];
+    const int item0 = hpair_begin[tb.hpair_lo(level)];  // `partial` slots count from the served batch's first item
     long long sg = 0, sh = 0;
     if (j < n_bins) {
         // every item counted at its own scale (item_shift): shift its sums to the tree's
@@ -568,7 +574,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
             const int h_bits = tb.quant->h_bits;
             const unsigned long long h_mask = (1ull << h_bits) - 1ull;
             for (int it = ib + ig; it < ie; it += kMergeGroups) {
-                const unsigned long long t = packed[(size_t)it * n_bins + j];
+                const unsigned long long t = packed[(size_t)(it - item0) * n_bins + j];
                 const int2 s = shift[it];
                 const unsigned long long lo = t & h_mask;
                 sg += ((long long)(t - lo) >> h_bits) << s.x;
@@ -576,7 +582,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
             }
         } else {
             for (int it = ib + ig; it < ie; it += kMergeGroups) {
-                longlong2 v = partial[(size_t)it * n_bins + j];
+                longlong2 v = partial[(size_t)(it - item0) * n_bins + j];
                 const int2 s = shift[it];
                 sg += v.x << s.x;
                 sh += v.y << s.y;
@@ -594,7 +600,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     }
     const int off = (1 << level) - 1;
     cur_q[(size_t)(built - off) * n_bins + j] = make_longlong2(sg, sh);
-    if (level > 0) {
+    if (level > 0 && !tb.singles(level)) {
         const int sib = (built & 1) ? built + 1 : built - 1;
         const longlong2 par = prev_q[(size_t)p * n_bins + j];
         cur_q[(size_t)(sib - off) * n_bins + j] = make_longlong2(par.x - sg, par.y - sh);
@@ -713,7 +719,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_zero_built(TreeBuffers tb_all, 
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     longlong2 *__restrict__ cur_q = tb.hist(level);
     const int n_bins = tb.n_bins;
-    const int built = tb.hpair_built[blockIdx.y];
+    const int built = tb.hpair_built[blockIdx.y + tb.hpair_lo(level)];
     if (built < 0) return;
     const int off = (1 << level) - 1;
     longlong2 *h = cur_q + (size_t)(built - off) * n_bins;
@@ -739,6 +745,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_csr(TreeBuffers tb_all, CsrBins
         s_info[0] = b;
         s_info[1] = min(sg.y, b + c.hchunk);
         s_info[2] = node - ((1 << level) - 1);
+        if (s_info[2] < tb.lvl_x0 || s_info[2] >= tb.lvl_x1) s_info[1] = b;  // not in the served batch: no rows
     }
     __syncthreads();
     const int begin = s_info[0], end = s_info[1];
@@ -784,6 +791,7 @@ void k_hist_csr_head(TreeBuffers tb_all, CsrBins bins, const GHPair *__restrict_
         s_info[0] = b;
         s_info[1] = min(sg.y, b + c.hchunk);
         s_info[2] = node - ((1 << level) - 1);
+        if (s_info[2] < tb.lvl_x0 || s_info[2] >= tb.lvl_x1) s_info[1] = b;  // not in the served batch: no rows
     }
     for (int i = threadIdx.x; i < 2 * bins.head_bins; i += kHistBlock) lds[i] = 0ull;
     __syncthreads();
@@ -939,7 +947,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
     __shared__ GHPair s_miss[kWaves][kEvalPackBins];
     const int lane = lane_id(), w = wave_id();
     const int pack = blockIdx.x * kWaves + w;
-    const int x_in = blockIdx.y;
+    const int x_in = blockIdx.y + tb.lvl_x0;
     const int x = (1 << level) - 1 + x_in;
     const TreeNode nd = tb.nodes[x];
     const bool active = pack < tb.n_packs && nd.is_valid;
@@ -953,7 +961,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
     const double inv_g = tb.quant->inv_g, inv_h = tb.quant->inv_h;
     // SUB: is this node the sibling of the pair's built node?
     const longlong2 *h_par = nullptr, *h_built = nullptr;
-    if (SUB && level > 0 && active) {
+    if (SUB && level > 0 && active && !tb.singles(level)) {
         const int built = tb.hpair_built[x_in >> 1];
         if (built >= 0 && built != x) {
             h_par = tb.hist(level + 1) + (size_t)(x_in >> 1) * tb.n_bins;
@@ -1113,7 +1121,7 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
     __shared__ float s_abs[kWaves];
     __shared__ int s_idx[kWaves];
     __shared__ int s_pack[kWaves];
-    const int x_in = blockIdx.x;
+    const int x_in = blockIdx.x + tb.lvl_x0;
     const int x = (1 << level) - 1 + x_in;
     TreeNode &node = tb.nodes[x];
     SplitPoint &sp = tb.sp[x_in];
@@ -1323,6 +1331,66 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
     }
     if (threadIdx.x == 0) tb.pitem_loff[n_p] = carry;
     __syncthreads();
+    if (tb.singles(level + 1)) {
+        // No parent histograms below this level (the arena is smaller than the level): every child of a split node
+        // is built from its own rows; the plan's "pairs" are the 2 nl single nodes of the next level.
+        int rows_sum = 0, n_built = 0;
+        for (int x_in = threadIdx.x; x_in < nl; x_in += kBlock) {
+            const TreeNode &nd = tb.nodes[off + x_in];
+            const int2 sg = tb.seg[off + x_in];
+            if (node_splits(nd)) {
+                const int nleft = tb.pitem_loff[pb_cur[x_in + 1]] - tb.pitem_loff[pb_cur[x_in]];
+                tb.node_nleft[x_in] = nleft;
+                tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
+                tb.seg[nd.rch_index] = make_int2(sg.x + nleft, sg.y);
+                tb.hpair_built[2 * x_in] = nd.lch_index;
+                tb.hpair_built[2 * x_in + 1] = nd.rch_index;
+                rows_sum += sg.y - sg.x;
+                n_built += 2;
+            } else {
+                tb.node_nleft[x_in] = 0;
+                tb.seg[nd.lch_index] = make_int2(0, 0);
+                tb.seg[nd.rch_index] = make_int2(0, 0);
+                tb.hpair_built[2 * x_in] = -1;
+                tb.hpair_built[2 * x_in + 1] = -1;
+            }
+        }
+        const int total_rows = block_sum(rows_sum, lds);
+        n_built = block_sum(n_built, lds);
+        const int room = max(tb.target_hitems / 4, tb.target_hitems - n_built);
+        int chunk = (total_rows + room - 1) / room;
+        chunk = max(kHistMinChunk, (chunk + 255) / 256 * 256);
+        int hcarry = 0, pcarry = 0;
+        for (int base = 0; base < 2 * nl; base += kBlock) {
+            const int c_in = base + threadIdx.x;
+            int cnt = 0, pc = 0;
+            if (c_in < 2 * nl) {
+                const int2 sg = tb.seg[2 * nl - 1 + c_in];  // the child's heap id: (2 nl - 1) + c_in
+                if (tb.hpair_built[c_in] >= 0) cnt = (sg.y - sg.x + chunk - 1) / chunk;
+                pc = (sg.y - sg.x + kPartChunk - 1) / kPartChunk;
+            }
+            int tot, ptot;
+            const int ex = block_excl_scan(cnt, lds, &tot);
+            const int pex = block_excl_scan(pc, lds, &ptot);
+            if (c_in < 2 * nl) {
+                tb.hpair_begin[c_in] = hcarry + ex;
+                pb_next[c_in] = pcarry + pex;
+            }
+            hcarry += tot;
+            pcarry += ptot;
+        }
+        if (threadIdx.x == 0) {
+            tb.hpair_begin[2 * nl] = hcarry;
+            pb_next[2 * nl] = pcarry;
+            LevelCtl c;
+            c.hchunk = chunk;
+            c.n_hitems = hcarry;
+            c.n_pitems = pcarry;
+            c.rows_built = total_rows;
+            tb.ctl[level + 1] = c;
+        }
+        return;
+    }
     if (nl <= kBlock) {
         // the usual case (levels up to 8): one node per thread, everything after the scan stays in registers
         const int x_in = threadIdx.x;
@@ -1936,7 +2004,7 @@ void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_cla
 template <int LPR, int SLOTS>
 static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                               int level, int n_class) {
-    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    const int n_pairs = tb.n_hpairs(level);
     dim3 grid(tb.max_hitems, bins.n_blocks, n_class);
     size_t lds = (size_t)tb.max_block_bins * sizeof(unsigned long long);
     if (lds > 64 * 1024) {
@@ -1986,7 +2054,7 @@ void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bi
 }
 
 void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_class) {
-    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    const int n_pairs = tb.hpair_hi(level) - tb.hpair_lo(level);  // of the served nodes
     if (tb.target_hitems <= 16) {
         // wide data: many feature blocks, so a node has only a handful of work items and very long histograms;
         // one thread per bin walks them (a block of 8 bins would leave most of its 32 groups without an item)
@@ -2024,9 +2092,9 @@ long device_count_bytes(hipStream_t s, const uint8_t *d_v, size_t n, uint8_t val
 
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
                      int n_class) {
-    const int n_pairs = level == 0 ? 1 : (1 << (level - 1));
+    const int n_pairs = tb.n_hpairs(level);
     const int zgrid = std::min(1024, (tb.n_bins + kBlock - 1) / kBlock);
-    k_hist_zero_built<<<dim3(zgrid, n_pairs, n_class), kBlock, 0, s>>>(tb, level);
+    k_hist_zero_built<<<dim3(zgrid, tb.hpair_hi(level) - tb.hpair_lo(level), n_class), kBlock, 0, s>>>(tb, level);
     const size_t lds = (size_t)bins.head_bins * 2 * sizeof(unsigned long long);
     if (bins.hist_word != nullptr && lds > 64 * 1024) {
         static size_t opted = 0;  // more than the default dynamic LDS window: opt in once
@@ -2057,13 +2125,13 @@ void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, 
 
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class,
                        bool store_sibling) {
-    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, 1 << level, n_class);
+    dim3 grid((tb.n_packs + kWaves - 1) / kWaves, tb.nodes_served(level), n_class);
     if (tb.sparse) k_eval_split<true><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, store_sibling);
     else k_eval_split<false><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, true);
 }
 
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class) {
-    k_best_update<<<dim3(1 << level, 1, n_class), kBlock, 0, s>>>(tb, level, rt_eps, lambda);
+    k_best_update<<<dim3(tb.nodes_served(level), 1, n_class), kBlock, 0, s>>>(tb, level, rt_eps, lambda);
 }
 
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class) {
