@@ -167,7 +167,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     if (sparse_) {
         // TGBM_SPARSE_PASS=0 keeps the row-list kernels with per-node histograms in HBM (tests compare the two)
         const char *pe = std::getenv("TGBM_SPARSE_PASS");
-        sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && !(pe != nullptr && std::string(pe) == "0");
+        sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && nnz_ < (1l << 31) && !(pe != nullptr && std::string(pe) == "0");
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
         // Head of the histogram: the most frequent features whose bins fit the LDS slots. Worth it when
         // they carry a real share of the stored values (skewed, e.g. Zipf-distributed, feature usage).
@@ -673,6 +673,11 @@ bool Trainer::sparse_feature_in_tables(int f) {
             if (h_cut_row_ptr_[q + 1] > h_cut_row_ptr_[q]) sparse_bin0_owner_ = q;
         const char *se = std::getenv("TGBM_SPARSE_SORTED");  // "0": every feature through the tables (tests)
         sparse_sorted_on_ = !(se != nullptr && std::string(se) == "0");
+        // the sorted pass keeps 40 bytes per stored value of its features for every class tree built together;
+        // it is left out when that would take more than a quarter of the free memory
+        size_t free_b = 0, total_b = 0;
+        HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+        if ((size_t)nnz_ * 40 * (size_t)std::max(1, param_.tree_per_rounds) > free_b / 4) sparse_sorted_on_ = false;
     }
     return !sparse_sorted_on_ || cuts_.feature_nnz[f] > kSortedTile || f == sparse_bin0_owner_;
 }
