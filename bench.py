@@ -34,8 +34,12 @@ CONFIGS = {
 }
 
 
-KERNEL_SOURCES = ["thundergbm_amd/csrc/tree_kernels.hip", "thundergbm_amd/csrc/trainer.hip",
+KERNEL_SOURCES = ["thundergbm_amd/csrc/tree_kernels.hip", "thundergbm_amd/csrc/sparse_kernels.hip",
+                  "thundergbm_amd/csrc/kernel_common.h", "thundergbm_amd/csrc/trainer.hip",
                   "thundergbm_amd/csrc/device_api.h"]
+# counter summary of a configuration's histogram kernels under profiles/
+PMC_SUMMARY = {2: "k_hist_dense_config2_pmc.txt", 3: "k_hist_dense_config3_pmc.txt",
+               4: "sparse_level_pass_config4_pmc.txt", 5: "k_hist_dense_config5_pmc.txt"}
 
 
 def kernel_sources_sha1():
@@ -50,10 +54,11 @@ def kernel_sources_sha1():
 
 
 def traffic_from_profile(config):
-    """HBM bytes per histogram launch from the committed rocprofv3 --pmc summary of this configuration (FETCH_SIZE
+    """HBM bytes per histogram launch (for the sparse level pass: per level, i.e. its table, chunk-sum and sorted
+    kernels together) from the committed rocprofv3 --pmc summary of this configuration (FETCH_SIZE
     and WRITE_SIZE runs, calibrated against a plain copy kernel), with where it comes from. The figure is only
     passed on when the summary was measured with the kernel sources as they are now; else it would be stale."""
-    rel = os.path.join("profiles", "k_hist_dense_config%d_pmc.txt" % config)
+    rel = os.path.join("profiles", PMC_SUMMARY[config])
     value = sha = None
     try:
         for line in open(os.path.join(ROOT, rel)):

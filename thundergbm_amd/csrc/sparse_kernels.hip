@@ -591,7 +591,7 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     const int i0 = threadIdx.x * kSoV;
     int Mn = M;  // values of the new order
     if (!LEVEL0) {
-        const unsigned short *__restrict__ nid16 = tb.nid16;
+        const ulonglong2 *__restrict__ row_side = tb.row_side;
         int row[kSoV];
         unsigned key[kSoV];
         GHPair pair[kSoV];
@@ -607,8 +607,15 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
         int xn[kSoV];
 #pragma unroll
         for (int j = 0; j < kSoV; ++j) {
-            xn[j] = row[j] >= 0 ? (int)nid16[row[j]] - off : -1;          // < 0: its node is a leaf
-            if ((key[j] & kSoNodeMask) == kSoNodeMask) xn[j] = -1;       // its run left the pass at the level above
+            // the value's node of the level above is in its key; the row -> node update left two bits per row: did
+            // the node split, and did the row go right
+            xn[j] = -1;  // the node is a leaf, or the run left the pass at the level above (mark in the key)
+            if (row[j] >= 0 && (key[j] & kSoNodeMask) != kSoNodeMask) {
+                const ulonglong2 sd = row_side[row[j] >> 6];
+                const int bit = row[j] & 63;
+                if ((sd.x >> bit) & 1ull)
+                    xn[j] = 2 * (int)((key[j] >> kSortedNodeShift) & 0xfffu) + (int)((sd.y >> bit) & 1ull);
+            }
         }
         SoCount fw[kSoV];
         bool head[kSoV], tail[kSoV];
@@ -811,24 +818,33 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_partition(TreeBuffers tb_al
     const int nl = 1 << level, off = nl - 1;
     for (int i = threadIdx.x; i < 2 * nl; i += kSpBlock) cnt[i] = 0;
     __syncthreads();
-    for (int r = blockIdx.x * kSpBlock + threadIdx.x; r < tb.n; r += gridDim.x * kSpBlock) {
-        const int node = tb.nid16[r];
-        if (node < off) continue;  // the row stays in a leaf of an earlier level
-        const TreeNode &nd = tb.nodes[node];
-        if (!node_splits(nd)) continue;
-        const int col = bins.col_of_feature != nullptr ? bins.col_of_feature[nd.split_feature_id] : -1;
-        bool right;
-        if (col >= 0) {
-            // a frequent feature: the row's local bin id is one byte away (same rule: missing -> default direction,
-            // else right iff the bin is not below the split bin)
-            const int b = bins.colbin[(size_t)col * bins.col_stride + r];
-            right = b == kMissingBin ? (bool)nd.default_right : (b >= (int)nd.split_bid);
-        } else {
-            const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
-            right = csr_goes_right(bins, r, cb, ce, cb + nd.split_bid, nd.default_right);
+    // (every wavefront takes 64 consecutive rows per step and stays together, for the ballots at the end of the step)
+    const int n64 = (tb.n + 63) & ~63;
+    for (int r = blockIdx.x * kSpBlock + threadIdx.x; r < n64; r += gridDim.x * kSpBlock) {
+        bool moved = false, right = false;
+        if (r < tb.n) {
+            const int node = tb.nid16[r];
+            if (node >= off) {  // (else the row stays in a leaf of an earlier level)
+                const TreeNode &nd = tb.nodes[node];
+                if (node_splits(nd)) {
+                    moved = true;
+                    const int col = bins.col_of_feature != nullptr ? bins.col_of_feature[nd.split_feature_id] : -1;
+                    if (col >= 0) {
+                        // a frequent feature: the row's local bin id is one byte away (same rule: missing -> default
+                        // direction, else right iff the bin is not below the split bin)
+                        const int b = bins.colbin[(size_t)col * bins.col_stride + r];
+                        right = b == kMissingBin ? (bool)nd.default_right : (b >= (int)nd.split_bid);
+                    } else {
+                        const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
+                        right = csr_goes_right(bins, r, cb, ce, cb + nd.split_bid, nd.default_right);
+                    }
+                    tb.nid16[r] = (unsigned short)(right ? nd.rch_index : nd.lch_index);
+                    atomicAdd(&cnt[2 * (node - off) + (right ? 1 : 0)], 1);
+                }
+            }
         }
-        tb.nid16[r] = (unsigned short)(right ? nd.rch_index : nd.lch_index);
-        atomicAdd(&cnt[2 * (node - off) + (right ? 1 : 0)], 1);
+        const unsigned long long mv = __ballot(moved), rt = __ballot(moved && right);
+        if (lane_id() == 0) tb.row_side[r >> 6] = make_ulonglong2(mv, rt);
     }
     __syncthreads();
     for (int i = threadIdx.x; i < 2 * nl; i += kSpBlock)
