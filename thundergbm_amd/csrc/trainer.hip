@@ -290,10 +290,6 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         } else {
             W = 32;
         }
-        if (const char *we = std::getenv("TGBM_DENSE_W")) {  // block width override (measurements)
-            const int w = atoi(we);
-            if (w == 4 || w == 8 || w == 16 || w == 32 || w == 64) W = w;
-        }
         const int n_blocks = (F_ + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;
