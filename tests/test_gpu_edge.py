@@ -712,3 +712,84 @@ def test_capped_histogram_arena_gives_the_same_trees(T, layout, objective, kind)
         return
     same = [[a == b for a, b in zip(runs[0], r)] for r in runs[1:]]  # (model, predictions, row -> node map)
     assert same == [[True] * 3] * 2, same
+
+
+def test_split_search_per_feature_and_node_equals_the_packed_one(T):
+    """The split search for features of any number of bins (one workgroup per (feature, node), chunks of 256 bins
+    with a carried prefix) against the packed one (a wavefront per run of whole features of at most 256 bins) on
+    data both can serve: same candidates, gains and tie rule, so the same bytes. TGBM_WIDE_EVAL=1 switches it on
+    for the CSR layout's per-node path."""
+    os.environ["TGBM_LAYOUT"] = "sparse"
+    os.environ["TGBM_SPARSE_PASS"] = "0"
+    n, F = 6000, 9
+    val, rp, col = _ragged(n, F, 41, 8)
+    runs = []
+    try:
+        for objective, kind in (("reg:linear", "reg"), ("binary:logistic", "bin")):
+            y = _target(val, rp, col, n, F, 41, kind)
+            for wide in ("0", "1"):
+                os.environ["TGBM_WIDE_EVAL"] = wide
+                s = T.Session(val, rp, col, y, objective=objective, n_trees=4, depth=6, max_num_bin=200, learning_rate=0.4,
+                              gamma=0.0)
+                assert s.info("wide_eval") == int(wide)
+                s.boost(4)
+                runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+                s.close()
+    finally:
+        os.environ.pop("TGBM_WIDE_EVAL", None)
+        os.environ.pop("TGBM_SPARSE_PASS", None)
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
+    assert [a == b for a, b in zip(runs[2], runs[3])] == [True] * 3
+
+
+def test_more_than_255_bins_per_feature(T):
+    """max_num_bin above 255 (the reference cannot go there: its split bin is a byte, include/thundergbm/tree.h:23,
+    so there is nothing to compare a tree with): the CSR layout's global bin ids carry any number of bins per
+    feature. Checked: cut points and bin ids against the oracle's restatement of the cut rule (bit-exact, it has no
+    such limit), every row's final node against a walk down the tree by the raw feature values and the stored
+    thresholds, the training prediction against the sum of the leaf values along those walks, the hessian sums of the
+    final nodes against a count of the rows that arrived, and a loss that goes down."""
+    rng = np.random.default_rng(7)
+    n, F = 8000, 5
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.1] = 0.0  # zeros are not stored: missing values
+    val, rp, col = D.dense_to_csr(X)
+    y = (np.sin(2 * X[:, 0]) + X[:, 1] * X[:, 2] + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    lr, depth, rounds = 0.3, 6, 6
+    s = T.Session(val, rp, col, y, objective="reg:linear", n_trees=rounds, depth=depth, max_num_bin=1024,
+                  learning_rate=lr, gamma=0.0)
+    assert s.info("wide_bins") == 1 and s.info("sparse") == 1
+    cut_val, crp, cut_fid = s.cuts()
+    assert np.diff(crp).max() > 255 and np.diff(crp).max() <= 1024
+    o_val, o_crp, o_fid = O.cut_points(val, col, F, 1024)
+    assert np.array_equal(crp, o_crp) and np.array_equal(cut_val, o_val) and np.array_equal(cut_fid, o_fid)
+    gb, local = s.global_bin_ids(rp, col)
+    assert np.array_equal(gb, O.bin_ids(val, col, o_val, o_crp))
+    assert local.max() > 255
+    base = float(s.base_score)
+    s.boost(rounds)
+    log = s.metric_log()
+    assert np.all(np.diff(log) < 0)
+    model = s.model()[:, 0, :]
+    nid = s.nid()
+    Xm = np.where(X == 0, np.nan, X)
+    pred = np.full(n, base, np.float64)
+    for t in range(rounds):
+        nodes = model[t]
+        cur = np.zeros(n, np.int64)
+        for _ in range(depth):
+            nd = nodes[cur]
+            stop = (nd["is_leaf"] == 1) | (nd["split_fid"] < 0)
+            v = Xm[np.arange(n), np.maximum(nd["split_fid"], 0)]
+            right = np.where(np.isnan(v), nd["default_right"] == 1, v >= nd["split_value"])
+            cur = np.where(stop, cur, np.where(right, nd["rch"], nd["lch"]))
+        assert not nodes["is_pruned"].any()  # gamma = 0: nothing is pruned, a row's weight is its final node's
+        if t == rounds - 1:
+            np.testing.assert_array_equal(nid, cur)
+            # node sums of the nodes that hold rows against an fp64 recount of unit hessians (squared loss)
+            cnt = np.bincount(cur, minlength=len(nodes))
+            held = cnt > 0
+            np.testing.assert_allclose(nodes["sum_h"][held], cnt[held], rtol=1e-6)
+        pred += lr * nodes["base_weight"].astype(np.float64)[cur]
+    np.testing.assert_allclose(s.y_pred(), pred, rtol=1e-4, atol=1e-4)
+    s.close()

@@ -233,6 +233,10 @@ struct TreeBuffers {
     const unsigned short *bin_meta = nullptr;  // [n_bins]
     int n_packs = 0;
     const uint8_t *ignored = nullptr;  // [F] columns whose candidates score 0 this round (nullptr: none)
+    // Features with more than 255 cut points (max_num_bin up to 65 535; CSR layout, per-node path): the node's split
+    // bin does not fit TreeNode::split_bid, a byte as in the reference's model format, so the row -> node update
+    // reads it from here. nullptr: every feature has at most 255 bins.
+    int *split_bin = nullptr;          // [n_nodes] local bin id of the node's split
     const int *cut_row_ptr = nullptr;
     const int *cut_fid = nullptr;
     const float *cut_val = nullptr;
@@ -310,6 +314,7 @@ struct TreeBuffers {
         t.sp += K * max_level_nodes;
         t.cand += K * max_level_nodes * n_packs;
         t.root_partial += K * n_grad_blocks;
+        if (split_bin != nullptr) t.split_bin += K * n_nodes;
         return t;
     }
 };
@@ -343,6 +348,9 @@ void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &b
 // last level
 void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class = 1,
                        bool store_sibling = true);
+// Split search with one workgroup per (feature, node): any number of bins per feature (n_packs = F candidates per node)
+void launch_eval_split_wide(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class = 1,
+                            bool store_sibling = true);
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class = 1);
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class = 1);
 // Sparse level pass (tb.nid16 set): split search of a level (candidates into tb.cand, one slot per task / big

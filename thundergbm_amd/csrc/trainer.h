@@ -89,6 +89,8 @@ class Trainer {
     CsrBins csr_;
     // sparse layout: one pass per level over the bin-major copy instead of per-node histograms (depth <= 11)
     bool sparse_pass_ = false;
+    bool wide_bins_ = false;        // a feature has more than 255 cut points (max_num_bin above 255)
+    bool wide_eval_ = false;        // split search with one workgroup per (feature, node)
     int hist_cap_level_ = -1;       // first level with more nodes than the histogram arena holds (-1: none)
     int sparse_bin0_owner_ = -2;    // -2: not looked up yet
     bool sparse_sorted_on_ = true;

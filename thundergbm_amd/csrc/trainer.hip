@@ -77,8 +77,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     nnz_ = ds.nnz;
     TGBM_CHECK(n_ > 0, "empty dataset");
     TGBM_CHECK(param.depth >= 1 && param.depth <= 14, "depth %d out of the supported range 1..14", param.depth);
-    TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 255,
-               "max_num_bin %d out of the supported range 2..255", param.max_num_bin);
+    TGBM_CHECK(param.max_num_bin >= 2 && param.max_num_bin <= 65535,
+               "max_num_bin %d out of the supported range 2..65535", param.max_num_bin);
     TGBM_CHECK(objective_supported(param.objective), "undefined objective %s", param.objective.c_str());
     TGBM_CHECK(param.column_sampling_rate > 0.f, "column_sampling_rate must be positive");
     // class bookkeeping of TreeTrainer::train (src/thundergbm/trainer.cu:24-37)
@@ -163,11 +163,23 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
     if (force != nullptr && std::string(force) == "dense") sparse_ = false;
     if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
+    // More than 255 cut points in a feature (max_num_bin above 255): the dense layout's byte matrix and LDS
+    // histograms do not apply; the CSR layout's global bin ids have no such limit. Its split search then runs one
+    // workgroup per (feature, node) and the split bin travels in a side array (TreeNode::split_bid is a byte).
+    int max_feature_bins = 0;
+    for (int f = 0; f < F_; ++f) max_feature_bins = std::max(max_feature_bins, h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f]);
+    const char *wide_env = std::getenv("TGBM_WIDE_EVAL");  // "1": that split search for any data (tests)
+    wide_bins_ = max_feature_bins > 255;
+    if (wide_bins_) sparse_ = true;
     log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
     if (sparse_) {
         // TGBM_SPARSE_PASS=0 keeps the row-list kernels with per-node histograms in HBM (tests compare the two)
         const char *pe = std::getenv("TGBM_SPARSE_PASS");
-        sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && nnz_ < (1l << 31) && !(pe != nullptr && std::string(pe) == "0");
+        sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && nnz_ < (1l << 31) && !(pe != nullptr && std::string(pe) == "0") &&
+                       !wide_bins_;
+        wide_eval_ = wide_bins_ || (!sparse_pass_ && wide_env != nullptr && std::string(wide_env) == "1");
+        if (wide_bins_)
+            log_info("features with up to %d bins: CSR layout, split search per (feature, node)", max_feature_bins);
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
         // Head of the histogram: the most frequent features whose bins fit the LDS slots. Worth it when
         // they carry a real share of the stored values (skewed, e.g. Zipf-distributed, feature usage).
@@ -469,7 +481,7 @@ void Trainer::alloc_tree_buffers() {
     for (int f = 0; f < F_; ++f) {
         int k = h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f];
         if (k == 0) continue;
-        TGBM_CHECK(k <= kEvalPackBins, "feature %d has %d cut points, more than %d", f, k, kEvalPackBins);
+        TGBM_CHECK(k <= kEvalPackBins || wide_eval_, "feature %d has %d cut points, more than %d", f, k, kEvalPackBins);
         if (cur + k > kEvalPackBins) {
             pack_begin.push_back(h_cut_row_ptr_[f]);
             cur = 0;
@@ -478,6 +490,10 @@ void Trainer::alloc_tree_buffers() {
     }
     pack_begin.push_back(n_bins_);
     tb.n_packs = sparse_pass_ ? sp_.n_cand_slots : (int)pack_begin.size() - 1;  // candidates per node
+    if (wide_eval_) {
+        tb.n_packs = F_;  // one candidate per feature
+        tb.split_bin = dalloc<int>(S * tb.n_nodes);
+    }
     if (sparse_pass_) {
         tb.best_key = dalloc<unsigned long long>(S * (size_t)max_level_nodes);
         HIP_CHECK(hipMemsetAsync(tb.best_key, 0, sizeof(unsigned long long) * S * (size_t)max_level_nodes, stream_));
@@ -805,7 +821,8 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
             cur -= (size_t)x0 * n_bins_;
             build_level_hist(tbb, level, gh, n_class);
             if (!sparse_) launch_hist_merge(stream_, tbb, level, n_class);
-            launch_eval_split(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
+            if (wide_eval_) launch_eval_split_wide(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
+            else launch_eval_split(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
             launch_best_update(stream_, tbb, level, param_.rt_eps, param_.lambda, n_class);
         }
         lookup_level_ = level;
@@ -830,8 +847,12 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
         if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
         // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them); the
         // last level that fits a capped arena keeps them for the batches of the next one
-        launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
-                          !(in_boost_ && level == param_.depth - 1));
+        if (wide_eval_)
+            launch_eval_split_wide(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
+                                   !(in_boost_ && level == param_.depth - 1));
+        else
+            launch_eval_split(stream_, tb, level, param_.min_child_weight, param_.lambda, n_class,
+                              !(in_boost_ && level == param_.depth - 1));
     }
     launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
@@ -1138,6 +1159,8 @@ int Trainer::info(const std::string &key) const {
     if (key == "n_sets") return n_sets_;
     if (key == "sparse") return sparse_ ? 1 : 0;
     if (key == "sparse_pass") return sparse_pass_ ? 1 : 0;
+    if (key == "wide_bins") return wide_bins_ ? 1 : 0;
+    if (key == "wide_eval") return wide_eval_ ? 1 : 0;
     if (key == "row_lists") return sparse_pass_ ? 0 : 1;  // the sparse level pass keeps a row -> node map only
     if (key == "dense_W") return bins_.W;
     if (key == "reorders_done") return reorders_done_;

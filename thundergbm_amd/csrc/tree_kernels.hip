@@ -910,7 +910,7 @@ __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, C
     const int pe = min(sg.y, pb + kPartChunk);
     const int f = nd.split_feature_id;
     const int cb = tb.cut_row_ptr[f], ce = tb.cut_row_ptr[f + 1];
-    const int sbid = cb + nd.split_bid;
+    const int sbid = cb + (tb.split_bin != nullptr ? tb.split_bin[off + x_in] : (int)nd.split_bid);
     const bool dr = nd.default_right;
     int nleft = 0;
 #pragma unroll
@@ -1114,6 +1114,156 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
     }
 }
 
+// Split search for features of any number of bins (max_num_bin above 255): one workgroup per (feature, node) walks the
+// feature's bins in chunks of kBlock with a block-wide inclusive scan of the exact 64-bit sums and a carry from
+// chunk to chunk. Same candidates, gains and tie rule as k_eval_split (whose wavefront holds a whole feature of at
+// most 256 bins); one candidate per feature. CSR layout only: the node of a pair that was not built from rows is
+// derived as parent - built while it is read (and stored for the next level).
+__device__ __forceinline__ longlong2 wide_bin(const longlong2 *h, const longlong2 *h_par, const longlong2 *h_built, int b) {
+    if (h_par == nullptr) return h[b];
+    const longlong2 pv = h_par[b], bv = h_built[b];
+    return make_longlong2(pv.x - bv.x, pv.y - bv.y);
+}
+
+__global__ __launch_bounds__(kBlock) void k_eval_split_wide(TreeBuffers tb_all, int level, float mcw, float lambda,
+                                                           bool store_sibling) {
+#pragma clang fp contract(off)
+    __shared__ long long s_g[kWaves], s_h[kWaves];
+    __shared__ float s_abs[kWaves];
+    __shared__ int s_idx[kWaves];
+    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const int f = blockIdx.x;
+    const int x_in = blockIdx.y + tb.lvl_x0;
+    const int x = (1 << level) - 1 + x_in;
+    const TreeNode nd = tb.nodes[x];
+    if (!nd.is_valid) return;  // (nobody reads the candidates of an invalid node)
+    const int cb = tb.cut_row_ptr[f], ce = tb.cut_row_ptr[f + 1];
+    SplitCand *out = &tb.cand[(size_t)x_in * tb.n_packs + f];
+    if (cb == ce) {
+        if (threadIdx.x == 0) out->index = 0x7fffffff;  // a feature without bins has no candidate
+        return;
+    }
+    const int lane = lane_id(), w = wave_id();
+    longlong2 *h = tb.hist(level) + (size_t)x_in * tb.n_bins;
+    const longlong2 *h_par = nullptr, *h_built = nullptr;
+    if (level > 0 && !tb.singles(level)) {
+        const int built = tb.hpair_built[x_in >> 1];
+        if (built >= 0 && built != x) {
+            h_par = tb.hist(level + 1) + (size_t)(x_in >> 1) * tb.n_bins;
+            h_built = tb.hist(level) + (size_t)(built - ((1 << level) - 1)) * tb.n_bins;
+        }
+    }
+    const GHPair S = nd.sum_gh_pair;
+    const double inv_g = tb.quant->inv_g, inv_h = tb.quant->inv_h;
+    const bool ign = tb.ignored != nullptr && tb.ignored[f] != 0;
+    // ---- the feature's total (missing = node sum - total), the derived sibling stored on the way
+    long long tg = 0, th = 0;
+    for (int b = cb + threadIdx.x; b < ce; b += kBlock) {
+        const longlong2 v = wide_bin(h, h_par, h_built, b);
+        if (h_par != nullptr && store_sibling) h[b] = v;
+        tg += v.x;
+        th += v.y;
+    }
+    tg = wave_sum_ll(tg);
+    th = wave_sum_ll(th);
+    if (lane == 0) {
+        s_g[w] = tg;
+        s_h[w] = th;
+    }
+    __syncthreads();
+    tg = th = 0;
+    for (int i = 0; i < kWaves; ++i) {
+        tg += s_g[i];
+        th += s_h[i];
+    }
+    __syncthreads();
+    const GHPair m{S.g - (float)((double)tg * inv_g), S.h - (float)((double)th * inv_h)};
+    // ---- candidates, chunk by chunk
+    long long carry_g = 0, carry_h = 0;
+    float best = -1.f, best_score = 0.f;
+    int best_idx = 0x7fffffff;
+    GHPair best_left{0, 0};
+    for (int base = cb; base < ce; base += kBlock) {
+        const int b = base + threadIdx.x;
+        longlong2 v = make_longlong2(0, 0);
+        if (b < ce) v = (h_par != nullptr && !store_sibling) ? wide_bin(h, h_par, h_built, b) : h[b];
+        long long ig = v.x, ih = v.y;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const long long pg = shfl_up_ll(ig, d), ph = shfl_up_ll(ih, d);
+            if (lane >= d) {
+                ig += pg;
+                ih += ph;
+            }
+        }
+        if (lane == 63) {
+            s_g[w] = ig;
+            s_h[w] = ih;
+        }
+        __syncthreads();
+        long long wg = 0, wh = 0, cg = 0, ch = 0;
+        for (int i = 0; i < kWaves; ++i) {
+            if (i < w) {
+                wg += s_g[i];
+                wh += s_h[i];
+            }
+            cg += s_g[i];
+            ch += s_h[i];
+        }
+        __syncthreads();
+        if (b < ce) {
+            const long long exg = carry_g + wg + ig - v.x, exh = carry_h + wh + ih - v.y;  // bins below b
+            const GHPair l{(float)((double)exg * inv_g), (float)((double)exh * inv_h)};
+            const float gr = split_gain(S, l, mcw, lambda);
+            const GHPair l2{l.g + m.g, l.h + m.h};
+            const float gl = split_gain(S, l2, mcw, lambda);
+            float score = (gl > gr) ? gl : -gr;
+            if (ign) score = 0.f;  // column sampling: hist_tree_builder_single.cu:304 / :663
+            const float a = fabsf(score);
+            if (a > best) {  // (a thread's bins ascend: the first maximum is the one with the smallest index)
+                best = a;
+                best_score = score;
+                best_idx = b;
+                best_left = l;
+            }
+        }
+        carry_g += cg;
+        carry_h += ch;
+    }
+    // workgroup arg-max: larger |score| wins, ties go to the smaller bin index (hist_tree_builder_single.cu:330-335)
+    float win = best;
+    int win_idx = best_idx;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const float oa = __shfl_xor(win, d);
+        const int oi = __shfl_xor(win_idx, d);
+        if (oa > win || (oa == win && oi < win_idx)) {
+            win = oa;
+            win_idx = oi;
+        }
+    }
+    if (lane == 0) {
+        s_abs[w] = win;
+        s_idx[w] = win_idx;
+    }
+    __syncthreads();
+    for (int i = 0; i < kWaves; ++i) {
+        if (s_abs[i] > win || (s_abs[i] == win && s_idx[i] < win_idx)) {
+            win = s_abs[i];
+            win_idx = s_idx[i];
+        }
+    }
+    if (best == win && best_idx == win_idx) {  // exactly one thread: bin indices are distinct
+        SplitCand c;
+        c.score = best_score;
+        c.index = best_idx;
+        c.miss = m;
+        c.left = best_left;
+        c.pad[0] = c.pad[1] = 0;
+        *out = c;
+    }
+}
+
 // Per node: reduce the wavefront candidates, fill the split record (hist_tree_builder_single.cu
 // :365-389) and apply it to the tree (update_tree, :860-899). One workgroup per node of the level.
 __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int level, float rt_eps, float lambda) {
@@ -1223,6 +1373,7 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
         node.split_feature_id = f;
         node.split_value = s.fval;
         node.split_bid = (unsigned char)s.split_bid;
+        if (tb.split_bin != nullptr) tb.split_bin[x] = c.index - fbegin;
         GHPair ls = s.lch_sum_gh;
         if (!s.default_right) {
             ls.g += s.fea_missing_gh.g;
@@ -1696,7 +1847,9 @@ __device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBi
     bool right;
     if (SPARSE) {
         const int cb = tb.cut_row_ptr[nd.split_feature_id], ce = tb.cut_row_ptr[nd.split_feature_id + 1];
-        right = csr_goes_right(cbins, row, cb, ce, cb + nd.split_bid, nd.default_right);
+        // (the node's own heap id is its children's parent index; wide features keep their split bin in a side array)
+        const int sb = tb.split_bin != nullptr ? tb.split_bin[(nd.lch_index - 1) / 2] : (int)nd.split_bid;
+        right = csr_goes_right(cbins, row, cb, ce, cb + sb, nd.default_right);
     } else {
         const int b = dbins.col[(size_t)nd.split_feature_id * dbins.col_stride + row];
         right = (b == kMissingBin) ? nd.default_right : (b >= nd.split_bid);
@@ -2128,6 +2281,12 @@ void launch_eval_split(hipStream_t s, const TreeBuffers &tb, int level, float mc
     dim3 grid((tb.n_packs + kWaves - 1) / kWaves, tb.nodes_served(level), n_class);
     if (tb.sparse) k_eval_split<true><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, store_sibling);
     else k_eval_split<false><<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, true);
+}
+
+void launch_eval_split_wide(hipStream_t s, const TreeBuffers &tb, int level, float mcw, float lambda, int n_class,
+                            bool store_sibling) {
+    dim3 grid(tb.F, tb.nodes_served(level), n_class);
+    k_eval_split_wide<<<grid, kBlock, 0, s>>>(tb, level, mcw, lambda, store_sibling);
 }
 
 void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float rt_eps, float lambda, int n_class) {
