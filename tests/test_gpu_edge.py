@@ -793,3 +793,25 @@ def test_more_than_255_bins_per_feature(T):
         pred += lr * nodes["base_weight"].astype(np.float64)[cur]
     np.testing.assert_allclose(s.y_pred(), pred, rtol=1e-4, atol=1e-4)
     s.close()
+
+
+def test_sparse_level_pass_at_its_deepest_level(T):
+    """Depth 11 (1024 nodes on the last level: the sparse level pass's limit, 12-bit node field of the sorted keys,
+    20 KB of per-node LDS state): sorted pass against tables, byte for byte."""
+    os.environ["TGBM_LAYOUT"] = "sparse"
+    n, F = 60000, 400
+    val, rp, col = _ragged(n, F, 51, 10)
+    y = _target(val, rp, col, n, F, 51, "bin")
+    runs = []
+    try:
+        for srt in ("1", "0"):
+            os.environ["TGBM_SPARSE_SORTED"] = srt
+            s = T.Session(val, rp, col, y, objective="binary:logistic", n_trees=2, depth=11, max_num_bin=48,
+                          learning_rate=0.5, gamma=0.0, min_child_weight=0.05)
+            assert s.info("sparse_pass") == 1
+            s.boost(2)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        os.environ.pop("TGBM_SPARSE_SORTED", None)
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
