@@ -218,8 +218,7 @@ __device__ void sp_search_batch(const TreeBuffers &tb, SpShared &sh, const longl
 
 // One task = a run of whole features (batched so that their tables fit the LDS) or one chunk of a big feature (its
 // table goes to the partial buffer, k_sparse_big adds the chunks up and searches them).
-__global__ __launch_bounds__(kSpBlock) __attribute__((amdgpu_waves_per_eu(8)))  // two workgroups per CU
-void k_sparse_level(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
+__global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
                                                           const GHPair *__restrict__ gh, int level, float mcw,
                                                           float lambda, int dump_hist, int n_cells) {
     extern __shared__ longlong2 cells[];  // [n_cells]
@@ -276,7 +275,7 @@ void k_sparse_level(TreeBuffers tb_all, CsrBins bins, SparsePass sp,
             for (int c = threadIdx.x; c < n_cells; c += kSpBlock) cells[c] = make_longlong2(0, 0);
             __syncthreads();
             // accumulate: four values in flight per thread (row -> node from the cache-resident map, then the pair)
-            constexpr int U = 4;
+            constexpr int U = 8;
             for (int e0 = v0 + threadIdx.x; e0 < v1; e0 += kSpBlock * U) {
                 int gb[U], row[U], x[U];
 #pragma unroll
