@@ -15,6 +15,14 @@ __device__ __forceinline__ int lanes_below(unsigned long long mask) {
 }
 
 
+// Round-to-nearest-even of a float (|x| < 2^51) as a 64-bit integer: the integer sits in the low mantissa bits of
+// x + 1.5 * 2^52 (bit pattern 0x4338000000000000, whose low word is zero: only the high word is corrected).
+__device__ __forceinline__ long long round_to_ll(float x) {
+    const long long b = __double_as_longlong((double)x + 6755399441055744.0);
+    const unsigned hi = (unsigned)((unsigned long long)b >> 32) - 0x43380000u;
+    return (long long)(((unsigned long long)hi << 32) | (unsigned)b);
+}
+
 __device__ __forceinline__ bool node_splits(const TreeNode &nd) {
     return nd.is_valid && !nd.is_leaf && nd.split_feature_id >= 0;
 }

@@ -291,7 +291,7 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, C
                 for (int u = 0; u < U; ++u) {
                     if ((unsigned)x[u] < (unsigned)nn) {
                         const GHPair s = csc_gh != nullptr ? csc_gh[e0 + u * kSpBlock] : gh[row[u]];
-                        const long long gq = __float2ll_rn(s.g * scale_g), hq = __float2ll_rn(s.h * scale_h);
+                        const long long gq = round_to_ll(s.g * scale_g), hq = round_to_ll(s.h * scale_h);
                         unsigned long long *cell = reinterpret_cast<unsigned long long *>(cells + (size_t)x[u] * nbins + (gb[u] - bin0));
                         atomicAdd(cell, (unsigned long long)gq);
                         atomicAdd(cell + 1, (unsigned long long)hq);
@@ -588,6 +588,7 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     }
     __syncthreads();
     const int i0 = threadIdx.x * kSoV;
+    const int pb = i0 + (threadIdx.x >> 2);  // so_phys(i0 + j) = pb + j: a thread's eight positions share one padding count
     int Mn = M;  // values of the new order
     if (!LEVEL0) {
         const ulonglong2 *__restrict__ row_side = tb.row_side;
@@ -597,9 +598,9 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
 #pragma unroll
         for (int j = 0; j < kSoV; ++j) {
             const int i = i0 + j;
-            row[j] = i < M ? s_row[so_phys(i)] : -1;
-            key[j] = i < M ? s_key[so_phys(i)] : 0xffffffffu;
-            pair[j] = i < M ? s_gh[so_phys(i)] : GHPair{0, 0};
+            row[j] = i < M ? s_row[pb + j] : -1;
+            key[j] = i < M ? s_key[pb + j] : 0xffffffffu;
+            pair[j] = i < M ? s_gh[pb + j] : GHPair{0, 0};
         }
         const unsigned prevk = (i0 > 0 && i0 - 1 < M) ? s_key[so_phys(i0 - 1)] : 0xffffffffu;
         const unsigned nextk = (i0 + kSoV < M) ? s_key[so_phys(i0 + kSoV)] : 0xffffffffu;
@@ -685,12 +686,12 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     for (int j = 0; j < kSoV; ++j) {
         const int p = i0 + j;
         const bool in = p < Mn;
-        key[j] = in ? s_key[so_phys(p)] : 0xffffffffu;
+        key[j] = in ? s_key[pb + j] : 0xffffffffu;
         fs[j] = SoSum{0, 0};
         if (in) {
-            const GHPair s = s_gh[so_phys(p)];
-            fs[j].g = __float2ll_rn(s.g * scale_g);
-            fs[j].h = __float2ll_rn(s.h * scale_h);
+            const GHPair s = s_gh[pb + j];
+            fs[j].g = round_to_ll(s.g * scale_g);
+            fs[j].h = round_to_ll(s.h * scale_h);
         }
     }
     {
@@ -727,7 +728,7 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     int start[kSoV];
 #pragma unroll
     for (int j = 0; j < kSoV; ++j) {
-        start[j] = (i0 + j < Mn) ? (int)s_aux[so_phys(i0 + j)] : 0;
+        start[j] = (i0 + j < Mn) ? (int)s_aux[pb + j] : 0;
         if (tail[j])
             s_gh[so_phys(start[j])] = GHPair{(float)((double)fs[j].g * inv_g), (float)((double)fs[j].h * inv_h)};
     }
@@ -748,7 +749,7 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
             tot[j] = s_gh[so_phys(start[j])];
             const float Sh = s_S[(key[j] >> kSortedNodeShift) & 0xfffu].h;
             drop[j] = !dump_hist && tot[j].h + Sh * 4.76837158e-7f < mcw;  // 2^-21
-            if (drop[j]) s_key[so_phys(p)] = key[j] | kSoNodeMask;
+            if (drop[j]) s_key[pb + j] = key[j] | kSoNodeMask;
         }
     }
     __syncthreads();

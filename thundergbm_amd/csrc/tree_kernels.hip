@@ -258,14 +258,6 @@ __device__ int item_shift(float qmax, int rows, int bits) {
     return ilogb(q / lim) + 1;  // 2^s > q / lim
 }
 
-// Round-to-nearest-even of a float (|x| < 2^51) as a 64-bit integer: the integer sits in the low mantissa bits of
-// x + 1.5 * 2^52 (bit pattern 0x4338000000000000, whose low word is zero: only the high word is corrected).
-__device__ __forceinline__ long long round_to_ll(float x) {
-    const long long b = __double_as_longlong((double)x + 6755399441055744.0);
-    const unsigned hi = (unsigned)((unsigned long long)b >> 32) - 0x43380000u;
-    return (long long)(((unsigned long long)hi << 32) | (unsigned)b);
-}
-
 // ------------------------------------------------------------------------------- tree init
 // Node array initialisation of the reference's Tree::init2 (src/thundergbm/tree.cu:8-39), root sum
 // from the block partials, root segment and the histogram plan of level 0. One workgroup.
@@ -362,8 +354,11 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         // The tree's scales keep the 64-bit sums over all n rows below 2^62; a dense work item coarsens them by its
         // own power of two so that its packed LDS fields hold the rows between two drains (item_shifts).
         QuantCtl q;
-        q.scale_g = pow2_scale(gm, tb.n, 4.6e18f);
-        q.scale_h = pow2_scale(hm, tb.n, 4.6e18f);
+        // (the sparse layout's kernels round with round_to_ll, good below 2^51: its scales are those of at least
+        // 4096 rows, which keeps every row's integers below 2^50)
+        const int scale_rows = tb.sparse ? max(tb.n, 4096) : tb.n;
+        q.scale_g = pow2_scale(gm, scale_rows, 4.6e18f);
+        q.scale_h = pow2_scale(hm, scale_rows, 4.6e18f);
         q.h_bits = 32;
         q.h_integer = 0;
         // every hessian a non-negative integer (squared loss; bagging multiplies by draw counts): the hessian field
