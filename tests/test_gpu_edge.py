@@ -27,11 +27,13 @@ def T():
 @pytest.fixture(autouse=True)
 def _default_layout():
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
-              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES"):
+              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
+              "TGBM_DENSE_BIN_BYTES"):
         os.environ.pop(k, None)
     yield
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
-              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES"):
+              "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
+              "TGBM_DENSE_BIN_BYTES"):
         os.environ.pop(k, None)
 
 
@@ -714,12 +716,13 @@ def test_capped_histogram_arena_gives_the_same_trees(T, layout, objective, kind)
     assert same == [[True] * 3] * 2, same
 
 
-def test_split_search_per_feature_and_node_equals_the_packed_one(T):
+@pytest.mark.parametrize("layout", ["sparse", "dense"])
+def test_split_search_per_feature_and_node_equals_the_packed_one(T, layout):
     """The split search for features of any number of bins (one workgroup per (feature, node), chunks of 256 bins
     with a carried prefix) against the packed one (a wavefront per run of whole features of at most 256 bins) on
     data both can serve: same candidates, gains and tie rule, so the same bytes. TGBM_WIDE_EVAL=1 switches it on
-    for the CSR layout's per-node path."""
-    os.environ["TGBM_LAYOUT"] = "sparse"
+    for the dense layout and the CSR layout's per-node path."""
+    os.environ["TGBM_LAYOUT"] = layout
     os.environ["TGBM_SPARSE_PASS"] = "0"
     n, F = 6000, 9
     val, rp, col = _ragged(n, F, 41, 8)
@@ -742,13 +745,17 @@ def test_split_search_per_feature_and_node_equals_the_packed_one(T):
     assert [a == b for a, b in zip(runs[2], runs[3])] == [True] * 3
 
 
-def test_more_than_255_bins_per_feature(T):
+@pytest.mark.parametrize("layout,max_bins", [("dense", 1024), ("dense", 3000), ("dense", 6000), ("sparse", 1024)])
+def test_more_than_255_bins_per_feature(T, layout, max_bins):
     """max_num_bin above 255 (the reference cannot go there: its split bin is a byte, include/thundergbm/tree.h:23,
-    so there is nothing to compare a tree with): the CSR layout's global bin ids carry any number of bins per
-    feature. Checked: cut points and bin ids against the oracle's restatement of the cut rule (bit-exact, it has no
-    such limit), every row's final node against a walk down the tree by the raw feature values and the stored
-    thresholds, the training prediction against the sum of the leaf values along those walks, the hessian sums of the
-    final nodes against a count of the rows that arrived, and a loss that goes down."""
+    so there is nothing to compare a tree with): the dense layout keeps 16-bit bins, the CSR layout's global bin ids
+    carry any number of bins per feature anyway (1024 bins: eight features per block of the dense layout; 3000: two,
+    with two histogram workgroups per CU; 6000: two, with one). Checked for both: cut points and bin ids against the oracle's
+    restatement of the cut rule (bit-exact, it has no such limit), every row's final node against a walk down the tree
+    by the raw feature values and the stored thresholds, the training prediction against the sum of the leaf values
+    along those walks, the hessian sums of the final nodes against a count of the rows that arrived, and a loss that
+    goes down."""
+    os.environ["TGBM_LAYOUT"] = layout
     rng = np.random.default_rng(7)
     n, F = 8000, 5
     X = rng.standard_normal((n, F)).astype(np.float32)
@@ -756,16 +763,25 @@ def test_more_than_255_bins_per_feature(T):
     val, rp, col = D.dense_to_csr(X)
     y = (np.sin(2 * X[:, 0]) + X[:, 1] * X[:, 2] + 0.1 * rng.standard_normal(n)).astype(np.float32)
     lr, depth, rounds = 0.3, 6, 6
-    s = T.Session(val, rp, col, y, objective="reg:linear", n_trees=rounds, depth=depth, max_num_bin=1024,
+    s = T.Session(val, rp, col, y, objective="reg:linear", n_trees=rounds, depth=depth, max_num_bin=max_bins,
                   learning_rate=lr, gamma=0.0)
-    assert s.info("wide_bins") == 1 and s.info("sparse") == 1
+    assert s.info("wide_bins") == 1 and s.info("wide_eval") == 1
+    if layout == "dense":
+        assert s.info("sparse") == 0 and s.info("dense_bin_bytes") == 2
+    else:
+        assert s.info("sparse") == 1
     cut_val, crp, cut_fid = s.cuts()
-    assert np.diff(crp).max() > 255 and np.diff(crp).max() <= 1024
-    o_val, o_crp, o_fid = O.cut_points(val, col, F, 1024)
+    assert np.diff(crp).max() > max_bins // 2 and np.diff(crp).max() <= max_bins
+    o_val, o_crp, o_fid = O.cut_points(val, col, F, max_bins)
     assert np.array_equal(crp, o_crp) and np.array_equal(cut_val, o_val) and np.array_equal(cut_fid, o_fid)
     gb, local = s.global_bin_ids(rp, col)
     assert np.array_equal(gb, O.bin_ids(val, col, o_val, o_crp))
     assert local.max() > 255
+    if layout == "dense":  # a feature without a stored value in a row holds the 16-bit sentinel
+        m = s.binmat()
+        W = s.info("dense_W")
+        dense = np.concatenate([m[b] for b in range(m.shape[0])], axis=1)[:, :F]
+        assert m.dtype == np.uint16 and np.array_equal(dense == 65535, X == 0)
     base = float(s.base_score)
     s.boost(rounds)
     log = s.metric_log()
@@ -793,6 +809,49 @@ def test_more_than_255_bins_per_feature(T):
         pred += lr * nodes["base_weight"].astype(np.float64)[cur]
     np.testing.assert_allclose(s.y_pred(), pred, rtol=1e-4, atol=1e-4)
     s.close()
+
+
+@pytest.mark.parametrize("objective,F,reorder", [("reg:linear", 5, "0"), ("binary:logistic", 40, "always"),
+                                                 ("multi:softmax", 11, "0"), ("binary:logistic", 3, "0")])
+def test_dense_16_bit_bins_equal_byte_bins(T, objective, F, reorder):
+    """The dense layout with 16-bit bins (TGBM_DENSE_BIN_BYTES=2 forces it for data that byte bins can hold) against
+    the byte layout: other feature blocks, the same exact integer sums per bin, so the same models, predictions and
+    row -> node maps byte for byte (every feature has rows without a value, so neither run takes the root's sums from
+    a complete feature's bins). With a re-ordering of the rows after every tree, with class trees built together, and
+    with the split search of wide features (TGBM_WIDE_EVAL=1) on top."""
+    os.environ["TGBM_LAYOUT"] = "dense"
+    os.environ["TGBM_REORDER"] = reorder
+    rng = np.random.default_rng(F)
+    n = 30000
+    X = np.round(rng.standard_normal((n, F)) * 2, 1).astype(np.float32)
+    X[rng.random((n, F)) < 0.15] = 0.0
+    val, rp, col = D.dense_to_csr(X)
+    score = X[:, 0] - 0.5 * X[:, 1] * X[:, 2] + 0.3 * rng.standard_normal(n)
+    if objective == "reg:linear":
+        y = score.astype(np.float32)
+    elif objective == "binary:logistic":
+        y = (score > 0).astype(np.float32)
+    else:
+        y = np.digitize(score, [-1.0, 0.0, 1.0]).astype(np.float32)
+    kw = dict(objective=objective, n_trees=4, depth=6, max_num_bin=100, learning_rate=0.4, gamma=0.0)
+    runs, mats = [], []
+    try:
+        for nbytes, wide in (("1", "0"), ("2", "0"), ("2", "1")):
+            os.environ["TGBM_DENSE_BIN_BYTES"] = nbytes
+            os.environ["TGBM_WIDE_EVAL"] = wide
+            s = T.Session(val, rp, col, y, **kw)
+            assert s.info("sparse") == 0 and s.info("dense_bin_bytes") == int(nbytes) and s.info("wide_eval") == int(wide)
+            m = s.binmat()
+            mats.append(np.concatenate([m[b] for b in range(m.shape[0])], axis=1)[:, :F].astype(np.int32))
+            s.boost(4)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        for k in ("TGBM_DENSE_BIN_BYTES", "TGBM_WIDE_EVAL", "TGBM_REORDER"):
+            os.environ.pop(k, None)
+    assert np.array_equal(np.where(mats[0] == 255, 65535, mats[0]), mats[1])
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
+    assert [a == b for a, b in zip(runs[0], runs[2])] == [True] * 3
 
 
 def test_sparse_level_pass_at_its_deepest_level(T):

@@ -26,6 +26,11 @@
 namespace tgbm {
 
 constexpr int kMissingBin = 255;   // dense matrix sentinel: the feature has no stored value in this row
+constexpr int kMissingBin16 = 65535;  // the same for 16-bit bins
+// 16-bit bins: bins of a feature block that leave the LDS room for two histogram workgroups per CU, and the most a
+// block may hold at all (160 KB of 8-byte bins)
+constexpr int kDense16BlockBins = 8192;
+constexpr int kDense16MaxBlockBins = 20480;
 constexpr int kPartChunk = 2048;   // rows per partition work item (256 threads x 8 rounds)
 constexpr int kEvalPackBins = 256; // bins scanned by one wavefront in split finding (4 per lane)
 constexpr int kCsrHeadBins = 4864;  // head slots of the sparse histogram: 2 x 8 bytes each, two workgroups per CU
@@ -82,13 +87,16 @@ struct SplitCand {
 // Dense column-blocked bin matrix: block b holds features [b*W, (b+1)*W) as n rows of W bytes.
 struct DenseBins {
     const uint8_t *data = nullptr;
-    int W = 0;          // bytes (features) per row of a block, multiple of 4
+    int W = 0;          // features per row of a block (a row of a block is W * bin_bytes bytes, a multiple of 4)
     int n_blocks = 0;
-    size_t block_stride = 0;  // bytes between blocks = n * W
-    // Column-major copy (feature f = n consecutive bytes at col + f * col_stride): the partition reads
-    // one feature of many rows, which costs one byte per row here instead of one sector per row.
+    size_t block_stride = 0;  // bytes between blocks = n * W * bin_bytes
+    // Column-major copy (feature f = n consecutive bins at col + f * col_stride * bin_bytes): the partition reads
+    // one feature of many rows, which costs one bin per row here instead of one sector per row.
     const uint8_t *col = nullptr;
-    size_t col_stride = 0;
+    size_t col_stride = 0;  // in bins
+    // 1: byte bins (at most 255 bins per feature, 255 = no stored value); 2: 16-bit bins for max_num_bin above 255
+    // (65535 = no stored value)
+    int bin_bytes = 1;
 };
 
 // Sparse layout for wide, mostly-missing data: the reference's own representation, CSR rows of global
@@ -390,7 +398,7 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 // data preparation
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride);
+                      size_t col_stride, int bin_bytes);
 // feat_slot (may be nullptr): first head slot of a feature or -1; then hist_word is written as well
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id, const int *feat_slot = nullptr, int *hist_word = nullptr);
@@ -448,7 +456,7 @@ void launch_reorder_keys(hipStream_t s, int n, int depth, const int *nid, unsign
 void launch_gather_rows(hipStream_t s, int n, int bytes_per_row, const int *from, const void *src, void *dst);
 void launch_gather_perm(hipStream_t s, int n, const int *from, const int *perm_old, int *perm_new);
 void launch_cols_from_rows(hipStream_t s, int n, int W, int F, int n_blocks, const uint8_t *binmat, size_t block_stride,
-                           uint8_t *colmat, size_t col_stride);
+                           uint8_t *colmat, size_t col_stride, int bin_bytes);
 
 // Largest of n ints in device memory (synchronises; 0 for n == 0); aborts when one of them is negative.
 int device_max_int(hipStream_t s, const int *d_v, long n);

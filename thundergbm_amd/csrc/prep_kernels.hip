@@ -267,18 +267,20 @@ __device__ __forceinline__ int local_bin(const float *__restrict__ cuts, int k, 
     return left;
 }
 
+// (BinT = uint8_t or uint16_t; block_stride and col_stride count bins)
+template <typename BinT>
 __global__ void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
                             const float *__restrict__ val, const float *__restrict__ cut_val,
-                            const int *__restrict__ cut_row_ptr, uint8_t *__restrict__ binmat, int W,
-                            size_t block_stride, uint8_t *__restrict__ colmat, size_t col_stride) {
+                            const int *__restrict__ cut_row_ptr, BinT *__restrict__ binmat, int W,
+                            size_t block_stride, BinT *__restrict__ colmat, size_t col_stride) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         for (int e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
             int f = col[e];
             int cb = cut_row_ptr[f];
             int k = cut_row_ptr[f + 1] - cb;
             int b = local_bin(cut_val + cb, k, val[e]);
-            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (uint8_t)b;
-            colmat[(size_t)f * col_stride + i] = (uint8_t)b;
+            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (BinT)b;
+            colmat[(size_t)f * col_stride + i] = (BinT)b;
         }
     }
 }
@@ -477,18 +479,20 @@ __global__ __launch_bounds__(256) void k_gather_perm(int n, const int *__restric
     perm_new[p] = perm_old != nullptr ? perm_old[f] : f;
 }
 
-// Column-major copy of one feature block from its row-major form: a tile of 256 rows x W bytes goes through
-// LDS so that both the reads (whole rows) and the writes (256 consecutive bytes of one feature) are coalesced.
+// Column-major copy of one feature block from its row-major form: a tile of 256 rows x W bins goes through
+// LDS so that both the reads (whole rows) and the writes (256 consecutive bins of one feature) are coalesced.
+template <typename BinT>
 __global__ __launch_bounds__(256) void k_cols_from_rows(int n, int W, int F, int block, const uint8_t *__restrict__ rows,
-                                                       uint8_t *__restrict__ colmat, size_t col_stride) {
-    extern __shared__ uint8_t tile[];  // [256][W + 4]: the padding spreads a column's bytes over the banks
+                                                       BinT *__restrict__ colmat, size_t col_stride) {
+    extern __shared__ uint8_t tile[];  // [256][row bytes + 4]: the padding spreads a column's bins over the banks
     const int r0 = blockIdx.x * 256;
-    const int pitch = W + 4;
-    const int words = W / 4;
+    const int row_bytes = W * (int)sizeof(BinT);
+    const int pitch = row_bytes + 4;
+    const int words = row_bytes / 4;
     for (int i = threadIdx.x; i < 256 * words; i += 256) {
         const int r = i / words, w = i % words;
         unsigned v = 0xffffffffu;
-        if (r0 + r < n) v = reinterpret_cast<const unsigned *>(rows + (size_t)(r0 + r) * W)[w];
+        if (r0 + r < n) v = reinterpret_cast<const unsigned *>(rows + (size_t)(r0 + r) * row_bytes)[w];
         *reinterpret_cast<unsigned *>(tile + r * pitch + w * 4) = v;
     }
     __syncthreads();
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(256) void k_cols_from_rows(int n, int W, int F, int
     if (r0 + r >= n) return;
     for (int j = 0; j < W; ++j) {
         const int f = block * W + j;
-        if (f < F) colmat[(size_t)f * col_stride + r0 + r] = tile[r * pitch + j];
+        if (f < F) colmat[(size_t)f * col_stride + r0 + r] = reinterpret_cast<const BinT *>(tile + r * pitch)[j];
     }
 }
 
@@ -517,11 +521,17 @@ void launch_gather_perm(hipStream_t s, int n, const int *from, const int *perm_o
 }
 
 void launch_cols_from_rows(hipStream_t s, int n, int W, int F, int n_blocks, const uint8_t *binmat, size_t block_stride,
-                           uint8_t *colmat, size_t col_stride) {
+                           uint8_t *colmat, size_t col_stride, int bin_bytes) {
     if (n <= 0) return;
-    for (int b = 0; b < n_blocks; ++b)
-        k_cols_from_rows<<<(n + 255) / 256, 256, (size_t)256 * (W + 4), s>>>(n, W, F, b, binmat + (size_t)b * block_stride,
-                                                                             colmat, col_stride);
+    const size_t lds = (size_t)256 * (W * bin_bytes + 4);
+    for (int b = 0; b < n_blocks; ++b) {
+        const uint8_t *rows = binmat + (size_t)b * block_stride;
+        if (bin_bytes == 2)
+            k_cols_from_rows<uint16_t><<<(n + 255) / 256, 256, lds, s>>>(n, W, F, b, rows,
+                                                                      reinterpret_cast<uint16_t *>(colmat), col_stride);
+        else
+            k_cols_from_rows<uint8_t><<<(n + 255) / 256, 256, lds, s>>>(n, W, F, b, rows, colmat, col_stride);
+    }
 }
 
 void ScanScratch::release() {
@@ -587,9 +597,14 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits) {
 
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride) {
-    k_bin_dense<<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride,
-                                              colmat, col_stride);
+                      size_t col_stride, int bin_bytes) {
+    if (bin_bytes == 2)
+        k_bin_dense<uint16_t><<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr,
+                                                        reinterpret_cast<uint16_t *>(binmat), W, block_stride / 2,
+                                                        reinterpret_cast<uint16_t *>(colmat), col_stride);
+    else
+        k_bin_dense<uint8_t><<<grid_for(n), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W,
+                                                       block_stride, colmat, col_stride);
 }
 
 void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, const int *sort_key,

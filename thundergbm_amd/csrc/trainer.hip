@@ -163,15 +163,23 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
     if (force != nullptr && std::string(force) == "dense") sparse_ = false;
     if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
-    // More than 255 cut points in a feature (max_num_bin above 255): the dense layout's byte matrix and LDS
-    // histograms do not apply; the CSR layout's global bin ids have no such limit. Its split search then runs one
-    // workgroup per (feature, node) and the split bin travels in a side array (TreeNode::split_bid is a byte).
+    // More than 255 cut points in a feature (max_num_bin above 255): the dense layout then keeps 16-bit bins in narrower
+    // feature blocks (their LDS histograms hold as many bins as the byte layout's), as long as one feature's bins fit
+    // the LDS; the CSR layout's global bin ids have no limit at all. Either way the split search runs one workgroup
+    // per (feature, node) and the split bin travels in a side array (TreeNode::split_bid is a byte).
     int max_feature_bins = 0;
     for (int f = 0; f < F_; ++f) max_feature_bins = std::max(max_feature_bins, h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f]);
     const char *wide_env = std::getenv("TGBM_WIDE_EVAL");  // "1": that split search for any data (tests)
+    const char *bytes_env = std::getenv("TGBM_DENSE_BIN_BYTES");  // "2": 16-bit bins whatever the bin counts (tests)
     wide_bins_ = max_feature_bins > 255;
-    if (wide_bins_) sparse_ = true;
-    log_info("layout: %s (density %.4f)", sparse_ ? "sparse CSR bin ids" : "dense column-blocked uint8", density);
+    int bin_bytes = (wide_bins_ || (bytes_env != nullptr && std::string(bytes_env) == "2")) ? 2 : 1;
+    if (bin_bytes == 2 && (2 * max_feature_bins > kDense16MaxBlockBins || (size_t)n_ * F_ * 4 > free_b / 2))
+        sparse_ = true;  // two features' bins of a block must fit the LDS, matrix and column copy the memory
+    if (sparse_) bin_bytes = 1;
+    log_info("layout: %s (density %.4f)",
+             sparse_ ? "sparse CSR bin ids" : (bin_bytes == 2 ? "dense column-blocked uint16" : "dense column-blocked uint8"),
+             density);
+    wide_eval_ = wide_bins_ || (wide_env != nullptr && std::string(wide_env) == "1");
     if (sparse_) {
         // TGBM_SPARSE_PASS=0 keeps the row-list kernels with per-node histograms in HBM (tests compare the two)
         const char *pe = std::getenv("TGBM_SPARSE_PASS");
@@ -292,9 +300,21 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         HIP_CHECK(hipFree(d_val));
         HIP_CHECK(hipFree(d_col));
     } else {
-        // dense column-blocked layout: blocks of W features, each block n rows x W bytes
+        // dense column-blocked layout: blocks of W features, each block n rows x W bins
         int W;
-        if (F_ <= 32) {
+        if (bin_bytes == 2) {
+            // 16-bit bins: the widest block (a power of two, at most 32 features = 64-byte rows) whose histogram
+            // leaves room for two workgroups per CU, else two features per block
+            auto block_bins = [&](int w) {
+                int most = 0;
+                for (int f0 = 0; f0 < F_; f0 += w)
+                    most = std::max(most, h_cut_row_ptr_[std::min(F_, f0 + w)] - h_cut_row_ptr_[f0]);
+                return most;
+            };
+            W = 32;
+            while (W > 2 && (W / 2 >= F_ || block_bins(W) > kDense16BlockBins)) W /= 2;
+            if (wide_bins_) log_info("features with up to %d bins: 16-bit bins, %d features per block", max_feature_bins, W);
+        } else if (F_ <= 32) {
             W = 4;
             while (W < F_) W *= 2;
         } else if (F_ <= 64 && n_bins_ <= 8192) {
@@ -305,17 +325,18 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         const int n_blocks = (F_ + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;
-        const size_t mat_bytes = (size_t)n_ * W * n_blocks;
-        bins_.block_stride = (size_t)n_ * W;
-        TGBM_CHECK(mat_bytes + (size_t)n_ * F_ < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
+        bins_.bin_bytes = bin_bytes;
+        const size_t mat_bytes = (size_t)n_ * W * n_blocks * bin_bytes;
+        bins_.block_stride = (size_t)n_ * W * bin_bytes;
+        TGBM_CHECK(mat_bytes + (size_t)n_ * F_ * bin_bytes < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
                    mat_bytes, free_b);
         d_binmat_ = dalloc<uint8_t>(mat_bytes);
-        launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);
+        launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);  // (all-ones: the sentinel of both widths)
         const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
-        uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_);
-        launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_);
+        uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_ * bin_bytes);
+        launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_ * bin_bytes);
         launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                         bins_.block_stride, d_colmat, col_stride);
+                         bins_.block_stride, d_colmat, col_stride, bin_bytes);
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
@@ -455,7 +476,7 @@ void Trainer::alloc_tree_buffers() {
     tb.complete_feature = -1;
     if (!sparse_) {
         for (int f = 0; f < F_ && tb.complete_feature < 0; ++f)
-            if (cuts_.feature_nnz[f] == (long)n_ &&
+            if (cuts_.feature_nnz[f] == (long)n_ && bins_.bin_bytes == 1 &&
                 device_count_bytes(stream_, bins_.col + (size_t)f * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
                 tb.complete_feature = f;
     }
@@ -1045,7 +1066,7 @@ void Trainer::reorder_rows() {
         reorder_sorter_.alloc(n_);
         d_perm_alt_ = dalloc<int>((size_t)n_);
         int *second = dalloc<int>((size_t)n_);
-        d_binmat_alt_ = dalloc<uint8_t>((size_t)n_ * bins_.W * bins_.n_blocks);
+        d_binmat_alt_ = dalloc<uint8_t>((size_t)n_ * bins_.W * bins_.n_blocks * bins_.bin_bytes);
         d_y_alt_ = dalloc<float>((size_t)n_);
         d_yp_alt_ = dalloc<float>((size_t)n_yp_);
         perm_spare_ = second;
@@ -1055,9 +1076,9 @@ void Trainer::reorder_rows() {
     launch_reorder_keys(stream_, n_, param_.depth, tb.nid, reorder_sorter_.keys[0], reorder_sorter_.vals[0]);
     const int cur = sort_pairs(stream_, reorder_sorter_, n_, param_.depth);
     const int *from = reorder_sorter_.vals[cur];
-    const size_t blk = (size_t)n_ * bins_.W;
+    const size_t blk = bins_.block_stride;
     for (int b = 0; b < bins_.n_blocks; ++b)
-        launch_gather_rows(stream_, n_, bins_.W, from, d_binmat_ + b * blk, d_binmat_alt_ + b * blk);
+        launch_gather_rows(stream_, n_, bins_.W * bins_.bin_bytes, from, d_binmat_ + b * blk, d_binmat_alt_ + b * blk);
     launch_gather_rows(stream_, n_, 4, from, d_y_, d_y_alt_);
     for (int k = 0; k < n_planes; ++k)
         launch_gather_rows(stream_, n_, 4, from, d_yp_ + (size_t)k * n_, d_yp_alt_ + (size_t)k * n_);
@@ -1073,7 +1094,7 @@ void Trainer::reorder_rows() {
     d_perm_ = perm_new;
     bins_.data = d_binmat_;
     launch_cols_from_rows(stream_, n_, bins_.W, F_, bins_.n_blocks, d_binmat_, bins_.block_stride,
-                          const_cast<uint8_t *>(bins_.col), bins_.col_stride);
+                          const_cast<uint8_t *>(bins_.col), bins_.col_stride, bins_.bin_bytes);
     h_perm_valid_ = false;
     nid_materialized_ = true;
     lookup_level_ = -1;
@@ -1142,7 +1163,7 @@ HistProfile Trainer::profile() {
             if (sparse_)  // CSR: 4-byte bin id per stored value + row pointer, gradient pair and row index per row
                 p.hist_bytes += (long long)((double)c.rows_built * ((double)nnz_ / n_ * 4 + 8 + 8 + (level > 0 ? 4 : 0)));
             else
-                p.hist_bytes += (long long)c.rows_built * (F_ + 8 + (level > 0 ? 4 : 0));
+                p.hist_bytes += (long long)c.rows_built * (F_ * bins_.bin_bytes + 8 + (level > 0 ? 4 : 0));
         }
     }
     (void)W;
@@ -1163,6 +1184,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "wide_eval") return wide_eval_ ? 1 : 0;
     if (key == "row_lists") return sparse_pass_ ? 0 : 1;  // the sparse level pass keeps a row -> node map only
     if (key == "dense_W") return bins_.W;
+    if (key == "dense_bin_bytes") return sparse_ ? 0 : bins_.bin_bytes;
     if (key == "reorders_done") return reorders_done_;
     if (key == "device_free_mb") {
         size_t free_b = 0, total_b = 0;
@@ -1188,7 +1210,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     if (name == "cut_val") src = cuts_.cut_val, bytes = sizeof(float) * (size_t)n_bins_;
     else if (name == "cut_row_ptr") src = cuts_.cut_row_ptr, bytes = sizeof(int) * (size_t)(F_ + 1);
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
-    else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks;
+    else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks * bins_.bin_bytes;
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
     else if (name == "nid") {
         // the map is kept as row lists; materialise it on demand (a re-ordering of the rows has done so already)
@@ -1223,7 +1245,7 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
         if (name == "nid" || name == "y") row_bytes = 4;
         else if (name == "y_pred") row_bytes = 4, n_planes = (size_t)(n_yp_ / n_);
         else if (name == "gh") row_bytes = sizeof(GHPair), n_planes = (size_t)param_.num_class;
-        else if (name == "binmat") row_bytes = (size_t)bins_.W, n_planes = (size_t)bins_.n_blocks;
+        else if (name == "binmat") row_bytes = (size_t)bins_.W * bins_.bin_bytes, n_planes = (size_t)bins_.n_blocks;
         const bool row_list = name == "ridx0" || name == "ridx1";
         static const std::vector<int> identity;
         const std::vector<int> &perm = (row_bytes || row_list) ? host_perm() : identity;

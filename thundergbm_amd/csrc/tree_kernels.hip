@@ -386,12 +386,12 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
 // rows, whose items therefore count finer: item_shift), so after at most that many rows every thread drains the
 // bins it owns into 64-bit register accumulators and clears them; at the end the registers go to the item's slot
 // of `partial`, at the item's scale (k_hist_merge shifts them to the tree's).
-// LPR consecutive lanes cover one row (one dword = four bin bytes per lane), so a wavefront load
-// instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
+// LPR consecutive lanes cover one row (one dword = four bin bytes per lane, or two 16-bit bins with BIN16), so a
+// wavefront load instruction reads 256 contiguous bytes and the 64 atomics of one step spread over many features.
 // (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
 // instead of two was measured: it halves the fetched bytes below the root, but the per-tree refresh of
 // the pairs costs what the gathers save.)
-template <int LPR, bool DIRECT, int BLK, int SLOTS>
+template <int LPR, bool DIRECT, int BLK, int SLOTS, bool BIN16>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
@@ -451,9 +451,10 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     static_assert(RPS * U <= kHistFlushRows, "one iteration must not exceed the flush interval");
     const int q = threadIdx.x % LPR;
     const int rsub = threadIdx.x / LPR;
-    const int W = LPR * 4;
-    const int *fo = feat_lds_off + fb * W + q * 4;
-    const int o0 = fo[0], o1 = fo[1], o2 = fo[2], o3 = fo[3];
+    constexpr int FPL = BIN16 ? 2 : 4;  // features per lane (one dword of the row)
+    constexpr int ROWB = LPR * 4;       // bytes per row of the block
+    const int *fo = feat_lds_off + fb * (LPR * FPL) + q * FPL;
+    const int o0 = fo[0], o1 = fo[1], o2 = BIN16 ? 0 : fo[2], o3 = BIN16 ? 0 : fo[3];
     const uint8_t *blk = bins.data + (size_t)fb * bins.block_stride + q * 4;
     long long accg[SLOTS], acch[SLOTS];
 #pragma unroll
@@ -468,7 +469,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
             bool ok = pos < end;
             int r = 0;
             if (ok) r = DIRECT ? pos : ridx[pos];
-            opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * W) : 0xffffffffu;
+            opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * ROWB) : 0xffffffffu;
             os[u] = ok ? gh[r] : GHPair{0, 0};
         }
     };
@@ -502,11 +503,17 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
             const long long gq = round_to_ll(s[u].g * scale_g);
             const long long hq = round_to_ll(fmaxf(s[u].h, 0.f) * scale_h);
             const unsigned long long add = ((unsigned long long)gq << h_bits) + (unsigned long long)hq;
-            const unsigned b0 = v & 0xff, b1 = (v >> 8) & 0xff, b2 = (v >> 16) & 0xff, b3 = v >> 24;
-            if (b0 != kMissingBin) atomicAdd(lds + o0 + b0, add);
-            if (b1 != kMissingBin) atomicAdd(lds + o1 + b1, add);
-            if (b2 != kMissingBin) atomicAdd(lds + o2 + b2, add);
-            if (b3 != kMissingBin) atomicAdd(lds + o3 + b3, add);
+            if (BIN16) {
+                const unsigned b0 = v & 0xffff, b1 = v >> 16;
+                if (b0 != kMissingBin16) atomicAdd(lds + o0 + b0, add);
+                if (b1 != kMissingBin16) atomicAdd(lds + o1 + b1, add);
+            } else {
+                const unsigned b0 = v & 0xff, b1 = (v >> 8) & 0xff, b2 = (v >> 16) & 0xff, b3 = v >> 24;
+                if (b0 != kMissingBin) atomicAdd(lds + o0 + b0, add);
+                if (b1 != kMissingBin) atomicAdd(lds + o1 + b1, add);
+                if (b2 != kMissingBin) atomicAdd(lds + o2 + b2, add);
+                if (b3 != kMissingBin) atomicAdd(lds + o3 + b3, add);
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -1112,8 +1119,9 @@ __global__ __launch_bounds__(kBlock) void k_eval_split(TreeBuffers tb_all, int l
 // Split search for features of any number of bins (max_num_bin above 255): one workgroup per (feature, node) walks the
 // feature's bins in chunks of kBlock with a block-wide inclusive scan of the exact 64-bit sums and a carry from
 // chunk to chunk. Same candidates, gains and tie rule as k_eval_split (whose wavefront holds a whole feature of at
-// most 256 bins); one candidate per feature. CSR layout only: the node of a pair that was not built from rows is
-// derived as parent - built while it is read (and stored for the next level).
+// most 256 bins); one candidate per feature. In the CSR layout the node of a pair that was not built from rows is
+// derived as parent - built while it is read (and stored for the next level); the dense layout's k_hist_merge has
+// done that already.
 __device__ __forceinline__ longlong2 wide_bin(const longlong2 *h, const longlong2 *h_par, const longlong2 *h_built, int b) {
     if (h_par == nullptr) return h[b];
     const longlong2 pv = h_par[b], bv = h_built[b];
@@ -1141,7 +1149,7 @@ __global__ __launch_bounds__(kBlock) void k_eval_split_wide(TreeBuffers tb_all, 
     const int lane = lane_id(), w = wave_id();
     longlong2 *h = tb.hist(level) + (size_t)x_in * tb.n_bins;
     const longlong2 *h_par = nullptr, *h_built = nullptr;
-    if (level > 0 && !tb.singles(level)) {
+    if (tb.sparse && level > 0 && !tb.singles(level)) {  // (the dense layout's k_hist_merge has derived the siblings)
         const int built = tb.hpair_built[x_in >> 1];
         if (built >= 0 && built != x) {
             h_par = tb.hist(level + 1) + (size_t)(x_in >> 1) * tb.n_bins;
@@ -1397,7 +1405,7 @@ __global__ __launch_bounds__(kBlock) void k_best_update(TreeBuffers tb_all, int 
 // Decide left/right for every row of a work item from the split feature's column of the bin matrix
 // (missing -> default direction, else right iff bin >= split bin; the reference's rule at
 // hist_tree_builder_single.cu:986-1011) and count the rows that go left.
-template <bool DIRECT>
+template <bool DIRECT, typename BinT>
 __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all, DenseBins bins, int level) {
     __shared__ int lds[kWaves];
     __shared__ int s_x;
@@ -1418,9 +1426,11 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     const int pb = sg.x + (item - tb.pbegin(level)[x_in]) * kPartChunk;
     const int pe = min(sg.y, pb + kPartChunk);
     const int f = nd.split_feature_id;
-    const int sbid = nd.split_bid;
+    // (features of more than 255 bins keep their split bin in a side array: TreeNode::split_bid is a byte)
+    const int sbid = tb.split_bin != nullptr ? tb.split_bin[off + x_in] : (int)nd.split_bid;
     const bool dr = nd.default_right;
-    const uint8_t *column = bins.col + (size_t)f * bins.col_stride;
+    constexpr int kMissing = sizeof(BinT) == 2 ? kMissingBin16 : kMissingBin;
+    const BinT *column = reinterpret_cast<const BinT *>(bins.col) + (size_t)f * bins.col_stride;
     int nleft = 0;
     // all row ids first, then all bin bytes, then the stores: the three phases keep a thread's eight
     // gathers in flight together (the byte store may alias the byte loads for the compiler)
@@ -1436,7 +1446,7 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
 #pragma unroll
     for (int k = 0; k < R; ++k) {
         if (row[k] >= 0) {
-            const bool right = (b[k] == kMissingBin) ? dr : (b[k] >= sbid);
+            const bool right = (b[k] == kMissing) ? dr : (b[k] >= sbid);
             tb.goes_right[pb + k * kBlock + threadIdx.x] = right ? 1 : 0;
             nleft += right ? 0 : 1;
         }
@@ -1845,6 +1855,10 @@ __device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBi
         // (the node's own heap id is its children's parent index; wide features keep their split bin in a side array)
         const int sb = tb.split_bin != nullptr ? tb.split_bin[(nd.lch_index - 1) / 2] : (int)nd.split_bid;
         right = csr_goes_right(cbins, row, cb, ce, cb + sb, nd.default_right);
+    } else if (dbins.bin_bytes == 2) {
+        const int b = reinterpret_cast<const uint16_t *>(dbins.col)[(size_t)nd.split_feature_id * dbins.col_stride + row];
+        const int sb = tb.split_bin != nullptr ? tb.split_bin[(nd.lch_index - 1) / 2] : (int)nd.split_bid;
+        right = (b == kMissingBin16) ? nd.default_right : (b >= sb);
     } else {
         const int b = dbins.col[(size_t)nd.split_feature_id * dbins.col_stride + row];
         right = (b == kMissingBin) ? nd.default_right : (b >= nd.split_bid);
@@ -1959,12 +1973,12 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
                 row[u] = node[u] == 0 ? p : tb.list(31 - __clz(node[u] + 1))[p];
             }
         }
-        if (SPARSE) {
+        if (SPARSE || dbins.bin_bytes == 2) {  // (16-bit bins: the packed split word has no room for the split bin)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (node[u] < 0) continue;
                 s_leaf[row[u] - r0] =
-                    split[u] >= 0 ? end_child_of<true>(tb, dbins, cbins, tb.nodes[node[u]], row[u]) : node[u];
+                    split[u] >= 0 ? end_child_of<SPARSE>(tb, dbins, cbins, tb.nodes[node[u]], row[u]) : node[u];
             }
         } else {
             int bin[U];
@@ -2149,7 +2163,7 @@ void launch_tree_init(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_cla
     }
 }
 
-template <int LPR, int SLOTS>
+template <int LPR, int SLOTS, bool BIN16>
 static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                               int level, int n_class) {
     const int n_pairs = tb.n_hpairs(level);
@@ -2160,44 +2174,51 @@ static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseB
         static size_t opted = 0;
         if (lds > opted) {
             HIP_CHECK(hipFuncSetAttribute(
-                reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS>),
+                reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS, BIN16>),
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             HIP_CHECK(hipFuncSetAttribute(
-                reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS>),
+                reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS, BIN16>),
                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             opted = lds;
         }
     }
     if (level == 0)
-        k_hist_dense<LPR, true, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
+        k_hist_dense<LPR, true, kHistBlock, SLOTS, BIN16><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
     else
-        k_hist_dense<LPR, false, kHistBlock, SLOTS><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
+        k_hist_dense<LPR, false, kHistBlock, SLOTS, BIN16><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
 }
 
 template <int LPR>
 static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                                 int level, int n_class) {
     const int slots = (tb.max_block_bins + kHistBlock - 1) / kHistBlock;  // bins drained per thread
-    if (slots <= 1) hist_dense_launch<LPR, 1>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 2) hist_dense_launch<LPR, 2>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 3) hist_dense_launch<LPR, 3>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 4) hist_dense_launch<LPR, 4>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 6) hist_dense_launch<LPR, 6>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 7) hist_dense_launch<LPR, 7>(s, tb, bins, gh, level, n_class);  // fewer accumulator registers
-    else if (slots <= 8) hist_dense_launch<LPR, 8>(s, tb, bins, gh, level, n_class);
-    else if (slots <= 20) hist_dense_launch<LPR, 20>(s, tb, bins, gh, level, n_class);
+    if (bins.bin_bytes == 2) {  // (fewer variants: the blocks of 16-bit bins are sized to fill the LDS)
+        if (slots <= 4) hist_dense_launch<LPR, 4, true>(s, tb, bins, gh, level, n_class);
+        else if (slots <= 8) hist_dense_launch<LPR, 8, true>(s, tb, bins, gh, level, n_class);
+        else if (slots <= 20) hist_dense_launch<LPR, 20, true>(s, tb, bins, gh, level, n_class);
+        else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
+        return;
+    }
+    if (slots <= 1) hist_dense_launch<LPR, 1, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 2) hist_dense_launch<LPR, 2, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 3) hist_dense_launch<LPR, 3, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 4) hist_dense_launch<LPR, 4, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 6) hist_dense_launch<LPR, 6, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 7) hist_dense_launch<LPR, 7, false>(s, tb, bins, gh, level, n_class);  // fewer accumulator registers
+    else if (slots <= 8) hist_dense_launch<LPR, 8, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 20) hist_dense_launch<LPR, 20, false>(s, tb, bins, gh, level, n_class);
     else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
 }
 
 void launch_hist_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh, int level,
                        int n_class) {
-    switch (bins.W) {
+    switch (bins.W * bins.bin_bytes) {  // bytes per row of a block = 4 x lanes per row
         case 4: hist_dense_dispatch<1>(s, tb, bins, gh, level, n_class); break;
         case 8: hist_dense_dispatch<2>(s, tb, bins, gh, level, n_class); break;
         case 16: hist_dense_dispatch<4>(s, tb, bins, gh, level, n_class); break;
         case 32: hist_dense_dispatch<8>(s, tb, bins, gh, level, n_class); break;
         case 64: hist_dense_dispatch<16>(s, tb, bins, gh, level, n_class); break;
-        default: fatal("unsupported dense block width %d", bins.W);
+        default: fatal("unsupported dense block width %d x %d bytes", bins.W, bins.bin_bytes);
     }
 }
 
@@ -2291,12 +2312,15 @@ void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float r
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class) {
     if (level == tb.depth - 1) return;  // the last level's children never get row lists (see k_tree_end)
     const dim3 one(1, 1, n_class), items(tb.max_pitems, 1, n_class);
+    const bool b16 = bins.bin_bytes == 2;
     if (level == 0) {
-        k_part_count_dense<true><<<items, kBlock, 0, s>>>(tb, bins, level);
+        if (b16) k_part_count_dense<true, uint16_t><<<items, kBlock, 0, s>>>(tb, bins, level);
+        else k_part_count_dense<true, uint8_t><<<items, kBlock, 0, s>>>(tb, bins, level);
         k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
         k_part_scatter<true><<<items, kBlock, 0, s>>>(tb, level);
     } else {
-        k_part_count_dense<false><<<items, kBlock, 0, s>>>(tb, bins, level);
+        if (b16) k_part_count_dense<false, uint16_t><<<items, kBlock, 0, s>>>(tb, bins, level);
+        else k_part_count_dense<false, uint8_t><<<items, kBlock, 0, s>>>(tb, bins, level);
         k_part_scan_plan<<<one, kBlock, 0, s>>>(tb, level);
         k_part_scatter<false><<<items, kBlock, 0, s>>>(tb, level);
     }

@@ -113,7 +113,7 @@ class Session:
 
     def binmat(self):
         W, nb = self.info("dense_W"), self.info("dense_blocks")
-        return self.get("binmat", np.uint8, (nb, self.n, W))
+        return self.get("binmat", np.uint16 if self.info("dense_bin_bytes") == 2 else np.uint8, (nb, self.n, W))
 
     def global_bin_ids(self, row_ptr, col):
         """Global bin id of every stored value (the reference's csr_bin_id) and its local bin id."""
