@@ -79,6 +79,7 @@ CASES = {
     "reg_logistic": (1200, 8, 8, "reg:logistic", "prob", dict(depth=4, max_num_bin=32), None),
     "softprob": (1500, 10, 8, "multi:softprob", "multi", dict(depth=3, max_num_bin=32), None),
     "wide_dense_blocks": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense"),
+    "wide_dense_blocks_16_bit_bins": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense-16"),
     "wide_sparse": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse"),
     # the same through the kernel without an LDS head (every value goes to HBM atomics)
     "wide_sparse_no_head": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse-nohead"),
@@ -121,18 +122,47 @@ def test_random_small_cases(T):
     assert ran > 120
 
 
+def test_random_small_cases_16_bit_bins(T):
+    """40 more seeded random shapes through the dense layout with 16-bit bins (forced: the data has at most 255 bins
+    per feature, so the oracle can follow), same teacher-forced comparison."""
+    objs = [("reg:linear", "reg"), ("binary:logistic", "bin"), ("reg:logistic", "prob"), ("multi:softmax", "multi")]
+    ran = 0
+    for seed in range(3000, 3040):
+        rng = np.random.default_rng(seed)
+        n = int(rng.choice([5, 64, 65, 700, 4097, 9000, 20000]))
+        F = int(rng.choice([1, 2, 3, 5, 9, 17, 40]))
+        depth = int(rng.integers(1, 7))
+        bins = int(rng.choice([2, 8, 33, 255]))
+        objective, kind = objs[int(rng.integers(0, 4))]
+        if kind in ("bin", "multi") and n < 8:
+            objective, kind = "reg:linear", "reg"
+        case = (n, F, int(rng.integers(1, F + 1)), objective, kind, dict(depth=depth, max_num_bin=bins), "dense-16")
+        if len(_ragged(n, F, seed, case[2])[0]) == 0:
+            continue
+        try:
+            run_case(T, case, seed)
+        except AssertionError as e:
+            raise AssertionError("seed %d case %r: %s" % (seed, case, e))
+        ran += 1
+    assert ran > 30
+
+
 def run_case(T, name, seed):
     n, F, max_len, objective, kind, kw, layout = CASES[name] if isinstance(name, str) else name
     if layout:
         os.environ["TGBM_LAYOUT"] = layout.split("-")[0]
         if layout.endswith("-nohead"):
             os.environ["TGBM_CSR_HEAD"] = "0"
+        if layout.endswith("-16"):
+            os.environ["TGBM_DENSE_BIN_BYTES"] = "2"
     val, rp, col = _ragged(n, F, seed, max_len)
     y = _target(val, rp, col, n, F, seed, kind)
     rounds = 4
     kw = dict(kw, objective=objective, n_trees=rounds, learning_rate=0.5)
     lam = kw.get("lambda_", 1.0)
     s = T.Session(val, rp, col, y, **kw)
+    if layout and layout.endswith("-16"):
+        assert s.info("dense_bin_bytes") == 2
     o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
     # data preparation: exact
     cv, crp, cf = s.cuts()
