@@ -841,6 +841,34 @@ def test_more_than_255_bins_per_feature(T, layout, max_bins):
     s.close()
 
 
+def test_more_than_255_bins_through_the_c_abi(T, tmp_path):
+    """fit / predict / save / load of the estimator (sparse_train_scikit, sparse_predict_scikit, save / load through
+    the model file) with 2000 bins per feature: the predictor follows split_value, so the prediction of the training
+    rows is the session's training prediction without the base score (the C-API predict path carries none), also
+    after a round trip through the model file, whose split_bid keeps only the split bin's low byte."""
+    rng = np.random.default_rng(11)
+    n, F = 20000, 7
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.05] = 0.0
+    y = (np.cos(3 * X[:, 0]) * X[:, 1] + 0.5 * X[:, 2] + 0.05 * rng.standard_normal(n)).astype(np.float32)
+    kw = dict(depth=6, n_trees=8, learning_rate=0.3, max_num_bin=2000)
+    m = T.TGBMRegressor(objective="reg:linear", verbose=0, **kw)
+    m.fit(X, y)
+    pred = np.asarray(m.predict(X)).ravel()
+    val, rp, col = D.dense_to_csr(X)
+    s = T.Session(val, rp, col, y, objective="reg:linear", **kw)
+    assert s.info("wide_bins") == 1 and s.info("dense_bin_bytes") == 2
+    s.boost(8)
+    np.testing.assert_allclose(pred, s.y_pred() - s.base_score, rtol=1e-5, atol=1e-5)
+    assert np.sqrt(np.mean((pred + s.base_score - y) ** 2)) < 0.6 * np.std(y)
+    s.close()
+    path = str(tmp_path / "wide.model")
+    m.save_model(path)
+    m2 = T.TGBMRegressor(objective="reg:linear", verbose=0)
+    m2.load_model(path)
+    assert np.array_equal(np.asarray(m2.predict(X)).ravel(), pred)
+
+
 @pytest.mark.parametrize("objective,F,reorder", [("reg:linear", 5, "0"), ("binary:logistic", 40, "always"),
                                                  ("multi:softmax", 11, "0"), ("binary:logistic", 3, "0")])
 def test_dense_16_bit_bins_equal_byte_bins(T, objective, F, reorder):
