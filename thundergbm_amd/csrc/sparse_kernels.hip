@@ -588,7 +588,8 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     }
     __syncthreads();
     const int i0 = threadIdx.x * kSoV;
-    const int pb = i0 + (threadIdx.x >> 2);  // so_phys(i0 + j) = pb + j: a thread's eight positions share one padding count
+    static_assert(32 % kSoV == 0, "a thread's positions must not straddle a padding element");
+    const int pb = so_phys(i0);  // so_phys(i0 + j) = pb + j: a thread's positions share one padding count
     int Mn = M;  // values of the new order
     if (!LEVEL0) {
         const ulonglong2 *__restrict__ row_side = tb.row_side;
