@@ -159,7 +159,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     size_t free_b = 0, total_b = 0;
     HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
     const char *force = std::getenv("TGBM_LAYOUT");  // "dense" / "sparse" override the heuristic (tests)
-    sparse_ = (F_ > 4096 && density < 0.05) || (size_t)n_ * F_ * 2 > free_b / 2;
+    sparse_ = (F_ > 4096 && density < 0.05) || (size_t)n_ * F_ * 2 > free_b / 2 || n_ >= (1 << 29);
     if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
     if (force != nullptr && std::string(force) == "dense") sparse_ = false;
     if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
@@ -322,6 +322,11 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         } else {
             W = 32;
         }
+        // (the histogram kernel addresses a block's rows, the gradient pairs and the row lists with unsigned 32-bit
+        // byte offsets: a block stays below 4 GiB, the rows below 2^29)
+        while (W * bin_bytes > 4 && (size_t)n_ * W * bin_bytes >= ((size_t)1 << 32)) W /= 2;
+        TGBM_CHECK((size_t)n_ * W * bin_bytes < ((size_t)1 << 32) && n_ < (1 << 29),
+                   "%d rows are more than the dense layout addresses; use TGBM_LAYOUT=sparse", n_);
         const int n_blocks = (F_ + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;

@@ -446,8 +446,9 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     const float scale_h = ldexpf(quant->scale_h, -__builtin_amdgcn_readfirstlane(s_range[3]));
     const unsigned long long h_mask = (1ull << h_bits) - 1ull;  // h_bits <= 32
     constexpr int RPS = BLK / LPR;  // rows per step of the whole block
-    // steps in flight per thread: three keep the 64-register variants (8 waves per SIMD) free of spills
-    constexpr int U = SLOTS <= 8 ? 3 : 4;
+    // rows per thread and stage: what the registers left over by the drain accumulators hold without spills (64
+    // registers per thread with two workgroups per CU)
+    constexpr int U = SLOTS <= 4 ? 4 : 2;
     static_assert(RPS * U <= kHistFlushRows, "one iteration must not exceed the flush interval");
     const int q = threadIdx.x % LPR;
     const int rsub = threadIdx.x / LPR;
@@ -455,29 +456,48 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     constexpr int ROWB = LPR * 4;       // bytes per row of the block
     const int *fo = feat_lds_off + fb * (LPR * FPL) + q * FPL;
     const int o0 = fo[0], o1 = fo[1], o2 = BIN16 ? 0 : fo[2], o3 = BIN16 ? 0 : fo[3];
-    const uint8_t *blk = bins.data + (size_t)fb * bins.block_stride + q * 4;
+    // (a block is smaller than 4 GiB and has fewer than 2^29 rows - checked when the layout is chosen -, so a lane
+    // addresses its dword, its gradient pair and its row id with an unsigned 32-bit offset from a uniform base)
+    const uint8_t *blk = bins.data + (size_t)fb * bins.block_stride;
+    const unsigned qoff = q * 4;
     long long accg[SLOTS], acch[SLOTS];
 #pragma unroll
     for (int k = 0; k < SLOTS; ++k) accg[k] = acch[k] = 0;
     int pending = 0;  // rows accumulated in LDS since the last drain (uniform across the block)
     unsigned pk[U], pk_next[U];
     GHPair s[U], s_next[U];
-    auto load_rows = [&](int base, unsigned(&opk)[U], GHPair(&os)[U]) {
+    // Three stages in flight per thread: the row ids of the step after next, the bins and gradient pairs of the next
+    // step (gathered through row ids that arrived during the previous iteration), the atomics of this step. All
+    // loads are unconditional - positions past the item's end are clamped to its last row and their bins replaced by
+    // the sentinel - and each stage's loads are issued back to back, so that no load waits for an unrelated one.
+    int r_next[U];
+    auto load_ids = [&](int base, int(&r)[U]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            int pos = base + rsub + u * RPS;
-            bool ok = pos < end;
-            int r = 0;
-            if (ok) r = DIRECT ? pos : ridx[pos];
-            opk[u] = ok ? *reinterpret_cast<const unsigned *>(blk + (size_t)r * ROWB) : 0xffffffffu;
-            os[u] = ok ? gh[r] : GHPair{0, 0};
+            const int pos = min(base + rsub + u * RPS, end - 1);
+            r[u] = DIRECT ? pos : *reinterpret_cast<const int *>(reinterpret_cast<const char *>(ridx) + (unsigned)pos * 4u);
         }
     };
-    if (begin < end) load_rows(begin, pk, s);
-    for (int base = begin; base < end; base += RPS * U) {
+    auto load_rows = [&](const int(&r)[U], unsigned(&opk)[U], GHPair(&os)[U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            opk[u] = *reinterpret_cast<const unsigned *>(blk + ((unsigned)r[u] * (unsigned)ROWB + qoff));
+            os[u] = *reinterpret_cast<const GHPair *>(reinterpret_cast<const char *>(gh) + (unsigned)r[u] * 8u);
+        }
+    };
+    constexpr int STEP = RPS * U;
+    if (begin < end) {
+        load_ids(begin, r_next);
+        load_rows(r_next, pk, s);
+        if (begin + STEP < end) load_ids(begin + STEP, r_next);
+    }
+    for (int base = begin; base < end; base += STEP) {
         // the next step's rows are requested before this step's atomics (and before a drain's
         // barriers), so the memory pipeline stays busy
-        if (base + RPS * U < end) load_rows(base + RPS * U, pk_next, s_next);
+        if (base + STEP < end) {
+            load_rows(r_next, pk_next, s_next);
+            if (base + 2 * STEP < end) load_ids(base + 2 * STEP, r_next);
+        }
         const int step_rows = min(RPS * U, end - base);
         if (pending + step_rows > kHistFlushRows) {
             __syncthreads();
@@ -498,7 +518,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         pending += step_rows;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const unsigned v = pk[u];
+            const unsigned v = (base + rsub + u * RPS < end) ? pk[u] : 0xffffffffu;  // (a clamped position adds nothing)
             // exact products (the scales are powers of two), rounded once to the nearest integer
             const long long gq = round_to_ll(s[u].g * scale_g);
             const long long hq = round_to_ll(fmaxf(s[u].h, 0.f) * scale_h);
