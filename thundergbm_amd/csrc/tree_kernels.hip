@@ -1452,24 +1452,30 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     constexpr int kMissing = sizeof(BinT) == 2 ? kMissingBin16 : kMissingBin;
     const BinT *column = reinterpret_cast<const BinT *>(bins.col) + (size_t)f * bins.col_stride;
     int nleft = 0;
-    // all row ids first, then all bin bytes, then the stores: the three phases keep a thread's eight
-    // gathers in flight together (the byte store may alias the byte loads for the compiler)
+    // All row ids first, then all bins, then the decisions, then the stores. Every load is unconditional (positions
+    // past the item's end are clamped to its last row), so each phase's loads are issued back to back and a thread's
+    // eight gathers are in flight together; a conditional load would make the compiler wait for everything
+    // outstanding, the previous store included, before the next one.
     constexpr int R = kPartChunk / kBlock;
     int row[R], b[R];
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-        const int pos = pb + k * kBlock + threadIdx.x;
-        row[k] = pos < pe ? (DIRECT ? pos : ridx[pos]) : -1;
+        const int pos = min(pb + k * kBlock + (int)threadIdx.x, pe - 1);
+        row[k] = DIRECT ? pos : ridx[pos];
     }
 #pragma unroll
-    for (int k = 0; k < R; ++k) b[k] = row[k] >= 0 ? column[row[k]] : 0;
+    for (int k = 0; k < R; ++k) b[k] = column[row[k]];
+    unsigned rights = 0;
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-        if (row[k] >= 0) {
-            const bool right = (b[k] == kMissing) ? dr : (b[k] >= sbid);
-            tb.goes_right[pb + k * kBlock + threadIdx.x] = right ? 1 : 0;
-            nleft += right ? 0 : 1;
-        }
+        const bool right = (b[k] == kMissing) ? dr : (b[k] >= sbid);
+        rights |= (right ? 1u : 0u) << k;
+        if (pb + k * kBlock + (int)threadIdx.x < pe) nleft += right ? 0 : 1;
+    }
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const int pos = pb + k * kBlock + threadIdx.x;
+        if (pos < pe) tb.goes_right[pos] = (uint8_t)((rights >> k) & 1u);
     }
     int tot = block_sum(nleft, lds);
     if (threadIdx.x == 0) tb.pitem_nleft[item] = tot;
@@ -1703,7 +1709,7 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
 template <bool DIRECT>
 __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int level) {
     __shared__ int s_x;
-    __shared__ int s_cnt[2][kWaves];
+    __shared__ int s_cnt[kPartChunk / kBlock][2][kWaves];
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     const int *__restrict__ ridx_cur = tb.list(level);
     int *__restrict__ ridx_next = tb.list(level + 1);
@@ -1722,26 +1728,37 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int
     int left_base = sg.x + loff;
     int right_base = sg.x + tb.node_nleft[x_in] + ((pb - sg.x) - loff);
     const int lane = lane_id(), w = wave_id();
-    for (int k = 0; k < kPartChunk / kBlock; ++k) {
-        int pos = pb + k * kBlock + threadIdx.x;
-        bool valid = pos < pe;
-        int row = 0;
-        bool right = false;
-        if (valid) {
-            row = DIRECT ? pos : ridx_cur[pos];
-            right = tb.goes_right[pos] != 0;
-        }
-        unsigned long long mL = __ballot(valid && !right);
-        unsigned long long mR = __ballot(valid && right);
+    // all loads of the item first (unconditional, clamped positions), one barrier for the wavefront counts of all
+    // eight steps, then all stores
+    constexpr int R = kPartChunk / kBlock;
+    int row[R];
+    unsigned rights = 0;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const int pos = min(pb + k * kBlock + (int)threadIdx.x, pe - 1);
+        row[k] = DIRECT ? pos : ridx_cur[pos];
+        rights |= (tb.goes_right[pos] != 0 ? 1u : 0u) << k;
+    }
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const bool valid = pb + k * kBlock + (int)threadIdx.x < pe;
+        const bool right = (rights >> k) & 1u;
+        const unsigned long long mL = __ballot(valid && !right), mR = __ballot(valid && right);
         if (lane == 0) {
-            s_cnt[0][w] = __popcll(mL);
-            s_cnt[1][w] = __popcll(mR);
+            s_cnt[k][0][w] = __popcll(mL);
+            s_cnt[k][1][w] = __popcll(mR);
         }
-        __syncthreads();
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const bool valid = pb + k * kBlock + (int)threadIdx.x < pe;
+        const bool right = (rights >> k) & 1u;
+        const unsigned long long mL = __ballot(valid && !right), mR = __ballot(valid && right);
         int bL = 0, bR = 0, tL = 0, tR = 0;
 #pragma unroll
         for (int i = 0; i < kWaves; ++i) {
-            int cl = s_cnt[0][i], cr = s_cnt[1][i];
+            const int cl = s_cnt[k][0][i], cr = s_cnt[k][1][i];
             if (i < w) {
                 bL += cl;
                 bR += cr;
@@ -1750,12 +1767,11 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int
             tR += cr;
         }
         if (valid) {
-            int dest = right ? right_base + bR + lanes_below(mR) : left_base + bL + lanes_below(mL);
-            ridx_next[dest] = row;
+            const int dest = right ? right_base + bR + lanes_below(mR) : left_base + bL + lanes_below(mL);
+            ridx_next[dest] = row[k];
         }
         left_base += tL;
         right_base += tR;
-        __syncthreads();
     }
 }
 
