@@ -1992,39 +1992,38 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
     }
     __syncthreads();
     for (int j0 = threadIdx.x; j0 < total; j0 += kBlock * U) {
+        // (every load is unconditional - entries past the end repeat the last one and are skipped when the results
+        // are stored -, so a thread's four list entries, then its four bins, are in flight together)
         int node[U], row[U], split[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int j = j0 + u * kBlock;
-            node[u] = -1;
-            if (j < total) {
-                int lo = 0, hi = n_list;  // last entry with s_off <= j
-                while (hi - lo > 1) {
-                    const int mid = (lo + hi) / 2;
-                    if (s_off[mid] <= j) lo = mid; else hi = mid;
-                }
-                node[u] = s_list[lo][0];
-                split[u] = s_split[lo];
-                const int p = s_list[lo][1] + (j - s_off[lo]);
-                row[u] = node[u] == 0 ? p : tb.list(31 - __clz(node[u] + 1))[p];
+            const int j = min(j0 + u * kBlock, total - 1);
+            int lo = 0, hi = n_list;  // last entry with s_off <= j
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) / 2;
+                if (s_off[mid] <= j) lo = mid; else hi = mid;
             }
+            node[u] = s_list[lo][0];
+            split[u] = s_split[lo];
+            const int p = s_list[lo][1] + (j - s_off[lo]);
+            const int listed = tb.list(31 - __clz(node[u] + 1))[p];  // (the root's list is the identity and not stored)
+            row[u] = node[u] == 0 ? p : listed;
         }
         if (SPARSE || dbins.bin_bytes == 2) {  // (16-bit bins: the packed split word has no room for the split bin)
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (node[u] < 0) continue;
+                if (j0 + u * kBlock >= total) continue;
                 s_leaf[row[u] - r0] =
                     split[u] >= 0 ? end_child_of<SPARSE>(tb, dbins, cbins, tb.nodes[node[u]], row[u]) : node[u];
             }
         } else {
             int bin[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                bin[u] = (node[u] >= 0 && split[u] >= 0)
-                             ? dbins.col[(size_t)(split[u] & 0xffff) * dbins.col_stride + row[u]] : 0;
+            for (int u = 0; u < U; ++u)  // (feature 0 for the entries of nodes that did not split)
+                bin[u] = dbins.col[(size_t)(split[u] >= 0 ? split[u] & 0xffff : 0) * dbins.col_stride + row[u]];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (node[u] < 0) continue;
+                if (j0 + u * kBlock >= total) continue;
                 int leaf = node[u];
                 if (split[u] >= 0) {
                     const bool right = bin[u] == kMissingBin ? (split[u] >> 24) != 0 : bin[u] >= ((split[u] >> 16) & 0xff);
