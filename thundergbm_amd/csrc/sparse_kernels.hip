@@ -277,21 +277,27 @@ __global__ __launch_bounds__(kSpBlock) void k_sparse_level(TreeBuffers tb_all, C
             // accumulate: four values in flight per thread (row -> node from the cache-resident map, then the pair)
             constexpr int U = 8;
             for (int e0 = v0 + threadIdx.x; e0 < v1; e0 += kSpBlock * U) {
+                // (every load is unconditional - a value index past the end repeats the last value and is skipped
+                // below -, so each stage's eight loads are issued together instead of one after the other)
                 int gb[U], row[U], x[U];
+                GHPair s[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int e = e0 + u * kSpBlock;
-                    const bool in = e < v1;
-                    gb[u] = in ? bins.csc_bin[e] : 0;
-                    row[u] = in ? bins.csc_row[e] : -1;
+                    const int e = min(e0 + u * kSpBlock, v1 - 1);
+                    gb[u] = bins.csc_bin[e];
+                    row[u] = bins.csc_row[e];
+                    if (csc_gh != nullptr) s[u] = csc_gh[e];
                 }
 #pragma unroll
-                for (int u = 0; u < U; ++u) x[u] = row[u] >= 0 ? (int)nid16[row[u]] - off - n0 : -1;
+                for (int u = 0; u < U; ++u) x[u] = (int)nid16[row[u]] - off - n0;
+                if (csc_gh == nullptr) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) s[u] = gh[row[u]];
+                }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    if ((unsigned)x[u] < (unsigned)nn) {
-                        const GHPair s = csc_gh != nullptr ? csc_gh[e0 + u * kSpBlock] : gh[row[u]];
-                        const long long gq = round_to_ll(s.g * scale_g), hq = round_to_ll(s.h * scale_h);
+                    if (e0 + u * kSpBlock < v1 && (unsigned)x[u] < (unsigned)nn) {
+                        const long long gq = round_to_ll(s[u].g * scale_g), hq = round_to_ll(s[u].h * scale_h);
                         unsigned long long *cell = reinterpret_cast<unsigned long long *>(cells + (size_t)x[u] * nbins + (gb[u] - bin0));
                         atomicAdd(cell, (unsigned long long)gq);
                         atomicAdd(cell + 1, (unsigned long long)hq);
