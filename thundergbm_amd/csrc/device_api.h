@@ -467,9 +467,17 @@ void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);
 
 // prediction of the n rows that row_ptr addresses (entry offsets into col / val); out[t * out_stride + i] for
 // class tree t and row i, out_stride = 0 means n (a slice of a larger row set passes the whole set's size)
+// `packed` (optional): the same nodes as 16-byte records (launch_pack_model); with them the trees are walked from LDS
 void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
                     const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
-                    float *out, size_t out_stride = 0);
+                    float *out, size_t out_stride = 0, const struct PackedNode *packed = nullptr);
+// What a traversal reads of a node, in one 16-byte record.
+struct PackedNode {
+    float split_value, base_weight;
+    unsigned children;  // left | right << 16 (a tree has at most 2^15 - 1 nodes)
+    unsigned meta;      // split feature (24 bits, all ones: not a feature of the data) | default_right << 30 | leaf << 31
+};
+void launch_pack_model(hipStream_t s, const TreeNode *model, long n_total, int n_nodes, PackedNode *packed);
 void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y);
 
 }  // namespace tgbm

@@ -51,14 +51,17 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     float *d_val = nullptr, *d_out = nullptr, *d_label = nullptr;
     int *d_col = nullptr, *d_row_ptr = nullptr;
     TreeNode *d_model = nullptr;
+    PackedNode *d_packed = nullptr;
     const size_t n_out = (size_t)n * nct;
     HIP_CHECK(hipMalloc(&d_val, sizeof(float) * (size_t)std::max(nnz, 1l)));
     HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz, 1l)));
     HIP_CHECK(hipMalloc(&d_row_ptr, sizeof(int) * (size_t)(n + 1)));
     HIP_CHECK(hipMalloc(&d_model, sizeof(TreeNode) * flat.size()));
+    HIP_CHECK(hipMalloc(&d_packed, sizeof(PackedNode) * flat.size()));
     HIP_CHECK(hipMalloc(&d_out, sizeof(float) * std::max(n_out, (size_t)1)));
     HIP_CHECK(hipMemcpyAsync(d_row_ptr, ds.row_ptr, sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, s));
     HIP_CHECK(hipMemcpyAsync(d_model, flat.data(), sizeof(TreeNode) * flat.size(), hipMemcpyHostToDevice, s));
+    launch_pack_model(s, d_model, (long)flat.size(), n_nodes, d_packed);
     launch_fill_f32(s, d_out, 0.f, n_out);
     // The column indices go up first (the feature count, which selects the traversal kernel, may have to be
     // taken from them), then the values in slices of whole rows on a second stream: the traversal of a
@@ -82,7 +85,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
             if (e1 > e0) upload_large(s_up, d_val + e0, ds.val + e0, sizeof(float) * (size_t)(e1 - e0));
             HIP_CHECK(hipStreamSynchronize(s_up));  // small copies return before they are done
             launch_predict(s, r1 - r0, F, d_row_ptr + r0, d_col, d_val, d_model, n_iter, nct, n_nodes,
-                           param.learning_rate, param.base_score, d_out + r0, (size_t)n);
+                           param.learning_rate, param.base_score, d_out + r0, (size_t)n, d_packed);
             HIP_CHECK_LAUNCHES("predict");
             r0 = r1;
         }
@@ -148,6 +151,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipFree(d_col));
     HIP_CHECK(hipFree(d_row_ptr));
     HIP_CHECK(hipFree(d_model));
+    HIP_CHECK(hipFree(d_packed));
     HIP_CHECK(hipFree(d_out));
     if (d_label) HIP_CHECK(hipFree(d_label));
     HIP_CHECK(hipStreamDestroy(s));
