@@ -841,6 +841,43 @@ def test_more_than_255_bins_per_feature(T, layout, max_bins):
     s.close()
 
 
+def test_dense_layout_keeps_the_later_of_two_entries_with_the_same_column(T):
+    """Rows that store a column twice (not something the wrappers produce: they sort and merge columns) - the dense
+    bin matrix has one cell per (row, feature) and keeps the bin of the later entry, in both bin widths."""
+    rng = np.random.default_rng(3)
+    n, F = 500, 6
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[X == 0] = 0.5
+    val, rp, col = D.dense_to_csr(X)
+    # every third row gets a second entry for column 2 right after the first, with another value
+    vals, cols, ptr = [], [], [0]
+    for r in range(n):
+        v, c = list(val[rp[r]:rp[r + 1]]), list(col[rp[r]:rp[r + 1]])
+        if r % 3 == 0:
+            k = c.index(2)
+            v.insert(k + 1, np.float32(-v[k]))
+            c.insert(k + 1, 2)
+        vals += v
+        cols += c
+        ptr.append(len(vals))
+    val2, col2, rp2 = np.array(vals, np.float32), np.array(cols, np.int32), np.array(ptr, np.int32)
+    y = X[:, 0].copy()
+    os.environ["TGBM_LAYOUT"] = "dense"
+    for nbytes in ("1", "2"):
+        os.environ["TGBM_DENSE_BIN_BYTES"] = nbytes
+        s = T.Session(val2, rp2, col2, y, objective="reg:linear", n_trees=1, depth=3, max_num_bin=32)
+        cut_val, crp, _ = s.cuts()
+        m = s.binmat()
+        dense = np.concatenate([m[b] for b in range(m.shape[0])], axis=1)[:, :F].astype(np.int64)
+        later = np.where(np.arange(n) % 3 == 0, -X[:, 2], X[:, 2])
+        cuts2 = cut_val[crp[2]:crp[3]]
+        # the bin rule (hist_tree_builder_single.cu:81-119): number of cut points <= value, at most k - 1
+        expect = np.minimum((cuts2[None, :] <= later[:, None]).sum(axis=1), len(cuts2) - 1)
+        assert np.array_equal(dense[:, 2], expect)
+        s.close()
+    os.environ.pop("TGBM_DENSE_BIN_BYTES", None)
+
+
 def test_more_than_255_bins_through_the_c_abi(T, tmp_path):
     """fit / predict / save / load of the estimator (sparse_train_scikit, sparse_predict_scikit, save / load through
     the model file) with 2000 bins per feature: the predictor follows split_value, so the prediction of the training

@@ -398,7 +398,7 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 // data preparation
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride, int bin_bytes);
+                      size_t col_stride, int bin_bytes, int F);
 // feat_slot (may be nullptr): first head slot of a feature or -1; then hist_word is written as well
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id, const int *feat_slot = nullptr, int *hist_word = nullptr);

@@ -341,7 +341,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_ * bin_bytes);
         launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_ * bin_bytes);
         launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                         bins_.block_stride, d_colmat, col_stride, bin_bytes);
+                         bins_.block_stride, d_colmat, col_stride, bin_bytes, F_);
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
