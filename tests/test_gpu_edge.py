@@ -878,6 +878,42 @@ def test_dense_layout_keeps_the_later_of_two_entries_with_the_same_column(T):
     os.environ.pop("TGBM_DENSE_BIN_BYTES", None)
 
 
+def test_dense_16_bit_bins_with_sampling_and_a_capped_arena(T):
+    """The 16-bit layout under the options that change which rows and columns a tree sees (bagging, column sampling;
+    same srand() seed for every run) and with a capped histogram arena (nodes in batches): same models, predictions
+    and row -> node maps as the byte layout, byte for byte."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    os.environ["TGBM_LAYOUT"] = "dense"
+    rng = np.random.default_rng(21)
+    n, F = 20000, 9
+    X = np.round(rng.standard_normal((n, F)) * 2, 1).astype(np.float32)
+    X[rng.random((n, F)) < 0.2] = 0.0
+    val, rp, col = D.dense_to_csr(X)
+    y = (X[:, 0] + X[:, 3] * X[:, 4] + 0.5 * rng.standard_normal(n)).astype(np.float32)  # squared loss: integer hessians
+    runs = []
+    try:
+        for nbytes, cap in (("1", None), ("2", None), ("2", "4")):
+            os.environ["TGBM_DENSE_BIN_BYTES"] = nbytes
+            os.environ.pop("TGBM_HIST_ARENA_NODES", None)
+            if cap:
+                os.environ["TGBM_HIST_ARENA_NODES"] = cap
+            s = T.Session(val, rp, col, y, objective="reg:linear", n_trees=4, depth=7, max_num_bin=64,
+                          learning_rate=0.4, gamma=0.0, min_child_weight=0.5)
+            assert s.info("dense_bin_bytes") == int(nbytes)
+            s.set_option("bagging", 1)
+            s.set_option("column_sampling_rate", 0.4)
+            libc.srand(99)
+            s.boost(4)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        os.environ.pop("TGBM_DENSE_BIN_BYTES", None)
+        os.environ.pop("TGBM_HIST_ARENA_NODES", None)
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
+    assert [a == b for a, b in zip(runs[0], runs[2])] == [True] * 3
+
+
 def test_more_than_255_bins_through_the_c_abi(T, tmp_path):
     """fit / predict / save / load of the estimator (sparse_train_scikit, sparse_predict_scikit, save / load through
     the model file) with 2000 bins per feature: the predictor follows split_value, so the prediction of the training
