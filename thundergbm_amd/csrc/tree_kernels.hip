@@ -395,7 +395,7 @@ template <int LPR, bool DIRECT, int BLK, int SLOTS, bool BIN16>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
-    __shared__ int s_range[5];
+    __shared__ int s_shift[2];  // the item's scale shifts (gradient, hessian)
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     gh += (size_t)blockIdx.z * tb.n;
     const int *__restrict__ ridx = tb.list(level);
@@ -415,35 +415,27 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     const int nb = blk_bin_begin[fb + 1] - bin0;
     if (nb == 0) return;
     const int h_bits = quant->h_bits;
+    // The item's node and rows: the same few look-ups in every lane (uniform addresses: scalar loads), so that the
+    // first row loads can be issued before the barrier that publishes the LDS histogram's clearing.
+    const int p = find_owner(hpair_begin, n_pairs, item);
+    const int node = hpair_built[p];
+    const int2 sg = seg[node];
+    const int begin = __builtin_amdgcn_readfirstlane(sg.x + (item - hpair_begin[p]) * c.hchunk);
+    const int end = __builtin_amdgcn_readfirstlane(min(sg.y, begin + c.hchunk));
+    const int x_in = node - ((1 << level) - 1);
+    if (x_in < tb.lvl_x0 || x_in >= tb.lvl_x1) return;  // not in the batch of nodes this launch serves
     if (threadIdx.x == 0) {
-        int p = find_owner(hpair_begin, n_pairs, item);
-        int node = hpair_built[p];
-        int2 sg = seg[node];
-        int b = sg.x + (item - hpair_begin[p]) * c.hchunk;
-        int e = min(sg.y, b + c.hchunk);
-        s_range[0] = b;
-        s_range[1] = e;
         // (the node's rows, not the item's: what a row adds must not depend on the item it falls into, or the sums
         // would change with the order of the rows)
         const int rows = max(1, min(sg.y - sg.x, kHistFlushRows));
         const int2 shift = make_int2(item_shift(quant->gq_max, rows, 63 - h_bits),
                                      quant->h_integer ? 0 : item_shift(quant->hq_max, rows, h_bits));
-        s_range[2] = shift.x;
-        s_range[3] = shift.y;
-        const int x_in = node - ((1 << level) - 1);
-        s_range[4] = (x_in < tb.lvl_x0 || x_in >= tb.lvl_x1) ? 1 : 0;  // not in the batch of nodes this launch serves
-        if (fb == 0 && !s_range[4]) tb.hitem_shift[item] = shift;
+        s_shift[0] = shift.x;
+        s_shift[1] = shift.y;
+        if (fb == 0) tb.hitem_shift[item] = shift;
     }
-    for (int i = threadIdx.x; i < nb; i += BLK) lds[i] = 0ull;
-    __syncthreads();
-    if (s_range[4]) return;
-    // (values that are the same for every lane are moved to scalar registers)
-    const int begin = __builtin_amdgcn_readfirstlane(s_range[0]), end = __builtin_amdgcn_readfirstlane(s_range[1]);
     // (slots of `partial` count from the first item of the served batch of nodes: item 0 unless the arena is capped)
     const int item0 = hpair_begin[tb.hpair_lo(level)];
-    // the item's scales: powers of two well inside the float range, so the products below are exact
-    const float scale_g = ldexpf(quant->scale_g, -__builtin_amdgcn_readfirstlane(s_range[2]));
-    const float scale_h = ldexpf(quant->scale_h, -__builtin_amdgcn_readfirstlane(s_range[3]));
     const unsigned long long h_mask = (1ull << h_bits) - 1ull;  // h_bits <= 32
     constexpr int RPS = BLK / LPR;  // rows per step of the whole block
     // rows per thread and stage: what the registers left over by the drain accumulators hold without spills (64
@@ -491,6 +483,12 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         load_rows(r_next, pk, s);
         if (begin + STEP < end) load_ids(begin + STEP, r_next);
     }
+    // the first rows are on their way: clear the histogram meanwhile
+    for (int i = threadIdx.x; i < nb; i += BLK) lds[i] = 0ull;
+    __syncthreads();
+    // the item's scales: powers of two well inside the float range, so the products below are exact
+    const float scale_g = ldexpf(quant->scale_g, -__builtin_amdgcn_readfirstlane(s_shift[0]));
+    const float scale_h = ldexpf(quant->scale_h, -__builtin_amdgcn_readfirstlane(s_shift[1]));
     for (int base = begin; base < end; base += STEP) {
         // the next step's rows are requested before this step's atomics (and before a drain's
         // barriers), so the memory pipeline stays busy
