@@ -478,6 +478,44 @@ def test_predict_wide_float_path_and_unseen_rows(T):
     s.close()
 
 
+@pytest.mark.parametrize("F,depth,num_class", [(20, 6, 1), (60, 3, 1), (96, 5, 3), (30, 12, 1), (12, 8, 4)])
+def test_predict_paths_of_the_dense_vector_kernels(T, F, depth, num_class):
+    """The predictor's kernels that spread a row into a dense vector in LDS (F <= 96): trees staged in LDS for 256 rows
+    per workgroup (F <= 48) or 128 (F <= 96), several trees per stage when they are small, and the walk through the
+    48-byte nodes in global memory when one tree does not fit the LDS (depth 12) - each against the oracle's
+    predictor on the same model and unseen rows."""
+    rng = np.random.default_rng(F + depth)
+    n = 3000
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.3] = 0
+    score = X[:, 0] - X[:, 1] * X[:, 2] + 0.1 * rng.standard_normal(n)
+    kw = dict(depth=depth, n_trees=5, learning_rate=0.4, max_num_bin=32, min_child_weight=0.1)
+    if num_class > 1:
+        y = np.digitize(score, np.quantile(score, np.linspace(0, 1, num_class + 1)[1:-1])).astype(np.float32)
+        kw["objective"] = "multi:softprob"
+    else:
+        y = score.astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    s = T.Session(val, rp, col, y, **kw)
+    s.boost(5)
+    Xt = rng.standard_normal((777, F)).astype(np.float32)
+    Xt[rng.random((777, F)) < 0.3] = 0
+    tv, trp, tc = D.dense_to_csr(Xt)
+    if len(tc) and tc.max() != F - 1:
+        tc[-1] = F - 1
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    k = s.tree_per_rounds
+    base = s.base_score if k == 1 else 0.0
+    ref = O.predict_raw(tv, trp, tc, F, s.model(), 0.4, base)
+    out = np.zeros(777 * k, np.float32)
+    L.tgbm_predict_raw(777, p(tv), p(trp), p(tc), model, 5, k, 0.4, base, p(out))
+    np.testing.assert_allclose(out, ref, rtol=1e-6, atol=1e-6)
+    L.model_free(C.byref(model))
+    s.close()
+
+
 @pytest.mark.parametrize("layout", ["dense", "sparse"])
 def test_a1a_quickstart_known_answer(T, layout):
     # README.md:76-80 of the reference: RMSE = 0.489562 (zero initial prediction, see the oracle test)
