@@ -380,14 +380,15 @@ void launch_sparse_gh_refresh(hipStream_t s, const TreeBuffers &tb, const CsrBin
 // whose split nodes still hold their children's rows (-1: none).
 void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                         int lookup_level);
+// (prune_gamma, here and below: prune the tree with this gamma first - launch_prune's work inside the same launches)
 void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
-                                int lookup_level, float *yp_class, float lr, int n_class = 1);
+                                int lookup_level, float *yp_class, float lr, int n_class = 1,
+                                const float *prune_gamma = nullptr);
 // prediction update + metric + next gradients + their block statistics (tb.root_partial); metric_scratch
 // holds row_blocks(n) doubles
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                       int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
-                      GHPair *gh, double *metric_scratch, float *metric_out);
-void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma, int n_class = 1);
+                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma = nullptr);
 // scratch: row_blocks(n) doubles
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);

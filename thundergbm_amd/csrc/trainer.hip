@@ -935,15 +935,15 @@ void Trainer::log_plan(const TreeBuffers &tb) {
 void Trainer::finish_tree(int k, bool fuse_round_end) {
     const TreeBuffers tb = set_of(k);
     rank_order_fresh_ = false;  // the scores change below
-    launch_prune(stream_, tb, param_.gamma);
+    // (the tree is pruned by a workgroup of the same launches)
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
         launch_round_end(stream_, tb, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
-                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_);
+                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_, &param_.gamma);
         next_round_ready_ = true;
     } else {
         launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_ + (size_t)k * n_,
-                                   param_.learning_rate);
+                                   param_.learning_rate, 1, &param_.gamma);
     }
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
@@ -967,8 +967,7 @@ void Trainer::build_round_together() {
         find_split_sets(tb, d_gh_, level, K);
         partition_sets(tb, level, K);
     }
-    launch_prune(stream_, tb, param_.gamma, K);
-    launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_, param_.learning_rate, K);
+    launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_, param_.learning_rate, K, &param_.gamma);
     TGBM_CHECK(trees_built_ + K <= model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
                              sizeof(TreeNode) * (size_t)tb.n_nodes * K, hipMemcpyDeviceToDevice, stream_));

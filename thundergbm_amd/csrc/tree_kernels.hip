@@ -1777,8 +1777,7 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int
 // Bottom-up, level-parallel form of the reference's Tree::prune_self (src/thundergbm/tree.cu:96-128):
 // a node whose two children are valid leaves and whose gain is below gamma becomes a leaf and its
 // children are marked pruned; then final ids are renumbered over valid, unpruned nodes.
-__global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb_all, float gamma) {
-    const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+__device__ void prune_tree(const TreeBuffers &tb, float gamma) {  // every thread of a kBlock-wide workgroup
     __shared__ int lds[kWaves];
     for (int level = tb.depth - 1; level >= 0; --level) {
         const int nl = 1 << level, off = nl - 1;
@@ -1815,6 +1814,10 @@ __global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb_all, float gamm
     }
 }
 
+__global__ __launch_bounds__(kBlock) void k_prune(TreeBuffers tb_all, float gamma) {
+    prune_tree(tb_all.for_class(blockIdx.z), gamma);
+}
+
 // -------------------------------------------------------------------------- end of a tree
 // The trainer keeps rows as per-node lists; everything that happens per row after the last split
 // search wants row order: the row -> node map (the reference's ins2node_id), the prediction update
@@ -1843,6 +1846,8 @@ struct TreeEndArgs {
     GHPair *gh;
     GradStats *stats;
     double *metric_partial;
+    int with_prune;  // prune the tree first (prune_self with `gamma`)
+    float gamma;
 };
 
 constexpr int kEndInline = 8;                        // shorter sub-ranges are handled by the finding thread
@@ -1904,11 +1909,19 @@ __device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBi
 // n_blocks), 0 everywhere for nodes that hold no rows: row block b then owns positions [bound[b][x],
 // bound[b + 1][x]) of every list. One thread per entry; neighbouring threads search neighbouring
 // boundaries of the same list.
-__global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb_all, int lookup_level, int n_blocks) {
+// with_prune: the launch has one workgroup more, which prunes the tree meanwhile (the searches read fields of the
+// nodes that pruning does not touch; what both produce is first read by k_tree_end).
+__global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb_all, int lookup_level, int n_blocks,
+                                                      int with_prune, float gamma) {
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
+    const int search_blocks = gridDim.x - (with_prune ? 1 : 0);
+    if (with_prune && blockIdx.x == search_blocks) {
+        prune_tree(tb, gamma);
+        return;
+    }
     const int n_holders = (1 << tb.depth) - 1;
     const size_t total = (size_t)n_holders * (n_blocks + 1);
-    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)gridDim.x * kBlock) {
+    for (size_t idx = (size_t)blockIdx.x * kBlock + threadIdx.x; idx < total; idx += (size_t)search_blocks * kBlock) {
         const int x = (int)(idx / (n_blocks + 1)), b = (int)(idx % (n_blocks + 1));
         const TreeNode &nd = tb.nodes[x];
         const int level = 31 - __clz(x + 1);
@@ -2387,7 +2400,10 @@ static void tree_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbin
     const int n_blocks = row_blocks(tb.n);
     const size_t entries = (size_t)((1 << tb.depth) - 1) * (n_blocks + 1);
     if (tb.nid16 == nullptr)
-        k_end_bounds<<<dim3(grid_for(entries, 8192), 1, n_class), kBlock, 0, s>>>(tb, a.lookup_level, n_blocks);
+        k_end_bounds<<<dim3(grid_for(entries, 8192) + (a.with_prune ? 1 : 0), 1, n_class), kBlock, 0, s>>>(
+            tb, a.lookup_level, n_blocks, a.with_prune, a.gamma);
+    else if (a.with_prune)
+        k_prune<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, a.gamma);
     if (tb.sparse) tree_end_launch<true>(s, tb, DenseBins{}, *cbins, mode, a, n_class);
     else tree_end_launch<false>(s, tb, *dbins, CsrBins{}, mode, a, n_class);
 }
@@ -2400,18 +2416,22 @@ void launch_nid_rebuild(hipStream_t s, const TreeBuffers &tb, const DenseBins *d
 }
 
 void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
-                                int lookup_level, float *yp_class, float lr, int n_class) {
+                                int lookup_level, float *yp_class, float lr, int n_class, const float *prune_gamma) {
     TreeEndArgs a{};
     a.lookup_level = lookup_level;
     a.yp = yp_class;
     a.lr = lr;
+    a.with_prune = prune_gamma != nullptr;
+    a.gamma = prune_gamma != nullptr ? *prune_gamma : 0.f;
     tree_end(s, tb, dbins, cbins, 1, a, n_class);
 }
 
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                       int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
-                      GHPair *gh, double *metric_scratch, float *metric_out) {
+                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma) {
     TreeEndArgs a{};
+    a.with_prune = prune_gamma != nullptr;
+    a.gamma = prune_gamma != nullptr ? *prune_gamma : 0.f;
     a.lookup_level = lookup_level;
     a.y = y;
     a.yp = yp;
@@ -2423,10 +2443,6 @@ void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbi
     a.metric_partial = metric_scratch;
     tree_end(s, tb, dbins, cbins, 2, a);
     k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, row_blocks(tb.n), metric_scratch, metric_out);
-}
-
-void launch_prune(hipStream_t s, const TreeBuffers &tb, float gamma, int n_class) {
-    k_prune<<<dim3(1, 1, n_class), kBlock, 0, s>>>(tb, gamma);
 }
 
 void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
