@@ -660,6 +660,16 @@ def test_full_size_properties_config2_reordered_rows(T):
                          max_num_bin=255)
 
 
+def test_full_size_properties_16_bit_bins_reordered_rows(T):
+    """4 M x 28 with up to 1024 bins per feature (the dense layout's 16-bit bins, four blocks of eight features),
+    rows re-ordered after the trees before: same properties."""
+    X, y = D.config2(4_000_000, seed=1)
+    val, rp, col = D.dense_to_csr(X)
+    del X
+    _check_boosted_round(T, val, rp, col, y, 100000, pre_rounds=3, objective="binary:logistic", depth=8,
+                         max_num_bin=1024)
+
+
 def test_full_size_properties_config5_softmax(T):
     """1 M x 54, 8 classes: the class trees of the round are built by common launches."""
     X, y = D.config5()
