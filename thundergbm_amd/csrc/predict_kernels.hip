@@ -222,7 +222,7 @@ void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *
     int grid = (n + kBlock - 1) / kBlock;
     // (TGBM_PREDICT_TPS: trees staged at a time, 0 = walk the 48-byte nodes in global memory; measurements)
     static const int tps_env = std::getenv("TGBM_PREDICT_TPS") ? atoi(std::getenv("TGBM_PREDICT_TPS")) : 4;
-    if (dense_path && packed != nullptr && tps_env > 0) {
+    if (dense_path && packed != nullptr && tps_env > 0 && n_nodes <= 0xffff) {  // (16-bit child indices)
         // trees in LDS: 256 rows per workgroup while their dense vectors take at most 48 KB, else 128; trees are staged
         // one at a time unless several fit next to the vectors in 40 KB (four workgroups per CU: measured on 10 M rows
         // x 40 trees of depth 8, 6.0 ms with one tree per stage, 8.0 ms with four, 14.3 ms from global memory)
