@@ -2132,6 +2132,28 @@ __global__ __launch_bounds__(kBlock) void k_metric_partial(int kind, int n, int 
     store_block_sum_d(acc, sd, out + blockIdx.x);
 }
 
+// The counting metrics (kind 1 and 2) do not depend on the order of their additions, so their partials come from
+// four times the threads per row block: the class predictions of a row are a chain of dependent-latency loads that
+// 256 threads per 4096 rows do not hide.
+constexpr int kCountBlock = 1024;
+__global__ __launch_bounds__(kCountBlock) void k_metric_count(int kind, int n, int K, const float *__restrict__ y,
+                                                             const float *__restrict__ yp, double *__restrict__ out) {
+    __shared__ double sd[kCountBlock / 64];
+    double acc = 0;
+    float accf = 0;
+    const int r0 = blockIdx.x * kRowBlock, r1 = min(n, r0 + kRowBlock);
+    for (int i = r0 + threadIdx.x; i < r1; i += kCountBlock) metric_row(kind, n, K, i, y[i], yp, yp[i], acc, accf);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d);
+    if (lane_id() == 0) sd[threadIdx.x / 64] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0;
+        for (int i = 0; i < kCountBlock / 64; ++i) t += sd[i];
+        out[blockIdx.x] = t;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void k_metric_final(int kind, int n, int n_blocks, const double *__restrict__ in,
                                                         float *__restrict__ out) {
     __shared__ double sd[kWaves];
@@ -2448,7 +2470,10 @@ void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbi
 void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
                    float *out) {
     int blocks = row_blocks(n);  // scratch: one double per block
-    k_metric_partial<<<blocks, kBlock, 0, s>>>(kind, n, num_class, y, yp, scratch);
+    if (kind == 0)
+        k_metric_partial<<<blocks, kBlock, 0, s>>>(kind, n, num_class, y, yp, scratch);
+    else
+        k_metric_count<<<blocks, kCountBlock, 0, s>>>(kind, n, num_class, y, yp, scratch);
     k_metric_final<<<1, kBlock, 0, s>>>(kind, n, blocks, scratch, out);
 }
 
