@@ -67,55 +67,99 @@ __global__ __launch_bounds__(kBlock) void k_radix_count(const unsigned long long
     for (int d = lane; d < 256; d += 64) counts[(size_t)d * n_tiles + tile] = cnt[w][d];
 }
 
-// A wavefront owns its tile and its row of running offsets, so the rounds need no workgroup barrier: the LDS
-// serves one wavefront's reads and writes in program order. Keys are fetched a batch of rounds ahead.
+// A workgroup owns one tile. Its keys are first ordered by digit inside LDS (every wavefront ranks its quarter of the
+// tile round by round, in order, so equal digits keep their order: per-wavefront digit counts, a scan over the digits
+// and the wavefronts, then a running position per wavefront and digit), then written out in that order: the keys of
+// one digit go to consecutive addresses (runs of 16 keys on average instead of single 8-byte stores).
 template <bool PAYLOAD>
 __global__ __launch_bounds__(kBlock) void k_radix_scatter(const unsigned long long *__restrict__ in,
                                                          unsigned long long *__restrict__ out, long n, int shift,
                                                          long n_tiles, const unsigned *__restrict__ offsets,
                                                          const int *__restrict__ in_val, int *__restrict__ out_val) {
-    __shared__ unsigned run[kWaves][256];
+    static_assert(kBlock == 256, "one thread per digit");
+    __shared__ unsigned long long s_key[kSortTile];
+    __shared__ int s_val[PAYLOAD ? kSortTile : 1];
+    __shared__ unsigned s_run[kWaves][256];  // per wavefront and digit: count, then the next local position
+    __shared__ unsigned s_delta[256];        // per digit: global position of its first key - local position of it
+    __shared__ unsigned s_wsum[kWaves];
     const int w = wave_id(), lane = lane_id();
-    const long tile = (long)blockIdx.x * kWaves + w;
-    if (tile >= n_tiles) return;
-    for (int d = lane; d < 256; d += 64) run[w][d] = offsets[(size_t)d * n_tiles + tile];
-    __builtin_amdgcn_wave_barrier();
+    const long tile = blockIdx.x;
     const long base = tile * kSortTile;
-    constexpr int kBatch = 8;
-    static_assert(kSortRounds % kBatch == 0, "rounds come in whole batches");
-    for (int r0 = 0; r0 < kSortRounds; r0 += kBatch) {
-        unsigned long long keys[kBatch];
-        int payload[kBatch];
+    const int count = (int)((n - base) < (long)kSortTile ? (n - base) : (long)kSortTile);
+    constexpr int kRounds = kSortTile / kBlock;  // rounds of 64 keys per wavefront
+    for (int d = lane; d < 256; d += 64) s_run[w][d] = 0;
+    unsigned long long keys[kRounds];
+    int payload[kRounds];
 #pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-            const long i = base + (long)(r0 + b) * 64 + lane;
-            keys[b] = i < n ? in[i] : 0ull;
-            payload[b] = (PAYLOAD && i < n) ? in_val[i] : 0;
+    for (int b = 0; b < kRounds; ++b) {
+        const int li = w * (kSortTile / kWaves) + b * 64 + lane;
+        const int lc = li < count ? li : count - 1;  // (clamped: unconditional loads; count >= 1)
+        keys[b] = in[base + lc];
+        payload[b] = PAYLOAD ? in_val[base + lc] : 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int b = 0; b < kRounds; ++b) {
+        const int li = w * (kSortTile / kWaves) + b * 64 + lane;
+        if (li < count) atomicAdd(&s_run[w][(unsigned)(keys[b] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    {
+        const int d = threadIdx.x;
+        unsigned c[kWaves], tot = 0;
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) {
+            c[i] = s_run[i][d];
+            tot += c[i];
         }
+        unsigned inc = tot;
 #pragma unroll
-        for (int b = 0; b < kBatch; ++b) {
-            const long i = base + (long)(r0 + b) * 64 + lane;
-            const bool valid = i < n;
-            const unsigned long long key = keys[b];
-            const unsigned d = (unsigned)(key >> shift) & 255u;
-            // lanes holding the same digit (match-any built from eight ballots)
-            unsigned long long mask = __ballot(valid);
-#pragma unroll
-            for (int bit_i = 0; bit_i < 8; ++bit_i) {
-                const bool bit = (d >> bit_i) & 1u;
-                const unsigned long long m = __ballot(bit);
-                mask &= bit ? m : ~m;
-            }
-            const unsigned first = valid ? run[w][d] : 0u;
-            const int rank = lanes_below(mask);
-            __builtin_amdgcn_wave_barrier();
-            if (valid) {
-                out[(size_t)first + rank] = key;
-                if (PAYLOAD) out_val[(size_t)first + rank] = payload[b];
-                if (rank == 0) run[w][d] = first + (unsigned)__popcll(mask);
-            }
-            __builtin_amdgcn_wave_barrier();
+        for (int k = 1; k < 64; k <<= 1) {
+            const unsigned t = __shfl_up(inc, k);
+            if (lane >= k) inc += t;
         }
+        if (lane == 63) s_wsum[w] = inc;
+        __syncthreads();
+        unsigned run = inc - tot;
+        for (int i = 0; i < w; ++i) run += s_wsum[i];
+        s_delta[d] = offsets[(size_t)d * n_tiles + tile] - run;  // (modulo 2^32; the sum below is a position < n)
+#pragma unroll
+        for (int i = 0; i < kWaves; ++i) {
+            s_run[i][d] = run;
+            run += c[i];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < kRounds; ++b) {
+        const int li = w * (kSortTile / kWaves) + b * 64 + lane;
+        const bool valid = li < count;
+        const unsigned long long key = keys[b];
+        const unsigned d = (unsigned)(key >> shift) & 255u;
+        // lanes holding the same digit (match-any built from eight ballots)
+        unsigned long long mask = __ballot(valid);
+#pragma unroll
+        for (int bit_i = 0; bit_i < 8; ++bit_i) {
+            const bool bit = (d >> bit_i) & 1u;
+            const unsigned long long m = __ballot(bit);
+            mask &= bit ? m : ~m;
+        }
+        const unsigned first = valid ? s_run[w][d] : 0u;
+        const int rank = lanes_below(mask);
+        __builtin_amdgcn_wave_barrier();
+        if (valid) {
+            s_key[first + rank] = key;
+            if (PAYLOAD) s_val[first + rank] = payload[b];
+            if (rank == 0) s_run[w][d] = first + (unsigned)__popcll(mask);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < count; i += kBlock) {
+        const unsigned long long key = s_key[i];
+        const unsigned pos = s_delta[(unsigned)(key >> shift) & 255u] + (unsigned)i;
+        out[pos] = key;
+        if (PAYLOAD) out_val[pos] = s_val[i];
     }
 }
 
@@ -371,7 +415,7 @@ DeviceCuts build_cut_points(hipStream_t s, int F, long nnz, const float *d_val, 
         const int shift = 8 * p;
         k_radix_count<<<sort_grid, kBlock, 0, s>>>(keys[cur], nnz, shift, n_tiles, counts);
         exclusive_scan<false>(s, counts, offsets, (long)n_counts, d_total, scratch);
-        k_radix_scatter<false><<<sort_grid, kBlock, 0, s>>>(keys[cur], keys[cur ^ 1], nnz, shift, n_tiles, offsets,
+        k_radix_scatter<false><<<(unsigned)n_tiles, kBlock, 0, s>>>(keys[cur], keys[cur ^ 1], nnz, shift, n_tiles, offsets,
                                                             nullptr, nullptr);
         cur ^= 1;
     }
@@ -595,7 +639,7 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits) {
         const int shift = 8 * p;
         k_radix_count<<<sort_grid, kBlock, 0, s>>>(ps.keys[cur], n, shift, n_tiles, ps.counts);
         exclusive_scan<false>(s, ps.counts, ps.offsets, (long)n_counts, ps.d_total, ps.scan);
-        k_radix_scatter<true><<<sort_grid, kBlock, 0, s>>>(ps.keys[cur], ps.keys[cur ^ 1], n, shift, n_tiles, ps.offsets,
+        k_radix_scatter<true><<<(unsigned)n_tiles, kBlock, 0, s>>>(ps.keys[cur], ps.keys[cur ^ 1], n, shift, n_tiles, ps.offsets,
                                                            ps.vals[cur], ps.vals[cur ^ 1]);
         cur ^= 1;
     }
