@@ -109,9 +109,15 @@ def test_rank_gradient_and_metric_parity(T, objective, name, ties):
     s.close()
 
 
-def test_rank_full_size_parity(T):
+@pytest.mark.parametrize("sort", ["counting", "radix"])
+def test_rank_full_size_parity(T, sort, monkeypatch):
     """About a million rows in 8 000 query groups (several thousand radix tiles, 40 000 label runs): order
-    bit-exact, gradients and both metrics against the oracle, which handles this size in a second."""
+    bit-exact, gradients and both metrics against the oracle, which handles this size in a second. Groups this
+    short are ordered by counting; TGBM_RANK_SORT=radix sends them through the radix sort that longer groups take."""
+    if sort == "radix":
+        monkeypatch.setenv("TGBM_RANK_SORT", "radix")
+    else:
+        monkeypatch.delenv("TGBM_RANK_SORT", raising=False)
     rng = np.random.default_rng(17)
     groups = rng.integers(40, 200, size=8000)
     n = int(groups.sum())

@@ -11,6 +11,11 @@ namespace tgbm {
 
 enum RankMetric { RANK_METRIC_MAP = 3, RANK_METRIC_NDCG = 4 };
 
+// Groups of at most this many rows are ordered by counting (every row counts the rows of its segment that go before
+// it: one launch, quadratic in the segment length); data with a longer group takes the radix sort.
+constexpr int kRankCountSortMax = 2048;
+constexpr int kRankCountSortMean = 384;  // ... and only while sum(len^2) / rows stays below this
+
 // One run of equal labels inside a query group, in the group's label-descending order. The run owns the
 // positions [begin, end) of that order; [first_l, end) are the positions that draw a partner (the reference's
 // loop over a group skips the first position of a run that follows a processed run,
@@ -19,7 +24,7 @@ struct RankRun {
     int group_begin, group_end;  // positions of the whole group
     int first_l, end;
     int group;
-    int pad;
+    int begin;
 };
 
 class RankContext {
@@ -68,6 +73,7 @@ class RankContext {
     PairSorter sorter_;
     int last_cur_ = 0;
     bool have_metric_order_ = false;  // sorter_.vals[last_cur_] is the (group, score) order of a metric() call
+    bool short_groups_ = false;       // groups short enough to be ordered by counting (kRankCountSortMax / Mean)
 };
 
 }  // namespace tgbm

@@ -15,6 +15,8 @@
 // whichever thread reaches the group first.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
+#include <string>
 
 #include "rank.h"
 
@@ -83,6 +85,54 @@ __global__ __launch_bounds__(kBlock) void k_rank_metric_keys(int n, const int *_
     if (row >= n) return;
     keys[row] = ((unsigned long long)(unsigned)group_of[row] << 32) | (unsigned)~float_key(score[row]);
     vals[row] = row;
+}
+
+// Stable order by descending score inside every segment through counting: the place of an element is the number of
+// elements of its segment with a smaller key (the radix sort's key: ~float_key(score)) or with the same key and an
+// earlier position - the order the stable radix sort of (segment, key) pairs gives, in one launch. Segments are short
+// (kRankCountSortMax at most) and the threads of a wavefront mostly walk the same one, so the loads of the walk are
+// shared. RUNS: segments are the runs of equal labels in the label-descending order (positions -> rows through
+// static_row); otherwise the query groups in row order.
+// (the keys of all elements in segment order first, so that the walk loads them from consecutive addresses)
+__global__ __launch_bounds__(kBlock) void k_rank_sort_keys(int n, const float *__restrict__ score,
+                                                          const int *__restrict__ static_row, unsigned *__restrict__ key) {
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p < n) key[p] = ~float_key(score[static_row != nullptr ? static_row[p] : p]);
+}
+
+template <bool RUNS>
+__global__ __launch_bounds__(kBlock) void k_rank_count_sort(int n, const unsigned *__restrict__ keys,
+                                                           const int *__restrict__ static_row,
+                                                           const int *__restrict__ run_of,
+                                                           const RankRun *__restrict__ runs,
+                                                           const int *__restrict__ group_of,
+                                                           const int *__restrict__ gptr, int *__restrict__ sorted) {
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= n) return;
+    int sb, se;
+    if (RUNS) {
+        const RankRun r = runs[run_of[p]];
+        sb = r.begin;
+        se = r.end;
+    } else {
+        const int g = group_of[p];
+        sb = gptr[g];
+        se = gptr[g + 1];
+    }
+    const unsigned key = keys[p];
+    int before = 0;
+    constexpr int kAhead = 8;
+    for (int j0 = sb; j0 < se; j0 += kAhead) {
+        unsigned kj[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) kj[u] = keys[min(j0 + u, se - 1)];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int j = j0 + u;
+            before += (j < se && (kj[u] < key || (kj[u] == key && j < p))) ? 1 : 0;
+        }
+    }
+    sorted[sb + before] = RUNS ? static_row[p] : p;
 }
 
 // One thread per position of the (label descending, score descending) order of its group; the body is the
@@ -280,7 +330,7 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
             r.end = j;
             r.first_l = std::min(j, i + (skip_first ? 1 : 0));
             r.group = g;
-            r.pad = 0;
+            r.begin = i;
             skip_first = r.first_l < j;  // a processed run makes the loop step over the next run's first position
             for (int k = i; k < j; ++k) {
                 run_of[k] = (int)runs.size();
@@ -293,6 +343,17 @@ RankContext::RankContext(hipStream_t s, const std::vector<float> &y, const std::
     ndcg_one_groups_ = ndcg_one;
     idcg_valid_ = labels_ok;
     n_runs_ = (int)runs.size();
+    // ordering by counting costs sum(len^2) steps (measured: 50 us for a million rows in groups of 120, where the radix
+    // sort takes 220 us): taken while the average row sits in a group of at most kRankCountSortMean rows
+    int longest = 0;
+    double steps = 0;
+    for (int g : group) {
+        longest = std::max(longest, g);
+        steps += (double)g * (double)g;
+    }
+    const char *sort_env = std::getenv("TGBM_RANK_SORT");  // "radix": the radix sort whatever the group sizes (tests)
+    short_groups_ = longest <= kRankCountSortMax && steps <= (double)kRankCountSortMean * (double)std::max(n_, 1) &&
+                    !(sort_env != nullptr && std::string(sort_env) == "radix");
     run_bits_ = bits_for(n_runs_);
     group_bits_ = bits_for(n_groups_);
 
@@ -335,7 +396,13 @@ RankContext::~RankContext() {
 void RankContext::gradient(const float *d_score, GHPair *d_gh, unsigned seed, bool order_is_fresh) {
     if (n_ == 0) return;
     const int grid = grid_for(n_);
-    if (order_is_fresh && have_metric_order_) {
+    if (short_groups_) {
+        last_cur_ = 0;
+        unsigned *keys = reinterpret_cast<unsigned *>(sorter_.keys[0]);
+        k_rank_sort_keys<<<grid, kBlock, 0, stream_>>>(n_, d_score, d_static_row_, keys);
+        k_rank_count_sort<true><<<grid, kBlock, 0, stream_>>>(n_, keys, d_static_row_, d_run_of_, d_runs_, nullptr, nullptr,
+                                                             sorter_.vals[0]);
+    } else if (order_is_fresh && have_metric_order_) {
         // rows already ordered by (group, score descending, row): a stable sort by run id yields
         // (run, score descending, row), the same order as the full sort below
         k_rank_run_keys<<<grid, kBlock, 0, stream_>>>(n_, d_run_of_row_, sorter_.vals[last_cur_], sorter_.keys[0],
@@ -356,8 +423,16 @@ void RankContext::gradient(const float *d_score, GHPair *d_gh, unsigned seed, bo
 void RankContext::metric(int kind, const float *d_score, float *d_out) {
     TGBM_CHECK(kind == RANK_METRIC_MAP || kind == RANK_METRIC_NDCG, "unknown ranking metric %d", kind);
     const int grid = grid_for(n_);
-    k_rank_metric_keys<<<grid, kBlock, 0, stream_>>>(n_, d_group_of_, d_score, sorter_.keys[0], sorter_.vals[0]);
-    const int cur = sort_pairs(stream_, sorter_, n_, 32 + group_bits_);
+    int cur = 0;
+    if (short_groups_) {
+        unsigned *keys = reinterpret_cast<unsigned *>(sorter_.keys[0]);
+        k_rank_sort_keys<<<grid, kBlock, 0, stream_>>>(n_, d_score, nullptr, keys);
+        k_rank_count_sort<false><<<grid, kBlock, 0, stream_>>>(n_, keys, nullptr, nullptr, nullptr, d_group_of_, d_gptr_,
+                                                              sorter_.vals[0]);
+    } else {
+        k_rank_metric_keys<<<grid, kBlock, 0, stream_>>>(n_, d_group_of_, d_score, sorter_.keys[0], sorter_.vals[0]);
+        cur = sort_pairs(stream_, sorter_, n_, 32 + group_bits_);
+    }
     const int *sorted = sorter_.vals[cur];
     double constant;
     if (kind == RANK_METRIC_NDCG) {
