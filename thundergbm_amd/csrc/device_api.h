@@ -363,9 +363,11 @@ void launch_best_update(hipStream_t s, const TreeBuffers &tb, int level, float r
 void launch_partition_dense(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, int level, int n_class = 1);
 // Sparse level pass (tb.nid16 set): split search of a level (candidates into tb.cand, one slot per task / big
 // feature; launch_best_update follows) and the row -> node update. dump_hist: also store the (node, bin) tables
-// into tb.hist(level) (stage-wise driving and tests; needs tb.hist_q).
+// into tb.hist(level) (stage-wise driving and tests; needs tb.hist_q). last_level: the tree's deepest level (the
+// sorted pass then keeps its new order to itself: no level reads it).
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
-                         const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1);
+                         const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class = 1,
+                         bool last_level = false);
 void launch_sparse_partition(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);
 // Byte columns of the frequent features (CsrBins::colbin, pre-filled with kMissingBin) from the bin-major copy.
 void launch_sparse_cols(hipStream_t s, long nnz, const int *csc_bin, const int *csc_row, const int *cut_fid,

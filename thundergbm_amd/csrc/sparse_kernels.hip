@@ -523,7 +523,7 @@ __device__ __forceinline__ float so_score(GHPair S, float fterm, GHPair m, GHPai
 template <bool LEVEL0>
 __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_all, SparsePass sp,
                                                                const GHPair *__restrict__ gh, int level, float mcw,
-                                                               float lambda, int dump_hist) {
+                                                               float lambda, int dump_hist, int last_level) {
 #pragma clang fp contract(off)
     extern __shared__ unsigned char so_dyn[];  // per node of the level: best key (8 bytes), sums (8), own gain term (4)
     __shared__ int s_row[kSoLds];
@@ -680,9 +680,12 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
     if (Mn == 0) return;
     // ---- rows and gradient pairs of the new order back to HBM (coalesced); the keys follow once the runs that leave
     // the pass are marked
-    for (int q = threadIdx.x; q < Mn; q += kSortedBlock) {
-        out_row[q] = s_row[so_phys(q)];
-        out_gh[q] = s_gh[so_phys(q)];
+    // (no level reads the order of the tree's last level)
+    if (!last_level) {
+        for (int q = threadIdx.x; q < Mn; q += kSortedBlock) {
+            out_row[q] = s_row[so_phys(q)];
+            out_gh[q] = s_gh[so_phys(q)];
+        }
     }
     unsigned key[kSoV];
     SoSum fs[kSoV];
@@ -760,7 +763,8 @@ __global__ __launch_bounds__(kSortedBlock) void k_sparse_sorted(TreeBuffers tb_a
         }
     }
     __syncthreads();
-    for (int q = threadIdx.x; q < Mn; q += kSortedBlock) out_key[q] = s_key[so_phys(q)];
+    if (!last_level)
+        for (int q = threadIdx.x; q < Mn; q += kSortedBlock) out_key[q] = s_key[so_phys(q)];
     // ---- candidates: raise the node's key in LDS, then the winners publish. A candidate without gain never
     // competes: the node's candidate at global bin 0 (a table feature's) has at least its key.
     float sc_head[kSoV], sc_bin[kSoV];
@@ -921,7 +925,8 @@ void launch_sparse_gh_refresh(hipStream_t s, const TreeBuffers &tb, const CsrBin
 }
 
 void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const SparsePass &sp,
-                         const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class) {
+                         const GHPair *gh, int level, float mcw, float lambda, bool dump_hist, int n_class,
+                         bool last_level) {
     // LDS table of a table task: room for one feature of 255 bins with every node of the level, at least 2048 and at
     // most kSparseCells cells (shallow levels: small tables, two workgroups per CU; deep levels: node ranges)
     int n_cells = 2048;
@@ -953,10 +958,10 @@ void launch_sparse_level(hipStream_t s, const TreeBuffers &tb, const CsrBins &bi
         const size_t so_lds = (size_t)(1 << level) * 20;
         if (level == 0)
             k_sparse_sorted<true><<<dim3(sp.n_sorted_tasks, 1, n_class), kSortedBlock, so_lds, s>>>(
-                tb, sp, gh, level, mcw, lambda, dh);
+                tb, sp, gh, level, mcw, lambda, dh, last_level ? 1 : 0);
         else
             k_sparse_sorted<false><<<dim3(sp.n_sorted_tasks, 1, n_class), kSortedBlock, so_lds, s>>>(
-                tb, sp, gh, level, mcw, lambda, dh);
+                tb, sp, gh, level, mcw, lambda, dh, last_level ? 1 : 0);
     }
 }
 

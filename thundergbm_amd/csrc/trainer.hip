@@ -889,7 +889,7 @@ void Trainer::build_level_hist(const TreeBuffers &tb, int level, const GHPair *g
     if (sparse_pass_) {
         // histogram and split search of the level in one pass; stage-wise driving also gets the per-node histograms
         launch_sparse_level(stream_, tb, csr_, sp_, gh, level, param_.min_child_weight, param_.lambda,
-                            !in_boost_ && tb_.hist_q[0] != nullptr, n_class);
+                            !in_boost_ && tb_.hist_q[0] != nullptr, n_class, level == param_.depth - 1);
     } else if (sparse_)
         launch_hist_csr(stream_, tb, csr_, gh, level, n_class);
     else
