@@ -408,9 +408,12 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     longlong2 *__restrict__ partial = tb.partial;
     const int n_bins = tb.n_bins;
     const LevelCtl c = tb.ctl[level];
-    const int item = blockIdx.x;
+    // (the feature blocks of an item are neighbours in the launch order: the item's row list and gradient pairs, which
+    // every block reads again, are then fetched while they still sit in an L2 - with the items of a block as
+    // neighbours, every block of 500 k x 2000 data fetched them from HBM again: 2.72 -> 2.29 ms per tree)
+    const int item = blockIdx.y;
     if (item >= c.n_hitems) return;
-    const int fb = blockIdx.y;
+    const int fb = blockIdx.x;
     const int bin0 = blk_bin_begin[fb];
     const int nb = blk_bin_begin[fb + 1] - bin0;
     if (nb == 0) return;
@@ -2235,7 +2238,7 @@ template <int LPR, int SLOTS, bool BIN16>
 static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseBins &bins, const GHPair *gh,
                               int level, int n_class) {
     const int n_pairs = tb.n_hpairs(level);
-    dim3 grid(tb.max_hitems, bins.n_blocks, n_class);
+    dim3 grid(bins.n_blocks, tb.max_hitems, n_class);
     size_t lds = (size_t)tb.max_block_bins * sizeof(unsigned long long);
     if (lds > 64 * 1024) {
         // more than the default dynamic LDS window: opt in once per kernel instance and size
