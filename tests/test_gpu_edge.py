@@ -28,12 +28,12 @@ def T():
 def _default_layout():
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
               "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
-              "TGBM_DENSE_BIN_BYTES"):
+              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W"):
         os.environ.pop(k, None)
     yield
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
               "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
-              "TGBM_DENSE_BIN_BYTES"):
+              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W"):
         os.environ.pop(k, None)
 
 
@@ -80,6 +80,10 @@ CASES = {
     "softprob": (1500, 10, 8, "multi:softprob", "multi", dict(depth=3, max_num_bin=32), None),
     "wide_dense_blocks": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense"),
     "wide_dense_blocks_16_bit_bins": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense-16"),
+    # blocks of 32 features (what small data with many bins per feature gets), and blocks of 64 features whose
+    # histogram fills the LDS of a CU (what large wide data gets)
+    "wide_dense_blocks_of_32": (700, 150, 90, "reg:linear", "reg", dict(depth=4, max_num_bin=16), "dense-w32"),
+    "wide_dense_blocks_of_64_255_bins": (3000, 150, 90, "reg:linear", "reg", dict(depth=5, max_num_bin=255), "dense-w64"),
     "wide_sparse": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse"),
     # the same through the kernel without an LDS head (every value goes to HBM atomics)
     "wide_sparse_no_head": (2500, 700, 12, "binary:logistic", "bin", dict(depth=5, max_num_bin=63), "sparse-nohead"),
@@ -155,6 +159,8 @@ def run_case(T, name, seed):
             os.environ["TGBM_CSR_HEAD"] = "0"
         if layout.endswith("-16"):
             os.environ["TGBM_DENSE_BIN_BYTES"] = "2"
+        if layout.endswith("-w32") or layout.endswith("-w64"):
+            os.environ["TGBM_DENSE_W"] = layout[-2:]
     val, rp, col = _ragged(n, F, seed, max_len)
     y = _target(val, rp, col, n, F, seed, kind)
     rounds = 4
@@ -163,6 +169,8 @@ def run_case(T, name, seed):
     s = T.Session(val, rp, col, y, **kw)
     if layout and layout.endswith("-16"):
         assert s.info("dense_bin_bytes") == 2
+    if layout and layout[-4:] in ("-w32", "-w64"):
+        assert s.info("dense_W") == int(layout[-2:])
     o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
     # data preparation: exact
     cv, crp, cf = s.cuts()

@@ -302,15 +302,15 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     } else {
         // dense column-blocked layout: blocks of W features, each block n rows x W bins
         int W;
+        auto block_bins = [&](int w) {  // bins of the largest block of w features
+            int most = 0;
+            for (int f0 = 0; f0 < F_; f0 += w)
+                most = std::max(most, h_cut_row_ptr_[std::min(F_, f0 + w)] - h_cut_row_ptr_[f0]);
+            return most;
+        };
         if (bin_bytes == 2) {
             // 16-bit bins: the widest block (a power of two, at most 32 features = 64-byte rows) whose histogram
             // leaves room for two workgroups per CU, else two features per block
-            auto block_bins = [&](int w) {
-                int most = 0;
-                for (int f0 = 0; f0 < F_; f0 += w)
-                    most = std::max(most, h_cut_row_ptr_[std::min(F_, f0 + w)] - h_cut_row_ptr_[f0]);
-                return most;
-            };
             W = 32;
             while (W > 2 && (W / 2 >= F_ || block_bins(W) > kDense16BlockBins)) W /= 2;
             if (wide_bins_) log_info("features with up to %d bins: 16-bit bins, %d features per block", max_feature_bins, W);
@@ -320,7 +320,18 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         } else if (F_ <= 64 && n_bins_ <= 8192) {
             W = 64;
         } else {
+            // Wide data. A 64-byte block row is one whole memory request of a gathered row (a 32-byte row shares it
+            // with a neighbour that the node mostly does not hold), but 64 features of 255 bins fill the LDS of a CU
+            // with one workgroup's histogram. Measured per tree, 32 against 64 features per block: 500 k x 2000
+            // 2.26 / 2.01 ms, 1 M x 200 1.15 / 1.09, 500 k x 300 with 63 bins (two workgroups fit either way)
+            // 0.53 / 0.48; but 2 M x 100 0.91 / 0.97, 200 k x 500 0.57 / 0.64, 100 k x 1000 0.57 / 0.77.
             W = 32;
+            const int bins64 = block_bins(64);
+            if (bins64 <= 8192 || (bins64 <= 16 * 1024 && F_ >= 128 && n_ >= 400000)) W = 64;
+            if (const char *we = std::getenv("TGBM_DENSE_W")) {  // 32 / 64: override (measurements)
+                const int w = atoi(we);
+                if ((w == 32 || w == 64) && block_bins(w) <= kDense16MaxBlockBins) W = w;
+            }
         }
         // (the histogram kernel addresses a block's rows, the gradient pairs and the row lists with unsigned 32-bit
         // byte offsets: a block stays below 4 GiB, the rows below 2^29)

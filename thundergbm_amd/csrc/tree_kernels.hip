@@ -443,7 +443,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     constexpr int RPS = BLK / LPR;  // rows per step of the whole block
     // rows per thread and stage: what the registers left over by the drain accumulators hold without spills (64
     // registers per thread with two workgroups per CU)
-    constexpr int U = SLOTS <= 4 ? 4 : 2;
+    constexpr int U = (SLOTS <= 4 || SLOTS == 16) ? 4 : 2;
     static_assert(RPS * U <= kHistFlushRows, "one iteration must not exceed the flush interval");
     const int q = threadIdx.x % LPR;
     const int rsub = threadIdx.x / LPR;
@@ -2277,6 +2277,7 @@ static void hist_dense_dispatch(hipStream_t s, const TreeBuffers &tb, const Dens
     else if (slots <= 6) hist_dense_launch<LPR, 6, false>(s, tb, bins, gh, level, n_class);
     else if (slots <= 7) hist_dense_launch<LPR, 7, false>(s, tb, bins, gh, level, n_class);  // fewer accumulator registers
     else if (slots <= 8) hist_dense_launch<LPR, 8, false>(s, tb, bins, gh, level, n_class);
+    else if (slots <= 16) hist_dense_launch<LPR, 16, false>(s, tb, bins, gh, level, n_class);
     else if (slots <= 20) hist_dense_launch<LPR, 20, false>(s, tb, bins, gh, level, n_class);
     else fatal("feature block with %d bins does not fit the histogram kernel", tb.max_block_bins);
 }
