@@ -28,12 +28,12 @@ def T():
 def _default_layout():
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
               "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
-              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W"):
+              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W", "TGBM_BUNDLE"):
         os.environ.pop(k, None)
     yield
     for k in ("TGBM_LAYOUT", "TGBM_CSR_HEAD", "TGBM_BATCH_CLASSES", "TGBM_CSC_ROOT", "TGBM_SPARSE_PASS",
               "TGBM_SPARSE_SORTED", "TGBM_SPARSE_COLS", "TGBM_HIST_ARENA_NODES", "TGBM_WIDE_EVAL",
-              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W"):
+              "TGBM_DENSE_BIN_BYTES", "TGBM_DENSE_W", "TGBM_BUNDLE"):
         os.environ.pop(k, None)
 
 
@@ -991,6 +991,73 @@ def test_dense_16_bit_bins_equal_byte_bins(T, objective, F, reorder):
     assert np.array_equal(np.where(mats[0] == 255, 65535, mats[0]), mats[1])
     assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
     assert [a == b for a, b in zip(runs[0], runs[2])] == [True] * 3
+
+
+def _one_hot_data(n, seed, groups, n_dense, empty_rate=0.0):
+    """n_dense quantised columns followed by one-hot groups of the given sizes (zeros are missing values); with
+    empty_rate some rows store nothing of a group."""
+    rng = np.random.default_rng(seed)
+    F = n_dense + sum(groups)
+    X = np.zeros((n, F), np.float32)
+    X[:, :n_dense] = np.floor(rng.random((n, n_dense)) * 40) + 1
+    c0 = n_dense
+    code = []
+    for g in groups:
+        k = rng.integers(0, g, size=n)
+        keep = rng.random(n) >= empty_rate
+        X[np.arange(n)[keep], c0 + k[keep]] = 1 + (rng.integers(0, 3, size=n)[keep] if g < 6 else 0)  # small groups: 3 values
+        code.append(np.where(keep, k, -1))
+        c0 += g
+    score = X[:, 0] / 20 - X[:, 1] / 30 + 0.7 * (code[0] % 3) - 0.4 * (code[-1] % 5) + 0.3 * rng.standard_normal(n)
+    return X, score
+
+
+@pytest.mark.parametrize("objective,reorder", [("reg:linear", "0"), ("binary:logistic", "always"), ("multi:softmax", "0")])
+@pytest.mark.parametrize("shape", ["two_groups", "group_wider_than_a_byte", "only_groups"])
+def test_bundled_columns_equal_one_column_per_feature(T, objective, reorder, shape):
+    """Runs of consecutive features that never meet in a row (one-hot groups) share a column of the dense matrix
+    (TGBM_BUNDLE=0: a column per feature). Same bins once taken apart, same exact integer sums, so the same models,
+    predictions and row -> node maps byte for byte - also when a group has more bins than a byte holds (it is split),
+    when rows store nothing of a group, with re-ordered rows and with class trees built together."""
+    os.environ["TGBM_LAYOUT"] = "dense"
+    os.environ["TGBM_REORDER"] = reorder
+    groups, n_dense = {"two_groups": ([4, 40], 6), "group_wider_than_a_byte": ([5, 300, 3], 3),
+                       "only_groups": ([3, 7, 9], 0)}[shape]
+    n = 20000
+    X, score = _one_hot_data(n, len(shape), groups, n_dense, empty_rate=0.1)
+    F = X.shape[1]
+    val, rp, col = D.dense_to_csr(X)
+    if objective == "reg:linear":
+        y = score.astype(np.float32)
+    elif objective == "binary:logistic":
+        y = (score > np.median(score)).astype(np.float32)
+    else:
+        y = np.digitize(score, np.quantile(score, [0.3, 0.6, 0.85])).astype(np.float32)
+    kw = dict(objective=objective, n_trees=4, depth=6, max_num_bin=64, learning_rate=0.4, gamma=0.0)
+    runs, mats, cols = [], [], []
+    try:
+        for bundle in ("1", "0"):
+            os.environ["TGBM_BUNDLE"] = bundle
+            s = T.Session(val, rp, col, y, **kw)
+            assert s.info("sparse") == 0
+            cols.append(s.info("dense_cols"))
+            m = s.binmat()
+            mats.append(np.concatenate([m[b] for b in range(m.shape[0])], axis=1)[:, :F].astype(np.int32))
+            s.boost(4)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        for k in ("TGBM_BUNDLE", "TGBM_REORDER"):
+            os.environ.pop(k, None)
+    assert cols[1] == F and cols[0] < F
+    if shape == "two_groups":
+        assert cols[0] == n_dense + 2
+    if shape == "group_wider_than_a_byte":
+        assert 3 + 1 + 2 <= cols[0] <= 3 + 1 + 3  # the group of 300 one-bin features needs two columns
+    if shape == "only_groups":
+        assert cols[0] == 3
+    assert np.array_equal(mats[0], mats[1])
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
 
 
 def test_sparse_level_pass_at_its_deepest_level(T):

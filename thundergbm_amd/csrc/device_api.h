@@ -97,6 +97,14 @@ struct DenseBins {
     // 1: byte bins (at most 255 bins per feature, 255 = no stored value); 2: 16-bit bins for max_num_bin above 255
     // (65535 = no stored value)
     int bin_bytes = 1;
+    // Bundles (byte bins only; nullptr: every feature has a column of its own). Consecutive features of which no row
+    // stores more than one (one-hot groups) share one column of the matrix: feature f sits in column feat_col[f] and
+    // its local bin b is stored as feat_lo[f] + b, where feat_lo[f] counts the bins of the bundle's features before
+    // f - the byte is the bin's distance from the bundle's first global bin, which is all the histogram kernel needs.
+    // A byte outside [feat_lo[f], feat_lo[f] + bins of f) means that f has no stored value in the row.
+    const int *feat_col = nullptr;
+    const uint8_t *feat_lo = nullptr;
+    int n_cols = 0;  // columns of the matrix (= features when nothing is bundled)
 };
 
 // Sparse layout for wide, mostly-missing data: the reference's own representation, CSR rows of global
@@ -399,9 +407,14 @@ void launch_calibration_copy(hipStream_t s, const void *src, void *dst, size_t b
 void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 
 // data preparation
+// F: columns of the matrix; feat_col / feat_lo: DenseBins' bundle tables or nullptr
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride, int bin_bytes, int F);
+                      size_t col_stride, int bin_bytes, int F, const int *feat_col = nullptr,
+                      const uint8_t *feat_lo = nullptr);
+// min_next[c] (pre-filled with INT_MAX) = smallest column index that follows column c in a row (equal neighbours, a
+// column stored twice, do not count); *descending is set when a row's columns do not ascend
+void launch_min_next_col(hipStream_t s, int n, const int *row_ptr, const int *col, int *min_next, int *descending);
 // feat_slot (may be nullptr): first head slot of a feature or -1; then hist_word is written as well
 void launch_bin_csr(hipStream_t s, long nnz, const int *col, const float *val, const float *cut_val,
                     const int *cut_row_ptr, int *bin_id, const int *feat_slot = nullptr, int *hist_word = nullptr);

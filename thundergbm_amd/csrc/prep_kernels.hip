@@ -321,7 +321,8 @@ template <typename BinT>
 __global__ __launch_bounds__(kBlock) void k_bin_dense(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
                                                      const float *__restrict__ val, const float *__restrict__ cut_val,
                                                      const int *__restrict__ cut_row_ptr, BinT *__restrict__ binmat,
-                                                     int W, size_t block_stride) {
+                                                     int W, size_t block_stride, const int *__restrict__ feat_col,
+                                                     const uint8_t *__restrict__ feat_lo) {
     constexpr int kLanes = 16;
     const int sub = threadIdx.x % kLanes;
     for (int i = blockIdx.x * (kBlock / kLanes) + threadIdx.x / kLanes; i < n; i += gridDim.x * (kBlock / kLanes)) {
@@ -331,7 +332,28 @@ __global__ __launch_bounds__(kBlock) void k_bin_dense(int n, const int *__restri
             if (e + 1 < e1 && col[e + 1] == f) continue;
             const int cb = cut_row_ptr[f];
             const int k = cut_row_ptr[f + 1] - cb;
-            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (BinT)local_bin(cut_val + cb, k, val[e]);
+            int c = f, b = local_bin(cut_val + cb, k, val[e]);
+            if (feat_col != nullptr) {  // (a bundled feature: its bins follow those of the bundle's earlier features)
+                c = feat_col[f];
+                b += feat_lo[f];
+            }
+            binmat[(size_t)(c / W) * block_stride + (size_t)i * W + (c % W)] = (BinT)b;
+        }
+    }
+}
+
+// Which columns follow which inside the rows (sixteen lanes per row, as above).
+__global__ __launch_bounds__(kBlock) void k_min_next_col(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
+                                                        int *__restrict__ min_next, int *__restrict__ descending) {
+    constexpr int kLanes = 16;
+    const int sub = threadIdx.x % kLanes;
+    for (int i = blockIdx.x * (kBlock / kLanes) + threadIdx.x / kLanes; i < n; i += gridDim.x * (kBlock / kLanes)) {
+        const int e1 = row_ptr[i + 1];
+        for (int e = row_ptr[i] + sub; e + 1 < e1; e += kLanes) {
+            const int c = col[e], next = col[e + 1];
+            if (next < c) *descending = 1;
+            // (the plain read keeps the atomics to the few that lower the entry)
+            if (next > c && next < min_next[c]) atomicMin(&min_next[c], next);
         }
     }
 }
@@ -648,14 +670,21 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits) {
 
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride, int bin_bytes, int F) {
+                      size_t col_stride, int bin_bytes, int F, const int *feat_col, const uint8_t *feat_lo) {
     const int grid = grid_for((size_t)n * 16, 1 << 20);
     if (bin_bytes == 2)
         k_bin_dense<uint16_t><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr,
-                                                     reinterpret_cast<uint16_t *>(binmat), W, block_stride / 2);
+                                                     reinterpret_cast<uint16_t *>(binmat), W, block_stride / 2, nullptr,
+                                                     nullptr);
     else
-        k_bin_dense<uint8_t><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride);
+        k_bin_dense<uint8_t><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride,
+                                                    feat_col, feat_lo);
     launch_cols_from_rows(s, n, W, F, (F + W - 1) / W, binmat, block_stride, colmat, col_stride, bin_bytes);
+}
+
+void launch_min_next_col(hipStream_t s, int n, const int *row_ptr, const int *col, int *min_next, int *descending) {
+    if (n == 0) return;
+    k_min_next_col<<<grid_for((size_t)n * 16, 1 << 20), kBlock, 0, s>>>(n, row_ptr, col, min_next, descending);
 }
 
 void launch_csc_keys(hipStream_t s, int n_rows, const int *row_ptr, const int *bin, const int *sort_key,

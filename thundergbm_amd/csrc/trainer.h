@@ -83,6 +83,8 @@ class Trainer {
     GHPair *d_gh_ = nullptr;
     DeviceCuts cuts_;
     std::vector<int> h_cut_row_ptr_;
+    std::vector<int> h_col_bin_begin_;  // dense layout: first global bin of every column of the matrix (+ the bin count)
+    std::vector<int> h_feat_col_;       // dense layout with bundles: column of every feature (else empty)
     uint8_t *d_binmat_ = nullptr;
     DenseBins bins_;
     bool sparse_ = false;

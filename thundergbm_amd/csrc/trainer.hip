@@ -300,24 +300,73 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         HIP_CHECK(hipFree(d_val));
         HIP_CHECK(hipFree(d_col));
     } else {
-        // dense column-blocked layout: blocks of W features, each block n rows x W bins
+        // dense column-blocked layout: blocks of W columns, each block n rows x W bins
+        // Bundles: a run of consecutive features of which no row stores more than one (the columns of a one-hot
+        // group) shares one column, as long as the run's bins fit a byte. No two features of [a, b) meet in a row
+        // if and only if no row has a column of [a, b) directly followed by another one of it (columns ascend inside
+        // a row), so the smallest successor of every column decides: one pass over the column indices.
+        h_col_bin_begin_ = h_cut_row_ptr_;
+        int P = F_;  // columns of the matrix
+        std::vector<int> h_feat_col;
+        std::vector<uint8_t> h_feat_lo;
+        const char *be = std::getenv("TGBM_BUNDLE");  // "0": one column per feature (tests, measurements)
+        if (bin_bytes == 1 && F_ > 1 && !(be != nullptr && std::string(be) == "0")) {
+            int *d_next = nullptr;
+            HIP_CHECK(hipMalloc(&d_next, sizeof(int) * ((size_t)F_ + 1)));
+            HIP_CHECK(hipMemsetAsync(d_next, 0x7f, sizeof(int) * (size_t)F_, stream_));  // 0x7f7f7f7f: above every column
+            HIP_CHECK(hipMemsetAsync(d_next + F_, 0, sizeof(int), stream_));
+            launch_min_next_col(stream_, n_, d_row_ptr, d_col, d_next, d_next + F_);
+            std::vector<int> next((size_t)F_ + 1);
+            HIP_CHECK(hipMemcpyAsync(next.data(), d_next, sizeof(int) * next.size(), hipMemcpyDeviceToHost, stream_));
+            HIP_CHECK(hipStreamSynchronize(stream_));
+            HIP_CHECK(hipFree(d_next));
+            if (next[F_] == 0) {  // (rows whose columns do not ascend: the argument above does not hold)
+                std::vector<int> col_of(F_), begin;
+                std::vector<uint8_t> lo(F_);
+                int p = 0;
+                for (int a = 0; a < F_; ++p) {
+                    auto nb = [&](int f) { return h_cut_row_ptr_[f + 1] - h_cut_row_ptr_[f]; };
+                    int limit = next[a], total = nb(a), b = a + 1;
+                    while (b < F_ && b < limit && total + nb(b) <= 255) {
+                        total += nb(b);
+                        limit = std::min(limit, next[b]);
+                        ++b;
+                    }
+                    begin.push_back(h_cut_row_ptr_[a]);
+                    for (int f = a; f < b; ++f) {
+                        col_of[f] = p;
+                        lo[f] = (uint8_t)(h_cut_row_ptr_[f] - h_cut_row_ptr_[a]);
+                    }
+                    a = b;
+                }
+                if (p < F_) {
+                    begin.push_back(n_bins_);
+                    h_col_bin_begin_ = begin;
+                    h_feat_col = col_of;
+                    h_feat_lo = lo;
+                    P = p;
+                    log_info("dense layout: %d features in %d columns (runs of features that never meet in a row share one)",
+                             F_, P);
+                }
+            }
+        }
         int W;
-        auto block_bins = [&](int w) {  // bins of the largest block of w features
+        auto block_bins = [&](int w) {  // bins of the largest block of w columns
             int most = 0;
-            for (int f0 = 0; f0 < F_; f0 += w)
-                most = std::max(most, h_cut_row_ptr_[std::min(F_, f0 + w)] - h_cut_row_ptr_[f0]);
+            for (int c0 = 0; c0 < P; c0 += w)
+                most = std::max(most, h_col_bin_begin_[std::min(P, c0 + w)] - h_col_bin_begin_[c0]);
             return most;
         };
         if (bin_bytes == 2) {
             // 16-bit bins: the widest block (a power of two, at most 32 features = 64-byte rows) whose histogram
             // leaves room for two workgroups per CU, else two features per block
             W = 32;
-            while (W > 2 && (W / 2 >= F_ || block_bins(W) > kDense16BlockBins)) W /= 2;
+            while (W > 2 && (W / 2 >= P || block_bins(W) > kDense16BlockBins)) W /= 2;
             if (wide_bins_) log_info("features with up to %d bins: 16-bit bins, %d features per block", max_feature_bins, W);
-        } else if (F_ <= 32) {
+        } else if (P <= 32) {
             W = 4;
-            while (W < F_) W *= 2;
-        } else if (F_ <= 64 && n_bins_ <= 8192) {
+            while (W < P) W *= 2;
+        } else if (P <= 64 && n_bins_ <= 8192) {
             W = 64;
         } else {
             // Wide data. A 64-byte block row is one whole memory request of a gathered row (a 32-byte row shares it
@@ -327,7 +376,7 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
             // 0.53 / 0.48; but 2 M x 100 0.91 / 0.97, 200 k x 500 0.57 / 0.64, 100 k x 1000 0.57 / 0.77.
             W = 32;
             const int bins64 = block_bins(64);
-            if (bins64 <= 8192 || (bins64 <= 16 * 1024 && F_ >= 128 && n_ >= 400000)) W = 64;
+            if (bins64 <= 8192 || (bins64 <= 16 * 1024 && P >= 128 && n_ >= 400000)) W = 64;
             if (const char *we = std::getenv("TGBM_DENSE_W")) {  // 32 / 64: override (measurements)
                 const int w = atoi(we);
                 if ((w == 32 || w == 64) && block_bins(w) <= kDense16MaxBlockBins) W = w;
@@ -338,21 +387,32 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         while (W * bin_bytes > 4 && (size_t)n_ * W * bin_bytes >= ((size_t)1 << 32)) W /= 2;
         TGBM_CHECK((size_t)n_ * W * bin_bytes < ((size_t)1 << 32) && n_ < (1 << 29),
                    "%d rows are more than the dense layout addresses; use TGBM_LAYOUT=sparse", n_);
-        const int n_blocks = (F_ + W - 1) / W;
+        const int n_blocks = (P + W - 1) / W;
         bins_.W = W;
         bins_.n_blocks = n_blocks;
         bins_.bin_bytes = bin_bytes;
+        bins_.n_cols = P;
+        if (!h_feat_col.empty()) {
+            int *d_fc = dalloc<int>((size_t)F_);
+            uint8_t *d_fl = dalloc<uint8_t>(((size_t)F_ + 3) / 4 * 4);
+            upload(stream_, d_fc, h_feat_col.data(), (size_t)F_);
+            upload(stream_, d_fl, h_feat_lo.data(), (size_t)F_);
+            HIP_CHECK(hipStreamSynchronize(stream_));  // (the host vectors go out of scope)
+            bins_.feat_col = d_fc;
+            bins_.feat_lo = d_fl;
+            h_feat_col_ = h_feat_col;
+        }
         const size_t mat_bytes = (size_t)n_ * W * n_blocks * bin_bytes;
         bins_.block_stride = (size_t)n_ * W * bin_bytes;
-        TGBM_CHECK(mat_bytes + (size_t)n_ * F_ * bin_bytes < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
+        TGBM_CHECK(mat_bytes + (size_t)n_ * P * bin_bytes < free_b / 2, "dense bin matrix of %zu bytes does not fit (free %zu)",
                    mat_bytes, free_b);
         d_binmat_ = dalloc<uint8_t>(mat_bytes);
         launch_fill_u8(stream_, d_binmat_, (uint8_t)kMissingBin, mat_bytes);  // (all-ones: the sentinel of both widths)
         const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
-        uint8_t *d_colmat = dalloc<uint8_t>(col_stride * F_ * bin_bytes);
-        launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * F_ * bin_bytes);
+        uint8_t *d_colmat = dalloc<uint8_t>(col_stride * P * bin_bytes);
+        launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * P * bin_bytes);
         launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                         bins_.block_stride, d_colmat, col_stride, bin_bytes, F_);
+                         bins_.block_stride, d_colmat, col_stride, bin_bytes, P, bins_.feat_col, bins_.feat_lo);
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
@@ -491,10 +551,16 @@ void Trainer::alloc_tree_buffers() {
     // would make the stored-value count lie): its bins add up to the root's sums
     tb.complete_feature = -1;
     if (!sparse_) {
-        for (int f = 0; f < F_ && tb.complete_feature < 0; ++f)
+        for (int f = 0; f < F_ && tb.complete_feature < 0; ++f) {
+            int c = f;
+            if (!h_feat_col_.empty()) {  // (only a feature with a column of its own)
+                c = h_feat_col_[f];
+                if ((f > 0 && h_feat_col_[f - 1] == c) || (f + 1 < F_ && h_feat_col_[f + 1] == c)) continue;
+            }
             if (cuts_.feature_nnz[f] == (long)n_ && bins_.bin_bytes == 1 &&
-                device_count_bytes(stream_, bins_.col + (size_t)f * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
+                device_count_bytes(stream_, bins_.col + (size_t)c * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
                 tb.complete_feature = f;
+        }
     }
     tb.hpair_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
     tb.leaf_value = dalloc<float>(S * tb.n_nodes);
@@ -576,12 +642,15 @@ void Trainer::alloc_tree_buffers() {
     const int W = bins_.W, nb = bins_.n_blocks;
     std::vector<int> blk_begin(nb + 1), feat_off((size_t)nb * W, 0);
     int max_block_bins = 0;
-    for (int b = 0; b <= nb; ++b) blk_begin[b] = h_cut_row_ptr_[std::min(b * W, F_)];
+    // (columns of the matrix: features, or bundles of features whose bins follow each other)
+    const std::vector<int> &cbb = sparse_ ? h_cut_row_ptr_ : h_col_bin_begin_;
+    const int n_cols = (int)cbb.size() - 1;
+    for (int b = 0; b <= nb; ++b) blk_begin[b] = cbb[std::min(b * W, n_cols)];
     for (int b = 0; b < nb; ++b) {
         max_block_bins = std::max(max_block_bins, blk_begin[b + 1] - blk_begin[b]);
         for (int j = 0; j < W; ++j) {
-            int f = b * W + j;
-            feat_off[(size_t)b * W + j] = f < F_ ? h_cut_row_ptr_[f] - blk_begin[b] : 0;
+            int c = b * W + j;
+            feat_off[(size_t)b * W + j] = c < n_cols ? cbb[c] - blk_begin[b] : 0;
         }
     }
     TGBM_CHECK(sparse_ || (size_t)max_block_bins * 8 <= 160 * 1024, "feature block histogram exceeds the LDS");
@@ -1108,7 +1177,7 @@ void Trainer::reorder_rows() {
     std::swap(d_yp_, d_yp_alt_);
     d_perm_ = perm_new;
     bins_.data = d_binmat_;
-    launch_cols_from_rows(stream_, n_, bins_.W, F_, bins_.n_blocks, d_binmat_, bins_.block_stride,
+    launch_cols_from_rows(stream_, n_, bins_.W, bins_.n_cols, bins_.n_blocks, d_binmat_, bins_.block_stride,
                           const_cast<uint8_t *>(bins_.col), bins_.col_stride, bins_.bin_bytes);
     h_perm_valid_ = false;
     nid_materialized_ = true;
@@ -1199,6 +1268,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "wide_eval") return wide_eval_ ? 1 : 0;
     if (key == "row_lists") return sparse_pass_ ? 0 : 1;  // the sparse level pass keeps a row -> node map only
     if (key == "dense_W") return bins_.W;
+    if (key == "dense_cols") return sparse_ ? 0 : bins_.n_cols;  // columns of the bin matrix (fewer than features: bundles)
     if (key == "dense_bin_bytes") return sparse_ ? 0 : bins_.bin_bytes;
     if (key == "reorders_done") return reorders_done_;
     if (key == "device_free_mb") {
@@ -1227,6 +1297,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else if (name == "cut_fid") src = cuts_.cut_fid, bytes = sizeof(int) * (size_t)n_bins_;
     else if (name == "binmat") src = d_binmat_, bytes = sparse_ ? 0 : (size_t)n_ * bins_.W * bins_.n_blocks * bins_.bin_bytes;
     else if (name == "csr_bin") src = csr_.bin, bytes = sparse_ ? sizeof(int) * (size_t)nnz_ : 0;
+    else if (name == "feat_col") src = bins_.feat_col, bytes = bins_.feat_col != nullptr ? sizeof(int) * (size_t)F_ : 0;
+    else if (name == "feat_lo") src = bins_.feat_lo, bytes = bins_.feat_lo != nullptr ? (size_t)F_ : 0;
     else if (name == "nid") {
         // the map is kept as row lists; materialise it on demand (a re-ordering of the rows has done so already)
         if (!nid_materialized_) launch_nid_rebuild(stream_, cur, &bins_, &csr_, lookup_level_);

@@ -1450,8 +1450,15 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     // (features of more than 255 bins keep their split bin in a side array: TreeNode::split_bid is a byte)
     const int sbid = tb.split_bin != nullptr ? tb.split_bin[off + x_in] : (int)nd.split_bid;
     const bool dr = nd.default_right;
-    constexpr int kMissing = sizeof(BinT) == 2 ? kMissingBin16 : kMissingBin;
-    const BinT *column = reinterpret_cast<const BinT *>(bins.col) + (size_t)f * bins.col_stride;
+    // A stored bin outside [lo, lo + span) means that the row has no value of the feature: the missing sentinel, or
+    // (a feature that shares its column with others, DenseBins::feat_col) a bin of another feature of the bundle.
+    int c = f, lo = 0, span = sizeof(BinT) == 2 ? kMissingBin16 : kMissingBin;
+    if (sizeof(BinT) == 1 && bins.feat_col != nullptr) {
+        c = bins.feat_col[f];
+        lo = bins.feat_lo[f];
+        span = tb.cut_row_ptr[f + 1] - tb.cut_row_ptr[f];
+    }
+    const BinT *column = reinterpret_cast<const BinT *>(bins.col) + (size_t)c * bins.col_stride;
     int nleft = 0;
     // All row ids first, then all bins, then the decisions, then the stores. Every load is unconditional (positions
     // past the item's end are clamped to its last row), so each phase's loads are issued back to back and a thread's
@@ -1469,7 +1476,8 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
     unsigned rights = 0;
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-        const bool right = (b[k] == kMissing) ? dr : (b[k] >= sbid);
+        const int t = b[k] - lo;
+        const bool right = ((unsigned)t >= (unsigned)span) ? dr : (t >= sbid);
         rights |= (right ? 1u : 0u) << k;
         if (pb + k * kBlock + (int)threadIdx.x < pe) nleft += right ? 0 : 1;
     }
@@ -1901,6 +1909,11 @@ __device__ __forceinline__ int end_child_of(const TreeBuffers &tb, const DenseBi
         const int b = reinterpret_cast<const uint16_t *>(dbins.col)[(size_t)nd.split_feature_id * dbins.col_stride + row];
         const int sb = tb.split_bin != nullptr ? tb.split_bin[(nd.lch_index - 1) / 2] : (int)nd.split_bid;
         right = (b == kMissingBin16) ? nd.default_right : (b >= sb);
+    } else if (dbins.feat_col != nullptr) {
+        const int f = nd.split_feature_id;
+        const int t = (int)dbins.col[(size_t)dbins.feat_col[f] * dbins.col_stride + row] - (int)dbins.feat_lo[f];
+        right = ((unsigned)t >= (unsigned)(tb.cut_row_ptr[f + 1] - tb.cut_row_ptr[f])) ? nd.default_right
+                                                                                     : (t >= (int)nd.split_bid);
     } else {
         const int b = dbins.col[(size_t)nd.split_feature_id * dbins.col_stride + row];
         right = (b == kMissingBin) ? nd.default_right : (b >= nd.split_bid);
@@ -2023,7 +2036,8 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
             const int listed = tb.list(31 - __clz(node[u] + 1))[p];  // (the root's list is the identity and not stored)
             row[u] = node[u] == 0 ? p : listed;
         }
-        if (SPARSE || dbins.bin_bytes == 2) {  // (16-bit bins: the packed split word has no room for the split bin)
+        // (16-bit bins and bundled columns: the packed split word has no room for what the decision needs)
+        if (SPARSE || dbins.bin_bytes == 2 || dbins.feat_col != nullptr) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (j0 + u * kBlock >= total) continue;

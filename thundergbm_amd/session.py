@@ -112,8 +112,23 @@ class Session:
         return self.get("cut_val", np.float32), self.get("cut_row_ptr", np.int32), self.get("cut_fid", np.int32)
 
     def binmat(self):
+        """Local bin of every (block, row, feature in block), 255 / 65535 where a row stores no value of the feature.
+        Features that share a column of the device matrix (runs of features that never meet in a row) are taken
+        apart here, so the result does not depend on that."""
         W, nb = self.info("dense_W"), self.info("dense_blocks")
-        return self.get("binmat", np.uint16 if self.info("dense_bin_bytes") == 2 else np.uint8, (nb, self.n, W))
+        m = self.get("binmat", np.uint16 if self.info("dense_bin_bytes") == 2 else np.uint8, (nb, self.n, W))
+        F, P = self.F, self.info("dense_cols")
+        if P == F:
+            return m
+        cols = m.transpose(1, 0, 2).reshape(self.n, nb * W).astype(np.int32)
+        fc, lo = self.get("feat_col", np.int32), self.get("feat_lo", np.uint8).astype(np.int32)
+        _, crp, _ = self.cuts()
+        t = cols[:, fc] - lo[None, :]
+        logical = np.where((t >= 0) & (t < np.diff(crp)[None, :]), t, 255).astype(np.uint8)
+        nbl = (F + W - 1) // W
+        out = np.full((self.n, nbl * W), 255, np.uint8)
+        out[:, :F] = logical
+        return np.ascontiguousarray(out.reshape(self.n, nbl, W).transpose(1, 0, 2))
 
     def global_bin_ids(self, row_ptr, col):
         """Global bin id of every stored value (the reference's csr_bin_id) and its local bin id."""
