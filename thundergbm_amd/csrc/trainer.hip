@@ -310,7 +310,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         std::vector<int> h_feat_col;
         std::vector<uint8_t> h_feat_lo;
         const char *be = std::getenv("TGBM_BUNDLE");  // "0": one column per feature (tests, measurements)
-        if (bin_bytes == 1 && F_ > 1 && !(be != nullptr && std::string(be) == "0")) {
+        // (rows that store every feature leave nothing to bundle)
+        if (bin_bytes == 1 && F_ > 1 && nnz_ < (long)n_ * F_ && !(be != nullptr && std::string(be) == "0")) {
             int *d_next = nullptr;
             HIP_CHECK(hipMalloc(&d_next, sizeof(int) * ((size_t)F_ + 1)));
             HIP_CHECK(hipMemsetAsync(d_next, 0x7f, sizeof(int) * (size_t)F_, stream_));  // 0x7f7f7f7f: above every column
