@@ -137,13 +137,16 @@ void tgbm_trainer_finish_tree(tgbm_trainer *t, int class_id);
 float tgbm_trainer_metric(tgbm_trainer *t);
 
 /* Integer facts: n, n_features, n_bins, num_class, tree_per_rounds, n_nodes, dense_W,
- * dense_blocks, trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems, n_sets (class trees
+ * dense_blocks, dense_cols (columns of the dense bin matrix: fewer than n_features when runs of features
+ * that never meet in a row share a column), trees_built, rounds_done, n_packs, depth, y_pred_size, max_hitems, n_sets (class trees
  * of a round built by common launches), reorders_done, device_free_mb (free device memory in MiB). */
 int tgbm_trainer_info(tgbm_trainer *t, const char *key);
 float tgbm_trainer_base_score(tgbm_trainer *t);
 
 /* Copies a device buffer to `out` when `cap` is large enough; always returns its size in bytes.
- * Names: cut_val, cut_row_ptr, cut_fid, binmat, nid, gh, y_pred, y, nodes, sp, hist_q0, hist_q1,
+ * Names: cut_val, cut_row_ptr, cut_fid, binmat (dense layout: [dense_blocks][n][dense_W] bins of the matrix's
+ * columns; with dense_cols < n_features feature f is column feat_col[f] and its local bin b is stored as
+ * feat_lo[f] + b), feat_col (int per feature), feat_lo (byte per feature), nid, gh, y_pred, y, nodes, sp, hist_q0, hist_q1,
  * quant, ctl, seg, ridx0, ridx1, model, metric_log, labels, rank_order (ranking objectives: the rows in
  * the order of the last gradient or metric pass). After tgbm_trainer_boost `gh` may already
  * hold the gradients of the next round (single-tree objectives compute them in the round's last pass). */
