@@ -1060,6 +1060,39 @@ def test_bundled_columns_equal_one_column_per_feature(T, objective, reorder, sha
     assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
 
 
+def test_bundle_of_a_complete_feature_and_an_empty_one(T):
+    """A feature stored in every row can only share its column with features that no row stores. The root's sums are
+    then still taken from that feature's bins, as without bundles (they are taken from the gradients otherwise, which
+    rounds differently): same bits with a re-ordering after every tree."""
+    os.environ["TGBM_LAYOUT"] = "dense"
+    os.environ["TGBM_REORDER"] = "always"
+    rng = np.random.default_rng(144)
+    n, g = 3000, 30
+    X = np.zeros((n, 6 + g), np.float32)
+    X[:, :3] = np.floor(rng.random((n, 3)) * 30)        # some zeros: not complete
+    X[:, 3] = 1 + rng.integers(0, 3, size=n)            # complete
+    # column 4 stays empty, column 5 is rare
+    X[rng.random(n) < 0.01, 5] = 2
+    X[np.arange(n), 6 + rng.integers(0, g, size=n)] = 1
+    y = ((X[:, 0] - X[:, 1]) / 10 + X[:, 3] + 0.5 * rng.standard_normal(n) > 2).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    runs = []
+    try:
+        for bundle in ("1", "0"):
+            os.environ["TGBM_BUNDLE"] = bundle
+            s = T.Session(val, rp, col, y, objective="binary:logistic", n_trees=4, depth=5, max_num_bin=8, learning_rate=0.5)
+            if bundle == "1":
+                fc = s.get("feat_col", np.int32)
+                assert fc[3] == fc[4] and s.info("dense_cols") < s.F
+            s.boost(4)
+            runs.append((s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()))
+            s.close()
+    finally:
+        for k in ("TGBM_BUNDLE", "TGBM_REORDER"):
+            os.environ.pop(k, None)
+    assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
+
+
 def test_sparse_level_pass_at_its_deepest_level(T):
     """Depth 11 (1024 nodes on the last level: the sparse level pass's limit, 12-bit node field of the sorted keys,
     20 KB of per-node LDS state): sorted pass against tables, byte for byte."""

@@ -554,9 +554,14 @@ void Trainer::alloc_tree_buffers() {
     if (!sparse_) {
         for (int f = 0; f < F_ && tb.complete_feature < 0; ++f) {
             int c = f;
-            if (!h_feat_col_.empty()) {  // (only a feature with a column of its own)
+            if (!h_feat_col_.empty()) {
+                // (a feature that shares its column: the others must be empty, so that every byte of the column that
+                // is not the missing sentinel is this feature's - the same choice as without bundles)
                 c = h_feat_col_[f];
-                if ((f > 0 && h_feat_col_[f - 1] == c) || (f + 1 < F_ && h_feat_col_[f + 1] == c)) continue;
+                bool alone = true;
+                for (int g = f - 1; g >= 0 && h_feat_col_[g] == c; --g) alone = alone && cuts_.feature_nnz[g] == 0;
+                for (int g = f + 1; g < F_ && h_feat_col_[g] == c; ++g) alone = alone && cuts_.feature_nnz[g] == 0;
+                if (!alone) continue;
             }
             if (cuts_.feature_nnz[f] == (long)n_ && bins_.bin_bytes == 1 &&
                 device_count_bytes(stream_, bins_.col + (size_t)c * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
