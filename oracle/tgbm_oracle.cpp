@@ -125,6 +125,7 @@ struct Oracle {
     std::vector<double> hist64_cur, hist64_prev;  // g,h interleaved
     // debug: per node of the whole tree
     std::vector<float> dbg_score;   // [n_nodes][n_bins], signed gain of every candidate
+    std::vector<float> dbg_dir_gap; // [n_nodes][n_bins], gain(missing -> left) - gain(missing -> right) of every candidate
     std::vector<GH> dbg_hist;       // [n_nodes][n_bins], raw hist
     std::vector<double> dbg_hist64; // [n_nodes][n_bins][2]
     std::vector<int> dbg_built;     // [n_nodes] 1 if built from rows, 0 if by subtraction
@@ -300,6 +301,7 @@ void tree_init(Oracle &o, int k) {
     o.cur_level = -1;
     if (o.keep_debug) {
         o.dbg_score.assign((size_t)n_max * o.n_bins, 0.f);
+        o.dbg_dir_gap.assign((size_t)n_max * o.n_bins, 0.f);
         o.dbg_hist.assign((size_t)n_max * o.n_bins, GH{0, 0});
         if (o.shadow64) o.dbg_hist64.assign((size_t)n_max * o.n_bins * 2, 0.0);
         o.dbg_built.assign(n_max, -1);
@@ -412,7 +414,10 @@ void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
         float gl = fmaxf(0.f, compute_gain(S, l2, r2, o.mcw, o.lambda));
         float score = (gl > gr) ? gl : -gr;
         if (!o.ignored.empty() && o.ignored[f]) score = 0;  // :304 / :663: an ignored column's gain is 0
-        if (dbg) dbg[b] = score;
+        if (dbg) {
+            dbg[b] = score;
+            o.dbg_dir_gap[(size_t)node * B + b] = gl - gr;
+        }
         // arg_abs_max (:330-335): larger |gain| wins, ties keep the smaller index
         if (first || fabsf(score) > fabsf(best_score)) {
             best = b;
@@ -1164,6 +1169,10 @@ void orc_get_level_hist(void *h, int node_in_level, float *out, double *out64) {
 void orc_get_tree_scores(void *h, float *out) {
     Oracle &o = *(Oracle *)h;
     std::copy(o.dbg_score.begin(), o.dbg_score.end(), out);
+}
+void orc_get_tree_dir_gaps(void *h, float *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.dbg_dir_gap.begin(), o.dbg_dir_gap.end(), out);
 }
 void orc_get_tree_hists(void *h, float *out, double *out64, int *built) {
     Oracle &o = *(Oracle *)h;

@@ -72,7 +72,7 @@ def lib():
             getattr(L, name).restype = C.c_long
         for name in ("orc_get_labels", "orc_get_y", "orc_get_bin_ids", "orc_get_y_pred", "orc_set_y_pred",
                      "orc_get_gh", "orc_set_gh", "orc_get_nid", "orc_set_nid", "orc_get_nodes", "orc_set_nodes",
-                     "orc_get_tree_scores", "orc_get_model"):
+                     "orc_get_tree_scores", "orc_get_tree_dir_gaps", "orc_get_model"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_void_p]
             getattr(L, name).restype = None
         L.orc_get_cuts.argtypes = [C.c_void_p] * 4
@@ -276,6 +276,12 @@ class Oracle:
     def tree_scores(self):
         out = np.zeros((self.n_nodes, self.n_bins), dtype=np.float32)
         self.L.orc_get_tree_scores(self.h, _p(out))
+        return out
+
+    def tree_dir_gaps(self):
+        """gain(missing -> left) - gain(missing -> right) of every candidate of every node of the current tree."""
+        out = np.zeros((self.n_nodes, self.n_bins), dtype=np.float32)
+        self.L.orc_get_tree_dir_gaps(self.h, _p(out))
         return out
 
     def tree_hists(self):

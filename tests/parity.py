@@ -83,9 +83,42 @@ class TreeDiff:
         self.compared = 0
         # (node, oracle best |gain|, oracle |gain| of the GPU's choice, magnitude of the oracle gain's terms)
         self.near_ties = []
+        # largest observed error / tolerance of the compared node sums, weights and gains (how much of the bound
+        # the two implementations actually use)
+        self.worst = {"sum": 0.0, "weight": 0.0, "gain": 0.0}
 
     def __repr__(self):
-        return "TreeDiff(compared=%d, near_ties=%r)" % (self.compared, self.near_ties)
+        return "TreeDiff(compared=%d, near_ties=%r, worst=%r)" % (self.compared, self.near_ties, self.worst)
+
+
+class Margins:
+    """Running maximum of error / tolerance per quantity over the comparisons of a test; report() prints it and,
+    when TGBM_MARGIN_LOG names a file, appends a line there."""
+
+    def __init__(self, name):
+        self.name = name
+        self.worst = {}
+        self.ties = 0
+
+    def add(self, diff_or_dict):
+        w = diff_or_dict.worst if hasattr(diff_or_dict, "worst") else diff_or_dict
+        for k, v in w.items():
+            self.worst[k] = max(self.worst.get(k, 0.0), float(v))
+
+    def note(self, key, err, tol):
+        r = float(np.max(np.asarray(err, np.float64) / np.maximum(np.asarray(tol, np.float64), 1e-300))) if np.size(err) else 0.0
+        self.worst[key] = max(self.worst.get(key, 0.0), r)
+
+    def report(self):
+        import json
+        import os
+        line = json.dumps({"case": self.name, "ties": self.ties,
+                           "worst_err_over_tol": {k: float("%.3g" % v) for k, v in sorted(self.worst.items())}})
+        print("\nmargins " + line, flush=True)
+        path = os.environ.get("TGBM_MARGIN_LOG")
+        if path:
+            with open(path, "a") as f:
+                f.write(line + "\n")
 
 
 def significant_ties(near_ties):
@@ -106,7 +139,8 @@ def rows_in_node(final_nid, x):
     return cur == x
 
 
-def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL, mcw=1.0):
+def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL, mcw=1.0,
+                  orc_dir_gaps=None):
     """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
 
     Where both trees split on the same candidate everything must agree: threshold and bin exactly,
@@ -114,7 +148,11 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     GPU's candidate must be within tolerance of the oracle's best (a near tie); the subtree below
     such a node is not compared. `default_right` is only compared where
     missing_rows(node, feature) > 0: without missing rows in the node the reference decides it by
-    float32 round-off of node_sum - feature_total.
+    float32 round-off of node_sum - feature_total. Where the node has missing rows the direction is the
+    larger of two gains of the same candidate (missing -> left against missing -> right, strict `>`,
+    hist_tree_builder_single.cu:300-323); orc_dir_gaps [n_nodes, n_bins] holds the oracle's difference of the
+    two, and a direction that differs is a near tie like any other when that difference is within the gain
+    tolerance (without orc_dir_gaps a differing direction fails).
 
     Tolerance: node sums are float32 results of a chain of histogram subtractions that starts at the
     root, so their error is relative to the root-level sums of |g| and |h| (abs_scale = (Ag, Ah)):
@@ -149,17 +187,33 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
         S = (float(o["sum_g"]), float(o["sum_h"]))
         assert abs(g["sum_g"] - o["sum_g"]) <= dG and abs(g["sum_h"] - o["sum_h"]) <= dH, \
             "node %d sum differs: gpu (%g,%g) oracle (%g,%g)" % (x, g["sum_g"], g["sum_h"], o["sum_g"], o["sum_h"])
+        diff.worst["sum"] = max(diff.worst["sum"], abs(float(g["sum_g"]) - float(o["sum_g"])) / dG,
+                                abs(float(g["sum_h"]) - float(o["sum_h"])) / dH)
         w = float(o["base_weight"])
-        assert abs(g["base_weight"] - w) <= (dG + abs(w) * dH) / (S[1] + lam) + rel * max(1.0, abs(w)), \
-            "node %d weight differs: %g vs %g" % (x, g["base_weight"], w)
+        w_tol = (dG + abs(w) * dH) / (S[1] + lam) + rel * max(1.0, abs(w))
+        assert abs(g["base_weight"] - w) <= w_tol, "node %d weight differs: %g vs %g" % (x, g["base_weight"], w)
+        diff.worst["weight"] = max(diff.worst["weight"], abs(float(g["base_weight"]) - w) / w_tol)
         split_g, split_o = g["split_fid"] >= 0, o["split_fid"] >= 0
         if not split_g and not split_o:
             continue
         if split_g and split_o and g["split_fid"] == o["split_fid"] and g["split_bid"] == o["split_bid"]:
             assert g["split_value"] == o["split_value"], "node %d threshold differs" % x
-            assert abs(g["gain"] - o["gain"]) <= gain_tol(x, o), "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
-            if missing_rows is not None and missing_rows(x, int(o["split_fid"])) > 0:
-                assert g["default_right"] == o["default_right"], "node %d default direction differs" % x
+            gt = gain_tol(x, o)
+            assert abs(g["gain"] - o["gain"]) <= gt, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
+            diff.worst["gain"] = max(diff.worst["gain"], abs(float(g["gain"]) - float(o["gain"])) / gt)
+            if (g["default_right"] != o["default_right"] and missing_rows is not None
+                    and missing_rows(x, int(o["split_fid"])) > 0):
+                gap = None
+                if orc_dir_gaps is not None and crp is not None:
+                    gap = abs(float(orc_dir_gaps[x][int(crp[o["split_fid"]]) + int(o["split_bid"])]))
+                assert gap is not None and gap <= 2 * gt, \
+                    "node %d default direction differs (oracle's gain difference between the directions: %r, tol %g)" % (
+                        x, gap, 2 * gt)
+                # the missing rows went to different children: nothing below is comparable
+                og = float(o["gain"])
+                diff.near_ties.append((x, og, og - gap, gain_scale(
+                    S, (float(orc[int(o["lch"])]["sum_g"]), float(orc[int(o["lch"])]["sum_h"])), lam)))
+                continue
             stack.extend([int(o["lch"]), int(o["rch"])])
             continue
         assert orc_scores is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (

@@ -211,6 +211,7 @@ def test_tree_lockstep(T, name):
     o.set_gh(gh_all)  # both sides build from bit-identical gradients
     lam = 1.0
     sparse = bool(s.info("sparse"))
+    margins = P.Margins("lockstep/" + name)
     for k in range(s.tree_per_rounds):
         gh = gh_all[k * n:(k + 1) * n]
         ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
@@ -261,6 +262,8 @@ def test_tree_lockstep(T, name):
                 _, h64 = o.level_hist(x)
                 what = "tree %d level %d node %d" % (k, level, x)
                 err = P.assert_hist_close(gh_level[x], h64, tol_level[x], what)
+                nz = tol_level[x] > 0
+                margins.note("hist", err[nz], tol_level[x][nz])
                 if built[x] and (sparse or quant["h_integer"]):
                     # wide fixed-point fields (64-bit sums in the sparse layout, 50-bit gradient fields for squared
                     # loss): also without the half-step allowance, every bin whose entries are not far below the
@@ -281,8 +284,10 @@ def test_tree_lockstep(T, name):
                     continue
                 assert a["fid"] == b["fid"] and a["bid"] == b["bid"] and a["fval"] == b["fval"]
                 assert abs(a["gain"] - b["gain"]) <= P.gain_tolerance(ws, b["gain"], dG, dH), what
+                margins.note("split_gain", abs(float(a["gain"]) - float(b["gain"])), P.gain_tolerance(ws, b["gain"], dG, dH))
                 for key, d in (("lch_g", dG), ("lch_h", dH), ("miss_g", dG), ("miss_h", dH)):
                     assert abs(a[key] - b[key]) <= d, (key, a[key], b[key])
+                    margins.note("split_sums", abs(float(a[key]) - float(b[key])), d)
             tol_prev = tol_level
             if diverged:
                 break
@@ -324,17 +329,24 @@ def test_tree_lockstep(T, name):
         o.predict_in_training(k)
         d = P.compare_trees(s.nodes(), o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(), abs_scale=(ghk[0], ghk[1]))
         assert not d.near_ties
+        margins.add(d)
         sl = slice(k * n, (k + 1) * n)
         tol = P.pred_tolerance(o.nodes(), o.nid(), 1.0, lam, (ghk[0], ghk[1]), o.y_pred()[sl])
-        assert np.all(np.abs(s.y_pred()[sl].astype(np.float64) - o.y_pred()[sl]) <= tol)
+        perr = np.abs(s.y_pred()[sl].astype(np.float64) - o.y_pred()[sl])
+        assert np.all(perr <= tol)
+        margins.note("pred", perr, tol)
+    margins.report()
     s.close()
 
 
 # -------------------------------------------------------------------- boosting, tree by tree
-@pytest.mark.parametrize("name,rounds", [("c1_regression", 40), ("missing_regression", 10), ("c2_binary", 10),
-                                         ("c3_wide_heavy_tails", 6), ("outlier_regression", 8), ("c5_softmax", 3), ("c4_sparse", 10), ("missing_regression@sparse", 10),
-                                         ("c1_regression@sparse", 5)])
-def test_boosting_teacher_forced(T, name, rounds):
+# (case, rounds, significant near ties allowed = the count observed on the MI355X + 1; the two of outlier_regression
+# are nodes of a few rows next to the 1e4x outliers)
+@pytest.mark.parametrize("name,rounds,tie_budget", [
+    ("c1_regression", 40, 1), ("missing_regression", 10, 1), ("c2_binary", 10, 1), ("c3_wide_heavy_tails", 6, 1),
+    ("outlier_regression", 8, 3), ("c5_softmax", 3, 1), ("c4_sparse", 10, 1), ("missing_regression@sparse", 10, 1),
+    ("c1_regression@sparse", 5, 1)])
+def test_boosting_teacher_forced(T, name, rounds, tie_budget):
     """Each round both sides start from the GPU's predictions, so every tree is compared on its own."""
     (val, rp, col), y, kw = case(name)
     kw = dict(kw, n_trees=rounds, learning_rate=0.1 if name == "c1_regression" else 0.3)
@@ -345,6 +357,7 @@ def test_boosting_teacher_forced(T, name, rounds):
     present = np.zeros((n, s.F), bool)
     present[np.repeat(np.arange(n), np.diff(rp)), col] = True
     total_ties = 0
+    margins = P.Margins("teacher_forced/" + name)
     for r in range(rounds):
         yp = s.y_pred()
         o.set_y_pred(yp)
@@ -362,19 +375,27 @@ def test_boosting_teacher_forced(T, name, rounds):
             o.build_tree(k)
             final_nid = o.nid()
             ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
-            d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(),
+            d = P.compare_trees(model[r, k], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(), orc_dir_gaps=o.tree_dir_gaps(),
                                 missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
                                 abs_scale=(ghk[0], ghk[1]))
             # candidates that cut a node's rows into the same two sets have equal gains in exact arithmetic and
             # differ by float round-off only (wide data, nodes of a few rows): those are not counted
             total_ties += len(P.significant_ties(d.near_ties))
             ok_round &= not d.near_ties
+            margins.add(d)
             sl = slice(k * n, (k + 1) * n)
             tol[sl] = P.pred_tolerance(o.nodes(), final_nid, kw["learning_rate"], 1.0, (ghk[0], ghk[1]), o.y_pred()[sl])
         if ok_round:
-            assert np.all(np.abs(s.y_pred().astype(np.float64) - o.y_pred()) <= tol)
+            perr = np.abs(s.y_pred().astype(np.float64) - o.y_pred())
+            assert np.all(perr <= tol)
+            margins.note("pred", perr, tol)
             np.testing.assert_allclose(s.metric_log()[-1], o.metric(), rtol=1e-4, atol=1e-5)
-    assert total_ties <= max(2, rounds * s.tree_per_rounds // 5), "too many near ties: %d" % total_ties
+    margins.ties = total_ties
+    margins.report()
+    assert total_ties <= tie_budget, "too many near ties: %d" % total_ties
+    # how much of the 1e-5 bounds the two implementations use (the GPU's sums are exact integers; what is left is the
+    # float32 prefix scan and subtraction chain of the reference's algorithm): at most 0.4 observed
+    assert max(margins.worst.values()) <= 0.8, margins.worst
     s.close()
 
 

@@ -195,7 +195,7 @@ def test_rank_boosting_teacher_forced(T, objective, name):
         o.build_tree(0)
         final_nid = o.nid()
         ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
-        d = P.compare_trees(s.model()[r, 0], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(),
+        d = P.compare_trees(s.model()[r, 0], o.nodes(), 1.0, crp=crp, orc_scores=o.tree_scores(), orc_dir_gaps=o.tree_dir_gaps(),
                             missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
                             abs_scale=(ghk[0], ghk[1]), mcw=0.1)
         total_ties += len(d.near_ties)
@@ -246,7 +246,7 @@ def test_rank_with_bagging_and_column_sampling(T, layout):
             o.set_gh(gh)
             o.build_tree(0)
             ghk = np.abs(gh.astype(np.float64)).sum(axis=0)
-            d = P.compare_trees(s.model()[r, 0], o.nodes(), 1.0, crp=s.cuts()[1], orc_scores=o.tree_scores(),
+            d = P.compare_trees(s.model()[r, 0], o.nodes(), 1.0, crp=s.cuts()[1], orc_scores=o.tree_scores(), orc_dir_gaps=o.tree_dir_gaps(),
                                 abs_scale=(ghk[0], ghk[1]), mcw=0.05)
             ties += len(d.near_ties)
         assert ties <= rounds
