@@ -139,10 +139,13 @@ def main():
     value = args.steps / dt
 
     roofline = None
+    phases = None
     if args.profile_steps > 0:
+        # (profiled iterations follow the timed ones: HIP events between the stages would perturb the timed region)
         s.set_profiling(True)
         s.boost(args.profile_steps)
         prof = s.profile()
+        phases = s.phase_profile()
         s.set_profiling(False)
         if prof["launches"] > 0 and prof["hist_ms"] > 0:
             achieved = prof["bytes"] / (prof["hist_ms"] * 1e-3) / 1e9
@@ -154,12 +157,26 @@ def main():
                         "bytes_per_launch": round(prof["bytes"] / prof["launches"], 1),
                         "avg_launch_us": round(prof["hist_ms"] * 1e3 / prof["launches"], 2),
                         "hist_ms_per_step": round(prof["hist_ms"] / args.profile_steps, 4),
-                        "rows_built_per_step": prof["rows_built"] // args.profile_steps}
+                        "rows_built_per_step": prof["rows_built"] // args.profile_steps,
+                        "measured_on": "the %d iterations that follow the timed ones (iterations %d-%d of the run), "
+                                       "HIP events on the trainer's stream around every stage" % (
+                                           args.profile_steps, args.warmup + args.steps + 1, total_rounds)}
+            for part in ("root", "below_root"):  # the root level streams its rows, the levels below gather theirs
+                h = phases["hist"][part]
+                if h["launches"] > 0 and h["ms"] > 0:
+                    gbs = h["bytes"] / (h["ms"] * 1e-3) / 1e9
+                    roofline[part] = {"launches": h["launches"], "bytes_per_launch": round(h["bytes"] / h["launches"], 1),
+                                      "avg_launch_us": round(h["ms"] * 1e3 / h["launches"], 2),
+                                      "achieved": round(gbs, 2), "frac": round(gbs / 8000.0, 4)}
     metric_log = s.metric_log()
     reorders = s.info("reorders_done")
     s.close()
 
-    aux = {"data_gen_s": round(t_gen, 2), "prep_s_upload_cuts_bins": round(t_prep, 3),
+    aux = {"phase_ms": None if phases is None else
+           {k: round(v / max(1, phases["rounds"]), 4) for k, v in phases["phase_ms"].items()},
+           "phase_ms_note": "milliseconds per iteration of the profiled iterations, by stage; their sum exceeds ms_per_step "
+                            "by what the event records between the stages cost",
+           "data_gen_s": round(t_gen, 2), "prep_s_upload_cuts_bins": round(t_prep, 3),
            "train_metric_last": float(metric_log[-1]) if len(metric_log) else None,
            "row_reorderings_before_or_inside_the_timed_steps": reorders}
     if args.config == 2 and args.full_run and args.rows == 0:

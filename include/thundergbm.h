@@ -159,6 +159,15 @@ void tgbm_trainer_set(tgbm_trainer *t, const char *name, const void *in, size_t 
  * out[3] = algorithmic bytes (rows x (features + 8 [+4 below the root])). */
 void tgbm_trainer_set_profiling(tgbm_trainer *t, int on);
 void tgbm_trainer_get_profile(tgbm_trainer *t, double *out4);
+/* Per-stage timing of the rounds boosted while profiling was on (the reference accumulates host timers for histogram
+ * build, evaluation and data partitioning under its `profiling` switch, hist_tree_builder_single.cu:19-27, :196-219,
+ * :392, :400-418; thundergbm_train.cpp:28-30). HIP events on the trainer's stream close every stage. Fills up to
+ * `cap` of: out[0] rounds; milliseconds of out[1] gradients + tree init, [2] histogram build, [3] merge + sibling
+ * subtraction + root sums, [4] split search + tree update, [5] partition, [6] end of tree (prune, prediction update,
+ * fused metric and next gradients), [7] metric as a pass of its own, [8] row re-ordering; then the histogram launches
+ * of the root level: [9] milliseconds, [10] launches, [11] algorithmic bytes; and of the levels below it: [12], [13],
+ * [14]. Returns the number of values it knows (15). */
+int tgbm_trainer_get_phase_profile(tgbm_trainer *t, double *out, int cap);
 
 /* Moves the trees built so far into a model handle usable with the Part 1 functions. */
 tgbm_model *tgbm_trainer_export_model(tgbm_trainer *t);

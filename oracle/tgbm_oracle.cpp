@@ -39,6 +39,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <new>
 #include <random>
 #include <string>
 #include <vector>
@@ -89,6 +90,45 @@ inline float compute_gain(GH f, GH l, GH r, float mcw, float lambda) {
     return 0.f;
 }
 
+// A level's histograms (nodes x bins): memory that is never touched by one thread alone. A wide sparse configuration
+// needs gigabytes per level, and a std::vector would fault its pages in and fill them sequentially.
+template <typename T>
+struct ZeroedBuffer {
+    T *p = nullptr;
+    size_t cap = 0, n = 0;
+    ZeroedBuffer() = default;
+    ZeroedBuffer(const ZeroedBuffer &) = delete;
+    ZeroedBuffer &operator=(const ZeroedBuffer &) = delete;
+    ~ZeroedBuffer() { std::free(p); }
+    T *data() { return p; }
+    const T *data() const { return p; }
+    size_t size() const { return n; }
+    void assign_zero(size_t count) {
+        if (count > cap) {
+            std::free(p);
+            p = (T *)std::malloc(std::max<size_t>(count, 1) * sizeof(T));
+            if (!p) throw std::bad_alloc();
+            cap = count;
+        }
+        n = count;
+        T *q = p;
+#pragma omp parallel for schedule(static) if (count > 200000)
+        for (long i = 0; i < (long)count; ++i) q[i] = T{};
+    }
+    void swap(ZeroedBuffer &o) {
+        std::swap(p, o.p);
+        std::swap(cap, o.cap);
+        std::swap(n, o.n);
+    }
+};
+
+struct ProbeResult {
+    float score;         // signed gain of the probed candidate (0 when the node was not evaluated)
+    float dir_gap;       // its gain(missing -> left) - gain(missing -> right)
+    float best;          // |gain| of the node's best candidate
+    float best_dir_gap;  // gain(missing -> left) - gain(missing -> right) of the best candidate
+};
+
 struct Oracle {
     float column_sampling_rate = 1.f;
     bool bagging = false;
@@ -121,14 +161,20 @@ struct Oracle {
     bool keep_debug = false;
     bool shadow64 = false;
     // raw (unscanned) histograms of the current and previous level, node-major
-    std::vector<GH> hist_cur, hist_prev;
-    std::vector<double> hist64_cur, hist64_prev;  // g,h interleaved
+    ZeroedBuffer<GH> hist_cur, hist_prev;
+    ZeroedBuffer<double> hist64_cur, hist64_prev;  // g,h interleaved
+    std::vector<double> hist_scratch;             // build_hist: one fp64 histogram per thread
+    std::vector<GH> eval_pre, eval_miss;          // evaluate_node: prefix sums per bin, missing sums per feature
     // debug: per node of the whole tree
     std::vector<float> dbg_score;   // [n_nodes][n_bins], signed gain of every candidate
     std::vector<float> dbg_dir_gap; // [n_nodes][n_bins], gain(missing -> left) - gain(missing -> right) of every candidate
     std::vector<GH> dbg_hist;       // [n_nodes][n_bins], raw hist
     std::vector<double> dbg_hist64; // [n_nodes][n_bins][2]
     std::vector<int> dbg_built;     // [n_nodes] 1 if built from rows, 0 if by subtraction
+    // Probes: the debug arrays above need n_nodes x n_bins floats, gigabytes for wide data. A probe names one
+    // candidate (global bin index, -1 = none) per node whose signed gain is recorded next to the node's best.
+    std::vector<int> probe;              // [n_nodes]
+    std::vector<ProbeResult> probe_out;  // [n_nodes]
     std::vector<std::vector<Node>> model;  // iteration-major, class inside
     std::vector<float> metric_log;
     long rows_built_total = 0;      // rows visited by histogram builds (for byte accounting)
@@ -319,10 +365,17 @@ void build_hist(Oracle &o, const int *rows, long cnt, GH *out, double *out64) {
     nt = omp_get_max_threads();
 #endif
     if (cnt < 4096) nt = 1;
+    // (a private histogram per thread is only worth its clearing and adding up when the node's stored entries
+    // outnumber the bins: wide sparse data has millions of bins and deep nodes of a few thousand rows)
+    const double entries = (double)cnt * (double)o.row_ptr[o.n] / (double)std::max(1, o.n);
+    nt = (int)std::max(1.0, std::min((double)nt, entries / (0.5 * (double)std::max(1, B))));
     // The reference adds with float atomics in no defined order, so its own result varies from run to run
     // by float round-off that grows with the number of rows per bin. The oracle accumulates in fp64 and
     // rounds once: the centre of those possible results, and what the 1e-5 parity tolerance refers to.
-    std::vector<double> priv64((size_t)nt * B * 2, 0.0);
+    std::vector<double> &priv64 = o.hist_scratch;
+    if (priv64.size() < (size_t)nt * B * 2) priv64.resize((size_t)nt * B * 2);
+#pragma omp parallel for schedule(static) if ((size_t)nt * B > 200000)
+    for (long i = 0; i < (long)nt * B * 2; ++i) priv64[i] = 0.0;
 #pragma omp parallel num_threads(nt)
     {
         int t = 0;
@@ -341,6 +394,7 @@ void build_hist(Oracle &o, const int *rows, long cnt, GH *out, double *out64) {
             }
         }
     }
+#pragma omp parallel for schedule(static) if (B > 100000)
     for (int b = 0; b < B; ++b) {
         double g = 0, h = 0;
         for (int t = 0; t < nt; ++t) {
@@ -382,10 +436,16 @@ void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
         s.nid = -1;
         return;
     }
-    std::vector<GH> pre(B);
-    std::vector<GH> miss(F, GH{0, 0});
+    std::vector<GH> &pre = o.eval_pre;
+    std::vector<GH> &miss = o.eval_miss;
+    pre.resize(B);
+    miss.assign(F, GH{0, 0});
     const GH S = nd.sum;
+    // (wide data: features in parallel; every feature's scan and every candidate's gain is computed exactly as in the
+    // sequential loop, and the arg-max below combines the threads' ranges in ascending order of their bins)
+    const bool par = B > 100000;
     // inclusive_scan_by_key over cut_fid (:257, :614): fp32 running sums restarting per feature
+#pragma omp parallel for schedule(static) if (par)
     for (int f = 0; f < F; ++f) {
         float g = 0, h = 0;
         for (int b = o.cut_row_ptr[f]; b < o.cut_row_ptr[f + 1]; ++b) {
@@ -403,27 +463,63 @@ void evaluate_node(Oracle &o, int node, const GH *raw, Split &s) {
     float best_score = 0;
     bool first = true;
     float *dbg = o.keep_debug ? o.dbg_score.data() + (size_t)node * B : nullptr;
-    for (int b = 0; b < B; ++b) {
-        int f = o.cut_fid[b];
+    int n_parts = 1;
+#ifdef _OPENMP
+    if (par) n_parts = omp_get_max_threads();
+#endif
+    std::vector<int> part_best(n_parts, -1);
+    std::vector<float> part_score(n_parts, 0.f);
+#pragma omp parallel for schedule(static, 1) if (par)
+    for (int part = 0; part < n_parts; ++part) {
+        const int b_lo = (int)((long)B * part / n_parts), b_hi = (int)((long)B * (part + 1) / n_parts);
+        int pb = -1;
+        float ps = 0;
+        for (int b = b_lo; b < b_hi; ++b) {
+            int f = o.cut_fid[b];
+            GH l = GH{0, 0};
+            if (o.cut_row_ptr[f] != b) l = pre[b - 1];
+            GH r = GH{S.g - l.g, S.h - l.h};
+            float gr = fmaxf(0.f, compute_gain(S, l, r, o.mcw, o.lambda));
+            GH l2 = GH{l.g + miss[f].g, l.h + miss[f].h};
+            GH r2 = GH{S.g - l2.g, S.h - l2.h};
+            float gl = fmaxf(0.f, compute_gain(S, l2, r2, o.mcw, o.lambda));
+            float score = (gl > gr) ? gl : -gr;
+            if (!o.ignored.empty() && o.ignored[f]) score = 0;  // :304 / :663: an ignored column's gain is 0
+            if (dbg) {
+                dbg[b] = score;
+                o.dbg_dir_gap[(size_t)node * B + b] = gl - gr;
+            }
+            if (!o.probe.empty() && (size_t)node < o.probe.size() && o.probe[node] == b)
+                o.probe_out[node] = ProbeResult{score, gl - gr, 0.f, 0.f};
+            // arg_abs_max (:330-335): larger |gain| wins, ties keep the smaller index
+            if (pb < 0 || fabsf(score) > fabsf(ps)) {
+                pb = b;
+                ps = score;
+            }
+        }
+        part_best[part] = pb;
+        part_score[part] = ps;
+    }
+    for (int part = 0; part < n_parts; ++part) {
+        if (part_best[part] < 0) continue;
+        if (first || fabsf(part_score[part]) > fabsf(best_score)) {
+            best = part_best[part];
+            best_score = part_score[part];
+            first = false;
+        }
+    }
+    if (!o.probe.empty() && (size_t)node < o.probe.size() && B > 0) {
+        // the chosen candidate's two direction gains once more, for the probe record
+        int f = o.cut_fid[best];
         GH l = GH{0, 0};
-        if (o.cut_row_ptr[f] != b) l = pre[b - 1];
+        if (o.cut_row_ptr[f] != best) l = pre[best - 1];
         GH r = GH{S.g - l.g, S.h - l.h};
         float gr = fmaxf(0.f, compute_gain(S, l, r, o.mcw, o.lambda));
         GH l2 = GH{l.g + miss[f].g, l.h + miss[f].h};
         GH r2 = GH{S.g - l2.g, S.h - l2.h};
         float gl = fmaxf(0.f, compute_gain(S, l2, r2, o.mcw, o.lambda));
-        float score = (gl > gr) ? gl : -gr;
-        if (!o.ignored.empty() && o.ignored[f]) score = 0;  // :304 / :663: an ignored column's gain is 0
-        if (dbg) {
-            dbg[b] = score;
-            o.dbg_dir_gap[(size_t)node * B + b] = gl - gr;
-        }
-        // arg_abs_max (:330-335): larger |gain| wins, ties keep the smaller index
-        if (first || fabsf(score) > fabsf(best_score)) {
-            best = b;
-            best_score = score;
-            first = false;
-        }
+        o.probe_out[node].best = fabsf(best_score);
+        o.probe_out[node].best_dir_gap = gl - gr;
     }
     std::memset(&s, 0, sizeof(Split));
     if (B == 0) {  // no candidate at all: behaves as a zero-gain split point
@@ -462,10 +558,10 @@ void find_split(Oracle &o, int level) {
     const int n_level = 1 << level;
     const int off = n_level - 1;
     o.sp.assign(n_level, Split{});
-    std::swap(o.hist_cur, o.hist_prev);
-    std::swap(o.hist64_cur, o.hist64_prev);
-    o.hist_cur.assign((size_t)n_level * B, GH{0, 0});
-    if (o.shadow64) o.hist64_cur.assign((size_t)n_level * B * 2, 0.0);
+    o.hist_cur.swap(o.hist_prev);
+    o.hist64_cur.swap(o.hist64_prev);
+    o.hist_cur.assign_zero((size_t)n_level * B);
+    if (o.shadow64) o.hist64_cur.assign_zero((size_t)n_level * B * 2);
     long built_rows_before = o.rows_built_total;
     if (level == 0) {
         build_hist(o, nullptr, o.n, o.hist_cur.data(), o.shadow64 ? o.hist64_cur.data() : nullptr);
@@ -507,6 +603,7 @@ void find_split(Oracle &o, int level) {
             double *hb64 = o.shadow64 ? o.hist64_cur.data() + (size_t)b * B * 2 : nullptr;
             build_hist(o, idx.data() + ptr[a], ptr[a + 1] - ptr[a], ha, ha64);
             const GH *par = o.hist_prev.data() + (size_t)p * B;  // raw parent histogram (:526-540)
+#pragma omp parallel for schedule(static) if (B > 100000)
             for (int i = 0; i < B; ++i) hb[i] = GH{par[i].g - ha[i].g, par[i].h - ha[i].h};
             if (o.shadow64) {
                 const double *par64 = o.hist64_prev.data() + (size_t)p * B * 2;
@@ -1169,6 +1266,23 @@ void orc_get_level_hist(void *h, int node_in_level, float *out, double *out64) {
 void orc_get_tree_scores(void *h, float *out) {
     Oracle &o = *(Oracle *)h;
     std::copy(o.dbg_score.begin(), o.dbg_score.end(), out);
+}
+// probe: n_nodes global candidate indices (-1 = none), or nullptr to switch probing off; results are collected
+// while the next tree is built
+void orc_set_probes(void *h, const int *probe) {
+    Oracle &o = *(Oracle *)h;
+    const int n_nodes = (1 << (o.depth + 1)) - 1;
+    if (probe == nullptr) {
+        o.probe.clear();
+        o.probe_out.clear();
+        return;
+    }
+    o.probe.assign(probe, probe + n_nodes);
+    o.probe_out.assign(n_nodes, ProbeResult{0.f, 0.f, 0.f, 0.f});
+}
+void orc_get_probes(void *h, ProbeResult *out) {
+    Oracle &o = *(Oracle *)h;
+    std::copy(o.probe_out.begin(), o.probe_out.end(), out);
 }
 void orc_get_tree_dir_gaps(void *h, float *out) {
     Oracle &o = *(Oracle *)h;

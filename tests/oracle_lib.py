@@ -27,6 +27,8 @@ SPLIT_DTYPE = np.dtype(
 )
 assert SPLIT_DTYPE.itemsize == 48
 
+PROBE_DTYPE = np.dtype([("score", "<f4"), ("dir_gap", "<f4"), ("best", "<f4"), ("best_dir_gap", "<f4")])
+
 _lib = None
 
 
@@ -75,6 +77,10 @@ def lib():
                      "orc_get_tree_scores", "orc_get_tree_dir_gaps", "orc_get_model"):
             getattr(L, name).argtypes = [C.c_void_p, C.c_void_p]
             getattr(L, name).restype = None
+        L.orc_set_probes.argtypes = [C.c_void_p, C.c_void_p]
+        L.orc_set_probes.restype = None
+        L.orc_get_probes.argtypes = [C.c_void_p, C.c_void_p]
+        L.orc_get_probes.restype = None
         L.orc_get_cuts.argtypes = [C.c_void_p] * 4
         L.orc_get_splits.argtypes = [C.c_void_p, C.c_void_p]
         L.orc_get_splits.restype = C.c_int
@@ -277,6 +283,22 @@ class Oracle:
         out = np.zeros((self.n_nodes, self.n_bins), dtype=np.float32)
         self.L.orc_get_tree_scores(self.h, _p(out))
         return out
+
+    def set_probes(self, probe):
+        """One candidate (global bin index, -1 = none) per node whose signed gain the next build_tree records next
+        to the node's best: what tree_scores / tree_dir_gaps give for all candidates, in O(nodes) memory."""
+        if probe is None:
+            self.L.orc_set_probes(self.h, None)
+            return
+        probe = np.ascontiguousarray(probe, dtype=np.int32)
+        assert len(probe) == self.n_nodes
+        self.L.orc_set_probes(self.h, _p(probe))
+        self._probe = probe
+
+    def probes(self):
+        out = np.zeros(self.n_nodes, dtype=PROBE_DTYPE)
+        self.L.orc_get_probes(self.h, _p(out))
+        return self._probe, out
 
     def tree_dir_gaps(self):
         """gain(missing -> left) - gain(missing -> right) of every candidate of every node of the current tree."""

@@ -83,6 +83,8 @@ class TreeDiff:
         self.compared = 0
         # (node, oracle best |gain|, oracle |gain| of the GPU's choice, magnitude of the oracle gain's terms)
         self.near_ties = []
+        # (node, feature) of nodes whose few rows without the split feature took different default directions
+        self.direction_ties = []
         # largest observed error / tolerance of the compared node sums, weights and gains (how much of the bound
         # the two implementations actually use)
         self.worst = {"sum": 0.0, "weight": 0.0, "gain": 0.0}
@@ -121,6 +123,50 @@ class Margins:
                 f.write(line + "\n")
 
 
+class FullScores:
+    """The oracle's candidate gains of one tree as compare_trees reads them, from the complete debug arrays
+    (Oracle.tree_scores(), Oracle.tree_dir_gaps(): [n_nodes, n_bins])."""
+
+    def __init__(self, scores, dir_gaps=None):
+        self.scores, self.dir_gaps = scores, dir_gaps
+
+    def best(self, x):
+        return float(np.abs(self.scores[x]).max())
+
+    def of(self, x, idx):
+        return abs(float(self.scores[x][idx]))
+
+    def dir_gap(self, x, idx):
+        return None if self.dir_gaps is None else abs(float(self.dir_gaps[x][idx]))
+
+
+class ProbeScores:
+    """The same from probes (Oracle.set_probes / probes()): per node the gain of one named candidate - the GPU's
+    choice - and of the oracle's best; for data whose n_nodes x n_bins arrays would take gigabytes."""
+
+    def __init__(self, probe, out):
+        self.probe, self.out = probe, out
+
+    def best(self, x):
+        return float(self.out[x]["best"])
+
+    def of(self, x, idx):
+        assert int(self.probe[x]) == int(idx), "node %d: candidate %d was not probed (%d was)" % (x, idx, self.probe[x])
+        return abs(float(self.out[x]["score"]))
+
+    def dir_gap(self, x, idx):
+        if int(self.probe[x]) == int(idx):
+            return abs(float(self.out[x]["dir_gap"]))
+        return abs(float(self.out[x]["best_dir_gap"]))  # (only asked for the oracle's own choice)
+
+
+def probes_for(gpu, crp):
+    """The GPU tree's chosen candidate per node as a global bin index (-1 where it did not split)."""
+    fid = gpu["split_fid"].astype(np.int64)
+    idx = np.asarray(crp)[np.maximum(fid, 0)].astype(np.int64) + gpu["split_bid"].astype(np.int64)
+    return np.where((fid >= 0) & (gpu["is_valid"] == 1), idx, -1).astype(np.int32)
+
+
 def significant_ties(near_ties):
     """Near ties that are more than float round-off between two candidates: candidates that cut a node's rows into
     the same two sets have equal gains in exact arithmetic, and which of them a float implementation prefers is
@@ -140,7 +186,7 @@ def rows_in_node(final_nid, x):
 
 
 def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL, mcw=1.0,
-                  orc_dir_gaps=None):
+                  orc_dir_gaps=None, few_missing_rows=0):
     """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
 
     Where both trees split on the same candidate everything must agree: threshold and bin exactly,
@@ -152,7 +198,11 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     larger of two gains of the same candidate (missing -> left against missing -> right, strict `>`,
     hist_tree_builder_single.cu:300-323); orc_dir_gaps [n_nodes, n_bins] holds the oracle's difference of the
     two, and a direction that differs is a near tie like any other when that difference is within the gain
-    tolerance (without orc_dir_gaps a differing direction fails).
+    tolerance (without orc_dir_gaps a differing direction fails). Such a node's subtree is not compared either -
+    unless the node has at most few_missing_rows rows without the feature (a handful of exact zeros in ten million
+    rows of continuous data): those few rows cannot move a sum beyond its bound, so the comparison goes on below the
+    node and the node is listed in TreeDiff.direction_ties, for the caller to excuse exactly those rows from the
+    comparison of the row -> node maps.
 
     Tolerance: node sums are float32 results of a chain of histogram subtractions that starts at the
     root, so their error is relative to the root-level sums of |g| and |h| (abs_scale = (Ag, Ah)):
@@ -162,11 +212,14 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     hessian sum sits within dH of min_child_weight (mcw): that gate (hist_tree_builder_single.cu
     compute_gain: both children need h >= min_child_weight) flips on the last ulps of a sum, e.g. four
     logistic rows with p = 0.5 give exactly 4 * 0.25 = 1.0 or one ulp less depending on the order.
-    orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle (None forbids any mismatch);
-    crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
+    orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle, or a FullScores / ProbeScores view of them
+    (None forbids any mismatch); crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
     """
     diff = TreeDiff()
     stack = [0]
+    view = orc_scores
+    if orc_scores is not None and not hasattr(orc_scores, "best"):
+        view = FullScores(orc_scores, orc_dir_gaps)
     if abs_scale is None:
         abs_scale = (max(1.0, abs(float(orc[0]["sum_g"])) + float(orc[0]["sum_h"])),) * 2
     dG, dH = sum_bounds(abs_scale, rel)
@@ -201,14 +254,20 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
             gt = gain_tol(x, o)
             assert abs(g["gain"] - o["gain"]) <= gt, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
             diff.worst["gain"] = max(diff.worst["gain"], abs(float(g["gain"]) - float(o["gain"])) / gt)
-            if (g["default_right"] != o["default_right"] and missing_rows is not None
-                    and missing_rows(x, int(o["split_fid"])) > 0):
+            n_missing = 0
+            if g["default_right"] != o["default_right"] and missing_rows is not None:
+                n_missing = missing_rows(x, int(o["split_fid"]))
+            if n_missing > 0:
                 gap = None
-                if orc_dir_gaps is not None and crp is not None:
-                    gap = abs(float(orc_dir_gaps[x][int(crp[o["split_fid"]]) + int(o["split_bid"])]))
+                if view is not None and crp is not None:
+                    gap = view.dir_gap(x, int(crp[o["split_fid"]]) + int(o["split_bid"]))
                 assert gap is not None and gap <= 2 * gt, \
                     "node %d default direction differs (oracle's gain difference between the directions: %r, tol %g)" % (
                         x, gap, 2 * gt)
+                if n_missing <= few_missing_rows:
+                    diff.direction_ties.append((x, int(o["split_fid"])))
+                    stack.extend([int(o["lch"]), int(o["rch"])])
+                    continue
                 # the missing rows went to different children: nothing below is comparable
                 og = float(o["gain"])
                 diff.near_ties.append((x, og, og - gap, gain_scale(
@@ -216,18 +275,17 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
                 continue
             stack.extend([int(o["lch"]), int(o["rch"])])
             continue
-        assert orc_scores is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (
+        assert view is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (
             x, g["split_fid"], g["split_bid"], o["split_fid"], o["split_bid"])
         on_gate = False
         for t, has in ((gpu, split_g), (orc, split_o)):
             if has:
                 hmin = min(float(t[int(t[x]["lch"])]["sum_h"]), float(t[int(t[x]["rch"])]["sum_h"]))
                 on_gate |= abs(hmin - mcw) <= dH
-        sc = orc_scores[x]
-        best = float(np.abs(sc).max())
+        best = view.best(x)
         tol = 2 * gain_tol(x, o)
         if split_g:
-            alt = abs(float(sc[int(crp[g["split_fid"]]) + int(g["split_bid"])]))
+            alt = view.of(x, int(crp[g["split_fid"]]) + int(g["split_bid"]))
             ok = best - alt <= tol
             msg = "node %d: gpu chose f%d b%d with oracle gain %g, oracle best %g (f%d b%d), tol %g" % (
                 x, g["split_fid"], g["split_bid"], alt, best, o["split_fid"], o["split_bid"], tol)
@@ -242,7 +300,7 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
         # magnitude of the three terms whose difference the gain is (float cancellation noise scales with it)
         terms = gain_scale(S, (float(orc[int(o["lch"])]["sum_g"]), float(orc[int(o["lch"])]["sum_h"])), lam) if split_o else 0.0
         diff.near_ties.append((x, best, alt, terms))
-    if not diff.near_ties:
+    if not diff.near_ties and not diff.direction_ties:
         for key in ("is_leaf", "is_pruned", "final_id", "lch", "rch", "parent"):
             valid = orc["is_valid"] == 1
             assert np.array_equal(gpu[key][valid], orc[key][valid]), "field %s differs" % key

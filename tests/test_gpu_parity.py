@@ -549,7 +549,107 @@ def test_a1a_quickstart_known_answer(T, layout):
     s.close()
 
 
-# --------------------------------------------- size-independent properties at the benchmark shape
+# ------------------------------------- the benchmark configurations at full size: properties, then the oracle
+_FULL = {}
+
+
+def _full_data(name):
+    """CSR arrays and labels of a full-size configuration; the tests of one configuration follow each other, and only
+    the last one asked for is kept."""
+    if name not in _FULL:
+        _FULL.clear()
+        if name == "c2":
+            X, y = D.config2(10_000_000, seed=1)
+        elif name == "c3":
+            X, y = D.config3()
+        elif name == "c5":
+            X, y = D.config5()
+        if name == "c4":
+            val, rp, col, y = D.config4()
+        else:
+            val, rp, col = D.dense_to_csr(X)
+            del X
+        _FULL[name] = (val, rp, col, y)
+    return _FULL[name]
+
+
+class _Stored:
+    """Which rows store which feature: lacking(f) = mask of the rows without feature f. Rows that store every
+    feature are skipped outright (continuous data has a handful of rows with an exact zero); data with many
+    incomplete rows gets a column-major copy when first asked (a direction that differs is rare)."""
+
+    def __init__(self, rp, col, F):
+        self.rp, self.col, self.F, self.n = rp, col, F, len(rp) - 1
+        self.incomplete = np.flatnonzero(np.diff(rp) < F)
+        self.csc = None
+
+    def lacking(self, f):
+        m = np.zeros(self.n, bool)
+        if len(self.incomplete) <= 10000:
+            for r in self.incomplete:
+                m[r] = f not in self.col[self.rp[r]:self.rp[r + 1]]
+            return m
+        if self.csc is None:
+            import scipy.sparse as sp
+            self.csc = sp.csr_matrix((np.ones(len(self.col), np.int8), self.col, self.rp), shape=(self.n, self.F)).tocsc()
+        m[:] = True
+        m[self.csc.indices[self.csc.indptr[f]:self.csc.indptr[f + 1]]] = False
+        return m
+
+
+def _oracle_tree_at_full_size(T, s, o, round_index, crp, lr, margins, stored):
+    """One boosting round of the library against the oracle started from the library's predictions and gradients:
+    every class tree through compare_trees (candidate gains from probes: the oracle records, per node, its best gain
+    and the gain of the candidate the GPU chose), the row -> node map bit for bit, predictions within the bound.
+    Returns the number of near ties."""
+    n, K = s.n, s.tree_per_rounds
+    o.set_y_pred(s.y_pred())
+    s.gradient()
+    gh = s.gh()
+    s.boost(1)
+    model = s.model()
+    o.compute_gradient()
+    np.testing.assert_allclose(gh, o.gh(), rtol=1e-5, atol=2e-7)
+    o.set_gh(gh)
+    ties = 0
+    for k in range(K):
+        gpu = model[round_index, k]
+        o.set_probes(P.probes_for(gpu, crp))
+        o.build_tree(k)
+        final_nid = o.nid()
+        ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
+
+        def rows_without(x, f):
+            m = stored.lacking(f)
+            return m & P.rows_in_node(final_nid, x) if m.any() else m
+
+        d = P.compare_trees(gpu, o.nodes(), 1.0, crp=crp, orc_scores=P.ProbeScores(*o.probes()),
+                            missing_rows=lambda x, f: int(rows_without(x, f).sum()), abs_scale=(ghk[0], ghk[1]),
+                            few_missing_rows=4)
+        margins.add(d)
+        ties += len(P.significant_ties(d.near_ties))
+        for t in d.near_ties:  # how close the candidates are that the two sides chose between
+            margins.worst["near_tie_rel_gap"] = max(margins.worst.get("near_tie_rel_gap", 0.0), (t[1] - t[2]) / max(t[1], 1e-30))
+        margins.worst["near_ties_all"] = margins.worst.get("near_ties_all", 0) + len(d.near_ties)
+        if d.near_ties:
+            continue
+        # rows that may sit elsewhere: the few without the split feature of a node where sending them left or right
+        # gains the same within the tolerance (continuous data holds a handful of exact zeros, which are not stored)
+        excused = np.zeros(n, bool)
+        for x, f in d.direction_ties:
+            excused |= rows_without(x, f)
+        assert excused.sum() <= 4 * len(d.direction_ties)
+        if k == K - 1:
+            assert np.array_equal(s.nid()[~excused], final_nid[~excused]), "row -> node map differs"
+        sl = slice(k * n, (k + 1) * n)
+        tol = P.pred_tolerance(o.nodes(), final_nid, lr, 1.0, (ghk[0], ghk[1]), o.y_pred()[sl])
+        perr = np.abs(s.y_pred()[sl].astype(np.float64) - o.y_pred()[sl])
+        assert np.all(perr[~excused] <= tol[~excused])
+        margins.note("pred", perr[~excused], tol[~excused])
+    o.set_probes(None)
+    return ties
+
+
 def test_full_size_properties_config2(T):
     n = int(os.environ.get("TGBM_TEST_FULL_ROWS", "10000000"))
     X, y = D.config2(n, seed=1)
@@ -674,11 +774,35 @@ def test_full_size_properties_config2_reordered_rows(T):
     """10 M x 28 after the rows were physically re-ordered (boost() does that after the second tree): the
     fourth tree's sums against an fp64 recount through the row -> node map, which like the gradients and the
     predictions comes back in the caller's row order, and the predictor against the training predictions."""
-    X, y = D.config2(10_000_000, seed=1)
-    val, rp, col = D.dense_to_csr(X)
-    del X
+    val, rp, col, y = _full_data("c2")
     _check_boosted_round(T, val, rp, col, y, 100000, pre_rounds=3, objective="binary:logistic", depth=8,
                          max_num_bin=255)
+
+
+def test_full_size_oracle_config2(T):
+    """10 M x 28, depth 8, 255 bins against the oracle at the full shape: the first tree (rows in the caller's order,
+    512-item plans, work items drained every 8192 rows) and the fifth (after three physical re-orderings of the
+    rows)."""
+    val, rp, col, y = _full_data("c2")
+    kw = dict(objective="binary:logistic", depth=8, max_num_bin=255, learning_rate=0.3, n_trees=5)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    cv, crp, cf = s.cuts()
+    ocv, ocrp, ocf = o.cuts()
+    assert np.array_equal(cv.view(np.uint32), ocv.view(np.uint32)) and np.array_equal(crp, ocrp)
+    gb, _ = s.global_bin_ids(rp, col)
+    assert np.array_equal(gb, o.bin_ids())
+    del gb
+    stored = _Stored(rp, col, s.F)
+    margins = P.Margins("full_size/config2")
+    ties = _oracle_tree_at_full_size(T, s, o, 0, crp, 0.3, margins, stored)
+    s.boost(3)
+    assert s.info("reorders_done") >= 3
+    ties += _oracle_tree_at_full_size(T, s, o, 4, crp, 0.3, margins, stored)
+    margins.ties = ties
+    margins.report()
+    assert ties <= 1
+    s.close()
 
 
 def test_full_size_properties_16_bit_bins_reordered_rows(T):
@@ -693,24 +817,81 @@ def test_full_size_properties_16_bit_bins_reordered_rows(T):
 
 def test_full_size_properties_config5_softmax(T):
     """1 M x 54, 8 classes: the class trees of the round are built by common launches."""
-    X, y = D.config5()
-    val, rp, col = D.dense_to_csr(X)
-    del X
+    val, rp, col, y = _full_data("c5")
     _check_boosted_round(T, val, rp, col, y, 100000, objective="multi:softmax", depth=8, max_num_bin=255)
+
+
+def test_full_size_oracle_config5_softmax(T):
+    """1 M x 54, 8 classes, depth 8 against the oracle at the full shape: the eight class trees of the first and of
+    the second round (bundled one-hot columns, class trees built by common launches)."""
+    val, rp, col, y = _full_data("c5")
+    kw = dict(objective="multi:softmax", depth=8, max_num_bin=255, learning_rate=0.3, n_trees=2)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    _, crp, _ = s.cuts()
+    assert np.array_equal(s.cuts()[0].view(np.uint32), o.cuts()[0].view(np.uint32)) and np.array_equal(crp, o.cuts()[1])
+    assert np.array_equal(s.global_bin_ids(rp, col)[0], o.bin_ids())
+    stored = _Stored(rp, col, s.F)
+    margins = P.Margins("full_size/config5")
+    ties = _oracle_tree_at_full_size(T, s, o, 0, crp, 0.3, margins, stored)
+    ties += _oracle_tree_at_full_size(T, s, o, 1, crp, 0.3, margins, stored)
+    margins.ties = ties
+    margins.report()
+    assert ties <= 2
+    s.close()
 
 
 def test_full_size_properties_config3_wide(T):
     """500k x 2000, depth 6: 63 feature blocks per work item, 4 MB of histogram per node."""
-    X, y = D.config3()
-    val, rp, col = D.dense_to_csr(X)
-    del X
+    val, rp, col, y = _full_data("c3")
     _check_boosted_round(T, val, rp, col, y, 20000, objective="reg:linear", depth=6, max_num_bin=255)
+
+
+def test_full_size_oracle_config3_wide(T):
+    """500k x 2000, depth 6 against the oracle at the full shape (blocks of 64 features, 510 000 bins): two trees."""
+    val, rp, col, y = _full_data("c3")
+    kw = dict(objective="reg:linear", depth=6, max_num_bin=255, learning_rate=0.3, n_trees=2)
+    s = T.Session(val, rp, col, y, **kw)
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    _, crp, _ = s.cuts()
+    assert np.array_equal(s.cuts()[0].view(np.uint32), o.cuts()[0].view(np.uint32)) and np.array_equal(crp, o.cuts()[1])
+    stored = _Stored(rp, col, s.F)
+    margins = P.Margins("full_size/config3")
+    ties = _oracle_tree_at_full_size(T, s, o, 0, crp, 0.3, margins, stored)
+    ties += _oracle_tree_at_full_size(T, s, o, 1, crp, 0.3, margins, stored)
+    margins.ties = ties
+    margins.report()
+    assert ties <= 1
+    s.close()
+    _FULL.clear()
 
 
 def test_full_size_properties_config4_sparse(T):
     """2 M x 100k CSR with Zipf-distributed feature ids: sparse layout with the LDS head."""
-    val, rp, col, y = D.config4()
+    val, rp, col, y = _full_data("c4")
     _check_boosted_round(T, val, rp, col, y, 100000, objective="binary:logistic", depth=8, max_num_bin=63)
+
+
+def test_full_size_oracle_config4_sparse(T):
+    """2 M x 100k CSR, depth 8, 63 bins against the oracle at the full shape (6.3 M cut points: the oracle keeps the
+    reference's histogram of all of them per node): the first tree of the level pass - 981 frequent features through
+    tables and byte columns, 99 k rare ones through the sorted pass."""
+    val, rp, col, y = _full_data("c4")
+    kw = dict(objective="binary:logistic", depth=8, max_num_bin=63, learning_rate=0.3, n_trees=1)
+    s = T.Session(val, rp, col, y, **kw)
+    assert s.info("sparse_pass") == 1
+    o = O.Oracle(val, rp, col, y, **kw).prepare()
+    _, crp, _ = s.cuts()
+    assert np.array_equal(s.cuts()[0].view(np.uint32), o.cuts()[0].view(np.uint32)) and np.array_equal(crp, o.cuts()[1])
+    assert np.array_equal(s.global_bin_ids(rp, col)[0], o.bin_ids())
+    stored = _Stored(rp, col, s.F)
+    margins = P.Margins("full_size/config4")
+    ties = _oracle_tree_at_full_size(T, s, o, 0, crp, 0.3, margins, stored)
+    margins.ties = ties
+    margins.report()
+    assert ties <= 1
+    s.close()
+    _FULL.clear()
 
 
 def test_estimator_cross_validation(T):

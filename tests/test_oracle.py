@@ -677,3 +677,43 @@ def test_bagging_scales_gradients_by_draw_counts():
     counts = np.bincount(O.bagging_draws(seed, 500), minlength=500)
     assert counts.sum() == 500 and counts.max() > 1 and (counts == 0).sum() > 100  # a bootstrap sample
     assert np.array_equal(o.gh(), plain * counts[:, None].astype(np.float32))
+
+
+def test_probes_equal_the_full_debug_arrays():
+    """Oracle.set_probes records, per node, the gain of one named candidate, the node's best gain and the direction
+    gaps of both: the same numbers as the [n_nodes, n_bins] debug arrays hold, and the tree is the same."""
+    import parity as P
+    X, y = D.config1(3000, 8, 0)
+    X[np.random.default_rng(1).random(X.shape) < 0.2] = 0  # missing values: direction gaps that are not round-off
+    val, rp, col = D.dense_to_csr(X)
+    o = O.Oracle(val, rp, col, y, depth=5, n_trees=2, debug=True).prepare()
+    o.compute_gradient()
+    o.build_tree(0)
+    nodes, sc, gaps, crp = o.nodes().copy(), o.tree_scores(), o.tree_dir_gaps(), o.cuts()[1]
+    rng = np.random.default_rng(0)
+    probe = P.probes_for(nodes, crp)
+    assert np.all(probe[(nodes["is_valid"] == 1) & (nodes["split_fid"] >= 0)] >= 0)
+    for x in range(0, len(probe), 3):  # some probes on other candidates than the chosen one
+        if probe[x] >= 0:
+            probe[x] = int(rng.integers(0, o.n_bins))
+    o2 = O.Oracle(val, rp, col, y, depth=5, n_trees=2).prepare()
+    o2.set_probes(probe)
+    o2.compute_gradient()
+    o2.build_tree(0)
+    _, out = o2.probes()
+    assert np.array_equal(o2.nodes(), nodes)
+    checked = 0
+    for x in np.flatnonzero(nodes["is_valid"] == 1):
+        if nodes[x]["lch"] < 0:
+            continue  # the deepest level is never evaluated
+        assert out[x]["best"] == np.abs(sc[x]).max()
+        if probe[x] >= 0:
+            assert out[x]["score"] == sc[x][probe[x]] and out[x]["dir_gap"] == gaps[x][probe[x]]
+            checked += 1
+        if nodes[x]["split_fid"] >= 0:
+            assert out[x]["best_dir_gap"] == gaps[x][crp[nodes[x]["split_fid"]] + nodes[x]["split_bid"]]
+    assert checked > 10
+    view = P.ProbeScores(probe, out)
+    full = P.FullScores(sc, gaps)
+    x = int(np.flatnonzero(probe >= 0)[0])
+    assert view.best(x) == full.best(x) and view.of(x, probe[x]) == full.of(x, probe[x])

@@ -44,6 +44,7 @@ SIGNATURES = {
     "tgbm_trainer_set": (None, [_P, C.c_char_p, _P, C.c_size_t]),
     "tgbm_trainer_set_profiling": (None, [_P, C.c_int]),
     "tgbm_trainer_get_profile": (None, [_P, _P]),
+    "tgbm_trainer_get_phase_profile": (C.c_int, [_P, _P, C.c_int]),
     "tgbm_trainer_export_model": (_P, [_P]),
     "tgbm_predict_raw": (None, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, _P]),
     "tgbm_predict_raw_noalloc": (C.c_int, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, _P]),

@@ -306,6 +306,17 @@ void tgbm_trainer_get_profile(tgbm_trainer *t, double *out4) {
     out4[2] = (double)p.rows_built;
     out4[3] = (double)p.hist_bytes;
 }
+int tgbm_trainer_get_phase_profile(tgbm_trainer *t, double *out, int cap) {
+    HistProfile p = t->impl->profile();
+    const double v[] = {(double)p.rounds,
+                        p.phase_ms[PH_GRADIENT], p.phase_ms[PH_HIST], p.phase_ms[PH_MERGE], p.phase_ms[PH_SPLIT],
+                        p.phase_ms[PH_PARTITION], p.phase_ms[PH_TREE_END], p.phase_ms[PH_METRIC], p.phase_ms[PH_REORDER],
+                        p.root_ms, (double)p.root_launches, (double)p.root_bytes,
+                        p.below_ms, (double)p.below_launches, (double)p.below_bytes};
+    const int n = (int)(sizeof(v) / sizeof(v[0]));
+    for (int i = 0; i < n && i < cap; ++i) out[i] = v[i];
+    return n;
+}
 tgbm_model *tgbm_trainer_export_model(tgbm_trainer *t) { return from_nested(t->impl->model_to_host()); }
 
 void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const int *col_ptr, tgbm_model *model,

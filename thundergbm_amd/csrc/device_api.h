@@ -357,6 +357,7 @@ void launch_hist_merge(hipStream_t s, const TreeBuffers &tb, int level, int n_cl
 void launch_root_sum(hipStream_t s, const TreeBuffers &tb, const GHPair *gh_class, float lambda, int n_class = 1);
 // Number of bytes equal to `value` among n bytes in device memory (synchronises).
 long device_count_bytes(hipStream_t s, const uint8_t *d_v, size_t n, uint8_t value);
+long device_count_u16(hipStream_t s, const uint16_t *d_v, size_t n, uint16_t value);
 void launch_hist_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, const GHPair *gh, int level,
                      int n_class = 1);
 void launch_partition_csr(hipStream_t s, const TreeBuffers &tb, const CsrBins &bins, int level, int n_class = 1);

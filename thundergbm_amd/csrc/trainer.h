@@ -13,11 +13,31 @@
 
 namespace tgbm {
 
+// Stages of a boosting round that the profiling switch times with HIP events on the trainer's stream (the
+// reference accumulates host timers for histogram, evaluation and data partitioning under its `profiling` switch,
+// hist_tree_builder_single.cu:19-27, :196-219, :392, :400-418).
+enum Phase {
+    PH_GRADIENT = 0,  // gradients, column sampling, tree initialisation
+    PH_HIST,          // histogram build of a level
+    PH_MERGE,         // sum of the work items' histograms, sibling = parent - built, exact root sums
+    PH_SPLIT,         // split search and tree update of a level
+    PH_PARTITION,     // row -> child decision and the next level's row lists
+    PH_TREE_END,      // pruning, prediction update (with metric and next gradients where fused), model copy
+    PH_METRIC,        // training metric when it is a pass of its own
+    PH_REORDER,       // physical re-ordering of the rows
+    PH_COUNT
+};
+
 struct HistProfile {
     double hist_ms = 0;          // summed duration of the histogram-build launches
     long long hist_launches = 0;
     long long rows_built = 0;    // rows visited by those launches
     long long hist_bytes = 0;    // algorithmic bytes of those launches
+    double phase_ms[PH_COUNT] = {0};
+    // the histogram launches of the root level and of the levels below it
+    double root_ms = 0, below_ms = 0;
+    long long root_launches = 0, below_launches = 0, root_bytes = 0, below_bytes = 0;
+    long long rounds = 0;
 };
 
 class Trainer {
@@ -130,12 +150,15 @@ class Trainer {
     bool next_round_ready_ = false;  // d_gh_ and the root statistics already belong to the next round
     // profiling
     bool profiling_ = false;
-    struct HistEvent {
-        hipEvent_t start, stop;
+    // a mark closes the stage that ran since the previous mark
+    struct PhaseMark {
+        hipEvent_t ev;
+        int phase;  // -1: start of a timed span (nothing is attributed to the interval before it)
         int level;
-        int tree;
     };
-    std::vector<HistEvent> events_;
+    std::vector<PhaseMark> marks_;
+    long long prof_rounds_ = 0;
+    void mark(int phase, int level = -1);
     std::vector<LevelCtl> ctl_log_;  // per tree, depth + 1 entries (copied at tree end when profiling)
     HistProfile prof_;
 };

@@ -563,9 +563,13 @@ void Trainer::alloc_tree_buffers() {
                 for (int g = f + 1; g < F_ && h_feat_col_[g] == c; ++g) alone = alone && cuts_.feature_nnz[g] == 0;
                 if (!alone) continue;
             }
-            if (cuts_.feature_nnz[f] == (long)n_ && bins_.bin_bytes == 1 &&
-                device_count_bytes(stream_, bins_.col + (size_t)c * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin) == 0)
-                tb.complete_feature = f;
+            if (cuts_.feature_nnz[f] != (long)n_) continue;
+            const long absent =
+                bins_.bin_bytes == 1
+                    ? device_count_bytes(stream_, bins_.col + (size_t)c * bins_.col_stride, (size_t)n_, (uint8_t)kMissingBin)
+                    : device_count_u16(stream_, reinterpret_cast<const uint16_t *>(bins_.col) + (size_t)c * bins_.col_stride,
+                                       (size_t)n_, (uint16_t)kMissingBin16);
+            if (absent == 0) tb.complete_feature = f;
         }
     }
     tb.hpair_begin = dalloc<int>(S * ((size_t)max_level_nodes + 1));
@@ -678,16 +682,23 @@ void Trainer::alloc_tree_buffers() {
 
 Trainer::~Trainer() {
     if (stream_) (void)hipStreamSynchronize(stream_);
-    for (auto &ev : events_) {
-        (void)hipEventDestroy(ev.start);
-        (void)hipEventDestroy(ev.stop);
-    }
+    for (auto &m : marks_) (void)hipEventDestroy(m.ev);
     reorder_sorter_.release();
     for (void *p : allocs_) (void)hipFree(p);
     if (stream_) (void)hipStreamDestroy(stream_);
 }
 
 void Trainer::sync() { HIP_CHECK(hipStreamSynchronize(stream_)); }
+
+void Trainer::mark(int phase, int level) {
+    if (!profiling_) return;
+    PhaseMark m;
+    HIP_CHECK(hipEventCreate(&m.ev));
+    m.phase = phase;
+    m.level = level;
+    HIP_CHECK(hipEventRecord(m.ev, stream_));
+    marks_.push_back(m);
+}
 
 // The first two steps of Booster::boost (include/thundergbm/booster.h:80-84): the objective's gradients, then
 // bagging when it is switched on.
@@ -924,6 +935,7 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
         // the level has more nodes than the histogram arena: batches of hist_nodes nodes, each through the whole
         // chain histogram -> merge -> split search -> update before the next one overwrites the arena
         const int nl = 1 << level;
+        mark(level == 0 ? PH_GRADIENT : PH_PARTITION, level);
         for (int x0 = 0; x0 < nl; x0 += tb.hist_nodes) {
             TreeBuffers tbb = tb;
             tbb.lvl_x0 = x0;
@@ -932,31 +944,25 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
             longlong2 *&cur = (level & 1) ? tbb.hist_q[1] : tbb.hist_q[0];
             cur -= (size_t)x0 * n_bins_;
             build_level_hist(tbb, level, gh, n_class);
+            mark(PH_HIST, level);
             if (!sparse_) launch_hist_merge(stream_, tbb, level, n_class);
+            mark(PH_MERGE, level);
             if (wide_eval_) launch_eval_split_wide(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
             else launch_eval_split(stream_, tbb, level, param_.min_child_weight, param_.lambda, n_class, false);
             launch_best_update(stream_, tbb, level, param_.rt_eps, param_.lambda, n_class);
+            mark(PH_SPLIT, level);
         }
         lookup_level_ = level;
         HIP_CHECK_LAUNCHES("find_split");
         return;
     }
-    if (profiling_) {
-        HistEvent ev;
-        HIP_CHECK(hipEventCreate(&ev.start));
-        HIP_CHECK(hipEventCreate(&ev.stop));
-        ev.level = level;
-        ev.tree = trees_built_;
-        HIP_CHECK(hipEventRecord(ev.start, stream_));
-        build_level_hist(tb, level, gh, n_class);
-        HIP_CHECK(hipEventRecord(ev.stop, stream_));
-        events_.push_back(ev);
-    } else {
-        build_level_hist(tb, level, gh, n_class);
-    }
+    mark(level == 0 ? PH_GRADIENT : PH_PARTITION, level);  // closes what ran before this level's histogram
+    build_level_hist(tb, level, gh, n_class);
+    mark(PH_HIST, level);
     if (!sparse_pass_) {
         if (!sparse_) launch_hist_merge(stream_, tb, level, n_class);
         if (level == 0) launch_root_sum(stream_, tb, gh, param_.lambda, n_class);
+        mark(PH_MERGE, level);
         // inside boost() nobody looks at the last level's derived histograms (the stage-wise API keeps them); the
         // last level that fits a capped arena keeps them for the batches of the next one
         if (wide_eval_)
@@ -967,6 +973,7 @@ void Trainer::find_split_sets(const TreeBuffers &tb, const GHPair *gh, int level
                               !(in_boost_ && level == param_.depth - 1));
     }
     launch_best_update(stream_, tb, level, param_.rt_eps, param_.lambda, n_class);
+    mark(PH_SPLIT, level);
     lookup_level_ = level;  // until partition(level) moves the rows into the children's lists
     HIP_CHECK_LAUNCHES("find_split");
 }
@@ -994,6 +1001,7 @@ void Trainer::partition_sets(const TreeBuffers &tb, int level, int n_class) {
         launch_partition_csr(stream_, tb, csr_, level, n_class);
     else
         launch_partition_dense(stream_, tb, bins_, level, n_class);
+    mark(PH_PARTITION, level);
     HIP_CHECK_LAUNCHES("partition");
 }
 
@@ -1034,6 +1042,7 @@ void Trainer::finish_tree(int k, bool fuse_round_end) {
     TGBM_CHECK(trees_built_ < model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
                              sizeof(TreeNode) * (size_t)tb.n_nodes, hipMemcpyDeviceToDevice, stream_));
+    mark(PH_TREE_END);
     if (profiling_) log_plan(tb);
     ++trees_built_;
     HIP_CHECK_LAUNCHES("finish_tree");
@@ -1057,6 +1066,7 @@ void Trainer::build_round_together() {
     TGBM_CHECK(trees_built_ + K <= model_cap_trees_, "more trees built than n_trees * tree_per_rounds");
     HIP_CHECK(hipMemcpyAsync(d_model_ + (size_t)trees_built_ * tb.n_nodes, tb.nodes,
                              sizeof(TreeNode) * (size_t)tb.n_nodes * K, hipMemcpyDeviceToDevice, stream_));
+    mark(PH_TREE_END);
     if (profiling_)
         for (int k = 0; k < K; ++k) log_plan(tb.for_class(k));
     trees_built_ += K;
@@ -1089,6 +1099,8 @@ void Trainer::boost(int rounds) {
         // (with bagging the next round's gradients are not the plain ones the fused pass would compute)
         const bool fuse = (objective_ == OBJ_SQUARE || objective_ == OBJ_LOGISTIC) && param_.tree_per_rounds == 1 &&
                           !param_.bagging;
+        mark(-1);  // a round's first interval starts here (log_plan of the previous round waited for the device)
+        if (profiling_) ++prof_rounds_;
         // the reference's order of the draws from rand(): gradients (ranking partner seed), bagging seed
         // (booster.h:80-84), then the column shuffle at the start of build_approximate (tree_builder.cu:150-152)
         if (!next_round_ready_) compute_gradient();
@@ -1109,7 +1121,11 @@ void Trainer::boost(int rounds) {
             }
         }
         float *slot = d_metric_ + rounds_done_;
-        if (!fuse) run_metric(slot);
+        if (!fuse) {
+            mark(-1);
+            run_metric(slot);
+            mark(PH_METRIC);
+        }
         if (g_verbose >= 1) {
             float v = 0;
             HIP_CHECK(hipMemcpyAsync(&v, slot, sizeof(float), hipMemcpyDeviceToHost, stream_));
@@ -1124,8 +1140,11 @@ void Trainer::boost(int rounds) {
         if (reorder_allowed() &&
             ((always != nullptr && std::string(always) == "always") ||
              (rounds_done_ >= reorder_first_ && rounds_done_ < reorder_first_ + reorder_burst_) ||
-             (reorder_every_ > 0 && rounds_done_ > reorder_first_ && (rounds_done_ - reorder_first_) % reorder_every_ == 0)))
+             (reorder_every_ > 0 && rounds_done_ > reorder_first_ && (rounds_done_ - reorder_first_) % reorder_every_ == 0))) {
+            mark(-1);
             reorder_rows();
+            mark(PH_REORDER);
+        }
         HIP_CHECK_LAUNCHES("boost");
     }
     in_boost_ = false;
@@ -1236,12 +1255,23 @@ void Trainer::set_profiling(bool on) {
 HistProfile Trainer::profile() {
     sync();
     HistProfile p;
-    const int W = bins_.W;
-    for (size_t i = 0; i < events_.size(); ++i) {
+    p.rounds = prof_rounds_;
+    for (size_t i = 1; i < marks_.size(); ++i) {
+        if (marks_[i].phase < 0) continue;
         float ms = 0;
-        HIP_CHECK(hipEventElapsedTime(&ms, events_[i].start, events_[i].stop));
-        p.hist_ms += ms;
-        p.hist_launches++;
+        HIP_CHECK(hipEventElapsedTime(&ms, marks_[i - 1].ev, marks_[i].ev));
+        p.phase_ms[marks_[i].phase] += ms;
+        if (marks_[i].phase == PH_HIST) {
+            p.hist_ms += ms;
+            p.hist_launches++;
+            if (marks_[i].level == 0) {
+                p.root_ms += ms;
+                p.root_launches++;
+            } else {
+                p.below_ms += ms;
+                p.below_launches++;
+            }
+        }
     }
     // algorithmic bytes: every visited row reads its bin bytes (one per feature), its gradient pair
     // and, below the root, its row index; every launch writes the level's built histograms once.
@@ -1250,13 +1280,15 @@ HistProfile Trainer::profile() {
         for (int level = 0; level < param_.depth; ++level) {
             const LevelCtl &c = ctl_log_[t * per_tree + level];
             p.rows_built += c.rows_built;
+            long long b;
             if (sparse_)  // CSR: 4-byte bin id per stored value + row pointer, gradient pair and row index per row
-                p.hist_bytes += (long long)((double)c.rows_built * ((double)nnz_ / n_ * 4 + 8 + 8 + (level > 0 ? 4 : 0)));
+                b = (long long)((double)c.rows_built * ((double)nnz_ / n_ * 4 + 8 + 8 + (level > 0 ? 4 : 0)));
             else
-                p.hist_bytes += (long long)c.rows_built * (F_ * bins_.bin_bytes + 8 + (level > 0 ? 4 : 0));
+                b = (long long)c.rows_built * (F_ * bins_.bin_bytes + 8 + (level > 0 ? 4 : 0));
+            p.hist_bytes += b;
+            (level == 0 ? p.root_bytes : p.below_bytes) += b;
         }
     }
-    (void)W;
     return p;
 }
 
@@ -1395,11 +1427,24 @@ std::vector<std::vector<Tree>> train(GBMParam &param, const DataSet &dataset) {
                param.tree_method.c_str());
     if (param.n_device != 1) log_info("n_gpus=%d requested; this build trains on one GPU", param.n_device);
     Trainer trainer(dataset, param);
+    // `profiling` (thundergbm_train.cpp:28-30 switches the reference's performance tracking on with it): per-stage
+    // timers around every launch group of the boosting loop, reported after the run
+    if (param.profiling) trainer.set_profiling(true);
     auto start = std::chrono::high_resolution_clock::now();
     trainer.boost(param.n_trees);
     trainer.sync();
     auto stop = std::chrono::high_resolution_clock::now();
     log_info("training time = %g", std::chrono::duration<float>(stop - start).count());
+    if (param.profiling) {
+        const HistProfile p = trainer.profile();
+        static const char *names[PH_COUNT] = {"gradients and tree init", "build hist", "merge and subtract",
+                                              "evaluate and update tree", "data partitioning", "end of tree",
+                                              "metric", "row re-ordering"};
+        for (int i = 0; i < PH_COUNT; ++i) log_info("profiling: %-26s %10.3f ms", names[i], p.phase_ms[i]);
+        log_info("profiling: histogram launches: root %lld x %.1f us, below the root %lld x %.1f us", p.root_launches,
+                 p.root_launches ? p.root_ms * 1e3 / p.root_launches : 0.0, p.below_launches,
+                 p.below_launches ? p.below_ms * 1e3 / p.below_launches : 0.0);
+    }
     std::vector<std::vector<Tree>> model = trainer.model_to_host();
     log_debug("model to host: %.3f s",
               std::chrono::duration<double>(std::chrono::high_resolution_clock::now() - stop).count());

@@ -733,6 +733,14 @@ __global__ __launch_bounds__(kBlock) void k_count_bytes(const uint8_t *__restric
     if (lane_id() == 0 && c) atomicAdd(out, c);
 }
 
+__global__ __launch_bounds__(kBlock) void k_count_u16(const uint16_t *__restrict__ v, size_t n, uint16_t value,
+                                                     unsigned long long *__restrict__ out) {
+    unsigned long long c = 0;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (size_t)gridDim.x * kBlock) c += v[i] == value;
+    c = (unsigned long long)wave_sum_ll((long long)c);
+    if (lane_id() == 0 && c) atomicAdd(out, c);
+}
+
 // --------------------------------------------------------------------------- sparse histogram
 // CSR rows of global bin ids: the histogram is too large for LDS (one slot per cut point of every
 // feature), so every stored value adds its row's fixed-point gradient pair to the node's histogram
@@ -2339,6 +2347,17 @@ long device_count_bytes(hipStream_t s, const uint8_t *d_v, size_t n, uint8_t val
     HIP_CHECK(hipMalloc(&d_out, sizeof(unsigned long long)));
     HIP_CHECK(hipMemsetAsync(d_out, 0, sizeof(unsigned long long), s));
     k_count_bytes<<<grid_for(n, 2048), kBlock, 0, s>>>(d_v, n, value, d_out);
+    HIP_CHECK(hipMemcpyAsync(&h, d_out, sizeof(h), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipFree(d_out));
+    return (long)h;
+}
+
+long device_count_u16(hipStream_t s, const uint16_t *d_v, size_t n, uint16_t value) {
+    unsigned long long *d_out = nullptr, h = 0;
+    HIP_CHECK(hipMalloc(&d_out, sizeof(unsigned long long)));
+    HIP_CHECK(hipMemsetAsync(d_out, 0, sizeof(unsigned long long), s));
+    k_count_u16<<<grid_for(n, 2048), kBlock, 0, s>>>(d_v, n, value, d_out);
     HIP_CHECK(hipMemcpyAsync(&h, d_out, sizeof(h), hipMemcpyDeviceToHost, s));
     HIP_CHECK(hipStreamSynchronize(s));
     HIP_CHECK(hipFree(d_out));

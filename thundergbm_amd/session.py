@@ -193,5 +193,18 @@ class Session:
         self.L.tgbm_trainer_get_profile(self.h, _p(out))
         return {"hist_ms": out[0], "launches": int(out[1]), "rows_built": int(out[2]), "bytes": int(out[3])}
 
+    PHASES = ("gradient_tree_init", "hist", "merge_subtract", "split_update", "partition", "tree_end", "metric", "reorder")
+
+    def phase_profile(self):
+        """Per-stage milliseconds of the rounds boosted with profiling on, and the histogram launches split into the
+        root level and the levels below it."""
+        out = np.zeros(15, dtype=np.float64)
+        self.L.tgbm_trainer_get_phase_profile(self.h, _p(out), 15)
+        split = {}
+        for i, name in enumerate(("root", "below_root")):
+            ms, launches, nbytes = out[9 + 3 * i:12 + 3 * i]
+            split[name] = {"ms": float(ms), "launches": int(launches), "bytes": int(nbytes)}
+        return {"rounds": int(out[0]), "phase_ms": {k: float(v) for k, v in zip(self.PHASES, out[1:9])}, "hist": split}
+
     def export_model(self):
         return self.L.tgbm_trainer_export_model(self.h)
