@@ -31,10 +31,10 @@ def item_shift(qmax, rows, bits):
     return int(np.floor(np.log2(qmax / lim))) + 1
 
 
-def node_quantum(quant, node_rows, sparse, flush_rows=8192):
+def node_quantum(quant, node_rows, sparse, flush_rows=32768):
     """Coarsest (g, h) step at which a row of a node with node_rows rows is counted. The library sums
     round(g * scale) as exact 64-bit integers; a dense work item coarsens the tree's scale by a power of two
-    that depends on the rows it adds between two drains of its packed LDS bins (at most min(node rows, 8192)).
+    that depends on the rows it adds between two drains of its packed LDS bins (at most min(node rows, 32768)).
     Every histogram built from rows is therefore exact up to half a step per stored entry."""
     qg, qh = float(quant["inv_g"]), float(quant["inv_h"])
     if sparse:

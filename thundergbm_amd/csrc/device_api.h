@@ -57,8 +57,8 @@ struct LevelCtl {
 // depend on the order of the rows;
 // k_hist_merge shifts every item's sums back to the tree's scale. h_bits: 32 in general; when every hessian of the
 // tree is a small non-negative integer (squared loss: 1, or the draw count under bagging) the hessian field gets
-// exactly the bits that kHistFlushRows * max h needs and the gradient field the rest (50 bits for h = 1), which
-// is what keeps heavy-tailed regression residuals at float-like resolution (2^-36 of the largest |g| per row).
+// exactly the bits that kHistFlushRows * max h needs and the gradient field the rest (47 bits for h = 1), which
+// is what keeps heavy-tailed regression residuals at float-like resolution (2^-32 of the largest |g| per row).
 // All sums after the LDS stage are 64-bit integers: exact, order-independent, bit-reproducible.
 struct QuantCtl {
     float scale_g, scale_h;  // value -> integer of the tree's histograms (powers of two)

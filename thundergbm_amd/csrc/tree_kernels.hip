@@ -14,7 +14,10 @@ constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / 64;
 constexpr int kHistMinChunk = 1024;
 constexpr int kHistBlock = 1024;      // threads per histogram workgroup (they share one LDS histogram)
-constexpr int kHistFlushRows = 8192;  // rows a packed 32+32-bit LDS bin may absorb before it is drained
+// Rows a packed 32+32-bit LDS bin may absorb before it is drained. 32768: the 512 root items of 10 M rows (19 712 rows
+// each) are never drained and leave as 8-byte packed words; a row of a node that large is counted at 2^-15 of the
+// tree's largest |g| (float hessians), fine against the 1e-5 bound on sums of tens of thousands of rows.
+constexpr int kHistFlushRows = 32768;
 
 // Exclusive scan of one int per thread over a 256-thread block; lds needs kWaves ints.
 __device__ int block_excl_scan(int v, int *lds, int *total) {
@@ -1501,13 +1504,29 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
 // Scan the per-item left counts, publish the children's row segments and plan the histogram work
 // of the next level: per sibling pair the child with fewer rows is built (ties: the left one, as
 // hist_tree_builder_single.cu:466-467), the other one comes from subtraction. One workgroup.
+constexpr int kScanLdsItems = 12 * 1024;  // item offsets that k_part_scan_plan keeps in LDS (25 M rows)
 __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, int level) {
     const TreeBuffers tb = tb_all.for_class(blockIdx.z);
     __shared__ int lds[kWaves];
+    __shared__ int s_loff[kScanLdsItems + 1];
     const int nl = 1 << level, off = nl - 1;
     const int n_p = tb.ctl[level].n_pitems;
     const int *pb_cur = tb.pbegin(level);
     int *pb_next = tb.pbegin(level + 1);
+    // the offsets of the items also stay in LDS when they fit, so that the per-node step below does not wait for
+    // its own global stores
+    const bool in_lds = n_p <= kScanLdsItems;
+    // (what the per-node step needs from global memory is requested here, next to the item counts: one round trip)
+    TreeNode my_node{};
+    int2 my_seg = make_int2(0, 0);
+    int my_pb0 = 0, my_pb1 = 0;
+    const bool fast = nl <= kBlock && !tb.singles(level + 1) && (int)threadIdx.x < nl;
+    if (fast) {
+        my_node = tb.nodes[off + threadIdx.x];
+        my_seg = tb.seg[off + threadIdx.x];
+        my_pb0 = pb_cur[threadIdx.x];
+        my_pb1 = pb_cur[threadIdx.x + 1];
+    }
     int carry = 0;
     constexpr int IPT = 20;  // items per thread and step (10 M rows are 4 883 items: one step)
     for (int base = 0; base < n_p; base += kBlock * IPT) {
@@ -1523,12 +1542,18 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         int run = carry + block_excl_scan(local, lds, &tot);
 #pragma unroll
         for (int j = 0; j < IPT; ++j) {
-            if (i0 + j < n_p) tb.pitem_loff[i0 + j] = run;
+            if (i0 + j < n_p) {
+                tb.pitem_loff[i0 + j] = run;
+                if (in_lds) s_loff[i0 + j] = run;
+            }
             run += v[j];
         }
         carry += tot;
     }
-    if (threadIdx.x == 0) tb.pitem_loff[n_p] = carry;
+    if (threadIdx.x == 0) {
+        tb.pitem_loff[n_p] = carry;
+        if (in_lds) s_loff[n_p] = carry;
+    }
     __syncthreads();
     if (tb.singles(level + 1)) {
         // No parent histograms below this level (the arena is smaller than the level): every child of a split node
@@ -1596,10 +1621,10 @@ __global__ __launch_bounds__(kBlock) void k_part_scan_plan(TreeBuffers tb_all, i
         int built = -1, rows = 0;
         int pl = 0, pr = 0;  // partition items of the two children
         if (x_in < nl) {
-            const TreeNode &nd = tb.nodes[off + x_in];
-            const int2 sg = tb.seg[off + x_in];
+            const TreeNode &nd = my_node;
+            const int2 sg = my_seg;
             if (node_splits(nd)) {
-                const int nleft = tb.pitem_loff[pb_cur[x_in + 1]] - tb.pitem_loff[pb_cur[x_in]];
+                const int nleft = in_lds ? s_loff[my_pb1] - s_loff[my_pb0] : tb.pitem_loff[my_pb1] - tb.pitem_loff[my_pb0];
                 const int nright = (sg.y - sg.x) - nleft;
                 tb.node_nleft[x_in] = nleft;
                 tb.seg[nd.lch_index] = make_int2(sg.x, sg.x + nleft);
@@ -1967,6 +1992,62 @@ __global__ __launch_bounds__(kBlock) void k_end_bounds(TreeBuffers tb_all, int l
     }
 }
 
+// The row-ordered part of the end of a tree: s_leaf holds the node of every row of the block.
+template <int MODE>
+__device__ __forceinline__ void tree_end_rows(const TreeBuffers &tb, const TreeEndArgs &a, const short *s_leaf, int r0, int r1) {
+    __shared__ float s_f[kStatsLds];
+    __shared__ double s_d[kWaves];
+    constexpr int U = 4;
+    if (MODE == 0) {
+        for (int i = r0 + threadIdx.x; i < r1; i += kBlock) {
+            const int x = s_leaf[i - r0];
+            if (x >= 0) tb.nid[i] = x;
+        }
+        return;
+    }
+    // rows in order; thread t takes rows t, t + kBlock, ... (the order every row-blocked reduction uses)
+    const float *__restrict__ y = a.y;
+    float *__restrict__ yp = a.yp;
+    GHPair *__restrict__ gh = a.gh;
+    const float *__restrict__ leaf_value = tb.leaf_value;
+    RowStats st;
+    double acc = 0;
+    float accf = 0;
+    for (int i0 = r0 + threadIdx.x; i0 < r1; i0 += kBlock * U) {
+        float p[U], w[U], yi[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * kBlock;
+            ok[u] = i < r1;
+            const int x = ok[u] ? s_leaf[i - r0] : -1;
+            p[u] = ok[u] ? yp[i] : 0.f;
+            yi[u] = (MODE == 2 && ok[u]) ? y[i] : 0.f;
+            w[u] = x >= 0 ? leaf_value[x] : 0.f;
+            ok[u] = ok[u] && (MODE == 2 || x >= 0);
+            if (x >= 0) p[u] += a.lr * w[u];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (!ok[u]) continue;
+            const int i = i0 + u * kBlock;
+            yp[i] = p[u];
+            if (MODE == 2) {
+                metric_row(a.metric_kind, tb.n, 1, i, yi[u], yp, p[u], acc, accf);
+                const GHPair o = pointwise_gradient(a.objective, yi[u], p[u]);
+                gh[i] = o;
+                st.add(o);
+            }
+        }
+    }
+    if (MODE == 2) {
+        store_block_stats(st, s_f, a.stats + blockIdx.x);
+        acc += (double)accf;
+        store_block_sum_d(acc, s_d, a.metric_partial + blockIdx.x);
+    }
+}
+
+
 template <int MODE, bool SPARSE>
 __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBins dbins, CsrBins cbins, TreeEndArgs a) {
     __shared__ short s_leaf[kRowBlock];  // node of every row of the block (depth <= 14: ids below 2^15), -1: none
@@ -1977,8 +2058,6 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
     __shared__ int s_off[kEndListCap];
     __shared__ int s_scan[kWaves];
     __shared__ int s_n;
-    __shared__ float s_f[kStatsLds];
-    __shared__ double s_d[kWaves];
     const int r0 = blockIdx.x * kRowBlock, r1 = min(tb.n, r0 + kRowBlock);
     constexpr int U = 4;
     if (tb.nid16 != nullptr) {
@@ -2071,53 +2150,7 @@ __global__ __launch_bounds__(kBlock) void k_tree_end(TreeBuffers tb_all, DenseBi
     }
     }  // row lists
     __syncthreads();
-    if (MODE == 0) {
-        for (int i = r0 + threadIdx.x; i < r1; i += kBlock) {
-            const int x = s_leaf[i - r0];
-            if (x >= 0) tb.nid[i] = x;
-        }
-        return;
-    }
-    // rows in order; thread t takes rows t, t + kBlock, ... (the order every row-blocked reduction uses)
-    const float *__restrict__ y = a.y;
-    float *__restrict__ yp = a.yp;
-    GHPair *__restrict__ gh = a.gh;
-    const float *__restrict__ leaf_value = tb.leaf_value;
-    RowStats st;
-    double acc = 0;
-    float accf = 0;
-    for (int i0 = r0 + threadIdx.x; i0 < r1; i0 += kBlock * U) {
-        float p[U], w[U], yi[U];
-        bool ok[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int i = i0 + u * kBlock;
-            ok[u] = i < r1;
-            const int x = ok[u] ? s_leaf[i - r0] : -1;
-            p[u] = ok[u] ? yp[i] : 0.f;
-            yi[u] = (MODE == 2 && ok[u]) ? y[i] : 0.f;
-            w[u] = x >= 0 ? leaf_value[x] : 0.f;
-            ok[u] = ok[u] && (MODE == 2 || x >= 0);
-            if (x >= 0) p[u] += a.lr * w[u];
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (!ok[u]) continue;
-            const int i = i0 + u * kBlock;
-            yp[i] = p[u];
-            if (MODE == 2) {
-                metric_row(a.metric_kind, tb.n, 1, i, yi[u], yp, p[u], acc, accf);
-                const GHPair o = pointwise_gradient(a.objective, yi[u], p[u]);
-                gh[i] = o;
-                st.add(o);
-            }
-        }
-    }
-    if (MODE == 2) {
-        store_block_stats(st, s_f, a.stats + blockIdx.x);
-        acc += (double)accf;
-        store_block_sum_d(acc, s_d, a.metric_partial + blockIdx.x);
-    }
+    tree_end_rows<MODE>(tb, a, s_leaf, r0, r1);
 }
 
 // ---------------------------------------------------------------------------------- metric
