@@ -7,7 +7,7 @@ data, cut points and the bin matrix are resident in HBM before the timed region 
 boosting call of K rounds, as in a training run, bracketed by device synchronisations. Prints one JSON line.
 
 The default workload is benchmark configuration 2 (10M x 28 dense, binary:logistic, depth 8, 255 bins), the one
-the headline metric is quoted on; --config 3, 4, 5 time the other full-size configurations the same way.
+the headline metric is quoted on; --config 1, 3, 4, 5 time the other configurations the same way.
 """
 import argparse
 import json
@@ -23,6 +23,8 @@ import numpy as np  # noqa: E402
 
 # objective, depth, bins, learning rate, trees of the configuration, histogram kernel
 CONFIGS = {
+    1: dict(objective="reg:linear", depth=6, max_num_bin=255, learning_rate=0.1, n_trees=40,
+            kernel="k_hist_dense", name="config 1: %d rows x %d dense features, reg:linear, depth %d, 255 bins"),
     2: dict(objective="binary:logistic", depth=8, max_num_bin=255, learning_rate=0.1, n_trees=100,
             kernel="k_hist_dense", name="config 2: %d rows x %d dense features, binary:logistic, depth %d, 255 bins"),
     3: dict(objective="reg:linear", depth=6, max_num_bin=255, learning_rate=0.1, n_trees=50,
@@ -38,7 +40,7 @@ KERNEL_SOURCES = ["thundergbm_amd/csrc/tree_kernels.hip", "thundergbm_amd/csrc/s
                   "thundergbm_amd/csrc/kernel_common.h", "thundergbm_amd/csrc/trainer.hip",
                   "thundergbm_amd/csrc/device_api.h"]
 # counter summary of a configuration's histogram kernels under profiles/
-PMC_SUMMARY = {2: "k_hist_dense_config2_pmc.txt", 3: "k_hist_dense_config3_pmc.txt",
+PMC_SUMMARY = {1: "none", 2: "k_hist_dense_config2_pmc.txt", 3: "k_hist_dense_config3_pmc.txt",
                4: "sparse_level_pass_config4_pmc.txt", 5: "k_hist_dense_config5_pmc.txt"}
 
 
@@ -77,7 +79,9 @@ def traffic_from_profile(config):
 
 def make_data(config, rows):
     import datasets as D
-    if config == 2:
+    if config == 1:
+        X, y = D.config1(rows or 10_000, 8, seed=0)
+    elif config == 2:
         X, y = D.config2(rows or 10_000_000, seed=1)
     elif config == 3:
         X, y = D.config3(rows or 500_000, 2000, seed=2)
@@ -89,6 +93,30 @@ def make_data(config, rows):
     n, F = X.shape
     val, rp, col = D.dense_to_csr(X)
     return val, rp, col, y, n, F
+
+
+def small_data_figures(T, torch):
+    """Milliseconds per tree on the two small workloads of the reference (its CPU-runnable configuration 1 and its
+    quick-start file): a tree there is a chain of dependent launches over a few thousand rows, so the figure is
+    launch latency, not bandwidth. One training call of 40 trees each, after a warm-up session."""
+    import datasets as D
+    out = {}
+    X, y = D.config1(10_000, 8, seed=0)
+    cases = {"config1_10000x8_depth6": (D.dense_to_csr(X), y, dict(objective="reg:linear", learning_rate=0.1)),
+             "a1a_1605x119_depth6": (None, None, dict(objective="reg:linear", learning_rate=1.0))}
+    val, rp, col, ya = D.read_libsvm(D.A1A)
+    cases["a1a_1605x119_depth6"] = ((val, rp, col), ya, cases["a1a_1605x119_depth6"][2])
+    for name, ((v, r, c), yy, kw) in cases.items():
+        for rep in range(2):  # the first session warms the code paths up
+            s = T.Session(v, r, c, yy, depth=6, n_trees=40, max_num_bin=255, verbose=0, **kw)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            s.boost(40)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            s.close()
+        out[name + "_ms_per_tree"] = round(dt / 40 * 1e3, 4)
+    return out
 
 
 def main():
@@ -190,13 +218,15 @@ def main():
         aux["iters_per_s_100_trees"] = round(cfg["n_trees"] / t_full, 2)
         aux["reorderings_in_100_trees"] = s.info("reorders_done")
         s.close()
+    if args.config == 2 and args.full_run and args.rows == 0:
+        aux["small_data"] = small_data_figures(T, torch)
     if args.calibration_copy_mb > 0:
         T.load().tgbm_calibration_copy(args.calibration_copy_mb << 20, 3)
 
     cpu = None
     if args.cpu_steps > 0:
         import oracle_lib as O
-        default_rows = {2: n, 3: 25_000, 4: 200_000, 5: 200_000}[args.config]
+        default_rows = {1: n, 2: n, 3: 25_000, 4: 200_000, 5: 200_000}[args.config]
         m = min(n, args.cpu_rows if args.cpu_rows > 0 else default_rows)
         crp = rp[: m + 1]
         nnz = int(crp[-1])

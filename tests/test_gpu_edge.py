@@ -90,6 +90,11 @@ CASES = {
     "lambda0_mcw5": (900, 6, 6, "reg:linear", "reg", dict(depth=4, max_num_bin=32, lambda_=0.0, min_child_weight=5.0),
                      None),
     "gamma_prunes_all": (600, 5, 5, "reg:linear", "reg", dict(depth=4, max_num_bin=16, gamma=1e9), None),
+    # depth 12: the sparse layout leaves its level pass (12-bit node ids) for per-node histograms in HBM
+    "sparse_depth12_per_node_path": (6000, 60, 8, "binary:logistic", "bin",
+                                     dict(depth=12, max_num_bin=16, gamma=0.0, min_child_weight=0.05), "sparse"),
+    "sparse_depth11_level_pass": (6000, 60, 8, "binary:logistic", "bin",
+                                  dict(depth=11, max_num_bin=16, gamma=0.0, min_child_weight=0.05), "sparse"),
     # A node whose chosen candidate gains 0.8363545 with the missing rows sent left and 0.8363642 with them sent right
     # (86 missing rows, fourth round, class 3, node 12): the direction is a near tie between two gains of one
     # candidate and may fall either way within the 1e-5 tolerance; found by random-shape testing.
@@ -181,6 +186,8 @@ def run_case(T, name, seed, margins=None):
     s = T.Session(val, rp, col, y, **kw)
     if layout and layout.endswith("-16"):
         assert s.info("dense_bin_bytes") == 2
+    if isinstance(name, str) and name.startswith("sparse_depth"):
+        assert s.info("sparse") == 1 and s.info("sparse_pass") == (1 if kw["depth"] <= 11 else 0)
     if layout and layout[-4:] in ("-w32", "-w64"):
         assert s.info("dense_W") == int(layout[-2:])
     o = O.Oracle(val, rp, col, y, debug=True, **kw).prepare()
@@ -902,6 +909,45 @@ def test_dense_layout_keeps_the_later_of_two_entries_with_the_same_column(T):
         assert np.array_equal(dense[:, 2], expect)
         s.close()
     os.environ.pop("TGBM_DENSE_BIN_BYTES", None)
+
+
+def test_dense_layout_with_unsorted_rows_that_repeat_a_column(T):
+    """Rows whose columns do not ascend and that store a column twice with other entries in between: the later entry
+    counts, the same bins on every run (sixteen lanes share a row of sorted data; such rows are filled by one thread
+    each, front to back)."""
+    rng = np.random.default_rng(8)
+    n, F = 3000, 9
+    vals, cols, ptr, later = [], [], [0], np.zeros((n, F), np.float32)
+    for r in range(n):
+        c = list(rng.permutation(F)[: int(rng.integers(3, F + 1))])
+        c += [c[0]] * int(rng.integers(0, 2))  # sometimes the first column once more at the end
+        v = list(np.round(rng.standard_normal(len(c)) * 2, 1).astype(np.float32) + np.float32(0.05))
+        for cc, vv in zip(c, v):
+            later[r, cc] = vv
+        cols += c
+        vals += v
+        ptr.append(len(cols))
+    val, col, rp = np.array(vals, np.float32), np.array(cols, np.int32), np.array(ptr, np.int32)
+    y = later[:, 0].copy()
+    os.environ["TGBM_LAYOUT"] = "dense"
+    mats = []
+    for nbytes in ("1", "2", "1"):
+        os.environ["TGBM_DENSE_BIN_BYTES"] = nbytes
+        s = T.Session(val, rp, col, y, objective="reg:linear", n_trees=1, depth=3, max_num_bin=32)
+        cut_val, crp, _ = s.cuts()
+        m = s.binmat()
+        dense = np.concatenate([m[b] for b in range(m.shape[0])], axis=1)[:, :F].astype(np.int64)
+        for f in range(F):
+            cf = cut_val[crp[f]:crp[f + 1]]
+            expect = np.minimum((cf[None, :] <= later[:, f][:, None]).sum(axis=1), len(cf) - 1)
+            stored = later[:, f] != 0
+            assert np.array_equal(dense[stored, f], expect[stored]), f
+            assert np.all(dense[~stored, f] == (255 if nbytes == "1" else 65535))
+        s.boost(1)
+        mats.append((dense, s.model().tobytes()))
+        s.close()
+    os.environ.pop("TGBM_DENSE_BIN_BYTES", None)
+    assert np.array_equal(mats[0][0], mats[2][0]) and mats[0][1] == mats[2][1]
 
 
 def test_dense_16_bit_bins_with_sampling_and_a_capped_arena(T):

@@ -412,7 +412,9 @@ void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
                       size_t col_stride, int bin_bytes, int F, const int *feat_col = nullptr,
-                      const uint8_t *feat_lo = nullptr);
+                      const uint8_t *feat_lo = nullptr, bool rows_ascend = true);
+// false when some row holds a column index below its predecessor's
+bool device_rows_ascend(hipStream_t s, int n, const int *row_ptr, const int *col);
 // min_next[c] (pre-filled with INT_MAX) = smallest column index that follows column c in a row (equal neighbours, a
 // column stored twice, do not count); *descending is set when a row's columns do not ascend
 void launch_min_next_col(hipStream_t s, int n, const int *row_ptr, const int *col, int *min_next, int *descending);

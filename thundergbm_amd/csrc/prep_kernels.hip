@@ -342,6 +342,39 @@ __global__ __launch_bounds__(kBlock) void k_bin_dense(int n, const int *__restri
     }
 }
 
+// The same for data with rows whose columns do not ascend (nothing the reference's wrappers produce: they sort the
+// indices of every row, thundergbm.py:103): a row may then store a column twice with other entries in between, and
+// sixteen lanes writing one cell would leave whichever bin arrived last. One thread walks its row front to back, so
+// the later entry counts, as for adjacent ones. (The reference adds both entries to the histogram and searches the
+// row's bin ids by bisection, which needs ascending columns: its own result for such rows is not defined.)
+template <typename BinT>
+__global__ __launch_bounds__(kBlock) void k_bin_dense_serial(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
+                                                            const float *__restrict__ val, const float *__restrict__ cut_val,
+                                                            const int *__restrict__ cut_row_ptr, BinT *__restrict__ binmat,
+                                                            int W, size_t block_stride) {
+    for (int i = blockIdx.x * kBlock + threadIdx.x; i < n; i += gridDim.x * kBlock) {
+        for (int e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
+            const int f = col[e];
+            const int cb = cut_row_ptr[f];
+            const int b = local_bin(cut_val + cb, cut_row_ptr[f + 1] - cb, val[e]);
+            binmat[(size_t)(f / W) * block_stride + (size_t)i * W + (f % W)] = (BinT)b;
+        }
+    }
+}
+
+// Sets *descending when a row holds a column index below its predecessor's.
+__global__ __launch_bounds__(kBlock) void k_rows_ascend(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
+                                                       int *__restrict__ descending) {
+    constexpr int kLanes = 16;
+    const int sub = threadIdx.x % kLanes;
+    bool bad = false;
+    for (int i = blockIdx.x * (kBlock / kLanes) + threadIdx.x / kLanes; i < n; i += gridDim.x * (kBlock / kLanes)) {
+        const int e1 = row_ptr[i + 1];
+        for (int e = row_ptr[i] + sub; e + 1 < e1; e += kLanes) bad |= col[e + 1] < col[e];
+    }
+    if (bad) *descending = 1;
+}
+
 // Which columns follow which inside the rows (sixteen lanes per row, as above).
 __global__ __launch_bounds__(kBlock) void k_min_next_col(int n, const int *__restrict__ row_ptr, const int *__restrict__ col,
                                                         int *__restrict__ min_next, int *__restrict__ descending) {
@@ -670,9 +703,17 @@ int sort_pairs(hipStream_t s, PairSorter &ps, long n, int key_bits) {
 
 void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, const float *val, const float *cut_val,
                       const int *cut_row_ptr, uint8_t *binmat, int W, size_t block_stride, uint8_t *colmat,
-                      size_t col_stride, int bin_bytes, int F, const int *feat_col, const uint8_t *feat_lo) {
+                      size_t col_stride, int bin_bytes, int F, const int *feat_col, const uint8_t *feat_lo,
+                      bool rows_ascend) {
     const int grid = grid_for((size_t)n * 16, 1 << 20);
-    if (bin_bytes == 2)
+    if (!rows_ascend) {  // (no bundles then: the layout is chosen with one column per feature)
+        if (bin_bytes == 2)
+            k_bin_dense_serial<uint16_t><<<grid_for((size_t)n, 1 << 20), kBlock, 0, s>>>(
+                n, row_ptr, col, val, cut_val, cut_row_ptr, reinterpret_cast<uint16_t *>(binmat), W, block_stride / 2);
+        else
+            k_bin_dense_serial<uint8_t><<<grid_for((size_t)n, 1 << 20), kBlock, 0, s>>>(n, row_ptr, col, val, cut_val,
+                                                                                      cut_row_ptr, binmat, W, block_stride);
+    } else if (bin_bytes == 2)
         k_bin_dense<uint16_t><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr,
                                                      reinterpret_cast<uint16_t *>(binmat), W, block_stride / 2, nullptr,
                                                      nullptr);
@@ -680,6 +721,18 @@ void launch_bin_dense(hipStream_t s, int n, const int *row_ptr, const int *col, 
         k_bin_dense<uint8_t><<<grid, kBlock, 0, s>>>(n, row_ptr, col, val, cut_val, cut_row_ptr, binmat, W, block_stride,
                                                     feat_col, feat_lo);
     launch_cols_from_rows(s, n, W, F, (F + W - 1) / W, binmat, block_stride, colmat, col_stride, bin_bytes);
+}
+
+bool device_rows_ascend(hipStream_t s, int n, const int *row_ptr, const int *col) {
+    if (n == 0) return true;
+    int *d_flag = nullptr, h = 0;
+    HIP_CHECK(hipMalloc(&d_flag, sizeof(int)));
+    HIP_CHECK(hipMemsetAsync(d_flag, 0, sizeof(int), s));
+    k_rows_ascend<<<grid_for((size_t)n * 16, 1 << 20), kBlock, 0, s>>>(n, row_ptr, col, d_flag);
+    HIP_CHECK(hipMemcpyAsync(&h, d_flag, sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipFree(d_flag));
+    return h == 0;
 }
 
 void launch_min_next_col(hipStream_t s, int n, const int *row_ptr, const int *col, int *min_next, int *descending) {

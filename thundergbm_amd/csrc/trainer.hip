@@ -162,7 +162,10 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
     sparse_ = (F_ > 4096 && density < 0.05) || (size_t)n_ * F_ * 2 > free_b / 2 || n_ >= (1 << 29);
     if (force != nullptr && std::string(force) == "sparse") sparse_ = true;
     if (force != nullptr && std::string(force) == "dense") sparse_ = false;
-    if (F_ >= 65536) sparse_ = true;  // the dense kernels keep feature ids in 16 bits
+    if (F_ >= 65536) {  // the dense kernels keep feature ids in 16 bits
+        if (!sparse_) log_info("%d features: sparse layout whatever the density (%.4f)", F_, density);
+        sparse_ = true;
+    }
     // More than 255 cut points in a feature (max_num_bin above 255): the dense layout then keeps 16-bit bins in narrower
     // feature blocks (their LDS histograms hold as many bins as the byte layout's), as long as one feature's bins fit
     // the LDS; the CSR layout's global bin ids have no limit at all. Either way the split search runs one workgroup
@@ -186,6 +189,15 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         sparse_pass_ = param_.depth <= 11 && nnz_ > 0 && nnz_ < (1l << 31) && !(pe != nullptr && std::string(pe) == "0") &&
                        !wide_bins_;
         wide_eval_ = wide_bins_ || (!sparse_pass_ && wide_env != nullptr && std::string(wide_env) == "1");
+        if (!sparse_pass_) {
+            // the per-node path keeps a histogram of all cut points per node in HBM (the reference's structure,
+            // hist_tree_builder_single.cu:811-832) and costs about three times the level pass per tree
+            const char *why = param_.depth > 11 ? "depth above 11 (the level pass keeps 12-bit node ids)"
+                              : wide_bins_      ? "features with more than 255 bins"
+                              : nnz_ >= (1l << 31) ? "2^31 stored values or more"
+                                                  : "switched off";
+            log_info("sparse layout: per-node histograms instead of the level pass: %s", why);
+        }
         if (wide_bins_)
             log_info("features with up to %d bins: CSR layout, split search per (feature, node)", max_feature_bins);
         int *d_bin = dalloc<int>((size_t)std::max(nnz_, 1l));
@@ -307,6 +319,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         // a row), so the smallest successor of every column decides: one pass over the column indices.
         h_col_bin_begin_ = h_cut_row_ptr_;
         int P = F_;  // columns of the matrix
+        bool rows_ascend = true;
+        bool ascend_known = false;
         std::vector<int> h_feat_col;
         std::vector<uint8_t> h_feat_lo;
         const char *be = std::getenv("TGBM_BUNDLE");  // "0": one column per feature (tests, measurements)
@@ -321,6 +335,8 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
             HIP_CHECK(hipMemcpyAsync(next.data(), d_next, sizeof(int) * next.size(), hipMemcpyDeviceToHost, stream_));
             HIP_CHECK(hipStreamSynchronize(stream_));
             HIP_CHECK(hipFree(d_next));
+            rows_ascend = next[F_] == 0;
+            ascend_known = true;
             if (next[F_] == 0) {  // (rows whose columns do not ascend: the argument above does not hold)
                 std::vector<int> col_of(F_), begin;
                 std::vector<uint8_t> lo(F_);
@@ -412,8 +428,11 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         const size_t col_stride = ((size_t)n_ + 3) / 4 * 4;
         uint8_t *d_colmat = dalloc<uint8_t>(col_stride * P * bin_bytes);
         launch_fill_u8(stream_, d_colmat, (uint8_t)kMissingBin, col_stride * P * bin_bytes);
+        // (rows that store every feature cannot hold a column twice)
+        if (!ascend_known && nnz_ != (long)n_ * F_) rows_ascend = device_rows_ascend(stream_, n_, d_row_ptr, d_col);
+        if (!rows_ascend) log_info("rows with descending column indices: the dense bins are filled row by row");
         launch_bin_dense(stream_, n_, d_row_ptr, d_col, d_val, cuts_.cut_val, cuts_.cut_row_ptr, d_binmat_, W,
-                         bins_.block_stride, d_colmat, col_stride, bin_bytes, P, bins_.feat_col, bins_.feat_lo);
+                         bins_.block_stride, d_colmat, col_stride, bin_bytes, P, bins_.feat_col, bins_.feat_lo, rows_ascend);
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
