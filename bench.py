@@ -221,7 +221,11 @@ def main():
     if args.config == 2 and args.full_run and args.rows == 0:
         aux["small_data"] = small_data_figures(T, torch)
     if args.calibration_copy_mb > 0:
-        T.load().tgbm_calibration_copy(args.calibration_copy_mb << 20, 3)
+        import ctypes
+        cal = ctypes.CDLL(os.path.join(ROOT, "thundergbm_amd", "libtgbm_calibration.so"))
+        cal.tgbm_calibration_copy.argtypes = [ctypes.c_size_t, ctypes.c_int]
+        cal.tgbm_calibration_copy.restype = None
+        cal.tgbm_calibration_copy(args.calibration_copy_mb << 20, 3)
 
     cpu = None
     if args.cpu_steps > 0:

@@ -177,16 +177,19 @@ tgbm_model *tgbm_trainer_export_model(tgbm_trainer *t);
 void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const int *col_ptr, tgbm_model *model,
                       int n_trees, int trees_per_iter, float learning_rate, float base_score, float *out);
 
-/* tgbm_predict_raw for callers that cannot allocate (tight serving loops, harnesses that forbid hipMalloc, code that
- * records the call's device work into a HIP graph). It has no counterpart in the reference. Same arguments, same
- * scores bit for bit, but no hipMalloc / hipFree / stream creation: the device copies of the rows, the model and
- * the scores live in a file-scope device array of about 34 MiB that every GPU used by the library holds until the
- * process ends (its address is resolved on the first call on a device). Limits per call: row_size <= 65536,
- * stored values <= 2^20, row_size * trees_per_iter <= 2^19, nodes of the trees used <= 2^19 (e.g. 800 trees of
- * depth 8). Returns 0, or 1 with a message on stderr when a limit is exceeded (nothing is computed then). Calls
- * share the device's array, which keeps the last call's contents; they are serialised inside one process, and
- * calls from several processes on one GPU do not interfere (every process has its own copy). The work runs on
- * the default stream and the call returns after the scores were copied to `out`. */
+/* tgbm_predict_raw for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. Same arguments, same scores bit for bit, but no hipMalloc /
+ * hipFree / stream creation: the device copies of the rows, the model and the scores live in a file-scope device
+ * array of about 34 MiB that every GPU used by the library holds until the process ends (its address is resolved on
+ * the first call on a device). Limits per call: row_size <= 65536, stored values <= 2^20,
+ * row_size * trees_per_iter <= 2^19, nodes of the trees used <= 2^19 (e.g. 800 trees of depth 8). Returns 0, or 1
+ * with a message on stderr when a limit is exceeded (nothing is computed then); malformed input (a null model, a
+ * row_ptr that does not ascend, a negative column index) aborts the process with a message, as in every other entry
+ * point. Calls share the device's array, which keeps the last call's contents; they are serialised inside one
+ * process, and calls from several processes on one GPU do not interfere (every process has its own copy). The work
+ * runs on the default stream with synchronous host copies (the call cannot be recorded into a HIP graph) and returns
+ * after the scores were copied to `out`. The trees are walked in their 48-byte node form (the packed LDS form of
+ * tgbm_predict_raw needs an allocation), so a call takes about twice the device time of tgbm_predict_raw. */
 int tgbm_predict_raw_noalloc(int row_size, const float *val, const int *row_ptr, const int *col_ptr,
                              tgbm_model *model, int n_trees, int trees_per_iter, float learning_rate,
                              float base_score, float *out);
@@ -196,11 +199,6 @@ int tgbm_predict_raw_noalloc(int row_size, const float *val, const int *row_ptr,
  * slot per stored value at most (row_ptr[row_size]); returns the number of cut points. */
 int tgbm_cut_points(int row_size, int n_features, const float *val, const int *row_ptr, const int *col_ptr,
                     int max_num_bin, float *cut_val, int *cut_row_ptr, int *cut_fid, int *bin_id);
-
-/* Runs `repeats` launches of a plain streaming copy kernel (k_calibration_copy) over `bytes` bytes.
- * It has no counterpart in the reference: it exists to calibrate a profiler's HBM byte counters
- * (FETCH_SIZE / WRITE_SIZE) against a transfer of known size. */
-void tgbm_calibration_copy(size_t bytes, int repeats);
 
 #ifdef __cplusplus
 }

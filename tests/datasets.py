@@ -124,3 +124,13 @@ def config5(n=1_000_000, seed=4):
     Z = Z + bias + rng.gumbel(size=Z.shape)
     y = Z.argmax(axis=1).astype(np.float32)
     return X, y
+
+
+def warm_up(T):
+    """One tiny training session: the first GPU call of a process initialises the runtime (which may draw from
+    rand() itself), so the tests' random streams do not depend on which of them runs first."""
+    X, y = config1(64, 3, seed=0)
+    val, rp, col = dense_to_csr(X)
+    s = T.Session(val, rp, col, y, depth=2, n_trees=1, max_num_bin=8)
+    s.boost(1)
+    s.close()

@@ -26,7 +26,7 @@ def T():
     L = thundergbm_amd.load()
     # the first GPU call of a process initialises the runtime (which may draw from rand() itself): do it here,
     # so that no test's random stream depends on which test runs first
-    L.tgbm_calibration_copy(1 << 20, 1)
+    D.warm_up(thundergbm_amd)
     return thundergbm_amd
 
 

@@ -48,7 +48,6 @@ SIGNATURES = {
     "tgbm_trainer_export_model": (_P, [_P]),
     "tgbm_predict_raw": (None, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, _P]),
     "tgbm_predict_raw_noalloc": (C.c_int, [C.c_int, _P, _P, _P, _P, C.c_int, C.c_int, C.c_float, C.c_float, _P]),
-    "tgbm_calibration_copy": (None, [C.c_size_t, C.c_int]),
     "tgbm_cut_points": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, C.c_int, _P, _P, _P, _P]),
 }
 

@@ -6,6 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libthundergbm.so")
+CALIBRATION_LIB = os.path.join(HERE, "libtgbm_calibration.so")
 BIN_DIR = os.path.join(HERE, "bin")
 
 HIP_SOURCES = ["tree_kernels.hip", "sparse_kernels.hip", "prep_kernels.hip", "predict_kernels.hip", "rank_kernels.hip", "trainer.hip",
@@ -49,6 +50,8 @@ def build(force=True):
     if failed:
         raise RuntimeError("hipcc failed")
     _run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs)
+    # the profiler calibration helper is a library of its own (not part of the training library's ABI)
+    _run([HIPCC] + COMMON + ["-shared", os.path.join(CSRC, "calibration_copy.hip"), "-o", CALIBRATION_LIB])
     os.makedirs(BIN_DIR, exist_ok=True)
     for name, src in (("thundergbm-train", "cli_train.cpp"), ("thundergbm-predict", "cli_predict.cpp")):
         _run([HIPCC, "-O2", "-std=c++17", os.path.join(CSRC, src), "-o", os.path.join(BIN_DIR, name),

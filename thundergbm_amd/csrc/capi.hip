@@ -334,18 +334,6 @@ void tgbm_predict_raw(int row_size, const float *val, const int *row_ptr, const 
     std::memcpy(out, r.data(), r.size() * sizeof(float));
 }
 
-void tgbm_calibration_copy(size_t bytes, int repeats) {
-    void *src = nullptr, *dst = nullptr;
-    HIP_CHECK(hipMalloc(&src, bytes));
-    HIP_CHECK(hipMalloc(&dst, bytes));
-    HIP_CHECK(hipMemset(src, 1, bytes));
-    HIP_CHECK(hipMemset(dst, 0, bytes));
-    for (int i = 0; i < repeats; ++i) launch_calibration_copy(nullptr, src, dst, bytes);
-    HIP_CHECK(hipDeviceSynchronize());
-    HIP_CHECK(hipFree(src));
-    HIP_CHECK(hipFree(dst));
-}
-
 int tgbm_cut_points(int row_size, int n_features, const float *val, const int *row_ptr, const int *col_ptr,
                     int max_num_bin, float *cut_val, int *cut_row_ptr, int *cut_fid, int *bin_id) {
     const long nnz = row_ptr[row_size];

@@ -404,7 +404,6 @@ void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbi
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);
 void launch_fill_f32(hipStream_t s, float *p, float v, size_t n);
-void launch_calibration_copy(hipStream_t s, const void *src, void *dst, size_t bytes);
 void launch_fill_u8(hipStream_t s, uint8_t *p, uint8_t v, size_t n);
 
 // data preparation

@@ -73,12 +73,6 @@ __device__ int find_owner(const int *begin, int n, int item) {
     return lo;
 }
 
-// Plain streaming copy of 16-byte words; used to calibrate the profiler's HBM byte counters.
-__global__ void k_calibration_copy(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = src[i];
-}
-
 // ------------------------------------------------------------------------------------ fills
 __global__ void k_fill_f32(float *p, float v, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
@@ -2243,12 +2237,6 @@ int grid_for(size_t n, int cap = 4096) {
 }  // namespace
 
 // =================================================================================== launchers
-void launch_calibration_copy(hipStream_t s, const void *src, void *dst, size_t bytes) {
-    size_t n = bytes / 16;
-    if (n == 0) return;
-    k_calibration_copy<<<grid_for(n, 16384), kBlock, 0, s>>>(static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), n);
-}
-
 void launch_fill_f32(hipStream_t s, float *p, float v, size_t n) {
     if (n == 0) return;
     k_fill_f32<<<grid_for(n), kBlock, 0, s>>>(p, v, n);
