@@ -31,15 +31,15 @@ def item_shift(qmax, rows, bits):
     return int(np.floor(np.log2(qmax / lim))) + 1
 
 
-def node_quantum(quant, node_rows, sparse, flush_rows=32768):
+def node_quantum(quant, node_rows, sparse):
     """Coarsest (g, h) step at which a row of a node with node_rows rows is counted. The library sums
     round(g * scale) as exact 64-bit integers; a dense work item coarsens the tree's scale by a power of two
-    that depends on the rows it adds between two drains of its packed LDS bins (at most min(node rows, 32768)).
+    that depends on the rows it adds between two drains of its packed LDS bins (at most min(node rows, flush_rows): 8192 with float hessians, 32768 with integer ones).
     Every histogram built from rows is therefore exact up to half a step per stored entry."""
     qg, qh = float(quant["inv_g"]), float(quant["inv_h"])
     if sparse:
         return np.array([qg, qh])
-    r = max(1, min(int(node_rows), flush_rows))
+    r = max(1, min(int(node_rows), int(quant["flush_rows"])))
     sg = item_shift(float(quant["gq_max"]), r, 63 - int(quant["h_bits"]))
     sh = 0 if quant["h_integer"] else item_shift(float(quant["hq_max"]), r, int(quant["h_bits"]))
     return np.array([qg * 2.0 ** sg, qh * 2.0 ** sh])

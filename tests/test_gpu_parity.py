@@ -219,12 +219,13 @@ def test_tree_lockstep(T, name):
         s.tree_init(k)
         o.tree_init(k)
         quant = s.quant()
-        # resolution of the fixed-point plan: the coarsest step (32768 rows between two drains) against the largest
-        # |g| of the tree; 47-bit gradient fields when every hessian is an integer (squared loss), 32 otherwise
+        # resolution of the fixed-point plan: the coarsest step against the largest |g| of the tree: 47-bit gradient
+        # fields and 32768 rows between two drains when every hessian is an integer (squared loss), else 32 bits
+        # and 8192 rows
         if not sparse:
             gmax = float(np.abs(gh[:, 0]).max())
             assert bool(quant["h_integer"]) == (kw["objective"] == "reg:linear")
-            assert P.node_quantum(quant, n, False)[0] <= gmax * 2.0 ** (-31 if quant["h_integer"] else -15)
+            assert P.node_quantum(quant, n, False)[0] <= gmax * 2.0 ** (-31 if quant["h_integer"] else -17)
         node_of_row = np.zeros(n, np.int64)
         tol_prev = None  # tolerance arrays of the previous level's nodes
         diverged = False
@@ -781,7 +782,7 @@ def test_full_size_properties_config2_reordered_rows(T):
 
 def test_full_size_oracle_config2(T):
     """10 M x 28, depth 8, 255 bins against the oracle at the full shape: the first tree (rows in the caller's order,
-    512-item plans of 19 712 rows each) and the fifth (after three physical re-orderings of the
+    512-item plans, work items drained every 8192 rows) and the fifth (after three physical re-orderings of the
     rows)."""
     val, rp, col, y = _full_data("c2")
     kw = dict(objective="binary:logistic", depth=8, max_num_bin=255, learning_rate=0.3, n_trees=5)

@@ -69,6 +69,16 @@ __device__ __forceinline__ bool csr_goes_right(const CsrBins &bins, int row, int
 }
 
 
+// Power of two by which the dense work items of a node that add at most `rows` rows between two drains coarsen one
+// of the tree's scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
+// scale, bits: magnitude bits of the packed field).
+__device__ int item_shift(float qmax, int rows, int bits) {
+    const double lim = ldexp(1.0, bits) / (double)rows * (1.0 - 1e-6) - 0.5;
+    const double q = (double)qmax;
+    if (!(q >= lim)) return 0;
+    return ilogb(q / lim) + 1;  // 2^s > q / lim
+}
+
 // ------------------------------------------------------------------------ split finding
 __device__ __forceinline__ float split_gain(GHPair f, GHPair l, float mcw, float lambda) {
 #pragma clang fp contract(off)

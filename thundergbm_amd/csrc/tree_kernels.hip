@@ -14,10 +14,6 @@ constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / 64;
 constexpr int kHistMinChunk = 1024;
 constexpr int kHistBlock = 1024;      // threads per histogram workgroup (they share one LDS histogram)
-// Rows a packed 32+32-bit LDS bin may absorb before it is drained. 32768: the 512 root items of 10 M rows (19 712 rows
-// each) are never drained and leave as 8-byte packed words; a row of a node that large is counted at 2^-15 of the
-// tree's largest |g| (float hessians), fine against the 1e-5 bound on sums of tens of thousands of rows.
-constexpr int kHistFlushRows = 32768;
 
 // Exclusive scan of one int per thread over a 256-thread block; lds needs kWaves ints.
 __device__ int block_excl_scan(int v, int *lds, int *total) {
@@ -245,16 +241,6 @@ __device__ float pow2_scale(float vmax, int rows, float limit) {
     return ldexpf(1.f, e - 1);     // 2^(e-1) <= bound
 }
 
-// Power of two by which the dense work items of a node that add at most `rows` rows between two drains coarsen one
-// of the tree's scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
-// scale, bits: magnitude bits of the packed field).
-__device__ int item_shift(float qmax, int rows, int bits) {
-    const double lim = ldexp(1.0, bits) / (double)rows * (1.0 - 1e-6) - 0.5;
-    const double q = (double)qmax;
-    if (!(q >= lim)) return 0;
-    return ilogb(q / lim) + 1;  // 2^s > q / lim
-}
-
 // ------------------------------------------------------------------------------- tree init
 // Node array initialisation of the reference's Tree::init2 (src/thundergbm/tree.cu:8-39), root sum
 // from the block partials, root segment and the histogram plan of level 0. One workgroup.
@@ -359,12 +345,14 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
         q.h_bits = 32;
         q.h_integer = 0;
         // every hessian a non-negative integer (squared loss; bagging multiplies by draw counts): the hessian field
-        // takes the bits that kHistFlushRows such rows need, the gradient field the rest
-        const float hrows = hm * (float)kHistFlushRows;
+        // takes the bits that kHistFlushRowsInt such rows need, the gradient field the rest
+        q.flush_rows = kHistFlushRows;
+        const float hrows = hm * (float)kHistFlushRowsInt;
         if (!tb.sparse && hf == 0.f && hm >= 1.f && hrows < 4.0e9f) {
             q.h_integer = 1;
             q.h_bits = ilogbf(hrows) + 1;
             q.scale_h = 1.f;
+            q.flush_rows = kHistFlushRowsInt;
         }
         q.inv_g = 1.f / q.scale_g;
         q.inv_h = 1.f / q.scale_h;
@@ -415,6 +403,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     const int nb = blk_bin_begin[fb + 1] - bin0;
     if (nb == 0) return;
     const int h_bits = quant->h_bits;
+    const int flush_rows = quant->flush_rows;
     // The item's node and rows: the same few look-ups in every lane (uniform addresses: scalar loads), so that the
     // first row loads can be issued before the barrier that publishes the LDS histogram's clearing.
     const int p = find_owner(hpair_begin, n_pairs, item);
@@ -427,7 +416,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     if (threadIdx.x == 0) {
         // (the node's rows, not the item's: what a row adds must not depend on the item it falls into, or the sums
         // would change with the order of the rows)
-        const int rows = max(1, min(sg.y - sg.x, kHistFlushRows));
+        const int rows = max(1, min(sg.y - sg.x, quant->flush_rows));
         const int2 shift = make_int2(item_shift(quant->gq_max, rows, 63 - h_bits),
                                      quant->h_integer ? 0 : item_shift(quant->hq_max, rows, h_bits));
         s_shift[0] = shift.x;
@@ -497,7 +486,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
             if (base + 2 * STEP < end) load_ids(base + 2 * STEP, r_next);
         }
         const int step_rows = min(RPS * U, end - base);
-        if (pending + step_rows > kHistFlushRows) {
+        if (pending + step_rows > flush_rows) {
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < SLOTS; ++k) {
@@ -540,7 +529,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         }
     }
     __syncthreads();
-    if (c.hchunk <= kHistFlushRows) {
+    if (c.hchunk <= flush_rows) {
         // an item this short was never drained: its packed LDS words are the complete sums and go out as
         // they are (8 bytes per bin instead of 16; k_hist_merge unpacks them)
         unsigned long long *out = reinterpret_cast<unsigned long long *>(partial) + (size_t)(item - item0) * n_bins + bin0;
@@ -589,7 +578,7 @@ __global__ __launch_bounds__(kBlock) void k_hist_merge(TreeBuffers tb_all, int l
     if (j < n_bins) {
         // every item counted at its own scale (item_shift): shift its sums to the tree's
         const int2 *__restrict__ shift = tb.hitem_shift;
-        if (tb.ctl[level].hchunk <= kHistFlushRows) {  // packed 8-byte partials (see k_hist_dense)
+        if (tb.ctl[level].hchunk <= tb.quant->flush_rows) {  // packed 8-byte partials (see k_hist_dense)
             const unsigned long long *packed = reinterpret_cast<const unsigned long long *>(partial);
             const int h_bits = tb.quant->h_bits;
             const unsigned long long h_mask = (1ull << h_bits) - 1ull;

@@ -21,7 +21,8 @@ SPLIT_DTYPE = np.dtype(
     ]
 )
 QUANT_DTYPE = np.dtype([("scale_g", "<f4"), ("scale_h", "<f4"), ("inv_g", "<f4"), ("inv_h", "<f4"),
-                        ("gq_max", "<f4"), ("hq_max", "<f4"), ("h_bits", "<i4"), ("h_integer", "<i4")])
+                        ("gq_max", "<f4"), ("hq_max", "<f4"), ("h_bits", "<i4"), ("h_integer", "<i4"),
+                        ("flush_rows", "<i4")])
 CTL_DTYPE = np.dtype([("hchunk", "<i4"), ("n_hitems", "<i4"), ("n_pitems", "<i4"), ("rows_built", "<i4")])
 
 
