@@ -131,6 +131,8 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=2, help="boosting iterations of the CPU baseline (0 = skip)")
     ap.add_argument("--full-run", type=int, default=1,
                     help="config 2: also time one training call of all the configuration's trees (0 = skip)")
+    ap.add_argument("--small-data", type=int, default=1,
+                    help="config 2: also time the two small workloads, 40 trees each (0 = skip, e.g. under a profiler)")
     ap.add_argument("--calibration-copy-mb", type=int, default=0,
                     help="also run 3 launches of a plain copy kernel of this many MiB (profiler counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU baseline sample (0 = a default per config)")
@@ -218,7 +220,7 @@ def main():
         aux["iters_per_s_100_trees"] = round(cfg["n_trees"] / t_full, 2)
         aux["reorderings_in_100_trees"] = s.info("reorders_done")
         s.close()
-    if args.config == 2 and args.full_run and args.rows == 0:
+    if args.config == 2 and args.small_data and args.rows == 0:
         aux["small_data"] = small_data_figures(T, torch)
     if args.calibration_copy_mb > 0:
         import ctypes
