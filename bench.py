@@ -119,6 +119,26 @@ def small_data_figures(T, torch):
     return out
 
 
+def predict_figures(T, s, val, rp, col, lr, n_trees=40):
+    """Wall time of the C ABI's prediction call on the training rows (host CSR in, raw scores out: the upload is
+    inside; the traversal kernel's own time is in the kernel trace under profiles/)."""
+    import ctypes as C
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    out = np.zeros(s.n, np.float32)
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    best = None
+    for _ in range(2):
+        out[:] = 0
+        t0 = time.perf_counter()
+        L.tgbm_predict_raw(s.n, p(val), p(rp), p(col), model, n_trees, 1, lr, s.base_score, p(out))
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    L.model_free(C.byref(model))
+    return {"rows": int(s.n), "trees": n_trees, "wall_s_host_buffers": round(best, 4),
+            "rows_per_s": round(s.n / best, 1), "mean_raw_score": float(out.mean())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,6 +153,9 @@ def main():
                     help="config 2: also time one training call of all the configuration's trees (0 = skip)")
     ap.add_argument("--small-data", type=int, default=1,
                     help="config 2: also time the two small workloads, 40 trees each (0 = skip, e.g. under a profiler)")
+    ap.add_argument("--predict", type=int, default=1,
+                    help="config 2 with --full-run: also time tgbm_predict_raw (host buffers in, scores out) on all rows "
+                         "with 40 of the trees (0 = skip)")
     ap.add_argument("--calibration-copy-mb", type=int, default=0,
                     help="also run 3 launches of a plain copy kernel of this many MiB (profiler counter calibration)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU baseline sample (0 = a default per config)")
@@ -219,6 +242,8 @@ def main():
         t_full = time.perf_counter() - t0
         aux["iters_per_s_100_trees"] = round(cfg["n_trees"] / t_full, 2)
         aux["reorderings_in_100_trees"] = s.info("reorders_done")
+        if args.predict:
+            aux["predict"] = predict_figures(T, s, val, rp, col, cfg["learning_rate"])
         s.close()
     if args.config == 2 and args.small_data and args.rows == 0:
         aux["small_data"] = small_data_figures(T, torch)

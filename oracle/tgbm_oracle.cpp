@@ -1021,7 +1021,9 @@ void predict_raw(int n, int F, const float *val, const int *row_ptr, const int *
                 while (!nd[cur].is_leaf) {
                     int f = nd[cur].split_fid;
                     const int *p = std::lower_bound(ci, ci + len, f);
-                    if (p != ci + len && *p == f) {
+                    // (the shared-memory path marks a missing value with +inf in the row's dense vector and tests
+                    // `fval < INFINITY`, predictor.cu:96-118: a stored +inf or NaN takes the default direction there)
+                    if (p != ci + len && *p == f && (!dense_path || cv[p - ci] < INFINITY)) {
                         float v = cv[p - ci];
                         cur = v < nd[cur].split_value ? nd[cur].lch : nd[cur].rch;
                     } else {

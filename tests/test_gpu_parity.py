@@ -538,6 +538,134 @@ def test_predict_paths_of_the_dense_vector_kernels(T, F, depth, num_class):
     s.close()
 
 
+def _model_file(path, objective, lr, base_score, labels, model):
+    """The reference's model file (parser.cpp:102-171) for trees given as NODE arrays [n_iter, trees per round, nodes]."""
+    import struct
+    n_iter, k, n_nodes = model.shape
+    out = struct.pack("<i", len(objective)) + objective
+    out += struct.pack("<fiif", lr, max(k, 1) if k > 1 else 1, n_iter, base_score)
+    out += struct.pack("<i", len(labels)) + struct.pack("<%df" % len(labels), *labels)
+    out += struct.pack("<i", n_iter)
+    for it in range(n_iter):
+        out += struct.pack("<i", k)
+        for t in range(k):
+            out += struct.pack("<Q", n_nodes) + np.ascontiguousarray(model[it, t]).tobytes()
+    with open(path, "wb") as f:
+        f.write(out)
+
+
+def _predict_variants(L, n, tv, trp, tc, model, n_iter, k, lr, base, settings):
+    """tgbm_predict_raw under each (TGBM_PREDICT_COMPACT, TGBM_PREDICT_TPS) setting; the switches are read per call."""
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+    outs = {}
+    try:
+        for compact, tps in settings:
+            os.environ["TGBM_PREDICT_COMPACT"], os.environ["TGBM_PREDICT_TPS"] = str(compact), str(tps)
+            out = np.zeros(n * k, np.float32)
+            L.tgbm_predict_raw(n, p(tv), p(trp), p(tc), model, n_iter, k, lr, base, p(out))
+            outs[(compact, tps)] = out
+    finally:
+        os.environ.pop("TGBM_PREDICT_COMPACT", None)
+        os.environ.pop("TGBM_PREDICT_TPS", None)
+    return outs
+
+
+@pytest.mark.parametrize("num_class,depth", [(1, 6), (3, 4)])
+def test_predict_kernels_agree_bit_for_bit(T, num_class, depth, tmp_path):
+    """The predictor's LDS kernels - 48-byte nodes in global memory, 16-byte records, 8-byte records with one or two
+    trees walked at a time, with and without the coalesced spreading of equal-length rows - give the same bits,
+    and the oracle's predictor agrees, on: dense rows (equal length, some stored +inf / NaN / -inf), the same rows with
+    one row's columns descending and one column repeated (the later entry counts), ragged rows, and rows that lack
+    the model's last features. The same trees with their nodes stored in another order (children not side by side:
+    the 8-byte records do not apply) predict the same bits too."""
+    rng = np.random.default_rng(7 + num_class)
+    n, F, n_iter, lr = 3000, 20, 7, 0.4
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.1] = 0
+    score = X[:, 0] - X[:, 1] * X[:, 2] + X[:, F - 1] + 0.1 * rng.standard_normal(n)
+    kw = dict(depth=depth, n_trees=n_iter, learning_rate=lr, max_num_bin=32, min_child_weight=0.1)
+    if num_class > 1:
+        y = np.digitize(score, np.quantile(score, np.linspace(0, 1, num_class + 1)[1:-1])).astype(np.float32)
+        kw["objective"] = "multi:softprob"
+    else:
+        y = score.astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    s = T.Session(val, rp, col, y, **kw)
+    s.boost(n_iter)
+    k = s.tree_per_rounds
+    base = s.base_score if k == 1 else 0.0
+    nodes = s.model().copy()
+    assert (nodes["split_fid"] == F - 1).any()
+    L = T.load()
+    model = C.c_void_p(s.export_model())
+    m = 1001  # not a multiple of the workgroup's rows
+    Xt = rng.standard_normal((m, F)).astype(np.float32)
+    Xt[5, 3], Xt[6, 0], Xt[7, 1] = np.inf, np.nan, -np.inf
+    full_rp = (np.arange(m + 1) * F).astype(np.int32)
+    full_col = np.tile(np.arange(F, dtype=np.int32), m)
+    full_val = Xt.reshape(-1).copy()
+    cases = {"dense": (full_val, full_rp, full_col, F)}
+    c2, v2 = full_col.copy(), full_val.copy()
+    c2[300 * F + 4], c2[300 * F + 5] = 5, 4        # row 300: columns 4 and 5 swapped (descending)
+    c2[700 * F + 9] = 8                              # row 700: column 8 stored twice, the later entry counts
+    cases["unsorted"] = (v2, full_rp, c2, F)
+    Xr = Xt.copy()
+    Xr[rng.random((m, F)) < 0.4] = 0
+    cases["ragged"] = D.dense_to_csr(Xr)[0], D.dense_to_csr(Xr)[1], D.dense_to_csr(Xr)[2], F
+    short = F - 3                                     # the data's last column is 16: the model's features 17..19 are missing
+    keep = np.tile(np.arange(F) < short, m)
+    cases["short"] = (full_val[keep], (np.arange(m + 1) * short).astype(np.int32), full_col[keep], short)
+    settings = [(0, 0), (0, 1), (0, 4), (1, 1), (1, 2), (2, 1), (2, 2)]
+    results = {}
+    for name, (tv, trp, tc, Fd) in cases.items():
+        tv, trp, tc = np.ascontiguousarray(tv), np.ascontiguousarray(trp), np.ascontiguousarray(tc)
+        outs = _predict_variants(L, m, tv, trp, tc, model, n_iter, k, lr, base, settings)
+        first = outs[settings[0]]
+        for key, out in outs.items():
+            assert np.array_equal(out, first, equal_nan=True), (name, key)
+        if name == "unsorted":
+            # what the row-per-thread loop defines: the later entry of a repeated column; order does not matter
+            srt = full_val.copy()
+            srt[300 * F + 4], srt[300 * F + 5] = full_val[300 * F + 5], full_val[300 * F + 4]
+            srt[700 * F + 8] = full_val[700 * F + 9]
+            gone = 700 * F + 9  # row 700 has no column 9 any more
+            rp_ref = full_rp.copy()
+            rp_ref[701:] -= 1
+            ref = O.predict_raw(np.delete(srt, gone), rp_ref, np.delete(full_col, gone), F, nodes, lr, base)
+        else:
+            ref = O.predict_raw(tv, trp, tc, Fd, nodes, lr, base)
+        np.testing.assert_allclose(first, ref, rtol=1e-6, atol=1e-6, err_msg=name)
+        results[name] = first
+    L.model_free(C.byref(model))
+    # the same trees with the nodes of every tree in another order
+    perm_nodes = nodes.copy()
+    n_nodes = nodes.shape[2]
+    for it in range(n_iter):
+        for t in range(k):
+            order = np.concatenate([[0], 1 + rng.permutation(n_nodes - 1)])  # new position -> old index; the root stays
+            where = np.empty(n_nodes, np.int64)
+            where[order] = np.arange(n_nodes)
+            tree = nodes[it, t][order].copy()
+            for name in ("lch", "rch", "parent"):
+                old = tree[name]
+                tree[name] = np.where(old >= 0, where[np.clip(old, 0, n_nodes - 1)], old)
+            perm_nodes[it, t] = tree
+    path = str(tmp_path / "perm.model")
+    labels = [float(v) for v in range(max(k, 2))]
+    _model_file(path, b"multi:softprob" if k > 1 else b"reg:linear", lr, base, labels, perm_nodes)
+    model2 = C.c_void_p(None)
+    f1, i1, i2, i3 = (C.c_float * 1)(), (C.c_int * 1)(), (C.c_int * 1)(), (C.c_int * 1)()
+    vp = lambda a: C.cast(a, C.c_void_p)
+    L.load_model(path.encode(), vp(f1), vp(i1), vp(i2), vp(i3), vp(C.byref(model2)))
+    assert i2[0] == n_iter * k or i2[0] == n_iter
+    tv, trp, tc, _ = cases["dense"]
+    outs = _predict_variants(L, m, tv, trp, tc, model2, n_iter, k, lr, base, [(1, 2), (0, 0)])
+    assert np.array_equal(outs[(1, 2)], results["dense"], equal_nan=True)
+    assert np.array_equal(outs[(0, 0)], results["dense"], equal_nan=True)
+    L.model_free(C.byref(model2))
+    s.close()
+
+
 @pytest.mark.parametrize("layout", ["dense", "sparse"])
 def test_a1a_quickstart_known_answer(T, layout):
     # README.md:76-80 of the reference: RMSE = 0.489562 (zero initial prediction, see the oracle test)

@@ -548,6 +548,28 @@ def test_predictor_equals_training_prediction(objective, K):
         assert np.mean(out == y) > 0.6
 
 
+def test_predictor_stored_infinity_by_hand():
+    """One split (feature 1 < 0.5 -> leaf 1.0, else leaf 2.0; default left). The reference's shared-memory path
+    (F <= 96) marks missing values with +inf and tests `fval < INFINITY` (predictor.cu:96-118), so a stored +inf or
+    NaN follows the default direction there; its binary-search path (wider data, :120-189) compares the stored value:
+    +inf and NaN are not less than the threshold and go right. -inf is an ordinary small value in both."""
+    nodes = np.zeros((1, 1, 3), dtype=O.NODE_DTYPE)
+    nodes["lch"], nodes["rch"], nodes["is_leaf"], nodes["is_valid"] = -1, -1, 1, 1
+    root = nodes[0, 0, 0:1]
+    root["lch"], root["rch"], root["is_leaf"] = 1, 2, 0
+    root["split_fid"], root["split_value"], root["default_right"] = 1, 0.5, 0
+    nodes[0, 0, 1]["base_weight"], nodes[0, 0, 2]["base_weight"] = 1.0, 2.0
+    vals = np.array([0.0, 1.0, np.inf, np.nan, -np.inf], np.float32)  # one row each: feature 1 only
+    rp = np.arange(len(vals) + 1, dtype=np.int32)
+    col = np.ones(len(vals), np.int32)
+    dense = O.predict_raw(vals, rp, col, 3, nodes, 1.0, 0.0)
+    assert dense.tolist() == [1.0, 2.0, 1.0, 1.0, 1.0]
+    wide = O.predict_raw(vals, rp, col, 200, nodes, 1.0, 0.0)
+    assert wide.tolist() == [1.0, 2.0, 2.0, 2.0, 1.0]
+    no_row = O.predict_raw(np.zeros(0, np.float32), np.zeros(2, np.int32), np.zeros(0, np.int32), 3, nodes, 1.0, 0.0)
+    assert no_row.tolist() == [1.0]  # not stored: default left
+
+
 def test_base_score_binary_closed_form():
     rng = np.random.default_rng(8)
     X = rng.standard_normal((500, 3)).astype(np.float32)

@@ -497,7 +497,8 @@ void upload_large(hipStream_t s, void *dst, const void *src, size_t bytes);
 // `packed` (optional): the same nodes as 16-byte records (launch_pack_model); with them the trees are walked from LDS
 void launch_predict(hipStream_t s, int n, int F, const int *row_ptr, const int *col, const float *val,
                     const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, float lr, float base_score,
-                    float *out, size_t out_stride = 0, const struct PackedNode *packed = nullptr);
+                    float *out, size_t out_stride = 0, const struct PackedNode *packed = nullptr,
+                    const uint2 *compact = nullptr, int compact_depth = 0);
 // What a traversal reads of a node, in one 16-byte record.
 struct PackedNode {
     float split_value, base_weight;
@@ -505,6 +506,16 @@ struct PackedNode {
     unsigned meta;      // split feature (24 bits, all ones: not a feature of the data) | default_right << 30 | leaf << 31
 };
 void launch_pack_model(hipStream_t s, const TreeNode *model, long n_total, int n_nodes, PackedNode *packed);
+// `compact` of launch_predict: eight-byte records (threshold or leaf weight; left child | address of the split feature's
+// values | flags) for a model and data of F features that compact_records_apply() accepts; `compact_depth`: what it
+// returned. The records depend on F (features the data lacks, rows per workgroup), so they are packed per data set.
+void launch_pack_compact(hipStream_t s, const TreeNode *model, int n_iter, int n_class_trees, int n_nodes, int F,
+                         uint2 *packed);
+// Do the eight-byte records describe this model on data of F features? Every split node keeps its children side by
+// side (right = left + 1) and below itself - then a walk needs one child index and ends after at most `depth` steps,
+// the number returned (0: they do not apply) -, and one tree fits the LDS next to the rows' dense vectors.
+int compact_records_apply(const TreeNode *model, size_t n_total, int n_nodes, int F);
+int compact_rows_per_group(int F);  // rows per workgroup of the kernel that walks the eight-byte records
 void launch_predict_transform(hipStream_t s, int kind, int n, int num_class, const float *label, float *y);
 
 }  // namespace tgbm

@@ -72,7 +72,7 @@ __device__ __forceinline__ bool csr_goes_right(const CsrBins &bins, int row, int
 // Power of two by which the dense work items of a node that add at most `rows` rows between two drains coarsen one
 // of the tree's scales: the smallest s >= 0 with rows * (qmax / 2^s + 0.5) < 2^bits (qmax: the most one row adds at the tree's
 // scale, bits: magnitude bits of the packed field).
-__device__ int item_shift(float qmax, int rows, int bits) {
+__device__ __forceinline__ int item_shift(float qmax, int rows, int bits) {
     const double lim = ldexp(1.0, bits) / (double)rows * (1.0 - 1e-6) - 0.5;
     const double q = (double)qmax;
     if (!(q >= lim)) return 0;

@@ -17,6 +17,29 @@ static int transform_kind(const std::string &objective) {
     return 0;
 }
 
+int compact_records_apply(const TreeNode *model, size_t n_total, int n_nodes, int F) {
+    if (n_nodes < 1 || n_nodes > 0x1fff || F < 1 || (size_t)F * 128 * sizeof(float) > 48 * 1024) return 0;
+    const size_t dense_bytes = (size_t)(F + 2) * compact_rows_per_group(F) * sizeof(float);
+    if (dense_bytes + (size_t)n_nodes * sizeof(uint2) > 64 * 1024) return 0;
+    int deepest = 0;
+    std::vector<int> level((size_t)n_nodes);
+    for (size_t t0 = 0; t0 + (size_t)n_nodes <= n_total; t0 += (size_t)n_nodes) {
+        std::fill(level.begin(), level.end(), -1);
+        level[0] = 0;
+        for (int self = 0; self < n_nodes; ++self) {
+            const TreeNode &nd = model[t0 + self];
+            const bool children_ok = nd.lch_index >= 0 && nd.lch_index < n_nodes && nd.rch_index >= 0 && nd.rch_index < n_nodes;
+            if (nd.is_leaf || !children_ok) continue;  // (a walk ends here)
+            if (nd.rch_index != nd.lch_index + 1 || nd.lch_index <= self) return 0;
+            if (nd.split_value != nd.split_value) return 0;  // (a NaN threshold: the two comparisons would disagree)
+            if (level[self] < 0) continue;  // (not reachable from the root)
+            level[nd.lch_index] = level[nd.rch_index] = level[self] + 1;
+            deepest = std::max(deepest, level[self] + 1);
+        }
+    }
+    return std::max(deepest, 1);
+}
+
 // Runs the traversal kernel and, if asked, the objective's transform and the training metric.
 static std::vector<float> run_predict(const GBMParam &param, const std::vector<std::vector<Tree>> &model,
                                       const DataSet &ds, bool transform, bool log_metric) {
@@ -52,6 +75,8 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     int *d_col = nullptr, *d_row_ptr = nullptr;
     TreeNode *d_model = nullptr;
     PackedNode *d_packed = nullptr;
+    uint2 *d_compact = nullptr;
+    int compact_depth = 0;
     const size_t n_out = (size_t)n * nct;
     HIP_CHECK(hipMalloc(&d_val, sizeof(float) * (size_t)std::max(nnz, 1l)));
     HIP_CHECK(hipMalloc(&d_col, sizeof(int) * (size_t)std::max(nnz, 1l)));
@@ -68,6 +93,11 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     // slice runs while the next slice crosses PCIe.
     if (nnz) upload_large(s, d_col, ds.col_idx, sizeof(int) * (size_t)nnz);
     if (!ds.features_counted) F = device_max_int(s, d_col, nnz) + 1;
+    compact_depth = compact_records_apply(flat.data(), flat.size(), n_nodes, F);  // (F is known only now)
+    if (compact_depth > 0) {
+        HIP_CHECK(hipMalloc(&d_compact, sizeof(uint2) * flat.size()));
+        launch_pack_compact(s, d_model, n_iter, nct, n_nodes, F, d_compact);
+    }
     HIP_CHECK(hipStreamSynchronize(s));
     lap("allocation, model and column indices");
     {
@@ -85,7 +115,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
             if (e1 > e0) upload_large(s_up, d_val + e0, ds.val + e0, sizeof(float) * (size_t)(e1 - e0));
             HIP_CHECK(hipStreamSynchronize(s_up));  // small copies return before they are done
             launch_predict(s, r1 - r0, F, d_row_ptr + r0, d_col, d_val, d_model, n_iter, nct, n_nodes,
-                           param.learning_rate, param.base_score, d_out + r0, (size_t)n, d_packed);
+                           param.learning_rate, param.base_score, d_out + r0, (size_t)n, d_packed, d_compact, compact_depth);
             HIP_CHECK_LAUNCHES("predict");
             r0 = r1;
         }
@@ -152,6 +182,7 @@ static std::vector<float> run_predict(const GBMParam &param, const std::vector<s
     HIP_CHECK(hipFree(d_row_ptr));
     HIP_CHECK(hipFree(d_model));
     HIP_CHECK(hipFree(d_packed));
+    if (d_compact) HIP_CHECK(hipFree(d_compact));
     HIP_CHECK(hipFree(d_out));
     if (d_label) HIP_CHECK(hipFree(d_label));
     HIP_CHECK(hipStreamDestroy(s));
