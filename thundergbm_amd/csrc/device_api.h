@@ -228,10 +228,11 @@ struct TreeBuffers {
     // sparse level pass only (else nullptr): node every row has reached (heap id) and rows per node
     unsigned short *nid16 = nullptr;  // [n + 2]
     int *node_rows = nullptr;         // [n_nodes]
-    // what the last row -> node update did with every row, one bit each: .x bit r % 64 of word r / 64 = the row moved
-    // to a child (its node split), .y = it moved to the right child. 2 bits per row instead of 16: the sorted pass,
-    // which knows a value's previous node from its key, looks its rows up here (the whole map stays in every L2).
-    ulonglong2 *row_side = nullptr;   // [(n + 63) / 64]
+    // what the last row -> node update did with every row: bit 0 = the row moved to a child (its node split), bit 1 =
+    // to the right child. A byte per row instead of the 16-bit node: the sorted pass, which knows a value's previous
+    // node from its key, looks its rows up here with one-byte loads, eight of them in flight per thread (the whole
+    // map stays in every L2).
+    uint8_t *row_move = nullptr;      // [n rounded up to 64]
     // sparse level pass: best candidate key of every node of the level over all tasks, and the candidate slot of
     // the task that searches a feature (k_best_update reads the winner's record from that slot)
     unsigned long long *best_key = nullptr;  // [max_level_nodes]
@@ -324,7 +325,7 @@ struct TreeBuffers {
         if (nid16 != nullptr) {
             t.nid16 += K * (((size_t)n + 2) / 2 * 2);
             t.node_rows += K * n_nodes;
-            t.row_side += K * (((size_t)n + 63) / 64);
+            t.row_move += K * (((size_t)n + 63) / 64 * 64);
             t.best_key += K * max_level_nodes;
         }
         t.leaf_value += K * n_nodes;

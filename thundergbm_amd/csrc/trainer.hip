@@ -561,7 +561,7 @@ void Trainer::alloc_tree_buffers() {
     } else {
         tb.nid16 = dalloc<unsigned short>(S * (((size_t)n_ + 2) / 2 * 2));
         tb.node_rows = dalloc<int>(S * tb.n_nodes);
-        tb.row_side = dalloc<ulonglong2>(S * (((size_t)n_ + 63) / 64));
+        tb.row_move = dalloc<uint8_t>(S * (((size_t)n_ + 63) / 64 * 64));
     }
     tb.partial = dalloc<longlong2>(S * tb.n_partial);
     tb.quant = dalloc<QuantCtl>(S);
