@@ -1175,3 +1175,51 @@ def test_sparse_level_pass_at_its_deepest_level(T):
     finally:
         os.environ.pop("TGBM_SPARSE_SORTED", None)
     assert [a == b for a, b in zip(runs[0], runs[1])] == [True] * 3
+
+
+@pytest.mark.parametrize("objective", ["reg:linear", "binary:logistic"])
+@pytest.mark.parametrize("F,reorder", [(28, "0"), (28, "always"), (12, "0"), (20, "always")])
+def test_gradient_words_in_the_bin_matrix_give_the_same_bits(T, objective, F, reorder):
+    """With a spare dword at the end of a row's bin-matrix record (features <= row bytes - 4), one tree per round and a
+    squared or 0/1-label logistic loss, the histogram kernels take a row's gradient pair from a 32-bit word stored in
+    that dword instead of gathering it from the gradient array (TGBM_GH_WORD=0: always gather). The word decodes to
+    the very floats of the gradient kernel, the sums are exact integers: models, predictions, row -> node maps and
+    the histograms of a level are the same byte for byte - also with missing values, with re-ordered rows, and when a
+    level is driven stage by stage after gradients were uploaded by hand (which the words do not know: the kernels
+    must fall back to the array)."""
+    os.environ["TGBM_LAYOUT"] = "dense"
+    os.environ["TGBM_REORDER"] = reorder
+    rng = np.random.default_rng(F)
+    n = 30000
+    X = rng.standard_normal((n, F)).astype(np.float32)
+    X[rng.random((n, F)) < 0.05] = 0
+    score = X[:, 0] - X[:, 1] * X[:, 2] + 0.3 * rng.standard_normal(n)
+    y = score.astype(np.float32) if objective == "reg:linear" else (score > 0).astype(np.float32)
+    val, rp, col = D.dense_to_csr(X)
+    kw = dict(objective=objective, n_trees=5, depth=6, max_num_bin=64, learning_rate=0.3)
+    runs = []
+    try:
+        for word in ("1", "0"):
+            os.environ["TGBM_GH_WORD"] = word
+            s = T.Session(val, rp, col, y, **kw)
+            assert s.info("sparse") == 0 and s.info("dense_blocks") == 1
+            s.boost(4)
+            out = [s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()]
+            # a level by hand with the round's own gradients, then with uploaded ones
+            s.gradient()
+            s.tree_init()
+            s.find_split(0)
+            out.append(s.level_hist(0).tobytes())
+            gh = s.gh().copy()
+            gh[:, 0] *= np.float32(0.5)
+            s.set("gh", gh)
+            s.tree_init()
+            s.find_split(0)
+            out.append(s.level_hist(0).tobytes())
+            runs.append(out)
+            s.close()
+    finally:
+        for k in ("TGBM_GH_WORD", "TGBM_REORDER", "TGBM_LAYOUT"):
+            os.environ.pop(k, None)
+    assert [a == b for a, b in zip(*runs)] == [True] * 5
+    assert runs[0][3] != runs[0][4]  # the uploaded gradients were used

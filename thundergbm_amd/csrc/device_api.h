@@ -114,6 +114,15 @@ struct DenseBins {
     const int *feat_col = nullptr;
     const uint8_t *feat_lo = nullptr;
     int n_cols = 0;  // columns of the matrix (= features when nothing is bundled)
+    // Lane (dword) of a row's record that is kept free of bins for the row's gradient word (the last lane of the
+    // row), -1: none. gh_fresh: gh_words[row] (launch_gh_words) matches the gradient array of this launch; the root
+    // level's histogram launch then decodes the words (gh_objective says how) instead of reading the pairs and copies
+    // them into the records, and the launches below the root take them from the records instead of gathering the
+    // pairs. That lane never adds bins either way.
+    int gh_lane = -1;
+    int gh_fresh = 0;
+    int gh_objective = 0;
+    const unsigned *gh_words = nullptr;  // [n]
 };
 
 // Sparse layout for wide, mostly-missing data: the reference's own representation, CSR rows of global
@@ -409,7 +418,11 @@ void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const Dens
 // holds row_blocks(n) doubles
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                       int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
-                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma = nullptr);
+                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma = nullptr,
+                      unsigned *gh_words = nullptr);
+// words[i] = the gradient word of row i (the pair of a squared or 0/1-label logistic loss in 32 bits, which the
+// histogram kernels decode to the very pair launch_gradient computes; see DenseBins::gh_lane)
+void launch_gh_words(hipStream_t s, int objective, int n, const float *y, const float *yp, unsigned *words);
 // scratch: row_blocks(n) doubles
 void launch_metric(hipStream_t s, int objective_metric, int n, int num_class, const float *y, const float *yp,
                    double *scratch, float *out);

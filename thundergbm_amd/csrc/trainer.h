@@ -95,6 +95,13 @@ class Trainer {
     int n_ = 0, F_ = 0, n_bins_ = 0;
     long nnz_ = 0;
     int objective_ = OBJ_SQUARE, metric_kind_ = 0;
+    // Dense layout with a spare dword at the end of every row's record, one tree per round, squared or binary logistic
+    // loss: the rows' gradient pairs also travel as one word in that dword (DenseBins::gh_lane), written by whatever
+    // computes the round's gradients (into an array of their own; the root level's histogram launch moves them).
+    int gh_word_lane_ = -1;
+    bool gh_words_fresh_ = false;   // d_gh_words_ matches d_gh_
+    bool gh_records_fresh_ = false;  // and the root level's histogram launch of this tree has copied it into the records
+    unsigned *d_gh_words_ = nullptr;  // [n]
     std::vector<void *> allocs_;
     // dataset
     float *d_y_ = nullptr;

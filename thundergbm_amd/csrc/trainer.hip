@@ -436,6 +436,19 @@ Trainer::Trainer(const DataSet &ds, GBMParam &param) {
         bins_.col = d_colmat;
         bins_.col_stride = col_stride;
         bins_.data = d_binmat_;
+        {
+            // (TGBM_GH_WORD=0: the histogram kernels always gather the pairs from the gradient array; tests)
+            const char *ge = std::getenv("TGBM_GH_WORD");
+            const bool off = ge != nullptr && std::string(ge) == "0";
+            const bool loss_ok = param.objective == "reg:linear" || param.objective == "binary:logistic";  // (labels 0 / 1)
+            if (!off && loss_ok && param.tree_per_rounds == 1 && bin_bytes == 1 && n_blocks == 1 && W >= 16 && P <= W - 4) {
+                gh_word_lane_ = W / 4 - 1;
+                bins_.gh_lane = gh_word_lane_;
+                d_gh_words_ = dalloc<unsigned>((size_t)n_);
+                bins_.gh_words = d_gh_words_;
+                log_info("gradient pairs ride in the spare bytes of the bin-matrix rows");
+            }
+        }
         HIP_CHECK(hipStreamSynchronize(stream_));
         HIP_CHECK(hipFree(d_val));
         HIP_CHECK(hipFree(d_col));
@@ -731,6 +744,11 @@ void Trainer::compute_gradient() {
     } else {
         launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
     }
+    gh_words_fresh_ = gh_records_fresh_ = false;
+    if (gh_word_lane_ >= 0 && !param_.bagging) {  // (bagging multiplies the pairs by draw counts)
+        launch_gh_words(stream_, objective_, n_, d_y_, d_yp_, d_gh_words_);
+        gh_words_fresh_ = true;
+    }
     if (param_.bagging) {
         const size_t N = (size_t)param_.num_class * n_;  // the whole gradient array, as in the reference
         TGBM_CHECK(N < ((size_t)1 << 31), "bagging: %zu gradient pairs exceed the int index range", N);
@@ -781,6 +799,7 @@ void Trainer::set_option(const std::string &key, double value) {
     } else if (key == "bagging") {
         param_.bagging = value != 0;
         next_round_ready_ = false;
+        gh_words_fresh_ = gh_records_fresh_ = false;
     } else {
         fatal("unknown trainer option %s", key.c_str());
     }
@@ -1004,8 +1023,14 @@ void Trainer::build_level_hist(const TreeBuffers &tb, int level, const GHPair *g
                             !in_boost_ && tb_.hist_q[0] != nullptr, n_class, level == param_.depth - 1);
     } else if (sparse_)
         launch_hist_csr(stream_, tb, csr_, gh, level, n_class);
-    else
-        launch_hist_dense(stream_, tb, bins_, gh, level, n_class);
+    else {
+        DenseBins b = bins_;
+        // (the root level's launch of a tree moves the words into the records; the levels below use them there)
+        if (level == 0) gh_records_fresh_ = gh_words_fresh_ && n_class == 1 && gh == d_gh_ && tb.lvl_x0 == 0;
+        b.gh_fresh = gh_records_fresh_ && n_class == 1 && gh == d_gh_;
+        b.gh_objective = objective_;
+        launch_hist_dense(stream_, tb, b, gh, level, n_class);
+    }
 }
 
 void Trainer::partition(int level) { partition_sets(set_of(cur_class_), level, 1); }
@@ -1052,7 +1077,10 @@ void Trainer::finish_tree(int k, bool fuse_round_end) {
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
         launch_round_end(stream_, tb, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
-                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_, &param_.gamma);
+                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_, &param_.gamma,
+                         d_gh_words_);
+        gh_words_fresh_ = d_gh_words_ != nullptr;
+        gh_records_fresh_ = false;  // (the records still hold the finished tree's words)
         next_round_ready_ = true;
     } else {
         launch_predict_in_training(stream_, tb, &bins_, &csr_, lookup_level_, d_yp_ + (size_t)k * n_,
@@ -1228,6 +1256,7 @@ void Trainer::reorder_rows() {
     lookup_level_ = -1;
     // gradients (of this or already of the next round) and their block statistics are in the old order
     next_round_ready_ = false;
+    gh_words_fresh_ = gh_records_fresh_ = false;
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
     ++reorders_done_;
 }
@@ -1384,6 +1413,12 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
     else fatal("unknown buffer %s", name.c_str());
     if (out != nullptr && cap >= bytes && bytes > 0) {
         HIP_CHECK(hipMemcpy(out, src, bytes, hipMemcpyDeviceToHost));
+        if (name == "binmat" && gh_word_lane_ >= 0) {
+            // (the records' spare dword carries the rows' gradient words: the matrix is handed out as bins only)
+            const size_t rb = (size_t)bins_.W;
+            unsigned char *m = static_cast<unsigned char *>(out);
+            for (int r = 0; r < n_; ++r) std::memset(m + (size_t)r * rb + rb - 4, kMissingBin, 4);
+        }
         // per-row buffers are handed out in the caller's row order, whatever the physical order is by now
         size_t row_bytes = 0, n_planes = 1;
         if (name == "nid" || name == "y") row_bytes = 4;
@@ -1417,7 +1452,7 @@ void Trainer::set(const std::string &name, const void *in, size_t bytes) {
     rank_order_fresh_ = false;
     void *dst = nullptr;
     size_t want = 0;
-    if (name == "gh") dst = d_gh_, want = sizeof(GHPair) * (size_t)param_.num_class * n_;
+    if (name == "gh") dst = d_gh_, want = sizeof(GHPair) * (size_t)param_.num_class * n_, gh_words_fresh_ = gh_records_fresh_ = false;
     else if (name == "y_pred") dst = d_yp_, want = sizeof(float) * (size_t)n_yp_;
     else fatal("buffer %s cannot be set", name.c_str());
     TGBM_CHECK(bytes == want, "set %s: got %zu bytes, expected %zu", name.c_str(), bytes, want);

@@ -98,6 +98,39 @@ __global__ void k_gradient_pointwise(int objective, int n, const float *__restri
         gh[i] = pointwise_gradient(objective, y[i], yp[i]);
 }
 
+// The gradient pair of a row as one 32-bit word that rides in the spare bytes of the row's bin-matrix record
+// (DenseBins::gh_lane), so that a histogram work item that gathers a row gets its pair with the same memory request
+// instead of a second one. Whatever computes a round's gradients also leaves the words in an array of their own
+// (launch_gh_words, k_tree_end); the root level's histogram launch, which streams every record anyway, reads them
+// there and writes the records back with the word in place - whole records, so that memory sees full-sector writes
+// (4 bytes of every 32 written by themselves cost a read-modify-write per sector: 90 us per tree on 10 M rows). Squared loss: the gradient itself (the hessian is 1). Logistic loss with 0/1 labels: the
+// sigmoid s (never negative) with the label in the sign bit; pair_from_word repeats pointwise_gradient's operations on
+// s, so both give the same bits.
+__device__ __forceinline__ unsigned word_from_row(int objective, float yi, float p) {
+    if (objective == OBJ_SQUARE) return __float_as_uint(p - yi);
+    const float s = 1.f / (1.f + expf(-p));
+    return __float_as_uint(s) | (yi != 0.f ? 0x80000000u : 0u);
+}
+__device__ __forceinline__ GHPair pair_from_word(int objective, unsigned w) {
+    GHPair o;
+    if (objective == OBJ_SQUARE) {
+        o.g = __uint_as_float(w);
+        o.h = 1.f;
+    } else {
+        const float s = __uint_as_float(w & 0x7fffffffu);
+        const float yi = (w >> 31) ? 1.f : 0.f;
+        o.g = s - yi;
+        o.h = fmaxf(s * (1.f - s), 1e-16f);
+    }
+    return o;
+}
+
+__global__ void k_gh_words(int objective, int n, const float *__restrict__ y, const float *__restrict__ yp,
+                           unsigned *__restrict__ words) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+        words[i] = word_from_row(objective, y[i], yp[i]);
+}
+
 // Softmax: src/thundergbm/objective/multiclass_obj.cu:6-35 (class-major predictions and gradients,
 // hessian 2p(1-p)).
 __global__ void k_gradient_softmax(int n, int K, const float *__restrict__ y, const float *__restrict__ yp,
@@ -376,7 +409,10 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
 // (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
 // instead of two was measured: it halves the fetched bytes below the root, but the per-tree refresh of
 // the pairs costs what the gathers save.)
-template <int LPR, bool DIRECT, int BLK, int SLOTS, bool BIN16>
+// GHW: the rows' gradient pairs come from 32-bit words (word_from_row). Below the root the word sits in the last
+// dword of the row's record, which the row's last lane has loaded with the bins anyway: no second gather per row. The
+// root launch (DIRECT) reads the words from their own array and puts them there, storing every record back.
+template <int LPR, bool DIRECT, int BLK, int SLOTS, bool BIN16, bool GHW = false>
 __global__ __launch_bounds__(BLK) __attribute__((amdgpu_waves_per_eu(SLOTS <= 8 ? 8 : 4)))  // two 1024-thread groups per CU
 void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__ gh, int level, int n_pairs) {
     extern __shared__ unsigned long long lds[];
@@ -404,6 +440,8 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
     if (nb == 0) return;
     const int h_bits = quant->h_bits;
     const int flush_rows = quant->flush_rows;
+    const int gh_objective = bins.gh_objective;
+    const bool word_lane = bins.gh_lane >= 0 && (int)(threadIdx.x % LPR) == bins.gh_lane;
     // The item's node and rows: the same few look-ups in every lane (uniform addresses: scalar loads), so that the
     // first row loads can be issued before the barrier that publishes the LDS histogram's clearing.
     const int p = find_owner(hpair_begin, n_pairs, item);
@@ -463,7 +501,9 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             opk[u] = *reinterpret_cast<const unsigned *>(blk + ((unsigned)r[u] * (unsigned)ROWB + qoff));
-            os[u] = *reinterpret_cast<const GHPair *>(reinterpret_cast<const char *>(gh) + (unsigned)r[u] * 8u);
+            if (!GHW) os[u] = *reinterpret_cast<const GHPair *>(reinterpret_cast<const char *>(gh) + (unsigned)r[u] * 8u);
+            if (GHW && DIRECT)  // (the word travels in the pair's first slot)
+                os[u].g = __uint_as_float(*reinterpret_cast<const unsigned *>(reinterpret_cast<const char *>(bins.gh_words) + (unsigned)r[u] * 4u));
         }
     };
     constexpr int STEP = RPS * U;
@@ -505,10 +545,23 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         pending += step_rows;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const unsigned v = (base + rsub + u * RPS < end) ? pk[u] : 0xffffffffu;  // (a clamped position adds nothing)
+            unsigned v = (base + rsub + u * RPS < end) ? pk[u] : 0xffffffffu;  // (a clamped position adds nothing)
+            GHPair sv = s[u];
+            if (GHW && DIRECT) {
+                const unsigned w = __float_as_uint(s[u].g);
+                sv = pair_from_word(gh_objective, w);
+                // the record goes back with the word in its last dword (whole records: full-sector writes)
+                const int pos = base + rsub + u * RPS;
+                if (pos < end)
+                    *reinterpret_cast<unsigned *>(const_cast<uint8_t *>(blk) + ((unsigned)pos * (unsigned)ROWB + qoff)) = word_lane ? w : pk[u];
+            } else if (GHW) {
+                // the row's last lane holds the word: every lane of the row takes it from there
+                sv = pair_from_word(gh_objective, (unsigned)__shfl((int)pk[u], (int)(threadIdx.x & 63u) | (LPR - 1)));
+            }
+            if (word_lane) v = 0xffffffffu;  // (that lane's dword holds no bins, whether the word is used or not)
             // exact products (the scales are powers of two), rounded once to the nearest integer
-            const long long gq = round_to_ll(s[u].g * scale_g);
-            const long long hq = round_to_ll(fmaxf(s[u].h, 0.f) * scale_h);
+            const long long gq = round_to_ll(sv.g * scale_g);
+            const long long hq = round_to_ll(fmaxf(sv.h, 0.f) * scale_h);
             const unsigned long long add = ((unsigned long long)gq << h_bits) + (unsigned long long)hq;
             if (BIN16) {
                 const unsigned b0 = v & 0xffff, b1 = v >> 16;
@@ -525,7 +578,7 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             pk[u] = pk_next[u];
-            s[u] = s_next[u];
+            if (!GHW || DIRECT) s[u] = s_next[u];
         }
     }
     __syncthreads();
@@ -1875,6 +1928,7 @@ struct TreeEndArgs {
     double *metric_partial;
     int with_prune;  // prune the tree first (prune_self with `gamma`)
     float gamma;
+    unsigned *gh_words;  // MODE 2: where the rows' gradient words go (word_from_row; nullptr: nowhere)
 };
 
 constexpr int kEndInline = 8;                        // shorter sub-ranges are handled by the finding thread
@@ -2019,6 +2073,7 @@ __device__ __forceinline__ void tree_end_rows(const TreeBuffers &tb, const TreeE
                 metric_row(a.metric_kind, tb.n, 1, i, yi[u], yp, p[u], acc, accf);
                 const GHPair o = pointwise_gradient(a.objective, yi[u], p[u]);
                 gh[i] = o;
+                if (a.gh_words != nullptr) a.gh_words[i] = word_from_row(a.objective, yi[u], p[u]);
                 st.add(o);
             }
         }
@@ -2285,6 +2340,27 @@ static void hist_dense_launch(hipStream_t s, const TreeBuffers &tb, const DenseB
             opted = lds;
         }
     }
+    if constexpr (!BIN16 && LPR >= 4) {
+        if (bins.gh_lane >= 0 && bins.gh_fresh) {
+            if (lds > 64 * 1024) {
+                static size_t opted_w = 0;
+                if (lds > opted_w) {
+                    HIP_CHECK(hipFuncSetAttribute(
+                        reinterpret_cast<const void *>(&k_hist_dense<LPR, true, kHistBlock, SLOTS, BIN16, true>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                    HIP_CHECK(hipFuncSetAttribute(
+                        reinterpret_cast<const void *>(&k_hist_dense<LPR, false, kHistBlock, SLOTS, BIN16, true>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                    opted_w = lds;
+                }
+            }
+            if (level == 0)
+                k_hist_dense<LPR, true, kHistBlock, SLOTS, BIN16, true><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
+            else
+                k_hist_dense<LPR, false, kHistBlock, SLOTS, BIN16, true><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
+            return;
+        }
+    }
     if (level == 0)
         k_hist_dense<LPR, true, kHistBlock, SLOTS, BIN16><<<grid, kHistBlock, lds, s>>>(tb, bins, gh, level, n_pairs);
     else
@@ -2497,8 +2573,10 @@ void launch_predict_in_training(hipStream_t s, const TreeBuffers &tb, const Dens
 
 void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbins, const CsrBins *cbins,
                       int lookup_level, int objective, int metric_kind, const float *y, float *yp, float lr,
-                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma) {
+                      GHPair *gh, double *metric_scratch, float *metric_out, const float *prune_gamma,
+                      unsigned *gh_words) {
     TreeEndArgs a{};
+    a.gh_words = gh_words;
     a.with_prune = prune_gamma != nullptr;
     a.gamma = prune_gamma != nullptr ? *prune_gamma : 0.f;
     a.lookup_level = lookup_level;
@@ -2512,6 +2590,11 @@ void launch_round_end(hipStream_t s, const TreeBuffers &tb, const DenseBins *dbi
     a.metric_partial = metric_scratch;
     tree_end(s, tb, dbins, cbins, 2, a);
     k_metric_final<<<1, kBlock, 0, s>>>(metric_kind, tb.n, row_blocks(tb.n), metric_scratch, metric_out);
+}
+
+void launch_gh_words(hipStream_t s, int objective, int n, const float *y, const float *yp, unsigned *words) {
+    if (n <= 0) return;
+    k_gh_words<<<std::min(4096, (n + kBlock - 1) / kBlock), kBlock, 0, s>>>(objective, n, y, yp, words);
 }
 
 void launch_metric(hipStream_t s, int kind, int n, int num_class, const float *y, const float *yp, double *scratch,
