@@ -409,6 +409,17 @@ __global__ __launch_bounds__(kBlock) void k_tree_init(TreeBuffers tb_all, float 
 // (Packing each row's gradient pair next to its bins so that a gathered row costs one 128-byte line
 // instead of two was measured: it halves the fetched bytes below the root, but the per-tree refresh of
 // the pairs costs what the gathers save.)
+// The value that the last of the LPR lanes of a row holds, in every lane of the row (LPR = 4, 8 or 16 consecutive
+// lanes): a DPP broadcast inside the 16-lane row of the wavefront, no trip through the LDS crossbar.
+template <int LPR>
+__device__ __forceinline__ unsigned last_lane_of_row(unsigned v) {
+    if (LPR == 4) return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0xff, 0xf, 0xf, false);  // quad_perm:[3,3,3,3]
+    const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x15f, 0xf, 0xf, false);  // row_newbcast:15
+    if (LPR == 16) return hi;
+    const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x157, 0xf, 0xf, false);  // row_newbcast:7
+    return (threadIdx.x & 8u) ? hi : lo;
+}
+
 // GHW: the rows' gradient pairs come from 32-bit words (word_from_row). Below the root the word sits in the last
 // dword of the row's record, which the row's last lane has loaded with the bins anyway: no second gather per row. The
 // root launch (DIRECT) reads the words from their own array and puts them there, storing every record back.
@@ -547,16 +558,16 @@ void k_hist_dense(TreeBuffers tb_all, DenseBins bins, const GHPair *__restrict__
         for (int u = 0; u < U; ++u) {
             unsigned v = (base + rsub + u * RPS < end) ? pk[u] : 0xffffffffu;  // (a clamped position adds nothing)
             GHPair sv = s[u];
-            if (GHW && DIRECT) {
+            if constexpr (GHW && DIRECT) {
                 const unsigned w = __float_as_uint(s[u].g);
                 sv = pair_from_word(gh_objective, w);
                 // the record goes back with the word in its last dword (whole records: full-sector writes)
                 const int pos = base + rsub + u * RPS;
                 if (pos < end)
                     *reinterpret_cast<unsigned *>(const_cast<uint8_t *>(blk) + ((unsigned)pos * (unsigned)ROWB + qoff)) = word_lane ? w : pk[u];
-            } else if (GHW) {
+            } else if constexpr (GHW) {
                 // the row's last lane holds the word: every lane of the row takes it from there
-                sv = pair_from_word(gh_objective, (unsigned)__shfl((int)pk[u], (int)(threadIdx.x & 63u) | (LPR - 1)));
+                sv = pair_from_word(gh_objective, last_lane_of_row<LPR>(pk[u]));
             }
             if (word_lane) v = 0xffffffffu;  // (that lane's dword holds no bins, whether the word is used or not)
             // exact products (the scales are powers of two), rounded once to the nearest integer
