@@ -1178,7 +1178,7 @@ def test_sparse_level_pass_at_its_deepest_level(T):
 
 
 @pytest.mark.parametrize("objective", ["reg:linear", "binary:logistic"])
-@pytest.mark.parametrize("F,reorder", [(28, "0"), (28, "always"), (12, "0"), (20, "always")])
+@pytest.mark.parametrize("F,reorder", [(28, "0"), (28, "always"), (12, "0"), (20, "always"), (40, "0"), (60, "always")])
 def test_gradient_words_in_the_bin_matrix_give_the_same_bits(T, objective, F, reorder):
     """With a spare dword at the end of a row's bin-matrix record (features <= row bytes - 4), one tree per round and a
     squared or 0/1-label logistic loss, the histogram kernels take a row's gradient pair from a 32-bit word stored in
@@ -1203,6 +1203,7 @@ def test_gradient_words_in_the_bin_matrix_give_the_same_bits(T, objective, F, re
             os.environ["TGBM_GH_WORD"] = word
             s = T.Session(val, rp, col, y, **kw)
             assert s.info("sparse") == 0 and s.info("dense_blocks") == 1
+            assert s.info("gh_word_lane") == (s.info("dense_W") // 4 - 1 if word == "1" else -1)
             s.boost(4)
             out = [s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()]
             # a level by hand with the round's own gradients, then with uploaded ones

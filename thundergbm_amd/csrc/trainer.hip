@@ -1354,6 +1354,7 @@ int Trainer::info(const std::string &key) const {
     if (key == "wide_eval") return wide_eval_ ? 1 : 0;
     if (key == "row_lists") return sparse_pass_ ? 0 : 1;  // the sparse level pass keeps a row -> node map only
     if (key == "dense_W") return bins_.W;
+    if (key == "gh_word_lane") return gh_word_lane_;  // dword of a row's record that carries its gradient word, -1: none
     if (key == "dense_cols") return sparse_ ? 0 : bins_.n_cols;  // columns of the bin matrix (fewer than features: bundles)
     if (key == "dense_bin_bytes") return sparse_ ? 0 : bins_.bin_bytes;
     if (key == "reorders_done") return reorders_done_;
