@@ -1206,7 +1206,13 @@ def test_gradient_words_in_the_bin_matrix_give_the_same_bits(T, objective, F, re
             assert s.info("gh_word_lane") == (s.info("dense_W") // 4 - 1 if word == "1" else -1)
             s.boost(4)
             out = [s.model().tobytes(), s.y_pred().tobytes(), s.nid().tobytes()]
-            # a level by hand with the round's own gradients, then with uploaded ones
+            # the next round's pairs (inside boost() they may exist as words only: the getter has them recomputed)
+            # and its root level by hand, started from what the fused end of the last round left
+            s.tree_init()
+            s.find_split(0)
+            out.append(s.gh().tobytes())
+            out.append(s.level_hist(0).tobytes())
+            # a level by hand with freshly computed gradients, then with uploaded ones
             s.gradient()
             s.tree_init()
             s.find_split(0)
@@ -1222,5 +1228,5 @@ def test_gradient_words_in_the_bin_matrix_give_the_same_bits(T, objective, F, re
     finally:
         for k in ("TGBM_GH_WORD", "TGBM_REORDER", "TGBM_LAYOUT"):
             os.environ.pop(k, None)
-    assert [a == b for a, b in zip(*runs)] == [True] * 5
-    assert runs[0][3] != runs[0][4]  # the uploaded gradients were used
+    assert [a == b for a, b in zip(*runs)] == [True] * 7
+    assert runs[0][4] == runs[0][5] and runs[0][5] != runs[0][6]  # the uploaded gradients were used

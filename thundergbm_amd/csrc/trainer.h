@@ -102,6 +102,12 @@ class Trainer {
     bool gh_words_fresh_ = false;   // d_gh_words_ matches d_gh_
     bool gh_records_fresh_ = false;  // and the root level's histogram launch of this tree has copied it into the records
     unsigned *d_gh_words_ = nullptr;  // [n]
+    // Inside boost() the fused end of a round leaves the next gradients as words only when nothing of the next tree
+    // reads the pair array (the histogram kernels take the words, the root's sums come from a complete feature's
+    // bins, the tree's scales from the pass's own statistics); whoever wants the array then - the stage-wise API, a
+    // getter - has it recomputed from the predictions first (the same kernel, the same values).
+    bool gh_array_stale_ = false;
+    void ensure_gh_array();
     std::vector<void *> allocs_;
     // dataset
     float *d_y_ = nullptr;

@@ -736,6 +736,7 @@ void Trainer::mark(int phase, int level) {
 // bagging when it is switched on.
 void Trainer::compute_gradient() {
     next_round_ready_ = false;
+    gh_array_stale_ = false;  // (recomputed below)
     if (objective_ == OBJ_RANK) {
         // the round's partner draws hang off the process-wide rand(), which is what the reference seeds its
         // per-group generators from (ranking_obj.cpp:53): srand() makes a run repeatable
@@ -797,6 +798,7 @@ void Trainer::set_option(const std::string &key, double value) {
     } else if (key == "reorder_min_rows") {
         reorder_min_rows_ = (long)value;
     } else if (key == "bagging") {
+        ensure_gh_array();
         param_.bagging = value != 0;
         next_round_ready_ = false;
         gh_words_fresh_ = gh_records_fresh_ = false;
@@ -809,6 +811,7 @@ void Trainer::set_option(const std::string &key, double value) {
 TreeBuffers Trainer::set_of(int k) const { return tb_.for_class(n_sets_ > 1 ? k : 0); }
 
 void Trainer::tree_init(int k) {
+    if (!in_boost_) ensure_gh_array();
     cur_class_ = k;
     HIP_CHECK_LAUNCHES("the stages before tree_init");  // gradients, bagging, column sampling, metric, re-ordering
     launch_tree_init(stream_, set_of(k), d_gh_ + (size_t)k * n_, param_.lambda, next_round_ready_);
@@ -817,7 +820,14 @@ void Trainer::tree_init(int k) {
     nid_materialized_ = false;
 }
 
+void Trainer::ensure_gh_array() {
+    if (!gh_array_stale_) return;
+    launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
+    gh_array_stale_ = false;
+}
+
 void Trainer::find_split(int level) {
+    if (!in_boost_) ensure_gh_array();
     if (sparse_pass_ && !in_boost_) ensure_hist_arena();
     find_split_sets(set_of(cur_class_), d_gh_ + (size_t)cur_class_ * n_, level, 1);
 }
@@ -1076,9 +1086,12 @@ void Trainer::finish_tree(int k, bool fuse_round_end) {
     // (the tree is pruned by a workgroup of the same launches)
     if (fuse_round_end) {
         // one tree per round: prediction update + metric + next gradients + their statistics in one pass
+        // (see gh_array_stale_: inside boost() the next tree may need the words only)
+        const bool words_only = in_boost_ && d_gh_words_ != nullptr && tb.complete_feature >= 0;
         launch_round_end(stream_, tb, &bins_, &csr_, lookup_level_, objective_, metric_kind_, d_y_, d_yp_,
-                         param_.learning_rate, d_gh_, d_metric_scratch_, d_metric_ + rounds_done_, &param_.gamma,
-                         d_gh_words_);
+                         param_.learning_rate, words_only ? nullptr : d_gh_, d_metric_scratch_, d_metric_ + rounds_done_,
+                         &param_.gamma, d_gh_words_);
+        gh_array_stale_ = words_only;
         gh_words_fresh_ = d_gh_words_ != nullptr;
         gh_records_fresh_ = false;  // (the records still hold the finished tree's words)
         next_round_ready_ = true;
@@ -1257,6 +1270,7 @@ void Trainer::reorder_rows() {
     // gradients (of this or already of the next round) and their block statistics are in the old order
     next_round_ready_ = false;
     gh_words_fresh_ = gh_records_fresh_ = false;
+    gh_array_stale_ = false;  // (recomputed here)
     launch_gradient(stream_, objective_, n_, param_.num_class, d_y_, d_yp_, d_gh_, nullptr, 0);
     ++reorders_done_;
 }
@@ -1392,7 +1406,11 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
         sync();
         src = cur.nid, bytes = sizeof(int) * (size_t)n_;
     }
-    else if (name == "gh") src = d_gh_, bytes = sizeof(GHPair) * (size_t)param_.num_class * n_;
+    else if (name == "gh") {
+        ensure_gh_array();
+        sync();
+        src = d_gh_, bytes = sizeof(GHPair) * (size_t)param_.num_class * n_;
+    }
     else if (name == "y_pred") src = d_yp_, bytes = sizeof(float) * (size_t)n_yp_;
     else if (name == "y") src = d_y_, bytes = sizeof(float) * (size_t)n_;
     else if (name == "nodes") src = cur.nodes, bytes = sizeof(TreeNode) * (size_t)tb_.n_nodes;
@@ -1448,6 +1466,8 @@ size_t Trainer::get(const std::string &name, void *out, size_t cap) {
 }
 
 void Trainer::set(const std::string &name, const void *in, size_t bytes) {
+    if (name == "gh") gh_array_stale_ = false;  // (overwritten below)
+    else ensure_gh_array();                      // (the pairs of the predictions as they are now)
     sync();
     next_round_ready_ = false;
     rank_order_fresh_ = false;

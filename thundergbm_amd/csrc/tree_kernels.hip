@@ -2083,7 +2083,7 @@ __device__ __forceinline__ void tree_end_rows(const TreeBuffers &tb, const TreeE
             if (MODE == 2) {
                 metric_row(a.metric_kind, tb.n, 1, i, yi[u], yp, p[u], acc, accf);
                 const GHPair o = pointwise_gradient(a.objective, yi[u], p[u]);
-                gh[i] = o;
+                if (gh != nullptr) gh[i] = o;  // (nullptr: the next tree reads the words only)
                 if (a.gh_words != nullptr) a.gh_words[i] = word_from_row(a.objective, yi[u], p[u]);
                 st.add(o);
             }
