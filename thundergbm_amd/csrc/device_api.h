@@ -226,7 +226,7 @@ struct TreeBuffers {
     int2 *seg = nullptr;           // [n_nodes] row-list segment [x, y) of every node
     int *nid = nullptr;            // [n]
     int *ridx[2] = {nullptr, nullptr};  // [n] row lists, ping-pong by level parity
-    uint8_t *goes_right = nullptr; // [n]
+    uint8_t *goes_right = nullptr; // [max_pitems * 256] per partition item and thread: bit k = its k-th row goes right
     longlong2 *hist_q[2] = {nullptr, nullptr};  // [max_level_nodes * n_bins] exact fixed-point histograms (g, h)
                                                 // of the nodes of a level, ping-pong by level parity
     longlong2 *partial = nullptr;  // [max_hitems * n_bins] per-item fixed-point sums (g, h)
@@ -324,7 +324,7 @@ struct TreeBuffers {
         t.nid += K * n;
         t.ridx[0] += K * n;
         t.ridx[1] += K * n;
-        t.goes_right += K * ((size_t)n + 4);
+        t.goes_right += K * (size_t)max_pitems * 256;
         t.hist_q[0] += K * hist_nodes * n_bins;
         t.hist_q[1] += K * hist_nodes * n_bins;
         t.partial += K * n_partial;

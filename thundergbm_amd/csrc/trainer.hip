@@ -567,7 +567,7 @@ void Trainer::alloc_tree_buffers() {
     tb.nid = dalloc<int>(S * n_);
     tb.ridx[0] = dalloc<int>(S * n_);
     tb.ridx[1] = dalloc<int>(S * n_);
-    tb.goes_right = dalloc<uint8_t>(S * ((size_t)n_ + 4));
+    tb.goes_right = dalloc<uint8_t>(S * (size_t)tb.max_pitems * 256);
     if (!sparse_pass_) {
         tb.hist_q[0] = dalloc<longlong2>(S * (size_t)hist_nodes * n_bins_);
         tb.hist_q[1] = dalloc<longlong2>(S * (size_t)hist_nodes * n_bins_);

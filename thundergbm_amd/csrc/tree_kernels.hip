@@ -994,16 +994,18 @@ __global__ __launch_bounds__(kBlock) void k_part_count_csr(TreeBuffers tb_all, C
     const int sbid = cb + (tb.split_bin != nullptr ? tb.split_bin[off + x_in] : (int)nd.split_bid);
     const bool dr = nd.default_right;
     int nleft = 0;
+    unsigned rights = 0;
 #pragma unroll
     for (int k = 0; k < kPartChunk / kBlock; ++k) {
         int pos = pb + k * kBlock + threadIdx.x;
         if (pos < pe) {
             int row = DIRECT ? pos : ridx[pos];
             bool right = csr_goes_right(bins, row, cb, ce, sbid, dr);
-            tb.goes_right[pos] = right ? 1 : 0;
+            rights |= (right ? 1u : 0u) << k;
             nleft += right ? 0 : 1;
         }
     }
+    tb.goes_right[(size_t)item * kBlock + threadIdx.x] = (uint8_t)rights;  // (see k_part_count_dense)
     int tot = block_sum(nleft, lds);
     if (threadIdx.x == 0) tb.pitem_nleft[item] = tot;
 }
@@ -1539,11 +1541,9 @@ __global__ __launch_bounds__(kBlock) void k_part_count_dense(TreeBuffers tb_all,
         rights |= (right ? 1u : 0u) << k;
         if (pb + k * kBlock + (int)threadIdx.x < pe) nleft += right ? 0 : 1;
     }
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-        const int pos = pb + k * kBlock + threadIdx.x;
-        if (pos < pe) tb.goes_right[pos] = (uint8_t)((rights >> k) & 1u);
-    }
+    // the decisions of a thread's eight rows as one byte (k_part_scatter gives the same rows to the same thread)
+    static_assert(R <= 8, "a byte per thread holds the decisions of its rows");
+    tb.goes_right[(size_t)item * kBlock + threadIdx.x] = (uint8_t)rights;
     int tot = block_sum(nleft, lds);
     if (threadIdx.x == 0) tb.pitem_nleft[item] = tot;
 }
@@ -1821,12 +1821,11 @@ __global__ __launch_bounds__(kBlock) void k_part_scatter(TreeBuffers tb_all, int
     // eight steps, then all stores
     constexpr int R = kPartChunk / kBlock;
     int row[R];
-    unsigned rights = 0;
+    const unsigned rights = tb.goes_right[(size_t)item * kBlock + threadIdx.x];  // bit k: the thread's k-th row goes right
 #pragma unroll
     for (int k = 0; k < R; ++k) {
         const int pos = min(pb + k * kBlock + (int)threadIdx.x, pe - 1);
         row[k] = DIRECT ? pos : ridx_cur[pos];
-        rights |= (tb.goes_right[pos] != 0 ? 1u : 0u) << k;
     }
 #pragma unroll
     for (int k = 0; k < R; ++k) {
