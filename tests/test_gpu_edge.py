@@ -100,8 +100,12 @@ CASES = {
     # candidate and may fall either way within the 1e-5 tolerance; found by random-shape testing.
     "softmax_direction_near_tie_16_bit_bins": (4097, 8, 2, "multi:softmax", "multi", dict(depth=6, max_num_bin=8), "dense-16"),
     "softmax_direction_near_tie": (4097, 8, 2, "multi:softmax", "multi", dict(depth=6, max_num_bin=8), "dense"),
+    # five labels of both signs whose mean is a hundredth of their size: the base score's 1e-5 is relative to the
+    # labels, not to the mean (two float sums in different orders differ by 4e-7 here)
+    "labels_cancel_in_the_base_score": (5, 60, 47, "reg:linear", "reg", dict(depth=4, max_num_bin=255), "sparse-nohead"),
 }
-CASE_SEEDS = {"softmax_direction_near_tie_16_bit_bins": 31479, "softmax_direction_near_tie": 31479}
+CASE_SEEDS = {"softmax_direction_near_tie_16_bit_bins": 31479, "softmax_direction_near_tie": 31479,
+              "labels_cancel_in_the_base_score": 80436}
 
 
 @pytest.mark.parametrize("name", sorted(CASES))
@@ -198,7 +202,8 @@ def run_case(T, name, seed, margins=None):
     gb, _ = s.global_bin_ids(rp, col)
     assert np.array_equal(gb, o.bin_ids())
     assert np.array_equal(s.y(), o.y()) and np.array_equal(s.labels(), o.labels())
-    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7)
+    # (a mean of labels of both signs: like every other sum, 1e-5 of the terms' absolute values, not of the result)
+    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7 + 1e-5 * float(np.abs(y).mean()))
     present = np.zeros((n, s.F), bool)
     present[np.repeat(np.arange(n), np.diff(rp)), col] = True
     for r in range(rounds):

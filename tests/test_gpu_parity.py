@@ -169,7 +169,8 @@ def test_session_cuts_bins_base_score(T, name):
     assert s.num_class == o.num_class and s.tree_per_rounds == o.tree_per_rounds
     assert np.array_equal(s.labels(), o.labels())
     assert np.array_equal(s.y(), o.y())
-    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7)
+    # (a mean of labels of both signs: like every other sum, 1e-5 of the terms' absolute values, not of the result)
+    np.testing.assert_allclose(s.base_score, o.base_score, rtol=1e-5, atol=1e-7 + 1e-5 * float(np.abs(y).mean()))
     np.testing.assert_allclose(s.y_pred(), o.y_pred(), rtol=1e-5, atol=1e-7)
     s.close()
 
