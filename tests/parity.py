@@ -186,7 +186,7 @@ def rows_in_node(final_nid, x):
 
 
 def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, abs_scale=None, rel=REL, mcw=1.0,
-                  orc_dir_gaps=None, few_missing_rows=0):
+                  orc_dir_gaps=None, few_missing_rows=0, gamma=1.0):
     """Top-down comparison of two heap-ordered trees (NODE_DTYPE arrays).
 
     Where both trees split on the same candidate everything must agree: threshold and bin exactly,
@@ -211,7 +211,11 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
     A choice that differs is also accepted as a near tie when one side's chosen split has a child whose
     hessian sum sits within dH of min_child_weight (mcw): that gate (hist_tree_builder_single.cu
     compute_gain: both children need h >= min_child_weight) flips on the last ulps of a sum, e.g. four
-    logistic rows with p = 0.5 give exactly 4 * 0.25 = 1.0 or one ulp less depending on the order.
+    logistic rows with p = 0.5 give exactly 4 * 0.25 = 1.0 or one ulp less depending on the order. The same gate
+    decides between the two default directions of one candidate (the direction whose child falls below it is not
+    a candidate), so a direction that differs on the gate is a near tie as well, whatever the two gains.
+    Pruning compares a node's gain with gamma (tree.cu:96-128): a node that only one side pruned is a near tie too
+    when its gain is within its tolerance of gamma (the flags and final ids of the trees are then not compared).
     orc_scores: [n_nodes, n_bins] signed candidate gains of the oracle, or a FullScores / ProbeScores view of them
     (None forbids any mismatch); crp: cut_row_ptr, to turn (feature, local bin) into a global candidate index.
     """
@@ -229,6 +233,14 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
         if o["lch"] >= 0:
             ws += [float(orc[o["lch"]]["base_weight"]), float(orc[o["rch"]]["base_weight"])]
         return gain_tolerance(ws, o["gain"], dG, dH, rel)
+
+    def on_mcw_gate(x, split_g, split_o):
+        on_gate = False
+        for t, has in ((gpu, split_g), (orc, split_o)):
+            if has:
+                hmin = min(float(t[int(t[x]["lch"])]["sum_h"]), float(t[int(t[x]["rch"])]["sum_h"]))
+                on_gate |= abs(hmin - mcw) <= dH
+        return on_gate
 
     while stack:
         x = stack.pop()
@@ -252,11 +264,16 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
         if split_g and split_o and g["split_fid"] == o["split_fid"] and g["split_bid"] == o["split_bid"]:
             assert g["split_value"] == o["split_value"], "node %d threshold differs" % x
             gt = gain_tol(x, o)
-            assert abs(g["gain"] - o["gain"]) <= gt, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
-            diff.worst["gain"] = max(diff.worst["gain"], abs(float(g["gain"]) - float(o["gain"])) / gt)
             n_missing = 0
             if g["default_right"] != o["default_right"] and missing_rows is not None:
                 n_missing = missing_rows(x, int(o["split_fid"]))
+            if n_missing > 0 and on_mcw_gate(x, True, True):
+                diff.near_ties.append((x, float("nan"), float("nan"), 0.0))
+                continue
+            assert abs(g["gain"] - o["gain"]) <= gt, "node %d gain %g vs %g" % (x, g["gain"], o["gain"])
+            diff.worst["gain"] = max(diff.worst["gain"], abs(float(g["gain"]) - float(o["gain"])) / gt)
+            if bool(g["is_leaf"]) != bool(o["is_leaf"]) and abs(float(o["gain"]) - gamma) <= gt:  # pruned on one side
+                diff.near_ties.append((x, float(o["gain"]), float(o["gain"]), 0.0))
             if n_missing > 0:
                 gap = None
                 if view is not None and crp is not None:
@@ -277,11 +294,7 @@ def compare_trees(gpu, orc, lam, crp=None, orc_scores=None, missing_rows=None, a
             continue
         assert view is not None and crp is not None, "node %d: split differs (gpu f%d b%d, oracle f%d b%d)" % (
             x, g["split_fid"], g["split_bid"], o["split_fid"], o["split_bid"])
-        on_gate = False
-        for t, has in ((gpu, split_g), (orc, split_o)):
-            if has:
-                hmin = min(float(t[int(t[x]["lch"])]["sum_h"]), float(t[int(t[x]["rch"])]["sum_h"]))
-                on_gate |= abs(hmin - mcw) <= dH
+        on_gate = on_mcw_gate(x, split_g, split_o)
         best = view.best(x)
         tol = 2 * gain_tol(x, o)
         if split_g:

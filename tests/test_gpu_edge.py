@@ -103,9 +103,16 @@ CASES = {
     # five labels of both signs whose mean is a hundredth of their size: the base score's 1e-5 is relative to the
     # labels, not to the mean (two float sums in different orders differ by 4e-7 here)
     "labels_cancel_in_the_base_score": (5, 60, 47, "reg:linear", "reg", dict(depth=4, max_num_bin=255), "sparse-nohead"),
+    # a candidate whose right child's hessians add up to min_child_weight or one ulp less: with the three rows that
+    # lack the feature it passes the gate on either side, without them on one side only, so the two sides take
+    # different default directions with gains of 1.33 and 2.00
+    "default_direction_on_the_min_child_weight_gate": (700, 5, 5, "binary:logistic", "bin", dict(depth=11, max_num_bin=8), "sparse-nohead"),
+    # a node of gain 1.0000001 against 0.99999994 with gamma = 1: pruned on one side only
+    "gain_on_the_pruning_threshold": (4097, 7, 6, "binary:logistic", "bin", dict(depth=9, max_num_bin=33), "sparse-nohead"),
 }
 CASE_SEEDS = {"softmax_direction_near_tie_16_bit_bins": 31479, "softmax_direction_near_tie": 31479,
-              "labels_cancel_in_the_base_score": 80436}
+              "labels_cancel_in_the_base_score": 80436, "default_direction_on_the_min_child_weight_gate": 73303,
+              "gain_on_the_pruning_threshold": 71740}
 
 
 @pytest.mark.parametrize("name", sorted(CASES))
@@ -223,7 +230,7 @@ def run_case(T, name, seed, margins=None):
             ghk = np.abs(gh[k * n:(k + 1) * n].astype(np.float64)).sum(axis=0)
             d = P.compare_trees(model[r, k], o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(), orc_dir_gaps=o.tree_dir_gaps(),
                                 missing_rows=lambda x, f: int((~present[P.rows_in_node(final_nid, x), f]).sum()),
-                                abs_scale=(ghk[0], ghk[1]), mcw=kw.get("min_child_weight", 1.0))
+                                abs_scale=(ghk[0], ghk[1]), mcw=kw.get("min_child_weight", 1.0), gamma=kw.get("gamma", 1.0))
             clean &= not d.near_ties
             if margins is not None:
                 margins.add(d)

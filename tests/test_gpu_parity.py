@@ -329,7 +329,8 @@ def test_tree_lockstep(T, name):
         s.finish_tree(k)
         o.prune()
         o.predict_in_training(k)
-        d = P.compare_trees(s.nodes(), o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(), abs_scale=(ghk[0], ghk[1]))
+        d = P.compare_trees(s.nodes(), o.nodes(), lam, crp=crp, orc_scores=o.tree_scores(), abs_scale=(ghk[0], ghk[1]),
+                            gamma=kw["gamma"])
         assert not d.near_ties
         margins.add(d)
         sl = slice(k * n, (k + 1) * n)
